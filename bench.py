@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): RMSNorm bf16 over X[8192,4096]
+(f32 accumulate, eps 1e-6, learned scale) followed by a fused pointwise MUL —
+one `step` is one such launch through the C ABI with inputs resident in HBM.
+Buffer sets are rotated so the 256 MB Infinity Cache cannot serve the reads.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s over the timed wall-clock
+region; `roofline` prices the kernel's own average duration (HIP events on the
+launch stream) against the 8 TB/s HBM peak; `cpu_baseline` is the CPU oracle's
+restatement of the same op timed on this box's host cores over a bounded
+sample; `others` carries the remaining BASELINE configs (TFLOP/s or GB/s and
+fraction of their rooflines), measured the same way.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from fusilli_amd import capi, synth  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}
+
+
+def timed_loop(ctx, launch, steps, warmup):
+    """W untimed + K timed launches; returns (wall ms/step, event ms/step)."""
+    for i in range(warmup):
+        launch(i)
+    ctx.sync()
+    e0, e1 = ctx.event(), ctx.event()
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        launch(i)
+    e1.record()
+    ctx.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e1.elapsed_ms_since(e0) / steps
+    return wall_ms, ev_ms
+
+
+# ---------------------------------------------------------------------------
+# C2: RMSNorm + MUL
+# ---------------------------------------------------------------------------
+def rmsnorm_desc(rows, cols, mul_kind):
+    d = capi.NormDesc()
+    d.x = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.scale = capi.TensorDesc.make([1, cols], [cols, 1], capi.BFLOAT16)
+    d.y = capi.TensorDesc.make([rows, cols], [cols, 1], capi.FLOAT)
+    d.out = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.epsilon = 1e-6
+    if mul_kind == "scalar":
+        op = capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16, scalar=0.5)
+    else:
+        op = capi.epilogue_op(
+            capi.PW["MUL"], capi.BFLOAT16, operand_index=0,
+            operand=capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16))
+    d.epilogue = capi.make_epilogue([op])
+    return d
+
+
+def bench_rmsnorm(ctx, steps, warmup, mul_kind="scalar", sets=5):
+    rows, cols = 8192, 4096
+    d = rmsnorm_desc(rows, cols, mul_kind)
+    assert ctx.lib.fhip_norm_fwd_supported(d) == 2, "tuned row kernel not chosen"
+    n = rows * cols
+    scale = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(2, 1, cols, 1.0, 0.02)))
+    xs, gs, ys = [], [], []
+    for s in range(sets):
+        xs.append(ctx.to_device(synth.f32_to_bf16_bits(synth.normal(2, 10 + s, n))))
+        ys.append(ctx.alloc(n * 2))
+        if mul_kind == "full":
+            gs.append(ctx.to_device(synth.f32_to_bf16_bits(synth.normal(2, 50 + s, n))))
+
+    def launch(i):
+        j = i % sets
+        ctx.norm_fwd(d, xs[j], scale, None, ys[j],
+                     epilogue_operands=[gs[j]] if gs else ())
+
+    wall_ms, ev_ms = timed_loop(ctx, launch, steps, warmup)
+    algo_bytes = 2 * n * 2 + cols * 2 + (n * 2 if mul_kind == "full" else 0)
+    return {"wall_ms": wall_ms, "kernel_ms": ev_ms, "bytes": algo_bytes,
+            "gbs_wall": algo_bytes / wall_ms / 1e6,
+            "gbs_kernel": algo_bytes / ev_ms / 1e6,
+            "sets": sets}
+
+
+def cpu_baseline_rmsnorm(seconds_budget=12.0):
+    """The oracle's bf16 RMSNorm * scalar on the host cores over a row sample."""
+    from oracle import oracle
+    rows, cols = 1024, 4096
+    x = synth.f32_to_bf16_bits(synth.normal(2, 10, rows * cols)).reshape(rows, cols)
+    s = synth.f32_to_bf16_bits(synth.normal(2, 1, cols, 1.0, 0.02))
+    oracle.rmsnorm_bf16_baseline(x, s, 1e-6, 0.5)  # warm
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        oracle.rmsnorm_bf16_baseline(x, s, 1e-6, 0.5)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds_budget or reps >= 200:
+            break
+    nbytes = (2 * rows * cols * 2 + cols * 2) * reps
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s",
+            "cores": threads, "kind": "port",
+            "sample": f"{reps} passes over {rows}x{cols} bf16 rows "
+                      f"(1/8 of the workload's rows), OpenMP, {dt:.1f} s; "
+                      "reference IREE llvm-cpu path unavailable offline"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-others", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path "
+              "(no collectives, no sharding); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    ctx = capi.Context(0)
+    r = bench_rmsnorm(ctx, args.steps, args.warmup, "scalar")
+    line = {
+        "metric": "GB/s (norms) on 1 MI355X, % roofline",
+        "value": round(r["gbs_wall"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "RMSNorm bf16 X[8192,4096] eps=1e-6 scale[4096] "
+                               "+ fused pointwise MUL (scalar operand), "
+                               f"{r['sets']} rotating buffer sets",
+                   "device": ctx.arch()},
+        "roofline": {"bound": "hbm", "achieved": round(r["gbs_kernel"], 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(r["gbs_kernel"] / HBM_PEAK_GBS, 4),
+                     "traffic": None,
+                     "algorithmic_bytes_per_launch": r["bytes"],
+                     "kernel_us": round(r["kernel_ms"] * 1e3, 2)},
+    }
+    if not args.no_others:
+        others = {}
+        r2 = bench_rmsnorm(ctx, args.steps, args.warmup, "full")
+        others["rmsnorm_bf16_8192x4096_mul_full_operand"] = {
+            "value": round(r2["gbs_kernel"], 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(r2["gbs_kernel"] / HBM_PEAK_GBS, 4),
+            "kernel_us": round(r2["kernel_ms"] * 1e3, 2), "bytes": r2["bytes"]}
+        try:
+            import bench_configs
+            others.update(bench_configs.run_all(ctx, args.steps, args.warmup))
+        except ImportError:
+            pass
+        line["others"] = others
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_rmsnorm()
+    ctx.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

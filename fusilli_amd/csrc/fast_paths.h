@@ -1,0 +1,30 @@
+// Tuned gfx950 kernels behind the op entry points.  Each op has a predicate
+// (does the tuned kernel accept this descriptor?) and a launcher.  Launchers
+// assume the descriptor passed the entry point's validation.
+#ifndef FUSILLI_AMD_CSRC_FAST_PATHS_H
+#define FUSILLI_AMD_CSRC_FAST_PATHS_H
+
+#include "common.h"
+
+bool fhip_fast_matmul_applicable(const fhip_matmul_desc *d);
+int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
+                     const void *b, const DevEpilogue &epi, void *out);
+
+bool fhip_fast_conv_applicable(const fhip_conv_desc *d);
+int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
+                   const void *w, const DevEpilogue &epi, void *out);
+
+bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d);
+int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
+                   const void *k, const void *v, void *o);
+
+bool fhip_fast_norm_applicable(const fhip_norm_desc *d);
+int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
+                   const void *scale, const void *bias, const DevEpilogue &epi,
+                   void *out, void *mean, void *inv_variance);
+
+bool fhip_fast_reduce_applicable(const fhip_reduce_desc *d);
+int fhip_fast_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
+                     void *y);
+
+#endif // FUSILLI_AMD_CSRC_FAST_PATHS_H

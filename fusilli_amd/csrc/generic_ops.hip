@@ -1,0 +1,1008 @@
+// Generic strided kernels: one straightforward gfx950 kernel per op that accepts
+// every layout, broadcast and element type the descriptors can express.  They
+// keep the API surface honest; the MFMA / bandwidth-tuned kernels in the other
+// files take over for the shapes they support.  This file also holds the op
+// entry points of the C ABI, which choose between the two.
+#include "common.h"
+#include "fast_paths.h"
+
+namespace {
+
+struct Dims {
+  int32_t rank;
+  int64_t dim[FHIP_MAX_RANK];
+};
+
+__device__ __forceinline__ void unravel(int64_t lin, const Dims &s,
+                                        int64_t *coord) {
+  for (int r = s.rank - 1; r >= 0; --r) {
+    const int64_t d = s.dim[r];
+    coord[r] = lin % d;
+    lin /= d;
+  }
+}
+
+struct Strides {
+  int64_t s[FHIP_MAX_RANK];
+};
+
+__device__ __forceinline__ int64_t dot(const int64_t *coord, const Strides &st,
+                                       int rank) {
+  int64_t off = 0;
+  for (int r = 0; r < rank; ++r)
+    off += coord[r] * st.s[r];
+  return off;
+}
+
+Dims make_dims(const fhip_tensor_desc &t) {
+  Dims d{};
+  d.rank = t.rank;
+  for (int i = 0; i < t.rank; ++i)
+    d.dim[i] = t.dim[i];
+  return d;
+}
+
+Strides make_strides(const fhip_tensor_desc &t) {
+  Strides s{};
+  for (int i = 0; i < t.rank; ++i)
+    s.s[i] = t.dim[i] == 1 ? 0 : t.stride[i];
+  return s;
+}
+
+inline unsigned grid_for(int64_t n, int block) {
+  int64_t g = (n + block - 1) / block;
+  return (unsigned)g;
+}
+
+// --------------------------------------------------------------------------
+// matmul
+// --------------------------------------------------------------------------
+struct MatmulArgs {
+  Dims out;          // logical output dims [..., M, N]
+  Strides a, b, o;   // strides on output coords (batch dims broadcast -> 0)
+  int64_t a_k, b_k;  // K strides
+  int64_t K;
+  int32_t a_dt, b_dt, c_dt, o_dt;
+  DevEpilogue epi;
+};
+
+template <typename Acc>
+__global__ void generic_matmul_kernel(MatmulArgs g, const void *a,
+                                      const void *b, void *out,
+                                      int64_t total) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= total)
+    return;
+  int64_t coord[FHIP_MAX_RANK];
+  unravel(lin, g.out, coord);
+  const int rank = g.out.rank;
+  // a uses (batch..., m), b uses (batch..., n)
+  int64_t ao = 0, bo = 0;
+  for (int r = 0; r < rank; ++r) {
+    ao += coord[r] * g.a.s[r];
+    bo += coord[r] * g.b.s[r];
+  }
+  Acc acc = 0;
+  for (int64_t k = 0; k < g.K; ++k) {
+    const Acc av = fhip_load<Acc>(a, g.a_dt, ao + k * g.a_k);
+    const Acc bv = fhip_load<Acc>(b, g.b_dt, bo + k * g.b_k);
+    acc += av * bv;
+  }
+  double v = fhip_round_through<double>(g.c_dt, (double)acc);
+  v = fhip_apply_epilogue<double>(g.epi, v, coord);
+  fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
+}
+
+// --------------------------------------------------------------------------
+// convolution forward (cross-correlation, zero padding, groups = C / fC)
+// --------------------------------------------------------------------------
+struct ConvArgs {
+  Dims y;            // [N, K, out spatial...]
+  Strides x, w, o;   // strides of X [N,C,sp..], W [K,fC,fsp..], OUT [N,K,sp..]
+  int64_t x_dim[FHIP_MAX_RANK];
+  int64_t w_dim[FHIP_MAX_RANK];
+  int32_t spatial;
+  int64_t pad[3], str[3], dil[3];
+  int64_t groups;
+  int32_t x_dt, w_dt, y_dt, o_dt;
+  DevEpilogue epi;
+};
+
+__global__ void generic_conv_kernel(ConvArgs g, const void *x, const void *w,
+                                    void *out, int64_t total) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= total)
+    return;
+  int64_t coord[FHIP_MAX_RANK];
+  unravel(lin, g.y, coord);
+  const int sp = g.spatial;
+  const int64_t n = coord[0], k = coord[1];
+  const int64_t fC = g.w_dim[1];
+  const int64_t kPerGroup = g.y.dim[1] / g.groups;
+  const int64_t grp = k / kPerGroup;
+  int64_t fvol = 1;
+  for (int i = 0; i < sp; ++i)
+    fvol *= g.w_dim[2 + i];
+  float acc = 0.f;
+  for (int64_t fc = 0; fc < fC; ++fc) {
+    const int64_t c = grp * fC + fc;
+    for (int64_t f = 0; f < fvol; ++f) {
+      int64_t rem = f;
+      int64_t xo = n * g.x.s[0] + c * g.x.s[1];
+      int64_t wo = k * g.w.s[0] + fc * g.w.s[1];
+      bool inside = true;
+      for (int i = sp - 1; i >= 0; --i) {
+        const int64_t fd = g.w_dim[2 + i];
+        const int64_t fi = rem % fd;
+        rem /= fd;
+        const int64_t xi = coord[2 + i] * g.str[i] - g.pad[i] + fi * g.dil[i];
+        if (xi < 0 || xi >= g.x_dim[2 + i])
+          inside = false;
+        xo += xi * g.x.s[2 + i];
+        wo += fi * g.w.s[2 + i];
+      }
+      if (inside)
+        acc += fhip_load<float>(x, g.x_dt, xo) * fhip_load<float>(w, g.w_dt, wo);
+    }
+  }
+  float v = fhip_round_through<float>(g.y_dt, acc);
+  v = fhip_apply_epilogue<float>(g.epi, v, coord);
+  fhip_store<float>(out, g.o_dt, dot(coord, g.o, g.y.rank), v);
+}
+
+// --------------------------------------------------------------------------
+// SDPA forward: one wavefront per query row, online softmax over 64-key chunks
+// --------------------------------------------------------------------------
+struct SdpaArgs {
+  int64_t B, Hq, Hkv, Sq, Skv, D, Dv;
+  int64_t q[4], k[4], v[4], o[4], m[4]; // element strides (mask: broadcast->0)
+  int32_t q_dt, k_dt, v_dt, o_dt, m_dt;
+  int32_t has_mask, causal;
+  float scale;
+};
+
+__device__ __forceinline__ float wave_max(float v) {
+  for (int o = 32; o > 0; o >>= 1)
+    v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  for (int o = 32; o > 0; o >>= 1)
+    v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+constexpr int kSdpaMaxDvPerLane = 8; // Dv <= 512
+
+__global__ __launch_bounds__(64) void generic_sdpa_kernel(SdpaArgs g,
+                                                          const void *q,
+                                                          const void *k,
+                                                          const void *v,
+                                                          const void *mask,
+                                                          void *o) {
+  __shared__ float p_lds[64];
+  const int lane = threadIdx.x;
+  int64_t row = blockIdx.x;
+  const int64_t sq = row % g.Sq;
+  row /= g.Sq;
+  const int64_t h = row % g.Hq;
+  const int64_t b = row / g.Hq;
+  const int64_t hk = h / (g.Hq / g.Hkv);
+  const int64_t qo = b * g.q[0] + h * g.q[1] + sq * g.q[2];
+  const int64_t ko = b * g.k[0] + hk * g.k[1];
+  const int64_t vo = b * g.v[0] + hk * g.v[1];
+  const int64_t mo = b * g.m[0] + h * g.m[1] + sq * g.m[2];
+  float acc[kSdpaMaxDvPerLane];
+  for (int i = 0; i < kSdpaMaxDvPerLane; ++i)
+    acc[i] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  int64_t kv_end = g.Skv;
+  if (g.causal && sq + 1 < kv_end)
+    kv_end = sq + 1;
+  for (int64_t j0 = 0; j0 < kv_end; j0 += 64) {
+    const int64_t j = j0 + lane;
+    float s = -INFINITY;
+    if (j < kv_end) {
+      float d = 0.f;
+      for (int64_t e = 0; e < g.D; ++e)
+        d += fhip_load<float>(q, g.q_dt, qo + e * g.q[3]) *
+             fhip_load<float>(k, g.k_dt, ko + j * g.k[2] + e * g.k[3]);
+      s = d * g.scale;
+      if (g.has_mask) {
+        if (g.m_dt == FHIP_BOOLEAN) {
+          if (((const uint8_t *)mask)[mo + j * g.m[3]] == 0)
+            s = -INFINITY;
+        } else {
+          s += fhip_load<float>(mask, g.m_dt, mo + j * g.m[3]);
+        }
+      }
+    }
+    const float m_new = fmaxf(m_run, wave_max(s));
+    const float p = (m_new == -INFINITY) ? 0.f : __expf(s - m_new);
+    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m_run - m_new);
+    l_run = l_run * corr + wave_sum(p);
+    m_run = m_new;
+    __syncthreads();
+    p_lds[lane] = p;
+    __syncthreads();
+    const int64_t cnt = (kv_end - j0 < 64) ? (kv_end - j0) : 64;
+    for (int i = 0; i < kSdpaMaxDvPerLane; ++i) {
+      const int64_t dv = lane + 64 * i;
+      if (dv < g.Dv) {
+        float a = acc[i] * corr;
+        for (int64_t jj = 0; jj < cnt; ++jj)
+          a += p_lds[jj] *
+               fhip_load<float>(v, g.v_dt, vo + (j0 + jj) * g.v[2] + dv * g.v[3]);
+        acc[i] = a;
+      }
+    }
+  }
+  const int64_t oo = b * g.o[0] + h * g.o[1] + sq * g.o[2];
+  for (int i = 0; i < kSdpaMaxDvPerLane; ++i) {
+    const int64_t dv = lane + 64 * i;
+    if (dv < g.Dv)
+      fhip_store<float>(o, g.o_dt, oo + dv * g.o[3], acc[i] / l_run);
+  }
+}
+
+// --------------------------------------------------------------------------
+// RMSNorm / LayerNorm forward over all dims but dim 0
+// --------------------------------------------------------------------------
+struct NormArgs {
+  Dims x;           // logical dims of X
+  Strides xs, ss, bs, os;
+  int64_t inner;    // product of dims 1..
+  int32_t x_dt, s_dt, b_dt, y_dt, o_dt, stats_dt;
+  int32_t has_scale, has_bias, is_layernorm, emit_stats;
+  float eps;
+  DevEpilogue epi;
+};
+
+__device__ __forceinline__ float block_sum_256(float v, float *lds) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0)
+    lds[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < (int)(blockDim.x >> 6); ++i)
+    t += lds[i];
+  return t;
+}
+
+__global__ __launch_bounds__(256) void generic_norm_kernel(
+    NormArgs g, const void *x, const void *scale, const void *bias, void *out,
+    void *mean_out, void *rstd_out) {
+  __shared__ float lds[4];
+  const int64_t b = blockIdx.x;
+  Dims inner{};
+  inner.rank = g.x.rank;
+  inner.dim[0] = 1;
+  for (int r = 1; r < g.x.rank; ++r)
+    inner.dim[r] = g.x.dim[r];
+  int64_t coord[FHIP_MAX_RANK];
+  float mean = 0.f;
+  if (g.is_layernorm) {
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < g.inner; i += blockDim.x) {
+      unravel(i, inner, coord);
+      coord[0] = b;
+      s += fhip_load<float>(x, g.x_dt, dot(coord, g.xs, g.x.rank));
+    }
+    mean = block_sum_256(s, lds) / (float)g.inner;
+  }
+  float ss = 0.f;
+  for (int64_t i = threadIdx.x; i < g.inner; i += blockDim.x) {
+    unravel(i, inner, coord);
+    coord[0] = b;
+    const float d =
+        fhip_load<float>(x, g.x_dt, dot(coord, g.xs, g.x.rank)) - mean;
+    ss += d * d;
+  }
+  const float var = block_sum_256(ss, lds) / (float)g.inner;
+  const float rstd = 1.0f / sqrtf(var + g.eps);
+  if (g.emit_stats && threadIdx.x == 0) {
+    fhip_store<float>(mean_out, g.stats_dt, b, mean);
+    fhip_store<float>(rstd_out, g.stats_dt, b, rstd);
+  }
+  for (int64_t i = threadIdx.x; i < g.inner; i += blockDim.x) {
+    unravel(i, inner, coord);
+    coord[0] = b;
+    float v =
+        (fhip_load<float>(x, g.x_dt, dot(coord, g.xs, g.x.rank)) - mean) * rstd;
+    if (g.has_scale)
+      v *= fhip_load<float>(scale, g.s_dt, dot(coord, g.ss, g.x.rank));
+    if (g.has_bias)
+      v += fhip_load<float>(bias, g.b_dt, dot(coord, g.bs, g.x.rank));
+    v = fhip_round_through<float>(g.y_dt, v);
+    v = fhip_apply_epilogue<float>(g.epi, v, coord);
+    fhip_store<float>(out, g.o_dt, dot(coord, g.os, g.x.rank), v);
+  }
+}
+
+// --------------------------------------------------------------------------
+// reduction (keep-dim)
+// --------------------------------------------------------------------------
+struct ReduceArgs {
+  Dims y;        // output logical dims (1 where reduced)
+  Dims red;      // reduced extents per dim (1 where kept)
+  Strides xs, ys;
+  int64_t red_count;
+  int32_t x_dt, y_dt, mode;
+};
+
+template <typename CT>
+__device__ __forceinline__ CT red_identity(int mode) {
+  switch (mode) {
+  case FHIP_RED_MUL:
+  case FHIP_RED_MUL_NO_ZEROS:
+    return (CT)1;
+  case FHIP_RED_MIN:
+    return (CT)INFINITY;
+  case FHIP_RED_MAX:
+    return (CT)-INFINITY;
+  default:
+    return (CT)0;
+  }
+}
+
+template <typename CT>
+__device__ __forceinline__ CT red_map(int mode, CT v) {
+  switch (mode) {
+  case FHIP_RED_AMAX:
+  case FHIP_RED_NORM1:
+    return fabs(v);
+  case FHIP_RED_NORM2:
+    return v * v;
+  case FHIP_RED_MUL_NO_ZEROS:
+    return v == (CT)0 ? (CT)1 : v;
+  default:
+    return v;
+  }
+}
+
+template <typename CT>
+__device__ __forceinline__ CT red_combine(int mode, CT a, CT b) {
+  switch (mode) {
+  case FHIP_RED_MUL:
+  case FHIP_RED_MUL_NO_ZEROS:
+    return a * b;
+  case FHIP_RED_MIN:
+    return (a != a || b != b) ? (a != a ? a : b) : (a < b ? a : b);
+  case FHIP_RED_MAX:
+  case FHIP_RED_AMAX:
+    return (a != a || b != b) ? (a != a ? a : b) : (a > b ? a : b);
+  default:
+    return a + b;
+  }
+}
+
+template <typename CT>
+__global__ __launch_bounds__(256) void generic_reduce_kernel(ReduceArgs g,
+                                                             const void *x,
+                                                             void *y) {
+  __shared__ CT lds[256];
+  int64_t ocoord[FHIP_MAX_RANK], rcoord[FHIP_MAX_RANK];
+  unravel((int64_t)blockIdx.x, g.y, ocoord);
+  const int rank = g.y.rank;
+  const int64_t base = dot(ocoord, g.xs, rank);
+  CT acc = g.mode == FHIP_RED_AMAX ? (CT)0 : red_identity<CT>(g.mode);
+  for (int64_t i = threadIdx.x; i < g.red_count; i += blockDim.x) {
+    unravel(i, g.red, rcoord);
+    const CT v = fhip_load<CT>(x, g.x_dt, base + dot(rcoord, g.xs, rank));
+    acc = red_combine<CT>(g.mode, acc, red_map<CT>(g.mode, v));
+  }
+  lds[threadIdx.x] = acc;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s)
+      lds[threadIdx.x] =
+          red_combine<CT>(g.mode, lds[threadIdx.x], lds[threadIdx.x + s]);
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    CT r = lds[0];
+    if (g.mode == FHIP_RED_AVG)
+      r = r / (CT)g.red_count;
+    else if (g.mode == FHIP_RED_NORM2)
+      r = sqrt(r);
+    fhip_store<CT>(y, g.y_dt, dot(ocoord, g.ys, rank), r);
+  }
+}
+
+// --------------------------------------------------------------------------
+// pointwise
+// --------------------------------------------------------------------------
+struct PointwiseArgs {
+  Dims out;
+  Strides in[3], os;
+  int32_t in_dt[3], o_dt;
+  int32_t is_scalar[3];
+  double scalar[3];
+  int32_t mode, num_inputs;
+  fhip_pointwise_params params;
+};
+
+template <typename CT>
+__global__ void generic_pointwise_kernel(PointwiseArgs g, const void *in0,
+                                         const void *in1, const void *in2,
+                                         void *out, int64_t total) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= total)
+    return;
+  int64_t coord[FHIP_MAX_RANK];
+  unravel(lin, g.out, coord);
+  const int rank = g.out.rank;
+  const void *ptr[3] = {in0, in1, in2};
+  CT v[3] = {(CT)0, (CT)0, (CT)0};
+  for (int i = 0; i < g.num_inputs; ++i)
+    v[i] = g.is_scalar[i]
+               ? (CT)g.scalar[i]
+               : fhip_load<CT>(ptr[i], g.in_dt[i], dot(coord, g.in[i], rank));
+  CT r;
+  if (g.num_inputs == 1)
+    r = fhip_pw_unary<CT>(g.mode, v[0], g.params);
+  else if (g.num_inputs == 2)
+    r = fhip_pw_binary<CT>(g.mode, v[0], v[1], g.params);
+  else
+    r = (v[0] != (CT)0) ? v[1] : v[2]; // BINARY_SELECT = where(in0, in1, in2)
+  fhip_store<CT>(out, g.o_dt, dot(coord, g.os, rank), r);
+}
+
+bool needs_double(int dt) {
+  return dt == FHIP_DOUBLE || dt == FHIP_INT32 || dt == FHIP_INT64;
+}
+
+// Whether dims of `t` equal the given list.
+bool dims_equal(const fhip_tensor_desc &t, int rank, const int64_t *dims) {
+  if (t.rank != rank)
+    return false;
+  for (int i = 0; i < rank; ++i)
+    if (t.dim[i] != dims[i])
+      return false;
+  return true;
+}
+
+} // namespace
+
+extern "C" {
+
+// ---- matmul ---------------------------------------------------------------
+static int matmul_validate(fhip_ctx *ctx, const fhip_matmul_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_matmul: null descriptor");
+  if (!fhip_check_desc(ctx, d->a, "matmul A") ||
+      !fhip_check_desc(ctx, d->b, "matmul B") ||
+      !fhip_check_desc(ctx, d->c, "matmul C") ||
+      !fhip_check_desc(ctx, d->out, "matmul OUT"))
+    return 1;
+  const int r = d->a.rank;
+  FHIP_REQUIRE(ctx, r >= 2 && d->b.rank == r && d->c.rank == r &&
+                        d->out.rank == r,
+               "fhip_matmul: A, B, C and OUT must share a rank >= 2");
+  FHIP_REQUIRE(ctx, d->a.dim[r - 1] == d->b.dim[r - 2],
+               "fhip_matmul: K mismatch (%lld vs %lld)",
+               (long long)d->a.dim[r - 1], (long long)d->b.dim[r - 2]);
+  FHIP_REQUIRE(ctx,
+               d->c.dim[r - 2] == d->a.dim[r - 2] &&
+                   d->c.dim[r - 1] == d->b.dim[r - 1],
+               "fhip_matmul: C dims do not match M x N");
+  for (int i = 0; i < r - 2; ++i) {
+    const int64_t ad = d->a.dim[i], bd = d->b.dim[i], cd = d->c.dim[i];
+    const int64_t mx = ad > bd ? ad : bd;
+    FHIP_REQUIRE(ctx, (ad == bd || ad == 1 || bd == 1) && cd == mx,
+                 "fhip_matmul: batch dim %d (%lld x %lld -> %lld) is not a "
+                 "1-to-N broadcast",
+                 i, (long long)ad, (long long)bd, (long long)cd);
+  }
+  FHIP_REQUIRE(ctx, dims_equal(d->out, r, d->c.dim),
+               "fhip_matmul: OUT dims differ from C dims");
+  FHIP_REQUIRE(ctx, d->out.dtype == d->out_dtype,
+               "fhip_matmul: out_dtype disagrees with OUT descriptor");
+  return 0;
+}
+
+int fhip_matmul_workspace_size(const fhip_matmul_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_matmul_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_matmul_supported(const fhip_matmul_desc *d) {
+  if (!d || matmul_validate(nullptr, d) != 0)
+    return 0;
+  return fhip_fast_matmul_applicable(d) ? 2 : 1;
+}
+
+int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
+                const void *b, const void *const *epilogue_operands, void *out,
+                void *workspace, size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_matmul: null context");
+  if (matmul_validate(ctx, d) != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, a && b && out, "fhip_matmul: null tensor pointer");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  const int r = d->a.rank;
+  DevEpilogue epi;
+  if (fhip_build_epilogue(ctx, d->epilogue, r, d->c.dim, epilogue_operands,
+                          &epi) != 0)
+    return 1;
+  if (fhip_fast_matmul_applicable(d))
+    return fhip_fast_matmul(ctx, d, a, b, epi, out);
+
+  MatmulArgs g{};
+  g.out = make_dims(d->c);
+  for (int i = 0; i < r; ++i) {
+    g.a.s[i] = (i < r - 2) ? (d->a.dim[i] == 1 ? 0 : d->a.stride[i]) : 0;
+    g.b.s[i] = (i < r - 2) ? (d->b.dim[i] == 1 ? 0 : d->b.stride[i]) : 0;
+    g.o.s[i] = d->out.dim[i] == 1 ? 0 : d->out.stride[i];
+  }
+  g.a.s[r - 2] = d->a.stride[r - 2]; // m
+  g.b.s[r - 1] = d->b.stride[r - 1]; // n
+  g.a_k = d->a.stride[r - 1];
+  g.b_k = d->b.stride[r - 2];
+  g.K = d->a.dim[r - 1];
+  g.a_dt = d->a.dtype;
+  g.b_dt = d->b.dtype;
+  g.c_dt = d->c.dtype;
+  g.o_dt = d->out.dtype;
+  g.epi = epi;
+  const int64_t total = fhip_desc_volume(d->c);
+  const bool int_path = fhip_dtype_is_int(d->a.dtype) &&
+                        fhip_dtype_is_int(d->b.dtype);
+  if (int_path)
+    hipLaunchKernelGGL(generic_matmul_kernel<int32_t>, dim3(grid_for(total, 256)),
+                       dim3(256), 0, ctx->stream, g, a, b, out, total);
+  else
+    hipLaunchKernelGGL(generic_matmul_kernel<float>, dim3(grid_for(total, 256)),
+                       dim3(256), 0, ctx->stream, g, a, b, out, total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- conv fprop -----------------------------------------------------------
+static int conv_validate(fhip_ctx *ctx, const fhip_conv_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_conv_fprop: null descriptor");
+  if (!fhip_check_desc(ctx, d->x, "conv X") ||
+      !fhip_check_desc(ctx, d->w, "conv W") ||
+      !fhip_check_desc(ctx, d->y, "conv Y") ||
+      !fhip_check_desc(ctx, d->out, "conv OUT"))
+    return 1;
+  const int sp = d->spatial_rank;
+  FHIP_REQUIRE(ctx, sp >= 1 && sp <= 3, "fhip_conv_fprop: spatial rank %d", sp);
+  FHIP_REQUIRE(ctx,
+               d->x.rank == sp + 2 && d->w.rank == sp + 2 &&
+                   d->y.rank == sp + 2 && d->out.rank == sp + 2,
+               "fhip_conv_fprop: tensor ranks must equal spatial rank + 2");
+  const int64_t C = d->x.dim[1], fC = d->w.dim[1], K = d->w.dim[0];
+  FHIP_REQUIRE(ctx, fC > 0 && C % fC == 0,
+               "fhip_conv_fprop: input channels %lld not divisible by filter "
+               "channels %lld",
+               (long long)C, (long long)fC);
+  const int64_t groups = C / fC;
+  FHIP_REQUIRE(ctx, K % groups == 0,
+               "fhip_conv_fprop: output channels %lld not divisible by groups "
+               "%lld",
+               (long long)K, (long long)groups);
+  FHIP_REQUIRE(ctx, d->y.dim[0] == d->x.dim[0] && d->y.dim[1] == K,
+               "fhip_conv_fprop: Y batch/channel dims mismatch");
+  for (int i = 0; i < sp; ++i) {
+    FHIP_REQUIRE(ctx, d->stride[i] >= 1 && d->dilation[i] >= 1 &&
+                          d->padding[i] >= 0,
+                 "fhip_conv_fprop: invalid stride/dilation/padding");
+    const int64_t expect =
+        1 + (d->x.dim[2 + i] + 2 * d->padding[i] -
+             d->dilation[i] * (d->w.dim[2 + i] - 1) - 1) /
+                d->stride[i];
+    FHIP_REQUIRE(ctx, d->y.dim[2 + i] == expect,
+                 "fhip_conv_fprop: Y spatial dim %d is %lld, expected %lld", i,
+                 (long long)d->y.dim[2 + i], (long long)expect);
+  }
+  FHIP_REQUIRE(ctx, dims_equal(d->out, d->y.rank, d->y.dim),
+               "fhip_conv_fprop: OUT dims differ from Y dims");
+  FHIP_REQUIRE(ctx, d->out.dtype == d->out_dtype,
+               "fhip_conv_fprop: out_dtype disagrees with OUT descriptor");
+  return 0;
+}
+
+int fhip_conv_fprop_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_conv_fprop_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_conv_fprop_supported(const fhip_conv_desc *d) {
+  if (!d || conv_validate(nullptr, d) != 0)
+    return 0;
+  return fhip_fast_conv_applicable(d) ? 2 : 1;
+}
+
+int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
+                    const void *w, const void *const *epilogue_operands,
+                    void *out, void *workspace, size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_conv_fprop: null context");
+  if (conv_validate(ctx, d) != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, x && w && out, "fhip_conv_fprop: null tensor pointer");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  DevEpilogue epi;
+  if (fhip_build_epilogue(ctx, d->epilogue, d->y.rank, d->y.dim,
+                          epilogue_operands, &epi) != 0)
+    return 1;
+  if (fhip_fast_conv_applicable(d))
+    return fhip_fast_conv(ctx, d, x, w, epi, out);
+
+  ConvArgs g{};
+  g.y = make_dims(d->y);
+  g.x = make_strides(d->x);
+  g.w = make_strides(d->w);
+  g.o = make_strides(d->out);
+  for (int i = 0; i < d->x.rank; ++i) {
+    g.x_dim[i] = d->x.dim[i];
+    g.w_dim[i] = d->w.dim[i];
+  }
+  g.spatial = d->spatial_rank;
+  for (int i = 0; i < 3; ++i) {
+    g.pad[i] = d->padding[i];
+    g.str[i] = d->stride[i];
+    g.dil[i] = d->dilation[i];
+  }
+  g.groups = d->x.dim[1] / d->w.dim[1];
+  g.x_dt = d->x.dtype;
+  g.w_dt = d->w.dtype;
+  g.y_dt = d->y.dtype;
+  g.o_dt = d->out.dtype;
+  g.epi = epi;
+  const int64_t total = fhip_desc_volume(d->y);
+  hipLaunchKernelGGL(generic_conv_kernel, dim3(grid_for(total, 256)), dim3(256),
+                     0, ctx->stream, g, x, w, out, total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- sdpa -----------------------------------------------------------------
+static int sdpa_validate(fhip_ctx *ctx, const fhip_sdpa_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_sdpa_fwd: null descriptor");
+  if (!fhip_check_desc(ctx, d->q, "sdpa Q") ||
+      !fhip_check_desc(ctx, d->k, "sdpa K") ||
+      !fhip_check_desc(ctx, d->v, "sdpa V") ||
+      !fhip_check_desc(ctx, d->o, "sdpa O"))
+    return 1;
+  FHIP_REQUIRE(ctx,
+               d->q.rank == 4 && d->k.rank == 4 && d->v.rank == 4 &&
+                   d->o.rank == 4,
+               "fhip_sdpa_fwd: Q, K, V, O must be rank 4");
+  const int64_t B = d->q.dim[0], Hq = d->q.dim[1], Sq = d->q.dim[2],
+                D = d->q.dim[3];
+  const int64_t Hkv = d->k.dim[1], Skv = d->k.dim[2];
+  FHIP_REQUIRE(ctx, d->k.dim[0] == B && d->v.dim[0] == B,
+               "fhip_sdpa_fwd: batch mismatch");
+  FHIP_REQUIRE(ctx, d->k.dim[3] == D, "fhip_sdpa_fwd: Q/K head dim mismatch");
+  FHIP_REQUIRE(ctx, d->v.dim[1] == Hkv && d->v.dim[2] == Skv,
+               "fhip_sdpa_fwd: K/V head count or sequence mismatch");
+  FHIP_REQUIRE(ctx, Hkv > 0 && Hq % Hkv == 0,
+               "fhip_sdpa_fwd: Hq %lld not divisible by Hkv %lld",
+               (long long)Hq, (long long)Hkv);
+  const int64_t Dv = d->v.dim[3];
+  FHIP_REQUIRE(ctx,
+               d->o.dim[0] == B && d->o.dim[1] == Hq && d->o.dim[2] == Sq &&
+                   d->o.dim[3] == Dv,
+               "fhip_sdpa_fwd: O dims must be [B, Hq, Sq, Dv]");
+  FHIP_REQUIRE(ctx, Dv <= 64 * kSdpaMaxDvPerLane,
+               "fhip_sdpa_fwd: value head dim %lld above %d", (long long)Dv,
+               64 * kSdpaMaxDvPerLane);
+  if (d->mask.rank != 0) {
+    if (!fhip_check_desc(ctx, d->mask, "sdpa MASK"))
+      return 1;
+    FHIP_REQUIRE(ctx, !d->is_causal,
+                 "fhip_sdpa_fwd: mask and is_causal are mutually exclusive");
+    int64_t dims[4] = {B, Hq, Sq, Skv};
+    int64_t st[4];
+    FHIP_REQUIRE(ctx, fhip_broadcast_strides(d->mask, 4, dims, st),
+                 "fhip_sdpa_fwd: mask is not broadcastable to [B,Hq,Sq,Skv]");
+  }
+  return 0;
+}
+
+int fhip_sdpa_fwd_workspace_size(const fhip_sdpa_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_sdpa_fwd_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_sdpa_fwd_supported(const fhip_sdpa_desc *d) {
+  if (!d || sdpa_validate(nullptr, d) != 0)
+    return 0;
+  return fhip_fast_sdpa_applicable(d) ? 2 : 1;
+}
+
+int fhip_sdpa_fwd(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
+                  const void *k, const void *v, const void *mask, void *o,
+                  void *workspace, size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_sdpa_fwd: null context");
+  if (sdpa_validate(ctx, d) != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, q && k && v && o, "fhip_sdpa_fwd: null tensor pointer");
+  FHIP_REQUIRE(ctx, (d->mask.rank != 0) == (mask != nullptr),
+               "fhip_sdpa_fwd: mask pointer and mask descriptor disagree");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  if (fhip_fast_sdpa_applicable(d))
+    return fhip_fast_sdpa(ctx, d, q, k, v, o);
+
+  SdpaArgs g{};
+  g.B = d->q.dim[0];
+  g.Hq = d->q.dim[1];
+  g.Sq = d->q.dim[2];
+  g.D = d->q.dim[3];
+  g.Hkv = d->k.dim[1];
+  g.Skv = d->k.dim[2];
+  g.Dv = d->v.dim[3];
+  for (int i = 0; i < 4; ++i) {
+    g.q[i] = d->q.stride[i];
+    g.k[i] = d->k.stride[i];
+    g.v[i] = d->v.stride[i];
+    g.o[i] = d->o.stride[i];
+    g.m[i] = 0;
+  }
+  g.q_dt = d->q.dtype;
+  g.k_dt = d->k.dtype;
+  g.v_dt = d->v.dtype;
+  g.o_dt = d->o.dtype;
+  g.has_mask = d->mask.rank != 0;
+  g.causal = d->is_causal;
+  if (g.has_mask) {
+    int64_t dims[4] = {g.B, g.Hq, g.Sq, g.Skv};
+    fhip_broadcast_strides(d->mask, 4, dims, g.m);
+    g.m_dt = d->mask.dtype;
+  }
+  g.scale = d->has_scale ? d->scale : 1.0f / sqrtf((float)g.D);
+  const int64_t rows = g.B * g.Hq * g.Sq;
+  hipLaunchKernelGGL(generic_sdpa_kernel, dim3((unsigned)rows), dim3(64), 0,
+                     ctx->stream, g, q, k, v, mask, o);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- norms ----------------------------------------------------------------
+static int norm_validate(fhip_ctx *ctx, const fhip_norm_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_norm_fwd: null descriptor");
+  if (!fhip_check_desc(ctx, d->x, "norm X") ||
+      !fhip_check_desc(ctx, d->y, "norm Y") ||
+      !fhip_check_desc(ctx, d->out, "norm OUT"))
+    return 1;
+  FHIP_REQUIRE(ctx, d->x.rank >= 2, "fhip_norm_fwd: X rank must be >= 2");
+  FHIP_REQUIRE(ctx, dims_equal(d->y, d->x.rank, d->x.dim) &&
+                        dims_equal(d->out, d->x.rank, d->x.dim),
+               "fhip_norm_fwd: Y / OUT dims differ from X dims");
+  int64_t sdim[FHIP_MAX_RANK];
+  for (int i = 0; i < d->x.rank; ++i)
+    sdim[i] = i == 0 ? 1 : d->x.dim[i];
+  if (d->scale.rank != 0) {
+    if (!fhip_check_desc(ctx, d->scale, "norm SCALE"))
+      return 1;
+    FHIP_REQUIRE(ctx, dims_equal(d->scale, d->x.rank, sdim),
+                 "fhip_norm_fwd: SCALE dims must equal X dims with dim 0 = 1");
+  }
+  if (d->bias.rank != 0) {
+    FHIP_REQUIRE(ctx, d->is_layernorm, "fhip_norm_fwd: RMSNorm takes no bias");
+    if (!fhip_check_desc(ctx, d->bias, "norm BIAS"))
+      return 1;
+    FHIP_REQUIRE(ctx, dims_equal(d->bias, d->x.rank, sdim),
+                 "fhip_norm_fwd: BIAS dims must equal X dims with dim 0 = 1");
+  }
+  if (d->emit_stats)
+    FHIP_REQUIRE(ctx, d->is_layernorm && fhip_dtype_is_float(d->stats_dtype),
+                 "fhip_norm_fwd: statistics are a LayerNorm training output "
+                 "of floating type");
+  FHIP_REQUIRE(ctx, d->out.dtype == d->out_dtype,
+               "fhip_norm_fwd: out_dtype disagrees with OUT descriptor");
+  return 0;
+}
+
+int fhip_norm_fwd_workspace_size(const fhip_norm_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_norm_fwd_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_norm_fwd_supported(const fhip_norm_desc *d) {
+  if (!d || norm_validate(nullptr, d) != 0)
+    return 0;
+  return fhip_fast_norm_applicable(d) ? 2 : 1;
+}
+
+int fhip_norm_fwd(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
+                  const void *scale, const void *bias,
+                  const void *const *epilogue_operands, void *out, void *mean,
+                  void *inv_variance, void *workspace, size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_norm_fwd: null context");
+  if (norm_validate(ctx, d) != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, x && out, "fhip_norm_fwd: null tensor pointer");
+  FHIP_REQUIRE(ctx, (d->scale.rank != 0) == (scale != nullptr),
+               "fhip_norm_fwd: scale pointer and descriptor disagree");
+  FHIP_REQUIRE(ctx, (d->bias.rank != 0) == (bias != nullptr),
+               "fhip_norm_fwd: bias pointer and descriptor disagree");
+  FHIP_REQUIRE(ctx, !d->emit_stats || (mean && inv_variance),
+               "fhip_norm_fwd: statistics requested but pointers are null");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  DevEpilogue epi;
+  if (fhip_build_epilogue(ctx, d->epilogue, d->x.rank, d->x.dim,
+                          epilogue_operands, &epi) != 0)
+    return 1;
+  if (fhip_fast_norm_applicable(d))
+    return fhip_fast_norm(ctx, d, x, scale, bias, epi, out, mean, inv_variance);
+
+  NormArgs g{};
+  g.x = make_dims(d->x);
+  g.xs = make_strides(d->x);
+  g.os = make_strides(d->out);
+  if (d->scale.rank)
+    g.ss = make_strides(d->scale);
+  if (d->bias.rank)
+    g.bs = make_strides(d->bias);
+  g.inner = fhip_desc_volume(d->x) / d->x.dim[0];
+  g.x_dt = d->x.dtype;
+  g.s_dt = d->scale.dtype;
+  g.b_dt = d->bias.dtype;
+  g.y_dt = d->y.dtype;
+  g.o_dt = d->out.dtype;
+  g.stats_dt = d->stats_dtype;
+  g.has_scale = d->scale.rank != 0;
+  g.has_bias = d->bias.rank != 0;
+  g.is_layernorm = d->is_layernorm;
+  g.emit_stats = d->emit_stats;
+  g.eps = d->epsilon;
+  g.epi = epi;
+  hipLaunchKernelGGL(generic_norm_kernel, dim3((unsigned)d->x.dim[0]),
+                     dim3(256), 0, ctx->stream, g, x, scale, bias, out, mean,
+                     inv_variance);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- reduction ------------------------------------------------------------
+static int reduce_validate(fhip_ctx *ctx, const fhip_reduce_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_reduce: null descriptor");
+  if (!fhip_check_desc(ctx, d->x, "reduce X") ||
+      !fhip_check_desc(ctx, d->y, "reduce Y"))
+    return 1;
+  FHIP_REQUIRE(ctx, d->x.rank == d->y.rank,
+               "fhip_reduce: X and Y must share a rank (keep-dim)");
+  for (int i = 0; i < d->x.rank; ++i)
+    FHIP_REQUIRE(ctx, d->y.dim[i] == d->x.dim[i] || d->y.dim[i] == 1,
+                 "fhip_reduce: Y dim %d must be 1 or equal X's", i);
+  FHIP_REQUIRE(ctx, d->mode > FHIP_RED_NOT_SET && d->mode <= FHIP_RED_MUL_NO_ZEROS,
+               "fhip_reduce: invalid mode %d", d->mode);
+  FHIP_REQUIRE(ctx, d->mode != FHIP_RED_AVG || fhip_dtype_is_float(d->x.dtype),
+               "fhip_reduce: AVG needs a floating-point input");
+  return 0;
+}
+
+int fhip_reduce_workspace_size(const fhip_reduce_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_reduce_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_reduce_supported(const fhip_reduce_desc *d) {
+  if (!d || reduce_validate(nullptr, d) != 0)
+    return 0;
+  return fhip_fast_reduce_applicable(d) ? 2 : 1;
+}
+
+int fhip_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
+                void *y, void *workspace, size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_reduce: null context");
+  if (reduce_validate(ctx, d) != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, x && y, "fhip_reduce: null tensor pointer");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  if (fhip_fast_reduce_applicable(d))
+    return fhip_fast_reduce(ctx, d, x, y);
+  ReduceArgs g{};
+  g.y = make_dims(d->y);
+  g.red.rank = d->x.rank;
+  g.red_count = 1;
+  for (int i = 0; i < d->x.rank; ++i) {
+    const bool reduced = d->y.dim[i] == 1 && d->x.dim[i] > 1;
+    g.red.dim[i] = reduced ? d->x.dim[i] : 1;
+    g.red_count *= g.red.dim[i];
+  }
+  g.xs = make_strides(d->x);
+  g.ys = make_strides(d->y);
+  g.x_dt = d->x.dtype;
+  g.y_dt = d->y.dtype;
+  g.mode = d->mode;
+  const int64_t outs = fhip_desc_volume(d->y);
+  if (needs_double(d->x.dtype))
+    hipLaunchKernelGGL(generic_reduce_kernel<double>, dim3((unsigned)outs),
+                       dim3(256), 0, ctx->stream, g, x, y);
+  else
+    hipLaunchKernelGGL(generic_reduce_kernel<float>, dim3((unsigned)outs),
+                       dim3(256), 0, ctx->stream, g, x, y);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- pointwise ------------------------------------------------------------
+static int pointwise_validate(fhip_ctx *ctx, const fhip_pointwise_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_pointwise: null descriptor");
+  FHIP_REQUIRE(ctx, d->mode > FHIP_PW_NOT_SET && d->mode < FHIP_PW_MODE_COUNT,
+               "fhip_pointwise: invalid mode %d", d->mode);
+  FHIP_REQUIRE(ctx, d->num_inputs == fhip_pw_arity(d->mode),
+               "fhip_pointwise: mode %d takes %d inputs, got %d", d->mode,
+               fhip_pw_arity(d->mode), d->num_inputs);
+  if (!fhip_check_desc(ctx, d->out, "pointwise OUT"))
+    return 1;
+  for (int i = 0; i < d->num_inputs; ++i) {
+    if (d->in_is_scalar[i])
+      continue;
+    if (!fhip_check_desc(ctx, d->in[i], "pointwise IN"))
+      return 1;
+    int64_t st[FHIP_MAX_RANK];
+    FHIP_REQUIRE(ctx,
+                 fhip_broadcast_strides(d->in[i], d->out.rank, d->out.dim, st),
+                 "fhip_pointwise: input %d does not broadcast to the output", i);
+  }
+  return 0;
+}
+
+int fhip_pointwise_supported(const fhip_pointwise_desc *d) {
+  if (!d || pointwise_validate(nullptr, d) != 0)
+    return 0;
+  return 1;
+}
+
+int fhip_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d, const void *in0,
+                   const void *in1, const void *in2, void *out) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_pointwise: null context");
+  if (pointwise_validate(ctx, d) != 0)
+    return 1;
+  const void *ptr[3] = {in0, in1, in2};
+  for (int i = 0; i < d->num_inputs; ++i)
+    FHIP_REQUIRE(ctx, d->in_is_scalar[i] || ptr[i] != nullptr,
+                 "fhip_pointwise: input %d pointer is null", i);
+  FHIP_REQUIRE(ctx, out != nullptr, "fhip_pointwise: null output pointer");
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  PointwiseArgs g{};
+  g.out = make_dims(d->out);
+  g.os = make_strides(d->out);
+  g.o_dt = d->out.dtype;
+  g.mode = d->mode;
+  g.num_inputs = d->num_inputs;
+  g.params = d->params;
+  bool dbl = needs_double(d->out.dtype);
+  for (int i = 0; i < d->num_inputs; ++i) {
+    g.is_scalar[i] = d->in_is_scalar[i];
+    g.scalar[i] = d->in_scalar[i];
+    if (!d->in_is_scalar[i]) {
+      fhip_broadcast_strides(d->in[i], d->out.rank, d->out.dim, g.in[i].s);
+      g.in_dt[i] = d->in[i].dtype;
+      dbl = dbl || needs_double(d->in[i].dtype);
+    }
+  }
+  const int64_t total = fhip_desc_volume(d->out);
+  if (dbl)
+    hipLaunchKernelGGL(generic_pointwise_kernel<double>,
+                       dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream, g,
+                       in0, in1, in2, out, total);
+  else
+    hipLaunchKernelGGL(generic_pointwise_kernel<float>,
+                       dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream, g,
+                       in0, in1, in2, out, total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,205 @@
+// RMSNorm / LayerNorm forward for rows that are dense in memory: the whole row
+// is held in registers (one 16-byte load per lane per 1 KiB of row), statistics
+// are reduced with wavefront shuffles, and the normalised row, the optional
+// scale/bias and the fused pointwise chain are applied before a single 16-byte
+// store per lane.  HBM traffic is the compulsory read of X plus write of OUT.
+//
+// Reference semantics: aten.rms_norm / aten.layer_norm over all dims except
+// dim 0 (reference support/asm_emitter.h:1592-1626, 1427-1503;
+// node/norm_utils.h:27-99).
+#include "common.h"
+#include "fast_paths.h"
+#include "rownorm_kernel.h"
+
+#include <algorithm>
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+namespace {
+
+// Inner dims (1..rank-1) of `t` that have extent > 1, ordered by stride.
+struct InnerLayout {
+  bool dense = false;
+  int64_t inner = 1;
+};
+
+InnerLayout inner_layout(const fhip_tensor_desc &t) {
+  InnerLayout r;
+  std::vector<std::pair<int64_t, int64_t>> ds; // (stride, dim)
+  for (int i = 1; i < t.rank; ++i) {
+    r.inner *= t.dim[i];
+    if (t.dim[i] > 1)
+      ds.emplace_back(t.stride[i], t.dim[i]);
+  }
+  std::sort(ds.begin(), ds.end());
+  int64_t expect = 1;
+  for (auto &p : ds) {
+    if (p.first != expect)
+      return r;
+    expect *= p.second;
+  }
+  r.dense = true;
+  return r;
+}
+
+// `t` walks the row exactly like `x` (same stride on every inner dim > 1).
+bool same_inner_strides(const fhip_tensor_desc &x, const int64_t *strides) {
+  for (int i = 1; i < x.rank; ++i)
+    if (x.dim[i] > 1 && strides[i] != x.stride[i])
+      return false;
+  return true;
+}
+
+bool zero_inner_strides(const fhip_tensor_desc &x, const int64_t *strides) {
+  for (int i = 1; i < x.rank; ++i)
+    if (x.dim[i] > 1 && strides[i] != 0)
+      return false;
+  return true;
+}
+
+bool fast_dtype(int dt) {
+  return dt == FHIP_BFLOAT16 || dt == FHIP_HALF || dt == FHIP_FLOAT;
+}
+
+constexpr int kMaxChunks = 16;
+
+// Picks (chunks per lane, wavefronts per row) for a row of `inner` elements.
+bool pick_shape(int64_t inner, int vec, int *chunks, int *wpr) {
+  const int64_t per_wave_chunk = 64 * (int64_t)vec;
+  int64_t need = (inner + per_wave_chunk - 1) / per_wave_chunk;
+  // One wavefront per row keeps the reduction barrier-free; use it while the
+  // row fits 8 loads per lane, else spread the row over the 4 wavefronts.
+  *wpr = need <= 8 ? 1 : 4;
+  if (*wpr == 4)
+    need = (need + 3) / 4;
+  if (need > kMaxChunks)
+    return false;
+  int c = 1;
+  while (c < need)
+    c *= 2;
+  *chunks = c;
+  return true;
+}
+
+} // namespace
+
+bool fhip_fast_norm_applicable(const fhip_norm_desc *d) {
+  const fhip_tensor_desc &x = d->x;
+  if (!fast_dtype(x.dtype) || d->out.dtype != x.dtype)
+    return false;
+  if (!fast_dtype(d->y.dtype) || !fhip_epilogue_is_fast(d->epilogue))
+    return false;
+  for (int i = 0; i < d->epilogue.count; ++i)
+    if (fhip_pw_is_transcendental(d->epilogue.op[i].mode))
+      return false;
+  const InnerLayout lay = inner_layout(x);
+  if (!lay.dense)
+    return false;
+  const int vec = 16 / fhip_dtype_size(x.dtype);
+  if (lay.inner % vec != 0)
+    return false;
+  int chunks, wpr;
+  if (!pick_shape(lay.inner, vec, &chunks, &wpr))
+    return false;
+  const int64_t xrs = x.dim[0] > 1 ? x.stride[0] : lay.inner;
+  const int64_t ors = d->out.dim[0] > 1 ? d->out.stride[0] : lay.inner;
+  if (xrs < lay.inner || ors < lay.inner || xrs % vec || ors % vec)
+    return false;
+  if (!same_inner_strides(x, d->out.stride))
+    return false;
+  auto operand_dtype_ok = [&](int dt) {
+    return dt == x.dtype || dt == FHIP_FLOAT;
+  };
+  if (d->scale.rank && (!same_inner_strides(x, d->scale.stride) ||
+                        !operand_dtype_ok(d->scale.dtype)))
+    return false;
+  if (d->bias.rank && (!same_inner_strides(x, d->bias.stride) ||
+                       !operand_dtype_ok(d->bias.dtype)))
+    return false;
+  if (d->emit_stats && !fast_dtype(d->stats_dtype))
+    return false;
+  for (int i = 0; i < d->epilogue.count; ++i) {
+    const fhip_epilogue_op &o = d->epilogue.op[i];
+    if (o.operand_kind != FHIP_OPERAND_TENSOR)
+      continue;
+    int64_t st[FHIP_MAX_RANK];
+    if (!fhip_broadcast_strides(o.operand, x.rank, x.dim, st) ||
+        !operand_dtype_ok(o.operand.dtype))
+      return false;
+    if (!same_inner_strides(x, st) && !zero_inner_strides(x, st))
+      return false;
+    if (same_inner_strides(x, st) && st[0] % vec != 0)
+      return false;
+  }
+  return true;
+}
+
+int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
+                   const void *scale, const void *bias, const DevEpilogue &epi,
+                   void *out, void *mean, void *inv_variance) {
+  const InnerLayout lay = inner_layout(d->x);
+  const int vec = 16 / fhip_dtype_size(d->x.dtype);
+  int chunks = 1, wpr = 1;
+  FHIP_REQUIRE(ctx, pick_shape(lay.inner, vec, &chunks, &wpr),
+               "rownorm: row of %lld elements exceeds the register-resident "
+               "kernel",
+               (long long)lay.inner);
+  RowNormArgs g{};
+  g.x = x;
+  g.scale = scale;
+  g.bias = bias;
+  g.out = out;
+  g.mean = mean;
+  g.rstd = inv_variance;
+  g.rows = d->x.dim[0];
+  g.inner = lay.inner;
+  g.x_row_stride = d->x.dim[0] > 1 ? d->x.stride[0] : lay.inner;
+  g.out_row_stride = d->out.dim[0] > 1 ? d->out.stride[0] : lay.inner;
+  g.scale_dt = d->scale.dtype;
+  g.bias_dt = d->bias.dtype;
+  g.y_dt = d->y.dtype;
+  g.stats_dt = d->stats_dtype;
+  g.is_layernorm = d->is_layernorm;
+  g.emit_stats = d->emit_stats;
+  g.eps = d->epsilon;
+  g.epi_count = epi.count;
+  for (int i = 0; i < epi.count; ++i) {
+    const DevEpiOp &s = epi.op[i];
+    FastEpiOp &o = g.epi[i];
+    o.mode = s.mode;
+    o.kind = s.kind;
+    o.acc_is_in1 = s.acc_is_in1;
+    o.result_dtype = s.result_dtype;
+    o.operand_dtype = s.operand_dtype;
+    o.scalar = s.scalar;
+    o.params = s.params;
+    o.ptr = s.ptr;
+    o.row_stride = s.stride[0];
+    o.col_unit = (s.kind == FHIP_OPERAND_TENSOR &&
+                  same_inner_strides(d->x, s.stride) && lay.inner > 1)
+                     ? 1
+                     : 0;
+  }
+  // 16-byte alignment of every vector-accessed base pointer.
+  auto aligned = [](const void *p) { return ((uintptr_t)p & 15u) == 0; };
+  FHIP_REQUIRE(ctx, aligned(x) && aligned(out) && aligned(scale) &&
+                        aligned(bias),
+               "rownorm: tensor base pointers must be 16-byte aligned");
+  for (int i = 0; i < epi.count; ++i)
+    FHIP_REQUIRE(ctx, g.epi[i].col_unit == 0 || aligned(g.epi[i].ptr),
+                 "rownorm: epilogue operand must be 16-byte aligned");
+  switch (d->x.dtype) {
+  case FHIP_BFLOAT16:
+    rownorm_launch_bf16(chunks, wpr, g.rows, ctx->stream, g);
+    break;
+  case FHIP_HALF:
+    rownorm_launch_f16(chunks, wpr, g.rows, ctx->stream, g);
+    break;
+  default:
+    rownorm_launch_f32(chunks, wpr, g.rows, ctx->stream, g);
+    break;
+  }
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}

@@ -1,0 +1,388 @@
+"""Matmul / conv / SDPA / reduction / pointwise through the C ABI vs the oracle
+and the reference samples' known answers (strided generic kernels and
+whichever tuned kernel the descriptor selects)."""
+import numpy as np
+import pytest
+
+from fusilli_amd import capi
+from oracle import oracle
+from helpers import HT, assert_close, rand
+
+pytestmark = pytest.mark.gpu
+
+
+# ---- matmul ---------------------------------------------------------------
+def run_matmul(ctx, a, b, c_dtype, *, out_dtype=None, epilogue=(),
+               epi_tensors=(), out_strides=None):
+    batch = np.broadcast_shapes(tuple(a.dims[:-2]), tuple(b.dims[:-2]))
+    cdims = list(batch) + [a.dims[-2], b.dims[-1]]
+    out_dtype = c_dtype if out_dtype is None else out_dtype
+    out = HT.empty(cdims, out_dtype, out_strides)
+    d = capi.MatmulDesc()
+    d.a, d.b = a.desc(), b.desc()
+    d.c = capi.TensorDesc.make(cdims, oracle.contiguous_strides(cdims), c_dtype)
+    d.out = out.desc()
+    d.out_dtype = out_dtype
+    d.epilogue = capi.make_epilogue(list(epilogue))
+    bufs = [t.upload(ctx) for t in epi_tensors]
+    da, db, dout = a.upload(ctx), b.upload(ctx), out.upload(ctx)
+    ctx.matmul(d, da, db, dout, epilogue_operands=bufs)
+    return out.fetch(ctx, dout)
+
+
+def test_matmul_config1_f32(ctx):
+    # BASELINE config 1: f32 A[1,256,512] x B[1,512,256], U[-1,1], rel 1e-4.
+    a = HT.from_logical(rand(1, 0, [1, 256, 512], "uniform"), capi.FLOAT)
+    b = HT.from_logical(rand(1, 1, [1, 512, 256], "uniform"), capi.FLOAT)
+    out = run_matmul(ctx, a, b, capi.FLOAT)
+    assert_close(out.logical(), oracle.matmul(a.logical(), b.logical()), capi.FLOAT)
+
+
+@pytest.mark.parametrize("transpose_b", [False, True])
+def test_matmul_all_ones_f16_equals_k(ctx, transpose_b):
+    # samples/matmul/matmul_basic.cpp:91-94,169-172: 64x128 * 128x256 => 128.
+    m, k, n = 64, 128, 256
+    a = HT.from_logical(np.ones([m, k]), capi.HALF)
+    b = HT.from_logical(np.ones([k, n]), capi.HALF,
+                        [1, k] if transpose_b else None)
+    out = run_matmul(ctx, a, b, capi.HALF)
+    assert np.all(out.logical() == 128.0)
+
+
+def test_matmul_bias_known_answer(ctx):
+    # samples/matmul/matmul_basic_with_bias.cpp:110-113: 128 + 2 = 130.
+    m, k, n = 64, 128, 256
+    a = HT.from_logical(np.ones([m, k]), capi.HALF)
+    b = HT.from_logical(np.ones([k, n]), capi.HALF)
+    bias = HT.from_logical(np.full([1, n], 2.0), capi.HALF)
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.HALF, operand=bias.desc())]
+    out = run_matmul(ctx, a, b, capi.HALF, epilogue=epi, epi_tensors=[bias])
+    assert np.all(out.logical() == 130.0)
+
+
+def test_matmul_batched_and_broadcast(ctx):
+    # samples/matmul/matmul_batched.cpp: [16,16,M,K] x [1,1,K,N].
+    a = HT.from_logical(rand(4, 0, [3, 4, 16, 24]), capi.FLOAT)
+    b = HT.from_logical(rand(4, 1, [1, 1, 24, 8]), capi.FLOAT)
+    out = run_matmul(ctx, a, b, capi.FLOAT)
+    assert_close(out.logical(), oracle.matmul(a.logical(), b.logical()), capi.FLOAT)
+    b2 = HT.from_logical(rand(4, 2, [3, 4, 24, 8]), capi.FLOAT)
+    out2 = run_matmul(ctx, a, b2, capi.FLOAT)
+    assert_close(out2.logical(), oracle.matmul(a.logical(), b2.logical()), capi.FLOAT)
+
+
+def test_matmul_strided_operands_and_output(ctx):
+    a = HT.from_logical(rand(6, 0, [2, 33, 17]), capi.BFLOAT16, [33 * 17, 1, 33])
+    b = HT.from_logical(rand(6, 1, [2, 17, 9]), capi.BFLOAT16, [17 * 9, 1, 17])
+    out = run_matmul(ctx, a, b, capi.BFLOAT16, out_strides=[33 * 9, 1, 33])
+    assert_close(out.logical(), oracle.matmul(a.logical(), b.logical()), capi.BFLOAT16)
+
+
+def test_matmul_int8_exact_small(ctx):
+    a = HT.from_logical(rand(5, 0, [70, 130], "int", lo=-127, hi=127), capi.INT8)
+    b = HT.from_logical(rand(5, 1, [130, 50], "int", lo=-127, hi=127), capi.INT8)
+    out = run_matmul(ctx, a, b, capi.INT32)
+    ref = oracle.matmul(a.logical().astype(np.int8), b.logical().astype(np.int8))
+    assert np.array_equal(out.logical(), ref)
+
+
+def test_matmul_one_hot_selects_columns(ctx):
+    a = HT.from_logical(rand(7, 0, [12, 10]), capi.FLOAT)
+    sel = np.zeros([10, 4])
+    for j, col in enumerate([7, 0, 3, 9]):
+        sel[col, j] = 1.0
+    out = run_matmul(ctx, a, HT.from_logical(sel, capi.FLOAT), capi.FLOAT)
+    assert np.array_equal(out.logical(), a.logical()[:, [7, 0, 3, 9]])
+
+
+# ---- conv -----------------------------------------------------------------
+def run_conv(ctx, x, w, pad, stride, dil, y_dtype, *, out_dtype=None,
+             epilogue=(), epi_tensors=(), channels_last_out=False):
+    ydims = oracle.conv_output_dims(x.dims, w.dims, pad, stride, dil)
+    out_dtype = y_dtype if out_dtype is None else out_dtype
+    ostr = oracle.channels_last_strides(ydims) if channels_last_out else None
+    out = HT.empty(ydims, out_dtype, ostr)
+    d = capi.ConvDesc()
+    d.x, d.w = x.desc(), w.desc()
+    d.y = capi.TensorDesc.make(ydims, out.strides, y_dtype)
+    d.out = out.desc()
+    d.out_dtype = out_dtype
+    d.spatial_rank = len(pad)
+    for i in range(len(pad)):
+        d.padding[i], d.stride[i], d.dilation[i] = pad[i], stride[i], dil[i]
+    d.epilogue = capi.make_epilogue(list(epilogue))
+    bufs = [t.upload(ctx) for t in epi_tensors]
+    dx, dw, dout = x.upload(ctx), w.upload(ctx), out.upload(ctx)
+    ctx.conv_fprop(d, dx, dw, dout, epilogue_operands=bufs)
+    return out.fetch(ctx, dout)
+
+
+@pytest.mark.parametrize("nhwc", [False, True])
+def test_conv_all_ones_1x1_known_answer(ctx, nhwc):
+    # tests/test_graph.cpp:198-223, samples/convolution/conv_fprop_nhwc_krsc.cpp:95:
+    # all-ones f16, 1x1, C = 128 => 128.
+    xd, wd = [4, 128, 8, 8], [32, 128, 1, 1]
+    xs = oracle.channels_last_strides(xd) if nhwc else None
+    ws = oracle.channels_last_strides(wd) if nhwc else None
+    x = HT.from_logical(np.ones(xd), capi.HALF, xs)
+    w = HT.from_logical(np.ones(wd), capi.HALF, ws)
+    out = run_conv(ctx, x, w, [0, 0], [1, 1], [1, 1], capi.HALF,
+                   channels_last_out=nhwc)
+    assert np.all(out.logical() == 128.0)
+
+
+def test_conv_bias_relu_known_answer(ctx):
+    # samples/convolution/conv_fprop_with_relu_and_bias.cpp:112 => 129.
+    xd, wd = [2, 128, 8, 8], [16, 128, 1, 1]
+    x = HT.from_logical(np.ones(xd), capi.HALF, oracle.channels_last_strides(xd))
+    w = HT.from_logical(np.ones(wd), capi.HALF, oracle.channels_last_strides(wd))
+    bias = HT(list([1, 16, 1, 1]), [16, 1, 16, 16], capi.HALF,
+              np.ones(16, np.float16))
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.HALF, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.HALF)]
+    out = run_conv(ctx, x, w, [0, 0], [1, 1], [1, 1], capi.HALF, epilogue=epi,
+                   epi_tensors=[bias], channels_last_out=True)
+    assert np.all(out.logical() == 129.0)
+
+
+def test_conv_3x3_same_pad_corner_known_answer(ctx):
+    # samples/convolution/conv_fprop_nhwc_krsc_with_pad.cpp:94: corner = 2*2*128.
+    xd, wd = [2, 128, 8, 8], [16, 128, 3, 3]
+    x = HT.from_logical(np.ones(xd), capi.HALF, oracle.channels_last_strides(xd))
+    w = HT.from_logical(np.ones(wd), capi.HALF, oracle.channels_last_strides(wd))
+    out = run_conv(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.HALF,
+                   channels_last_out=True)
+    lg = out.logical()
+    assert lg[0, 0, 0, 0] == 512.0 and lg[0, 0, 1, 1] == 1152.0 \
+        and lg[1, 3, 0, 4] == 768.0
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=[2, 6, 9, 11], w=[4, 6, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    dict(x=[2, 6, 9, 11], w=[4, 3, 3, 2], pad=[0, 1], s=[2, 1], d=[1, 2]),
+    dict(x=[1, 8, 13], w=[6, 2, 4], pad=[2], s=[3], d=[2]),
+    dict(x=[1, 4, 5, 6, 7], w=[2, 4, 2, 3, 3], pad=[1, 0, 1], s=[1, 2, 1], d=[1, 1, 1]),
+])
+@pytest.mark.parametrize("dtype", [capi.FLOAT, capi.BFLOAT16])
+def test_conv_random_vs_oracle(ctx, case, dtype):
+    x = HT.from_logical(rand(31, 0, case["x"]), dtype,
+                        oracle.channels_last_strides(case["x"]))
+    w = HT.from_logical(rand(31, 1, case["w"], std=0.2), dtype,
+                        oracle.channels_last_strides(case["w"]))
+    out = run_conv(ctx, x, w, case["pad"], case["s"], case["d"], dtype,
+                   channels_last_out=True)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"],
+                            case["d"])
+    assert_close(out.logical(), ref, dtype, str(case))
+
+
+# ---- sdpa -----------------------------------------------------------------
+def run_sdpa(ctx, q, k, v, *, mask=None, causal=False, scale=None, o_dtype=None):
+    o_dtype = q.dtype if o_dtype is None else o_dtype
+    out = HT.empty([q.dims[0], q.dims[1], q.dims[2], v.dims[3]], o_dtype)
+    d = capi.SdpaDesc()
+    d.q, d.k, d.v, d.o = q.desc(), k.desc(), v.desc(), out.desc()
+    if mask is not None:
+        d.mask = mask.desc()
+    d.is_causal = int(causal)
+    if scale is not None:
+        d.has_scale, d.scale = 1, scale
+    bufs = [t.upload(ctx) for t in (q, k, v)]
+    dm = mask.upload(ctx) if mask is not None else None
+    dout = out.upload(ctx)
+    ctx.sdpa_fwd(d, bufs[0], bufs[1], bufs[2], dout, mask=dm)
+    return out.fetch(ctx, dout)
+
+
+@pytest.mark.parametrize("variant", ["mha", "causal", "mask", "gqa", "cross"])
+def test_sdpa_constant_fill_equals_v(ctx, variant):
+    # samples/sdpa/*.cpp via samples/sdpa_utils.cpp:184-247: q = k = v = 0.01
+    # (mask -1) => output == v within 1e-2; B1 H8 S64 D64 f16.
+    B, Hq, Hkv, Sq, Skv, D = 1, 8, 8, 64, 64, 64
+    if variant == "gqa":
+        Hkv = 2
+    if variant == "cross":
+        Sq, Skv = 32, 128
+    q = HT.from_logical(np.full([B, Hq, Sq, D], 0.01), capi.HALF)
+    k = HT.from_logical(np.full([B, Hkv, Skv, D], 0.01), capi.HALF)
+    v = HT.from_logical(np.full([B, Hkv, Skv, D], 0.01), capi.HALF)
+    mask = HT.from_logical(np.full([B, 1, Sq, Skv], -1.0), capi.HALF) \
+        if variant == "mask" else None
+    out = run_sdpa(ctx, q, k, v, mask=mask, causal=(variant == "causal"))
+    assert np.allclose(out.logical(), v.logical()[0, 0, 0, 0], atol=1e-2)
+
+
+@pytest.mark.parametrize("case", [
+    dict(B=2, Hq=4, Hkv=4, Sq=70, Skv=70, D=32, Dv=32, causal=True),
+    dict(B=1, Hq=6, Hkv=2, Sq=33, Skv=129, D=16, Dv=24, causal=False),
+    dict(B=2, Hq=2, Hkv=1, Sq=17, Skv=65, D=64, Dv=64, causal=False, mask="float"),
+    dict(B=1, Hq=2, Hkv=2, Sq=40, Skv=40, D=128, Dv=128, causal=False, mask="bool"),
+])
+@pytest.mark.parametrize("dtype", [capi.FLOAT, capi.BFLOAT16])
+def test_sdpa_random_vs_oracle(ctx, case, dtype):
+    c = case
+    q = HT.from_logical(rand(41, 0, [c["B"], c["Hq"], c["Sq"], c["D"]]), dtype)
+    k = HT.from_logical(rand(41, 1, [c["B"], c["Hkv"], c["Skv"], c["D"]]), dtype)
+    v = HT.from_logical(rand(41, 2, [c["B"], c["Hkv"], c["Skv"], c["Dv"]]), dtype)
+    mask, mref = None, None
+    if c.get("mask") == "float":
+        mask = HT.from_logical(rand(41, 3, [c["B"], 1, c["Sq"], c["Skv"]]), dtype)
+        mref = mask.logical()
+    elif c.get("mask") == "bool":
+        keep = rand(41, 3, [1, 1, c["Sq"], c["Skv"]], "uniform") > -0.5
+        keep[..., 0] = True
+        mask = HT.from_logical(keep, capi.BOOLEAN)
+        mref = keep
+    out = run_sdpa(ctx, q, k, v, mask=mask, causal=c["causal"])
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), mask=mref,
+                      is_causal=c["causal"])
+    assert_close(out.logical(), ref, dtype, str(case))
+
+
+# ---- reduction ------------------------------------------------------------
+@pytest.mark.parametrize("mode", ["ADD", "SUM", "MUL", "MIN", "MAX", "AMAX",
+                                  "AVG", "NORM1", "NORM2", "MUL_NO_ZEROS"])
+@pytest.mark.parametrize("dtype", [capi.INT32, capi.HALF, capi.FLOAT])
+def test_reduction_reference_table(ctx, mode, dtype):
+    # samples/reduction/reduction_ops.cpp:31-64, 83-273: [2,16,8,8] -> [2,16,1,1];
+    # inputs i % 100 - 50 (sums) or ones with a 2 and a 3 (products).
+    if mode == "AVG" and dtype == capi.INT32:
+        pytest.skip("integer AVG is rejected at validation (reduction_node.h:122-127)")
+    dims, odims = [2, 16, 8, 8], [2, 16, 1, 1]
+    n = int(np.prod(dims))
+    if mode in ("MUL", "MUL_NO_ZEROS"):
+        vals = np.ones(n)
+        vals[0], vals[1] = 2.0, 3.0
+        if mode == "MUL_NO_ZEROS":
+            vals[2] = 0.0
+    else:
+        vals = (np.arange(n) % 100 - 50).astype(np.float64)
+    x = HT.from_logical(vals.reshape(dims), dtype)
+    out = HT.empty(odims, dtype)
+    d = capi.ReduceDesc()
+    d.x, d.y, d.mode = x.desc(), out.desc(), capi.RED[mode]
+    dx, dy = x.upload(ctx), out.upload(ctx)
+    ctx.reduce(d, dx, dy)
+    out.fetch(ctx, dy)
+    ref = oracle.reduction(x.logical(), odims, capi.RED[mode])
+    if dtype == capi.INT32:
+        assert np.array_equal(out.logical(), ref.astype(np.int64))
+    else:
+        assert np.all(np.abs(out.logical() - ref) < max(0.01, 2e-3 * np.abs(ref).max()))
+
+
+def test_reduction_middle_dim_strided(ctx):
+    dims, odims = [3, 50, 7], [3, 1, 7]
+    x = HT.from_logical(rand(51, 0, dims), capi.FLOAT, [7, 21, 1])
+    out = HT.empty(odims, capi.FLOAT)
+    d = capi.ReduceDesc()
+    d.x, d.y, d.mode = x.desc(), out.desc(), capi.RED["NORM2"]
+    dx, dy = x.upload(ctx), out.upload(ctx)
+    ctx.reduce(d, dx, dy)
+    assert_close(out.fetch(ctx, dy).logical(),
+                 oracle.reduction(x.logical(), odims, capi.RED["NORM2"]), capi.FLOAT)
+
+
+# ---- pointwise ------------------------------------------------------------
+def run_pointwise(ctx, mode, ins, out_dtype, out_dims=None, params=None,
+                  scalars=None):
+    scalars = scalars or {}
+    shapes = [tuple(t.dims) for t in ins if t is not None]
+    odims = list(np.broadcast_shapes(*shapes)) if out_dims is None else out_dims
+    out = HT.empty(odims, out_dtype)
+    d = capi.PointwiseDesc()
+    d.mode = capi.PW[mode]
+    d.num_inputs = len(ins)
+    d.params = params or capi.PointwiseParams.default()
+    bufs = []
+    for i, t in enumerate(ins):
+        if t is None:
+            d.in_is_scalar[i] = 1
+            d.in_scalar[i] = scalars[i]
+            bufs.append(None)
+        else:
+            d.in_[i] = t.desc()
+            bufs.append(t.upload(ctx))
+    d.out = out.desc()
+    bufs += [None] * (3 - len(bufs))
+    dout = out.upload(ctx)
+    ctx.pointwise(d, bufs[0], bufs[1], bufs[2], dout)
+    return out.fetch(ctx, dout)
+
+
+UNARY = ["ABS", "CEIL", "ELU_FWD", "ERF", "EXP", "FLOOR", "GELU_APPROX_TANH_FWD",
+         "GELU_FWD", "IDENTITY", "LOG", "NEG", "RECIPROCAL", "RELU_FWD", "RSQRT",
+         "SIGMOID_FWD", "SIN", "SOFTPLUS_FWD", "SQRT", "SWISH_FWD", "TAN",
+         "TANH_FWD", "LOGICAL_NOT"]
+BINARY = ["ADD", "ADD_SQUARE", "DIV", "MAX_OP", "MIN_OP", "MUL", "SUB", "CMP_EQ",
+          "CMP_GE", "CMP_GT", "CMP_LE", "CMP_LT", "CMP_NEQ", "LOGICAL_AND",
+          "LOGICAL_OR", "RELU_BWD", "TANH_BWD", "GELU_BWD",
+          "GELU_APPROX_TANH_BWD", "SWISH_BWD"]
+
+
+@pytest.mark.parametrize("mode", UNARY)
+@pytest.mark.parametrize("dtype", [capi.FLOAT, capi.HALF])
+def test_pointwise_unary_vs_oracle(ctx, mode, dtype):
+    vals = rand(61, 0, [4, 37], "uniform", lo=-3.0, hi=3.0)
+    if mode in ("LOG", "RSQRT", "SQRT"):
+        vals = np.abs(vals) + 0.1
+    if mode in ("RECIPROCAL", "TAN"):
+        vals = np.where(np.abs(vals) < 0.2, 0.7, vals) * (0.4 if mode == "TAN" else 1)
+    x = HT.from_logical(vals, dtype)
+    params = capi.PointwiseParams(1.5, 2.0, 3.0, 0.75)
+    odt = capi.BOOLEAN if mode == "LOGICAL_NOT" else dtype
+    out = run_pointwise(ctx, mode, [x], odt, params=params)
+    ref = oracle.pointwise(capi.PW[mode], [x.logical()], elu_alpha=1.5,
+                           softplus_beta=2.0, softplus_threshold=3.0,
+                           swish_beta=0.75)
+    if odt == capi.BOOLEAN:
+        assert np.array_equal(out.logical(), ref.astype(np.int64))
+    else:
+        assert_close(out.logical(), ref, dtype, mode,
+                     rtol=1e-4 if dtype == capi.FLOAT else 2e-2)
+
+
+@pytest.mark.parametrize("mode", BINARY)
+def test_pointwise_binary_broadcast_vs_oracle(ctx, mode):
+    a = HT.from_logical(np.round(rand(62, 0, [3, 1, 8], "uniform", lo=-2, hi=2), 1),
+                        capi.FLOAT)
+    b = HT.from_logical(np.round(rand(62, 1, [5, 8], "uniform", lo=-2, hi=2), 1) + 0.05,
+                        capi.FLOAT)
+    boolean = mode.startswith("CMP") or mode.startswith("LOGICAL")
+    out = run_pointwise(ctx, mode, [a, b], capi.BOOLEAN if boolean else capi.FLOAT)
+    ref = oracle.pointwise(capi.PW[mode], [a.logical(), b.logical()])
+    if boolean:
+        assert np.array_equal(out.logical(), ref.astype(np.int64))
+    else:
+        assert_close(out.logical(), ref, capi.FLOAT, mode)
+
+
+def test_pointwise_add_transposed_known_answer(ctx):
+    # samples/pointwise/pointwise_add_transposed.cpp:22-112: a = {1..6} as 3x2
+    # row-major, b = same bytes viewed with dim {3,2} stride {1,3}.
+    data = np.arange(1, 7, dtype=np.float32)
+    a = HT([3, 2], [2, 1], capi.FLOAT, data.copy())
+    b = HT([3, 2], [1, 3], capi.FLOAT, data.copy())
+    out = run_pointwise(ctx, "ADD", [a, b], capi.FLOAT)
+    assert out.storage.tolist() == [2, 6, 5, 9, 8, 12]
+
+
+def test_pointwise_scalar_mul_known_answer(ctx):
+    # samples/pointwise/pointwise_scalar_mul.cpp:22-78: 3 * 2 = 6, the scalar is
+    # a constant, not a buffer.
+    a = HT.from_logical(np.full([2, 5], 3.0), capi.FLOAT)
+    out = run_pointwise(ctx, "MUL", [a, None], capi.FLOAT, scalars={1: 2.0})
+    assert np.all(out.logical() == 6.0)
+
+
+def test_pointwise_int32_add_and_select(ctx):
+    # samples/aot/single_backend.cpp:52-110: int32 2 + 3 = 5.
+    a = HT.from_logical(np.full([4, 4], 2), capi.INT32)
+    b = HT.from_logical(np.full([4, 4], 3), capi.INT32)
+    assert np.all(run_pointwise(ctx, "ADD", [a, b], capi.INT32).logical() == 5)
+    big = HT.from_logical(np.full([4, 4], 2_000_000_011), capi.INT32)
+    assert np.all(run_pointwise(ctx, "IDENTITY", [big], capi.INT32).logical()
+                  == 2_000_000_011)
+    cond = HT.from_logical(np.eye(4), capi.BOOLEAN)
+    sel = run_pointwise(ctx, "BINARY_SELECT", [cond, a, b], capi.INT32).logical()
+    assert np.array_equal(sel, np.where(np.eye(4) != 0, 2, 3))
