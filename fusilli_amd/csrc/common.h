@@ -469,6 +469,78 @@ __device__ __forceinline__ float fhip_pw_fast_unary(int mode, float x,
   }
 }
 
+// Vector forms: one uniform branch per call, straight-line code per case.
+// (Per-element mode dispatch costs a scalar branch per element and dominates
+// bandwidth-bound kernels.)
+template <bool TRANSCENDENTAL, int N>
+__device__ __forceinline__ void fhip_pw_fast_unary_vec(int mode, float (&y)[N],
+                                                       float swish_beta) {
+#define FHIP_VEC_CASE(MODE)                                                    \
+  case MODE:                                                                   \
+    _Pragma("unroll") for (int i = 0; i < N; ++i) y[i] =                       \
+        fhip_pw_fast_unary<TRANSCENDENTAL>(MODE, y[i], swish_beta);            \
+    break;
+  switch (mode) {
+    FHIP_VEC_CASE(FHIP_PW_RELU_FWD)
+    FHIP_VEC_CASE(FHIP_PW_NEG)
+    FHIP_VEC_CASE(FHIP_PW_ABS)
+    FHIP_VEC_CASE(FHIP_PW_SIGMOID_FWD)
+    FHIP_VEC_CASE(FHIP_PW_SWISH_FWD)
+  default:
+    if constexpr (TRANSCENDENTAL) {
+      switch (mode) {
+        FHIP_VEC_CASE(FHIP_PW_TANH_FWD)
+        FHIP_VEC_CASE(FHIP_PW_GELU_FWD)
+        FHIP_VEC_CASE(FHIP_PW_GELU_APPROX_TANH_FWD)
+      default:
+        break;
+      }
+    }
+    break;
+  }
+#undef FHIP_VEC_CASE
+}
+
+template <int N>
+__device__ __forceinline__ void
+fhip_pw_fast_binary_vec(int mode, bool acc_is_in1, float (&y)[N],
+                        const float (&o)[N]) {
+#define FHIP_VEC_CASE(MODE)                                                    \
+  case MODE:                                                                   \
+    if (acc_is_in1) {                                                          \
+      _Pragma("unroll") for (int i = 0; i < N; ++i) y[i] =                     \
+          fhip_pw_fast_binary(MODE, o[i], y[i]);                               \
+    } else {                                                                   \
+      _Pragma("unroll") for (int i = 0; i < N; ++i) y[i] =                     \
+          fhip_pw_fast_binary(MODE, y[i], o[i]);                               \
+    }                                                                          \
+    break;
+  switch (mode) {
+    FHIP_VEC_CASE(FHIP_PW_ADD)
+    FHIP_VEC_CASE(FHIP_PW_SUB)
+    FHIP_VEC_CASE(FHIP_PW_MUL)
+    FHIP_VEC_CASE(FHIP_PW_DIV)
+    FHIP_VEC_CASE(FHIP_PW_MAX_OP)
+    FHIP_VEC_CASE(FHIP_PW_MIN_OP)
+  default:
+    break;
+  }
+#undef FHIP_VEC_CASE
+}
+
+template <int N>
+__device__ __forceinline__ void fhip_round_fast_vec(int dt, float (&y)[N]) {
+  if (dt == FHIP_BFLOAT16) {
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      y[i] = (float)(__bf16)y[i];
+  } else if (dt == FHIP_HALF) {
+#pragma unroll
+    for (int i = 0; i < N; ++i)
+      y[i] = (float)(_Float16)y[i];
+  }
+}
+
 __host__ __device__ inline bool fhip_pw_is_transcendental(int mode) {
   return mode == FHIP_PW_TANH_FWD || mode == FHIP_PW_GELU_FWD ||
          mode == FHIP_PW_GELU_APPROX_TANH_FWD;

@@ -329,53 +329,37 @@ struct ReduceArgs {
   Dims red;      // reduced extents per dim (1 where kept)
   Strides xs, ys;
   int64_t red_count;
-  int32_t x_dt, y_dt, mode;
+  int32_t x_dt, y_dt;
+  int32_t map_kind, comb_kind, post_kind;
+  double identity;
 };
 
-template <typename CT>
-__device__ __forceinline__ CT red_identity(int mode) {
-  switch (mode) {
-  case FHIP_RED_MUL:
-  case FHIP_RED_MUL_NO_ZEROS:
-    return (CT)1;
-  case FHIP_RED_MIN:
-    return (CT)INFINITY;
-  case FHIP_RED_MAX:
-    return (CT)-INFINITY;
-  default:
-    return (CT)0;
-  }
-}
+// The host splits a reduction mode into: a per-element map, a combine, an
+// identity and a final step.
+enum { RMAP_NONE = 0, RMAP_ABS, RMAP_SQUARE, RMAP_ZERO_TO_ONE };
+enum { RCOMB_ADD = 0, RCOMB_MUL, RCOMB_MIN, RCOMB_MAX };
+enum { RPOST_NONE = 0, RPOST_MEAN, RPOST_SQRT };
 
 template <typename CT>
-__device__ __forceinline__ CT red_map(int mode, CT v) {
-  switch (mode) {
-  case FHIP_RED_AMAX:
-  case FHIP_RED_NORM1:
-    return fabs(v);
-  case FHIP_RED_NORM2:
+__device__ __forceinline__ CT red_map(int kind, CT v) {
+  if (kind == RMAP_ABS)
+    return v < (CT)0 ? -v : v;
+  if (kind == RMAP_SQUARE)
     return v * v;
-  case FHIP_RED_MUL_NO_ZEROS:
+  if (kind == RMAP_ZERO_TO_ONE)
     return v == (CT)0 ? (CT)1 : v;
-  default:
-    return v;
-  }
+  return v;
 }
 
 template <typename CT>
-__device__ __forceinline__ CT red_combine(int mode, CT a, CT b) {
-  switch (mode) {
-  case FHIP_RED_MUL:
-  case FHIP_RED_MUL_NO_ZEROS:
+__device__ __forceinline__ CT red_combine(int kind, CT a, CT b) {
+  if (kind == RCOMB_MUL)
     return a * b;
-  case FHIP_RED_MIN:
+  if (kind == RCOMB_MIN)
     return (a != a || b != b) ? (a != a ? a : b) : (a < b ? a : b);
-  case FHIP_RED_MAX:
-  case FHIP_RED_AMAX:
+  if (kind == RCOMB_MAX)
     return (a != a || b != b) ? (a != a ? a : b) : (a > b ? a : b);
-  default:
-    return a + b;
-  }
+  return a + b;
 }
 
 template <typename CT>
@@ -387,25 +371,25 @@ __global__ __launch_bounds__(256) void generic_reduce_kernel(ReduceArgs g,
   unravel((int64_t)blockIdx.x, g.y, ocoord);
   const int rank = g.y.rank;
   const int64_t base = dot(ocoord, g.xs, rank);
-  CT acc = g.mode == FHIP_RED_AMAX ? (CT)0 : red_identity<CT>(g.mode);
+  CT acc = (CT)g.identity;
   for (int64_t i = threadIdx.x; i < g.red_count; i += blockDim.x) {
     unravel(i, g.red, rcoord);
     const CT v = fhip_load<CT>(x, g.x_dt, base + dot(rcoord, g.xs, rank));
-    acc = red_combine<CT>(g.mode, acc, red_map<CT>(g.mode, v));
+    acc = red_combine<CT>(g.comb_kind, acc, red_map<CT>(g.map_kind, v));
   }
   lds[threadIdx.x] = acc;
   __syncthreads();
   for (int s = 128; s > 0; s >>= 1) {
     if ((int)threadIdx.x < s)
       lds[threadIdx.x] =
-          red_combine<CT>(g.mode, lds[threadIdx.x], lds[threadIdx.x + s]);
+          red_combine<CT>(g.comb_kind, lds[threadIdx.x], lds[threadIdx.x + s]);
     __syncthreads();
   }
   if (threadIdx.x == 0) {
     CT r = lds[0];
-    if (g.mode == FHIP_RED_AVG)
+    if (g.post_kind == RPOST_MEAN)
       r = r / (CT)g.red_count;
-    else if (g.mode == FHIP_RED_NORM2)
+    else if (g.post_kind == RPOST_SQRT)
       r = sqrt(r);
     fhip_store<CT>(y, g.y_dt, dot(ocoord, g.ys, rank), r);
   }
@@ -923,7 +907,45 @@ int fhip_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
   g.ys = make_strides(d->y);
   g.x_dt = d->x.dtype;
   g.y_dt = d->y.dtype;
-  g.mode = d->mode;
+  g.map_kind = RMAP_NONE;
+  g.comb_kind = RCOMB_ADD;
+  g.post_kind = RPOST_NONE;
+  g.identity = 0.0;
+  switch (d->mode) {
+  case FHIP_RED_MUL:
+    g.comb_kind = RCOMB_MUL;
+    g.identity = 1.0;
+    break;
+  case FHIP_RED_MUL_NO_ZEROS:
+    g.comb_kind = RCOMB_MUL;
+    g.map_kind = RMAP_ZERO_TO_ONE;
+    g.identity = 1.0;
+    break;
+  case FHIP_RED_MIN:
+    g.comb_kind = RCOMB_MIN;
+    g.identity = (double)INFINITY;
+    break;
+  case FHIP_RED_MAX:
+    g.comb_kind = RCOMB_MAX;
+    g.identity = -(double)INFINITY;
+    break;
+  case FHIP_RED_AMAX:
+    g.comb_kind = RCOMB_MAX;
+    g.map_kind = RMAP_ABS;
+    break;
+  case FHIP_RED_AVG:
+    g.post_kind = RPOST_MEAN;
+    break;
+  case FHIP_RED_NORM1:
+    g.map_kind = RMAP_ABS;
+    break;
+  case FHIP_RED_NORM2:
+    g.map_kind = RMAP_SQUARE;
+    g.post_kind = RPOST_SQRT;
+    break;
+  default:
+    break;
+  }
   const int64_t outs = fhip_desc_volume(d->y);
   if (needs_double(d->x.dtype))
     hipLaunchKernelGGL(generic_reduce_kernel<double>, dim3((unsigned)outs),

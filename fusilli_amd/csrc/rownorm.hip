@@ -12,6 +12,7 @@
 #include "rownorm_kernel.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 #include <vector>
@@ -62,24 +63,31 @@ bool fast_dtype(int dt) {
   return dt == FHIP_BFLOAT16 || dt == FHIP_HALF || dt == FHIP_FLOAT;
 }
 
-constexpr int kMaxChunks = 16;
-
-// Picks (chunks per lane, wavefronts per row) for a row of `inner` elements.
+// Picks (chunks per lane, wavefronts per row) for a row of `inner` elements:
+// the first instantiated pair that covers the row.  FUSILLI_HIP_ROWNORM_SHAPE
+// ("wpr,chunks") overrides the choice for tuning runs.
 bool pick_shape(int64_t inner, int vec, int *chunks, int *wpr) {
   const int64_t per_wave_chunk = 64 * (int64_t)vec;
-  int64_t need = (inner + per_wave_chunk - 1) / per_wave_chunk;
-  // One wavefront per row keeps the reduction barrier-free; use it while the
-  // row fits 8 loads per lane, else spread the row over the 4 wavefronts.
-  *wpr = need <= 8 ? 1 : 4;
-  if (*wpr == 4)
-    need = (need + 3) / 4;
-  if (need > kMaxChunks)
-    return false;
-  int c = 1;
-  while (c < need)
-    c *= 2;
-  *chunks = c;
-  return true;
+  const int64_t need = (inner + per_wave_chunk - 1) / per_wave_chunk;
+  if (const char *env = getenv("FUSILLI_HIP_ROWNORM_SHAPE")) {
+    int w = 0, c = 0;
+    if (sscanf(env, "%d,%d", &w, &c) == 2 && (int64_t)w * c >= need) {
+      for (const RowNormShape &sh : kRowNormShapes)
+        if (sh.wpr == w && sh.chunks == c) {
+          *wpr = w;
+          *chunks = c;
+          return true;
+        }
+    }
+  }
+  for (const RowNormShape &sh : kRowNormShapes) {
+    if ((int64_t)sh.wpr * sh.chunks >= need) {
+      *wpr = sh.wpr;
+      *chunks = sh.chunks;
+      return true;
+    }
+  }
+  return false;
 }
 
 } // namespace
@@ -189,17 +197,39 @@ int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
   for (int i = 0; i < epi.count; ++i)
     FHIP_REQUIRE(ctx, g.epi[i].col_unit == 0 || aligned(g.epi[i].ptr),
                  "rownorm: epilogue operand must be 16-byte aligned");
+  // Choose the compile-time specialisation that matches this call exactly.
+  int variant = RN_GENERAL;
+  const bool scale_same = scale && d->scale.dtype == d->x.dtype;
+  const bool bias_same = bias && d->bias.dtype == d->x.dtype;
+  if (!d->is_layernorm && scale_same && !bias) {
+    if (epi.count == 0) {
+      variant = RN_RMS_SCALE;
+    } else if (epi.count == 1 && g.epi[0].mode == FHIP_PW_MUL) {
+      if (g.epi[0].kind == FHIP_OPERAND_SCALAR)
+        variant = RN_RMS_SCALE_MULS;
+      else if (g.epi[0].kind == FHIP_OPERAND_TENSOR && g.epi[0].col_unit &&
+               g.epi[0].operand_dtype == d->x.dtype)
+        variant = RN_RMS_SCALE_MULT;
+    }
+  } else if (d->is_layernorm && scale_same && bias_same && epi.count == 0) {
+    variant = RN_LN_SCALE_BIAS;
+  }
+  if (getenv("FUSILLI_HIP_ROWNORM_GENERAL"))
+    variant = RN_GENERAL; // tuning / test hook: force the general kernel
+  bool launched;
   switch (d->x.dtype) {
   case FHIP_BFLOAT16:
-    rownorm_launch_bf16(chunks, wpr, g.rows, ctx->stream, g);
+    launched = rownorm_launch_bf16(chunks, wpr, variant, g.rows, ctx->stream, g);
     break;
   case FHIP_HALF:
-    rownorm_launch_f16(chunks, wpr, g.rows, ctx->stream, g);
+    launched = rownorm_launch_f16(chunks, wpr, variant, g.rows, ctx->stream, g);
     break;
   default:
-    rownorm_launch_f32(chunks, wpr, g.rows, ctx->stream, g);
+    launched = rownorm_launch_f32(chunks, wpr, variant, g.rows, ctx->stream, g);
     break;
   }
+  FHIP_REQUIRE(ctx, launched, "rownorm: no kernel for shape (%d, %d)", wpr,
+               chunks);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }

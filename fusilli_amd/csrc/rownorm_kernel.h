@@ -7,7 +7,6 @@
 
 #include <type_traits>
 
-
 struct FastEpiOp {
   int32_t mode, kind, acc_is_in1, result_dtype, operand_dtype;
   int32_t col_unit; // operand varies along the row (stride 1) or not (0)
@@ -33,6 +32,19 @@ struct RowNormArgs {
   FastEpiOp epi[FHIP_MAX_EPILOGUE];
 };
 
+// Compile-time specialisations of the per-row work.  Everything a variant
+// fixes is resolved at compile time so the hot loop is straight-line code; the
+// general variant decides the same things with wavefront-uniform branches.
+enum RowNormVariant {
+  RN_GENERAL = 0,        // any combination the predicate admits
+  RN_RMS_SCALE = 1,      // RMSNorm, scale of the row's type, no epilogue
+  RN_RMS_SCALE_MULS = 2, // ... followed by one MUL with a scalar
+  RN_RMS_SCALE_MULT = 3, // ... followed by one MUL with a full-size tensor
+                         //     of the row's type
+  RN_LN_SCALE_BIAS = 4,  // LayerNorm, scale and bias of the row's type
+  RN_VARIANT_COUNT = 5
+};
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T> struct VecOf {
@@ -40,11 +52,18 @@ template <typename T> struct VecOf {
 };
 
 template <typename T, int VEC>
-__device__ __forceinline__ void unpack16(const u32x4 &raw, float *out) {
+__device__ __forceinline__ void unpack16(const u32x4 &raw, float (&out)[VEC]) {
   const T *p = reinterpret_cast<const T *>(&raw);
 #pragma unroll
   for (int i = 0; i < VEC; ++i)
     out[i] = (float)p[i];
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec_same(const void *base, int64_t off,
+                                              float (&out)[VEC]) {
+  const u32x4 raw = *reinterpret_cast<const u32x4 *>((const T *)base + off);
+  unpack16<T, VEC>(raw, out);
 }
 
 // Loads VEC consecutive elements starting at element offset `off` as floats.
@@ -52,10 +71,9 @@ __device__ __forceinline__ void unpack16(const u32x4 &raw, float *out) {
 template <typename T, int VEC>
 __device__ __forceinline__ void load_vec_as_float(const void *base, int dt,
                                                   int dt_of_T, int64_t off,
-                                                  float *out) {
+                                                  float (&out)[VEC]) {
   if (dt == dt_of_T) {
-    const u32x4 raw = *reinterpret_cast<const u32x4 *>((const T *)base + off);
-    unpack16<T, VEC>(raw, out);
+    load_vec_same<T, VEC>(base, off, out);
   } else { // FHIP_FLOAT (the predicate admits no third type)
 #pragma unroll
     for (int i = 0; i < VEC / 4; ++i) {
@@ -80,11 +98,25 @@ template <> struct DtypeOf<float> {
   static constexpr int value = FHIP_FLOAT;
 };
 
+// Sum over the 64 lanes, result in every lane.  DPP row operations (no LDS
+// crossbar traffic) reduce each row of 16 lanes; the four row sums are then
+// read through scalar registers.
 __device__ __forceinline__ float wave_sum64(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1)
-    v += __shfl_xor(v, o, 64);
-  return v;
+  auto dpp_add = [](float x, auto ctrl) {
+    constexpr int kCtrl = decltype(ctrl)::value;
+    const int moved = __builtin_amdgcn_update_dpp(
+        0, __builtin_bit_cast(int, x), kCtrl, 0xF, 0xF, false);
+    return x + __builtin_bit_cast(float, moved);
+  };
+  v = dpp_add(v, std::integral_constant<int, 0xB1>{});  // quad_perm [1,0,3,2]
+  v = dpp_add(v, std::integral_constant<int, 0x4E>{});  // quad_perm [2,3,0,1]
+  v = dpp_add(v, std::integral_constant<int, 0x124>{}); // row_ror 4
+  v = dpp_add(v, std::integral_constant<int, 0x128>{}); // row_ror 8
+  const int bits = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
 }
 
 template <int N, typename F>
@@ -95,16 +127,47 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-// WPR = wavefronts cooperating on one row (1 or 4); a 256-thread workgroup
-// therefore covers 4 / WPR rows.  CHUNKS = 16-byte loads per lane.  The row
-// stays packed in registers (4 VGPRs per chunk) between the statistics pass
-// and the apply pass.
-template <typename T, int CHUNKS, int WPR, bool EPI>
-__global__ __launch_bounds__(256) void rownorm_kernel(RowNormArgs g) {
+// WPR = wavefronts cooperating on one row (1, 2, 4, 8 or 16); a workgroup has
+// max(4, WPR) wavefronts and covers max(1, 4 / WPR) rows.  CHUNKS = 16-byte
+// loads per lane.  Few chunks per lane and many resident wavefronts is what
+// saturates HBM on this part: occupancy, not per-lane instruction-level
+// parallelism, hides the memory latency.
+template <int WPR> struct RowNormGeom {
+  static constexpr int kWaves = WPR < 4 ? 4 : WPR;
+  static constexpr int kThreads = 64 * kWaves;
+  static constexpr int kRowsPerWg = kWaves / WPR;
+};
+
+template <int WPR>
+__device__ __forceinline__ float row_sum(float v, float *lds, int wave,
+                                         int lane) {
+  v = wave_sum64(v);
+  if constexpr (WPR > 1) {
+    __syncthreads(); // previous use of lds is complete
+    if (lane == 0)
+      lds[wave] = v;
+    __syncthreads();
+    const int first = (wave / WPR) * WPR;
+    v = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i)
+      v += lds[first + i];
+  }
+  return v;
+}
+
+// One workgroup pass: the whole row is loaded with one 16-byte load per lane
+// per chunk and stays packed in registers (4 VGPRs per chunk) between the
+// statistics pass and the apply pass.
+template <typename T, int CHUNKS, int WPR, int VARIANT>
+__global__ __launch_bounds__(RowNormGeom<WPR>::kThreads) void rownorm_kernel(
+    RowNormArgs g) {
   constexpr int VEC = VecOf<T>::kVec;
   constexpr int DT = DtypeOf<T>::value;
-  constexpr int ROWS_PER_WG = 4 / WPR;
-  __shared__ float lds[4];
+  constexpr int ROWS_PER_WG = RowNormGeom<WPR>::kRowsPerWg;
+  constexpr bool GENERAL = VARIANT == RN_GENERAL;
+  constexpr bool LAYERNORM_FIXED = VARIANT == RN_LN_SCALE_BIAS;
+  __shared__ float lds[RowNormGeom<WPR>::kWaves];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -126,10 +189,33 @@ __global__ __launch_bounds__(256) void rownorm_kernel(RowNormArgs g) {
     else
       raw[c] = u32x4{0, 0, 0, 0};
   });
+  // The specialised variants fetch everything the apply pass needs together
+  // with the row, so nothing but arithmetic follows the reduction.
+  constexpr bool PREFETCH = !GENERAL && CHUNKS <= 4;
+  constexpr int PF = PREFETCH ? CHUNKS : 1;
+  u32x4 scale_raw[PF], bias_raw[PF], mult_raw[PF];
+  if constexpr (PREFETCH) {
+    static_for<CHUNKS>([&](auto ci) {
+      constexpr int c = decltype(ci)::value;
+      const int col = col0 + c * COL_STEP;
+      if (row_ok && col < inner) {
+        scale_raw[c] =
+            *reinterpret_cast<const u32x4 *>((const T *)g.scale + col);
+        if constexpr (VARIANT == RN_LN_SCALE_BIAS)
+          bias_raw[c] =
+              *reinterpret_cast<const u32x4 *>((const T *)g.bias + col);
+        if constexpr (VARIANT == RN_RMS_SCALE_MULT)
+          mult_raw[c] = __builtin_nontemporal_load(
+              reinterpret_cast<const u32x4 *>((const T *)g.epi[0].ptr +
+                                              row * g.epi[0].row_stride + col));
+      }
+    });
+  }
 
+  const bool layernorm = GENERAL ? g.is_layernorm != 0 : LAYERNORM_FIXED;
   const float inv_n = 1.0f / (float)inner;
   float mean = 0.f;
-  if (g.is_layernorm) {
+  if (layernorm) {
     float s = 0.f;
     static_for<CHUNKS>([&](auto ci) {
       constexpr int c = decltype(ci)::value;
@@ -139,39 +225,32 @@ __global__ __launch_bounds__(256) void rownorm_kernel(RowNormArgs g) {
       for (int i = 0; i < VEC; ++i)
         s += v[i];
     });
-    s = wave_sum64(s);
-    if (WPR > 1) {
-      if (lane == 0)
-        lds[wave] = s;
-      __syncthreads();
-      s = lds[0] + lds[1] + lds[2] + lds[3];
-      __syncthreads();
-    }
-    mean = s * inv_n;
+    mean = row_sum<WPR>(s, lds, wave, lane) * inv_n;
   }
   float ss = 0.f;
   static_for<CHUNKS>([&](auto ci) {
     constexpr int c = decltype(ci)::value;
-    const bool live = col0 + c * COL_STEP < inner;
     float v[VEC];
     unpack16<T, VEC>(raw[c], v);
+    if (layernorm) {
+      const bool live = col0 + c * COL_STEP < inner;
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      const float d = live ? v[i] - mean : 0.f;
-      ss += d * d;
+      for (int i = 0; i < VEC; ++i) {
+        const float d = live ? v[i] - mean : 0.f;
+        ss += d * d;
+      }
+    } else { // padding chunks hold zeros
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        ss += v[i] * v[i];
     }
   });
-  ss = wave_sum64(ss);
-  if (WPR > 1) {
-    if (lane == 0)
-      lds[wave] = ss;
-    __syncthreads();
-    ss = lds[0] + lds[1] + lds[2] + lds[3];
-  }
+  ss = row_sum<WPR>(ss, lds, wave, lane);
   const float rstd = 1.0f / sqrtf(ss * inv_n + g.eps);
   if (!row_ok)
     return;
-  if (g.emit_stats && lane == 0 && wave_in_row == 0) {
+  if ((GENERAL || LAYERNORM_FIXED) && g.emit_stats && lane == 0 &&
+      wave_in_row == 0) {
     if (g.stats_dt == FHIP_FLOAT) {
       ((float *)g.mean)[row] = mean;
       ((float *)g.rstd)[row] = rstd;
@@ -192,61 +271,95 @@ __global__ __launch_bounds__(256) void rownorm_kernel(RowNormArgs g) {
       return;
     float y[VEC];
     unpack16<T, VEC>(raw[c], y);
+    if (layernorm) {
 #pragma unroll
-    for (int i = 0; i < VEC; ++i)
-      y[i] = (y[i] - mean) * rstd;
-    if (g.scale) {
+      for (int i = 0; i < VEC; ++i)
+        y[i] = (y[i] - mean) * rstd;
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        y[i] *= rstd;
+    }
+
+    if constexpr (GENERAL) {
+      if (g.scale) {
+        float s[VEC];
+        load_vec_as_float<T, VEC>(g.scale, g.scale_dt, DT, col, s);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          y[i] *= s[i];
+      }
+      if (g.bias) {
+        float b[VEC];
+        load_vec_as_float<T, VEC>(g.bias, g.bias_dt, DT, col, b);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i)
+          y[i] += b[i];
+      }
+    } else {
       float s[VEC];
-      load_vec_as_float<T, VEC>(g.scale, g.scale_dt, DT, col, s);
+      if constexpr (PREFETCH)
+        unpack16<T, VEC>(scale_raw[c], s);
+      else
+        load_vec_same<T, VEC>(g.scale, col, s);
 #pragma unroll
       for (int i = 0; i < VEC; ++i)
         y[i] *= s[i];
-    }
-    if (g.bias) {
-      float b[VEC];
-      load_vec_as_float<T, VEC>(g.bias, g.bias_dt, DT, col, b);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i)
-        y[i] += b[i];
-    }
-    if (g.y_dt != FHIP_FLOAT) {
-#pragma unroll
-      for (int i = 0; i < VEC; ++i)
-        y[i] = fhip_round_fast(g.y_dt, y[i]);
-    }
-    for (int e = 0; EPI && e < g.epi_count; ++e) {
-      const FastEpiOp &o = g.epi[e];
-      if (o.kind == FHIP_OPERAND_NONE) {
+      if constexpr (VARIANT == RN_LN_SCALE_BIAS) {
+        float b[VEC];
+        if constexpr (PREFETCH)
+          unpack16<T, VEC>(bias_raw[c], b);
+        else
+          load_vec_same<T, VEC>(g.bias, col, b);
 #pragma unroll
         for (int i = 0; i < VEC; ++i)
-          y[i] = fhip_pw_fast_unary<false>(o.mode, y[i], o.params.swish_beta);
-      } else {
-        float other[VEC];
-        if (o.kind == FHIP_OPERAND_SCALAR) {
-#pragma unroll
-          for (int i = 0; i < VEC; ++i)
-            other[i] = o.scalar;
-        } else if (o.col_unit) {
-          load_vec_as_float<T, VEC>(o.ptr, o.operand_dtype, DT,
-                                    row * o.row_stride + col, other);
-        } else {
-          const float s =
-              o.operand_dtype == DT
-                  ? (float)((const T *)o.ptr)[row * o.row_stride]
-                  : ((const float *)o.ptr)[row * o.row_stride];
-#pragma unroll
-          for (int i = 0; i < VEC; ++i)
-            other[i] = s;
-        }
-#pragma unroll
-        for (int i = 0; i < VEC; ++i)
-          y[i] = o.acc_is_in1 ? fhip_pw_fast_binary(o.mode, other[i], y[i])
-                              : fhip_pw_fast_binary(o.mode, y[i], other[i]);
+          y[i] += b[i];
       }
-      if (o.result_dtype != FHIP_FLOAT) {
+    }
+    fhip_round_fast_vec<VEC>(g.y_dt, y);
+
+    if constexpr (VARIANT == RN_RMS_SCALE_MULS) {
+      const float m = g.epi[0].scalar;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i)
-          y[i] = fhip_round_fast(o.result_dtype, y[i]);
+      for (int i = 0; i < VEC; ++i)
+        y[i] *= m;
+      fhip_round_fast_vec<VEC>(g.epi[0].result_dtype, y);
+    } else if constexpr (VARIANT == RN_RMS_SCALE_MULT) {
+      float o[VEC];
+      if constexpr (PREFETCH)
+        unpack16<T, VEC>(mult_raw[c], o);
+      else
+        load_vec_same<T, VEC>(g.epi[0].ptr, row * g.epi[0].row_stride + col, o);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i)
+        y[i] *= o[i];
+      fhip_round_fast_vec<VEC>(g.epi[0].result_dtype, y);
+    } else if constexpr (GENERAL) {
+      for (int e = 0; e < g.epi_count; ++e) {
+        const FastEpiOp &o = g.epi[e];
+        if (o.kind == FHIP_OPERAND_NONE) {
+          fhip_pw_fast_unary_vec<false, VEC>(o.mode, y, o.params.swish_beta);
+        } else {
+          float other[VEC];
+          if (o.kind == FHIP_OPERAND_SCALAR) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+              other[i] = o.scalar;
+          } else if (o.col_unit) {
+            load_vec_as_float<T, VEC>(o.ptr, o.operand_dtype, DT,
+                                      row * o.row_stride + col, other);
+          } else {
+            const float s =
+                o.operand_dtype == DT
+                    ? (float)((const T *)o.ptr)[row * o.row_stride]
+                    : ((const float *)o.ptr)[row * o.row_stride];
+#pragma unroll
+            for (int i = 0; i < VEC; ++i)
+              other[i] = s;
+          }
+          fhip_pw_fast_binary_vec<VEC>(o.mode, o.acc_is_in1 != 0, y, other);
+        }
+        fhip_round_fast_vec<VEC>(o.result_dtype, y);
       }
     }
     u32x4 packed;
@@ -258,58 +371,73 @@ __global__ __launch_bounds__(256) void rownorm_kernel(RowNormArgs g) {
   });
 }
 
+// (wavefronts per row, chunks per lane) pairs that are instantiated.  A row of
+// N 16-byte-per-lane wavefront-chunks uses the first pair whose product
+// covers N.
+struct RowNormShape {
+  int wpr, chunks;
+};
+constexpr RowNormShape kRowNormShapes[] = {
+    {1, 1}, {1, 2}, {2, 2}, {4, 2}, {8, 2}, {16, 2}, {16, 4}, {16, 8}, {16, 16},
+};
 
-template <typename T, int WPR, bool EPI>
-void launch_chunks(int chunks, dim3 grid, hipStream_t s, const RowNormArgs &g) {
-  switch (chunks) {
-  case 1:
-    if constexpr (WPR == 1)
-      hipLaunchKernelGGL((rownorm_kernel<T, 1, WPR, EPI>), grid, dim3(256), 0, s, g);
-    else
-      hipLaunchKernelGGL((rownorm_kernel<T, 4, WPR, EPI>), grid, dim3(256), 0, s, g);
+template <typename T, int WPR, int CHUNKS>
+void rownorm_launch_one(int variant, int64_t rows, hipStream_t s,
+                        const RowNormArgs &g) {
+  constexpr int rpw = RowNormGeom<WPR>::kRowsPerWg;
+  const dim3 grid((unsigned)((rows + rpw - 1) / rpw));
+  const dim3 block(RowNormGeom<WPR>::kThreads);
+  switch (variant) {
+  case RN_RMS_SCALE:
+    hipLaunchKernelGGL((rownorm_kernel<T, CHUNKS, WPR, RN_RMS_SCALE>), grid,
+                       block, 0, s, g);
     break;
-  case 2:
-    if constexpr (WPR == 1)
-      hipLaunchKernelGGL((rownorm_kernel<T, 2, WPR, EPI>), grid, dim3(256), 0, s, g);
-    else
-      hipLaunchKernelGGL((rownorm_kernel<T, 4, WPR, EPI>), grid, dim3(256), 0, s, g);
+  case RN_RMS_SCALE_MULS:
+    hipLaunchKernelGGL((rownorm_kernel<T, CHUNKS, WPR, RN_RMS_SCALE_MULS>),
+                       grid, block, 0, s, g);
     break;
-  case 4:
-    hipLaunchKernelGGL((rownorm_kernel<T, 4, WPR, EPI>), grid, dim3(256), 0, s, g);
+  case RN_RMS_SCALE_MULT:
+    hipLaunchKernelGGL((rownorm_kernel<T, CHUNKS, WPR, RN_RMS_SCALE_MULT>),
+                       grid, block, 0, s, g);
     break;
-  case 8:
-    hipLaunchKernelGGL((rownorm_kernel<T, 8, WPR, EPI>), grid, dim3(256), 0, s, g);
+  case RN_LN_SCALE_BIAS:
+    hipLaunchKernelGGL((rownorm_kernel<T, CHUNKS, WPR, RN_LN_SCALE_BIAS>), grid,
+                       block, 0, s, g);
     break;
   default:
-    if constexpr (WPR == 4)
-      hipLaunchKernelGGL((rownorm_kernel<T, 16, WPR, EPI>), grid, dim3(256), 0, s, g);
+    hipLaunchKernelGGL((rownorm_kernel<T, CHUNKS, WPR, RN_GENERAL>), grid,
+                       block, 0, s, g);
     break;
   }
 }
 
+// Returns false when (wpr, chunks) is not an instantiated pair.
 template <typename T>
-void rownorm_launch_typed(int chunks, int wpr, int64_t rows, hipStream_t s,
-                          const RowNormArgs &g) {
-  const dim3 grid1((unsigned)((rows + 3) / 4)), grid4((unsigned)rows);
-  if (g.epi_count == 0) {
-    if (wpr == 1)
-      launch_chunks<T, 1, false>(chunks, grid1, s, g);
-    else
-      launch_chunks<T, 4, false>(chunks, grid4, s, g);
-  } else {
-    if (wpr == 1)
-      launch_chunks<T, 1, true>(chunks, grid1, s, g);
-    else
-      launch_chunks<T, 4, true>(chunks, grid4, s, g);
+bool rownorm_launch_typed(int chunks, int wpr, int variant, int64_t rows,
+                          hipStream_t s, const RowNormArgs &g) {
+#define FHIP_ROWNORM_CASE(W, C)                                                \
+  if (wpr == W && chunks == C) {                                               \
+    rownorm_launch_one<T, W, C>(variant, rows, s, g);                          \
+    return true;                                                               \
   }
+  FHIP_ROWNORM_CASE(1, 1)
+  FHIP_ROWNORM_CASE(1, 2)
+  FHIP_ROWNORM_CASE(2, 2)
+  FHIP_ROWNORM_CASE(4, 2)
+  FHIP_ROWNORM_CASE(8, 2)
+  FHIP_ROWNORM_CASE(16, 2)
+  FHIP_ROWNORM_CASE(16, 4)
+  FHIP_ROWNORM_CASE(16, 8)
+  FHIP_ROWNORM_CASE(16, 16)
+#undef FHIP_ROWNORM_CASE
+  return false;
 }
 
-
-void rownorm_launch_bf16(int chunks, int wpr, int64_t rows, hipStream_t s,
-                         const RowNormArgs &g);
-void rownorm_launch_f16(int chunks, int wpr, int64_t rows, hipStream_t s,
-                        const RowNormArgs &g);
-void rownorm_launch_f32(int chunks, int wpr, int64_t rows, hipStream_t s,
-                        const RowNormArgs &g);
+bool rownorm_launch_bf16(int chunks, int wpr, int variant, int64_t rows,
+                         hipStream_t s, const RowNormArgs &g);
+bool rownorm_launch_f16(int chunks, int wpr, int variant, int64_t rows,
+                        hipStream_t s, const RowNormArgs &g);
+bool rownorm_launch_f32(int chunks, int wpr, int variant, int64_t rows,
+                        hipStream_t s, const RowNormArgs &g);
 
 #endif // FUSILLI_AMD_CSRC_ROWNORM_KERNEL_H

@@ -160,7 +160,7 @@ def test_conv_3x3_same_pad_corner_known_answer(ctx):
 @pytest.mark.parametrize("case", [
     dict(x=[2, 6, 9, 11], w=[4, 6, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
     dict(x=[2, 6, 9, 11], w=[4, 3, 3, 2], pad=[0, 1], s=[2, 1], d=[1, 2]),
-    dict(x=[1, 8, 13], w=[6, 2, 4], pad=[2], s=[3], d=[2]),
+    dict(x=[1, 8, 13], w=[8, 2, 4], pad=[2], s=[3], d=[2]),
     dict(x=[1, 4, 5, 6, 7], w=[2, 4, 2, 3, 3], pad=[1, 0, 1], s=[1, 2, 1], d=[1, 1, 1]),
 ])
 @pytest.mark.parametrize("dtype", [capi.FLOAT, capi.BFLOAT16])
