@@ -1,4 +1,206 @@
+// MFMA GEMM for gfx950: C[b] = A[b] x B[b] with fused pointwise epilogue.
+//
+//   * element types: bf16 / f16 (v_mfma_f32_32x32x16), int8
+//     (v_mfma_i32_32x32x32_i8, exact int32 accumulate) and OCP fp8 e4m3 / e5m2
+//     (v_mfma_f32_32x32x64_f8f6f4);
+//   * either operand may be K-contiguous or M/N-contiguous (the reference
+//     expresses transposes purely by strides, node/matmul_node.h:240-252):
+//     K-contiguous tiles are read from LDS with 16-byte loads, the other kind
+//     with the gfx950 transposing LDS reads (ds_read_b64_tr_b16 / _tr_b8), so
+//     no operand is ever transposed in registers or in HBM;
+//   * 256 threads = 2 x 2 wavefronts per workgroup, each wavefront owning a
+//     (BM/2) x (BN/2) block of 32x32 MFMA tiles; K advances in 128-byte slices
+//     through double-buffered, bank-conflict-padded LDS with the next slice's
+//     global loads in flight during the MFMAs of the current one;
+//   * workgroup ids are remapped so that the workgroups resident on one XCD
+//     (one L2) cover a compact block of output tiles.
+//
+// Reference semantics: aten.matmul (reference support/asm_emitter.h:1669-1696).
 #include "common.h"
 #include "fast_paths.h"
-bool fhip_fast_matmul_applicable(const fhip_matmul_desc *) { return false; }
-int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *, const void *, const void *, const DevEpilogue &, void *) { return fhip_fail(ctx, "no fast matmul"); }
+#include "gemm_kernel.h"
+
+#include <cstdlib>
+#include <type_traits>
+
+namespace {
+
+// ---- host side --------------------------------------------------------------
+bool kind_for(int a_dt, int b_dt, int *kind) {
+  if (a_dt != b_dt)
+    return false;
+  switch (a_dt) {
+  case FHIP_BFLOAT16:
+    *kind = GK_BF16;
+    return true;
+  case FHIP_HALF:
+    *kind = GK_F16;
+    return true;
+  case FHIP_INT8:
+    *kind = GK_I8;
+    return true;
+  case FHIP_FP8E4M3:
+    *kind = GK_FP8E4M3;
+    return true;
+  case FHIP_FP8E5M2:
+    *kind = GK_FP8E5M2;
+    return true;
+  default:
+    return false;
+  }
+}
+
+GemmPlan make_plan(const fhip_matmul_desc *d) {
+  GemmPlan p;
+  const int r = d->a.rank;
+  if (r != 2 && r != 3)
+    return p;
+  if (!kind_for(d->a.dtype, d->b.dtype, &p.kind))
+    return p;
+  const int elem = fhip_dtype_size(d->a.dtype);
+  p.M = d->a.dim[r - 2];
+  p.K = d->a.dim[r - 1];
+  p.N = d->b.dim[r - 1];
+  p.batch = r == 3 ? d->c.dim[0] : 1;
+  // operand orientation from strides
+  const int64_t a_sm = d->a.stride[r - 2], a_sk = d->a.stride[r - 1];
+  const int64_t b_sk = d->b.stride[r - 2], b_sn = d->b.stride[r - 1];
+  if (a_sk == 1 || p.K == 1) {
+    p.a_kc = true;
+    p.a_ld = p.M == 1 ? p.K : a_sm;
+  } else if (a_sm == 1 || p.M == 1) {
+    p.a_kc = false;
+    p.a_ld = a_sk;
+  } else {
+    return p;
+  }
+  if (b_sk == 1 || p.K == 1) {
+    p.b_kc = true;
+    p.b_ld = p.N == 1 ? p.K : b_sn;
+  } else if (b_sn == 1 || p.N == 1) {
+    p.b_kc = false;
+    p.b_ld = b_sk;
+  } else {
+    return p;
+  }
+  // whole 128-byte K slices; 16-byte aligned rows; tiles no larger than the
+  // matrix so edge clamping stays in bounds
+  if ((p.K * elem) % kTileKBytes != 0)
+    return p;
+  if ((p.a_ld * elem) % 16 != 0 || (p.b_ld * elem) % 16 != 0)
+    return p;
+  if (p.a_kc ? p.a_ld < p.K : p.a_ld < p.M)
+    return p;
+  if (p.b_kc ? p.b_ld < p.K : p.b_ld < p.N)
+    return p;
+  if (p.M < 128 || p.N < 128)
+    return p;
+  // M/N-contiguous operands are moved in 16-byte column chunks
+  if (!p.a_kc && (p.M * elem) % 16 != 0)
+    return p;
+  if (!p.b_kc && (p.N * elem) % 16 != 0)
+    return p;
+  if (r == 3) {
+    p.a_batch = d->a.dim[0] == 1 ? 0 : d->a.stride[0];
+    p.b_batch = d->b.dim[0] == 1 ? 0 : d->b.stride[0];
+    p.o_batch = d->out.dim[0] == 1 ? 0 : d->out.stride[0];
+    if ((p.a_batch * elem) % 16 != 0 || (p.b_batch * elem) % 16 != 0)
+      return p;
+  }
+  p.o_sm = d->out.stride[r - 2];
+  p.o_sn = d->out.stride[r - 1];
+  // result / epilogue constraints
+  if (p.kind == GK_I8) {
+    if (d->c.dtype != FHIP_INT32 || d->out.dtype != FHIP_INT32 ||
+        d->epilogue.count != 0)
+      return p;
+  } else {
+    auto f = [](int dt) {
+      return dt == FHIP_FLOAT || dt == FHIP_BFLOAT16 || dt == FHIP_HALF;
+    };
+    if (!f(d->c.dtype) || !f(d->out.dtype) ||
+        !fhip_epilogue_is_fast(d->epilogue))
+      return p;
+    for (int i = 0; i < d->epilogue.count; ++i) {
+      const fhip_epilogue_op &o = d->epilogue.op[i];
+      if (o.operand_kind == FHIP_OPERAND_TENSOR && !f(o.operand.dtype))
+        return p;
+    }
+  }
+  // tile shape: biggest tile that still gives every CU work
+  p.bm = p.M >= 256 ? 256 : 128;
+  p.bn = p.N >= 256 && p.bm == 256 ? 256 : 128;
+  const int64_t big_tiles =
+      ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn) * p.batch;
+  if (big_tiles < 200) {
+    if (p.bm == 256 && p.bn == 256)
+      p.bn = 128;
+    const int64_t t2 =
+        ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn) * p.batch;
+    if (t2 < 200 && p.bm == 256)
+      p.bm = 128;
+  }
+  if (const char *env = getenv("FUSILLI_HIP_GEMM_TILE")) {
+    int bm = 0, bn = 0;
+    if (sscanf(env, "%d,%d", &bm, &bn) == 2 && (bm == 128 || bm == 256) &&
+        (bn == 128 || bn == 256) && bm >= bn && bm <= p.M && bn <= p.N)
+      p.bm = bm, p.bn = bn;
+  }
+  p.ok = true;
+  return p;
+}
+
+} // namespace
+
+bool fhip_fast_matmul_applicable(const fhip_matmul_desc *d) {
+  return make_plan(d).ok;
+}
+
+int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
+                     const void *b, const DevEpilogue &epi, void *out) {
+  const GemmPlan p = make_plan(d);
+  FHIP_REQUIRE(ctx, p.ok, "gemm: descriptor not supported by the MFMA kernel");
+  FHIP_REQUIRE(ctx, ((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0,
+               "gemm: A and B must be 16-byte aligned");
+  GemmArgs g{};
+  g.a = (const char *)a;
+  g.b = (const char *)b;
+  g.out = (char *)out;
+  g.M = p.M;
+  g.N = p.N;
+  g.K = p.K;
+  g.a_ld = p.a_ld;
+  g.b_ld = p.b_ld;
+  g.a_batch = p.a_batch;
+  g.b_batch = p.b_batch;
+  g.o_sm = p.o_sm;
+  g.o_sn = p.o_sn;
+  g.o_batch = p.o_batch;
+  g.c_dt = d->c.dtype;
+  g.o_dt = d->out.dtype;
+  g.tiles_m = (int)((p.M + p.bm - 1) / p.bm);
+  g.tiles_n = (int)((p.N + p.bn - 1) / p.bn);
+  // epilogue strides on (batch, m, n)
+  g.epi = epi;
+  g.epi.rank = 3;
+  const int r = d->a.rank;
+  for (int i = 0; i < epi.count; ++i) {
+    const DevEpiOp &s = epi.op[i];
+    DevEpiOp &o = g.epi.op[i];
+    o.stride[0] = r == 3 ? s.stride[0] : 0;
+    o.stride[1] = s.stride[r - 2];
+    o.stride[2] = s.stride[r - 1];
+  }
+  switch (p.kind) {
+  case GK_BF16:
+    return gemm_launch_bf16(ctx, p, g);
+  case GK_F16:
+    return gemm_launch_f16(ctx, p, g);
+  case GK_I8:
+    return gemm_launch_i8(ctx, p, g);
+  case GK_FP8E4M3:
+    return gemm_launch_fp8e4m3(ctx, p, g);
+  default:
+    return gemm_launch_fp8e5m2(ctx, p, g);
+  }
+}
