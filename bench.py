@@ -96,6 +96,48 @@ def bench_rmsnorm(ctx, steps, warmup, mul_kind="scalar", sets=5):
             "sets": sets}
 
 
+# ---------------------------------------------------------------------------
+# Matmul configs (C5a int8 -> int32, C5b fp8 -> bf16 with scales, bf16 GEMM)
+# ---------------------------------------------------------------------------
+def matmul_desc(m, n, k, in_dt, c_dt, out_dt, epilogue=()):
+    d = capi.MatmulDesc()
+    d.a = capi.TensorDesc.make([m, k], [k, 1], in_dt)
+    d.b = capi.TensorDesc.make([k, n], [n, 1], in_dt)
+    d.c = capi.TensorDesc.make([m, n], [n, 1], c_dt)
+    d.out = capi.TensorDesc.make([m, n], [n, 1], out_dt)
+    d.out_dtype = out_dt
+    d.epilogue = capi.make_epilogue(list(epilogue))
+    return d
+
+
+def bench_matmul(ctx, steps, warmup, kind, m=4096, n=4096, k=8192):
+    if kind == "int8":
+        in_dt, c_dt, out_dt, epi = capi.INT8, capi.INT32, capi.INT32, ()
+        gen = lambda tid, cnt: synth.integers(5, tid, cnt, -127, 127).astype(np.int8)
+        peak = PEAK_TFLOPS["int8"]
+    elif kind == "fp8":
+        in_dt, c_dt, out_dt = capi.FP8E4M3, capi.FLOAT, capi.BFLOAT16
+        epi = (capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16, scalar=1.0 / (448.0 * 448.0)),)
+        gen = lambda tid, cnt: synth.f32_to_fp8_bits(synth.uniform(6, tid, cnt) * 448.0, 4)
+        peak = PEAK_TFLOPS["fp8"]
+    else:
+        in_dt, c_dt, out_dt, epi = capi.BFLOAT16, capi.FLOAT, capi.BFLOAT16, ()
+        gen = lambda tid, cnt: synth.f32_to_bf16_bits(synth.normal(7, tid, cnt))
+        peak = PEAK_TFLOPS["bf16"]
+    d = matmul_desc(m, n, k, in_dt, c_dt, out_dt, epi)
+    assert ctx.lib.fhip_matmul_supported(d) == 2, "MFMA kernel not chosen"
+    a = ctx.to_device(gen(0, m * k))
+    b = ctx.to_device(gen(1, k * n))
+    out = ctx.alloc(m * n * capi.DTYPE_SIZE[out_dt])
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.matmul(d, a, b, out),
+                                steps, warmup)
+    flop = 2.0 * m * n * k
+    return {"value": round(flop / ev_ms / 1e9, 1),
+            "unit": "TOP/s" if kind == "int8" else "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / peak, 4),
+            "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
+
+
 def cpu_baseline_rmsnorm(seconds_budget=12.0):
     """The oracle's bf16 RMSNorm * scalar on the host cores over a row sample."""
     from oracle import oracle
@@ -166,11 +208,13 @@ def main():
             "value": round(r2["gbs_kernel"], 1), "unit": "GB/s",
             "frac_of_hbm_peak": round(r2["gbs_kernel"] / HBM_PEAK_GBS, 4),
             "kernel_us": round(r2["kernel_ms"] * 1e3, 2), "bytes": r2["bytes"]}
-        try:
-            import bench_configs
-            others.update(bench_configs.run_all(ctx, args.steps, args.warmup))
-        except ImportError:
-            pass
+        ksteps, kwarm = max(10, args.steps // 10), max(3, args.warmup // 5)
+        others["matmul_int8_4096x8192x4096_i32"] = bench_matmul(
+            ctx, ksteps, kwarm, "int8")
+        others["matmul_fp8e4m3_4096x8192x4096_scaled_bf16_out"] = bench_matmul(
+            ctx, ksteps, kwarm, "fp8")
+        others["matmul_bf16_4096x4096x4096"] = bench_matmul(
+            ctx, ksteps, kwarm, "bf16", 4096, 4096, 4096)
         line["others"] = others
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_rmsnorm()

@@ -1,0 +1,467 @@
+// Graph: the user-facing builder and executor.
+//
+// Same surface as the reference's graph/graph.h:75-401 (builders, validate,
+// compile, compileToArtifact, loadFromArtifact, getWorkspaceSize, execute) and
+// the same state machine and error behaviour (NotValidated / NotCompiled /
+// VariantPackError / InvalidArgument cases of backend/runtime.h:383-529).
+// compile() plans kernels (plan.h) instead of emitting MLIR for iree-compile;
+// execute() launches them through the C ABI instead of invoking a VM.
+#ifndef FUSILLI_GRAPH_H
+#define FUSILLI_GRAPH_H
+
+#include <array>
+#include <optional>
+#include <set>
+#include <span>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "plan.h"
+
+namespace fusilli {
+
+class Graph : public INode {
+public:
+  Graph() : INode(Context{}) {}
+  Graph(const Graph &) = delete;
+  Graph &operator=(const Graph &) = delete;
+  Graph(Graph &&) noexcept = default;
+  Graph &operator=(Graph &&) noexcept = default;
+  ~Graph() = default;
+
+  const std::string &getName() const override final {
+    return context.getName();
+  }
+  Type getType() const override final { return Type::Composite; }
+
+  Graph &setName(const std::string &name) {
+    context.setName(name);
+    return *this;
+  }
+  Graph &setIODataType(DataType t) {
+    context.setIODataType(t);
+    return *this;
+  }
+  Graph &setComputeDataType(DataType t) {
+    context.setComputeDataType(t);
+    return *this;
+  }
+  Graph &setIntermediateDataType(DataType t) {
+    context.setIntermediateDataType(t);
+    return *this;
+  }
+
+  // ---- validation -----------------------------------------------------------
+  ErrorObject validate() {
+    FUSILLI_LOG_LABEL_ENDL("INFO: Validating Graph");
+    FUSILLI_RETURN_ERROR_IF(getName().empty(), ErrorCode::AttributeNotSet,
+                            "Graph name not set");
+    FUSILLI_CHECK_ERROR(validateSubtree());
+    for (const auto &in : fullGraphInputs_)
+      FUSILLI_CHECK_ERROR(in->validate());
+    for (const auto &out : fullGraphOutputs_) {
+      FUSILLI_CHECK_ERROR(out->validate());
+      FUSILLI_RETURN_ERROR_IF(
+          out->hasBroadcastDims(), ErrorCode::InvalidAttribute,
+          "Tensor '" + out->getName() +
+              "' has broadcast strides (stride=0) on an operation output, "
+              "which is not yet supported");
+    }
+    isValidated_ = true;
+    return ok();
+  }
+
+  // ---- compilation ------------------------------------------------------------
+  // JIT: plan for the handle's backend and load the plan.
+  ErrorObject compile(const Handle &handle, bool remove = false) {
+    FUSILLI_ASSIGN_OR_RETURN(auto bytes,
+                             compileToArtifact(handle.getBackend(), remove));
+    return loadFromArtifact(handle, bytes);
+  }
+
+  // AOT: the serialised plan.  Needs no handle; does not disturb a loaded
+  // plan.  `remove` is accepted for source compatibility (there is no
+  // on-disk cache to clean).
+  ErrorOr<std::vector<uint8_t>> compileToArtifact(Backend backend,
+                                                  bool remove = false) {
+    (void)remove;
+    FUSILLI_RETURN_ERROR_IF(!isValidated_, ErrorCode::NotValidated,
+                            "Graph must be validated before being compiled");
+    plan::Planner planner(subNodes_, fullGraphInputsSorted_,
+                          fullGraphOutputsSorted_, backend);
+    FUSILLI_ASSIGN_OR_RETURN(plan::Plan p, planner.run());
+    return ok(plan::serialize(p));
+  }
+
+  // Loads a plan produced by this or an identically built graph.  Replaces
+  // any previously loaded plan; on failure the graph is left not loaded.
+  ErrorObject loadFromArtifact(const Handle &handle,
+                               std::span<const uint8_t> bytes) {
+    FUSILLI_RETURN_ERROR_IF(
+        !isValidated_, ErrorCode::NotValidated,
+        "Graph must be validated before loading a compiled artifact");
+    clearRuntimeState();
+    auto parsed = plan::deserialize(bytes);
+    if (isError(parsed))
+      return ErrorObject(parsed);
+    FUSILLI_RETURN_ERROR_IF(
+        parsed->backend != static_cast<uint32_t>(handle.getBackend()),
+        ErrorCode::RuntimeFailure,
+        std::string("Artifact was compiled for backend ") +
+            backendName(static_cast<Backend>(parsed->backend)) +
+            " but the handle is for backend " +
+            backendName(handle.getBackend()));
+    // The artifact must describe this graph: re-plan and compare signatures.
+    plan::Planner planner(subNodes_, fullGraphInputsSorted_,
+                          fullGraphOutputsSorted_, handle.getBackend());
+    auto own = planner.run();
+    if (isError(own))
+      return ErrorObject(own);
+    FUSILLI_RETURN_ERROR_IF(own->signature != parsed->signature,
+                            ErrorCode::RuntimeFailure,
+                            "Artifact does not match this graph (signature "
+                            "mismatch)");
+    loadedPlan_ = std::move(*parsed);
+    loadedBackend_ = handle.getBackend();
+    return ok();
+  }
+
+  // nullopt until a plan is loaded; must be called before execute().
+  ErrorOr<std::optional<size_t>> getWorkspaceSize() {
+    if (!loadedPlan_.has_value())
+      return ok(std::optional<size_t>());
+    const size_t need = static_cast<size_t>(loadedPlan_->workspaceBytes);
+    if (!workspaceSize_.has_value() || need > *workspaceSize_)
+      workspaceSize_ = need;
+    return ok(workspaceSize_);
+  }
+  [[deprecated("Use Graph::getWorkspaceSize() instead.")]]
+  ErrorOr<std::optional<size_t>> getWorkspaceSizeOrError() {
+    return getWorkspaceSize();
+  }
+
+  // ---- execution ----------------------------------------------------------------
+  // Results are written in place into the caller's output buffers; on AMDGPU
+  // the call returns once the kernels are queued on the handle's stream.
+  ErrorObject
+  execute(const Handle &handle,
+          const std::unordered_map<std::shared_ptr<TensorAttr>,
+                                   std::shared_ptr<Buffer>> &variantPack,
+          const std::shared_ptr<Buffer> &workspace) const {
+    FUSILLI_LOG_LABEL_ENDL("INFO: Executing Graph");
+    FUSILLI_RETURN_ERROR_IF(!loadedPlan_.has_value(), ErrorCode::NotCompiled,
+                            "Graph::execute requires a successful compile() "
+                            "first (no plan loaded)");
+    FUSILLI_RETURN_ERROR_IF(!loadedBackend_.has_value(), ErrorCode::NotCompiled,
+                            "Graph::execute requires a successful compile() "
+                            "first (loaded backend not set)");
+    FUSILLI_RETURN_ERROR_IF(
+        handle.getBackend() != *loadedBackend_, ErrorCode::InvalidArgument,
+        std::string("Graph::execute got a handle for backend ") +
+            backendName(handle.getBackend()) +
+            ", but the loaded artifact uses backend " +
+            backendName(*loadedBackend_));
+    FUSILLI_RETURN_ERROR_IF(
+        !workspaceSize_.has_value(), ErrorCode::InvalidArgument,
+        "Graph::execute requires getWorkspaceSize() to be called before "
+        "workspace allocation and execution");
+
+    std::vector<void *> args;
+    args.reserve(loadedPlan_->args.size());
+    auto push = [&](const std::shared_ptr<TensorAttr> &t) -> ErrorObject {
+      const std::shared_ptr<Buffer> &buf = variantPack.at(t);
+      FUSILLI_RETURN_ERROR_IF(!buf || buf->data() == nullptr,
+                              ErrorCode::VariantPackError,
+                              "Tensor '" + t->getName() +
+                                  "' has a null buffer in variantPack");
+      const plan::ArgInfo &info = loadedPlan_->args[args.size()];
+      FUSILLI_RETURN_ERROR_IF(
+          buf->sizeInBytes() < info.minBytes, ErrorCode::VariantPackError,
+          "Buffer for tensor '" + t->getName() + "' holds " +
+              std::to_string(buf->sizeInBytes()) + " bytes but the tensor "
+              "needs " + std::to_string(info.minBytes));
+      // A typed buffer must at least agree on the element width (raw byte
+      // carriers for fp8 and workspaces are untyped or one byte wide).
+      FUSILLI_RETURN_ERROR_IF(
+          buf->isTyped() &&
+              dataTypeSize(buf->getDataType()) !=
+                  dataTypeSize(static_cast<DataType>(info.dtype)),
+          ErrorCode::VariantPackError,
+          "Buffer for tensor '" + t->getName() + "' has element type " +
+              dataTypeAsm(buf->getDataType()) + " but the tensor is " +
+              dataTypeAsm(static_cast<DataType>(info.dtype)));
+      args.push_back(buf->data());
+      return ok();
+    };
+    for (const auto &out : fullGraphOutputsSorted_) {
+      if (out->isVirtual()) {
+        FUSILLI_RETURN_ERROR_IF(variantPack.contains(out),
+                                ErrorCode::VariantPackError,
+                                "Virtual output tensor found in variantPack");
+        continue;
+      }
+      FUSILLI_RETURN_ERROR_IF(!variantPack.contains(out),
+                              ErrorCode::VariantPackError,
+                              "Output tensor missing from variantPack");
+      FUSILLI_CHECK_ERROR(push(out));
+    }
+    for (const auto &in : fullGraphInputsSorted_) {
+      if (in->isScalar()) {
+        FUSILLI_RETURN_ERROR_IF(variantPack.contains(in),
+                                ErrorCode::VariantPackError,
+                                "Scalar constant tensor found in variantPack");
+        continue;
+      }
+      FUSILLI_RETURN_ERROR_IF(!variantPack.contains(in),
+                              ErrorCode::VariantPackError,
+                              "Input tensor missing from variantPack");
+      FUSILLI_CHECK_ERROR(push(in));
+    }
+
+    void *workspacePtr = nullptr;
+    if (*workspaceSize_ > 0) {
+      FUSILLI_RETURN_ERROR_IF(
+          workspace == nullptr, ErrorCode::InvalidArgument,
+          "Workspace buffer required but not provided (size=" +
+              std::to_string(*workspaceSize_) + " bytes)");
+      FUSILLI_RETURN_ERROR_IF(
+          workspace->sizeInBytes() < *workspaceSize_,
+          ErrorCode::InvalidArgument,
+          "Workspace buffer too small: provided " +
+              std::to_string(workspace->sizeInBytes()) + " bytes, required " +
+              std::to_string(*workspaceSize_) + " bytes");
+      workspacePtr = workspace->data();
+    } else if (workspace != nullptr) {
+      FUSILLI_LOG_LABEL_ENDL("WARNING: Workspace buffer provided but not "
+                             "needed (size=0), ignoring");
+    }
+
+    FUSILLI_RETURN_ERROR_IF(
+        handle.getBackend() != Backend::AMDGPU, ErrorCode::NotImplemented,
+        "Backend::CPU has no execution engine in this build: graphs run on "
+        "Backend::AMDGPU (gfx950) only");
+    for (const auto &kv : variantPack)
+      FUSILLI_RETURN_ERROR_IF(kv.second && !kv.second->isDeviceMemory(),
+                              ErrorCode::VariantPackError,
+                              "Tensor '" + kv.first->getName() +
+                                  "' is backed by host memory; AMDGPU "
+                                  "execution needs device buffers");
+    return plan::execute(handle.getContext(), *loadedPlan_, args, workspacePtr);
+  }
+
+  // ---- builders ---------------------------------------------------------------
+  std::shared_ptr<TensorAttr> tensor(const TensorAttr &t) {
+    FUSILLI_LOG_LABEL_ENDL("INFO: Adding input tensor '" << t.getName()
+                                                         << "' to Graph inputs");
+    auto p = std::make_shared<TensorAttr>(t);
+    fullGraphInputs_.insert(p);
+    return p;
+  }
+
+  std::shared_ptr<TensorAttr> convFProp(const TensorPtr &x, const TensorPtr &w,
+                                        ConvFPropAttr &attr) {
+    nameNode(attr, "conv_fprop");
+    nameTensor(x, attr, "X");
+    nameTensor(w, attr, "W");
+    attr.setX(x).setW(w);
+    auto y = outputTensor(attr.getName() + "_Y");
+    attr.setY(y);
+    subNodes_.emplace_back(
+        std::make_shared<ConvFPropNode>(std::move(attr), context));
+    return y;
+  }
+
+  std::shared_ptr<TensorAttr> matmul(const TensorPtr &a, const TensorPtr &b,
+                                     MatmulAttr &attr) {
+    nameNode(attr, "matmul");
+    nameTensor(a, attr, "A");
+    nameTensor(b, attr, "B");
+    attr.setA(a).setB(b);
+    auto c = outputTensor(attr.getName() + "_C");
+    attr.setC(c);
+    subNodes_.emplace_back(
+        std::make_shared<MatmulNode>(std::move(attr), context));
+    return c;
+  }
+
+  std::shared_ptr<TensorAttr> pointwise(const TensorPtr &in,
+                                        PointwiseAttr &attr) {
+    return pointwiseImpl({in}, attr);
+  }
+  std::shared_ptr<TensorAttr> pointwise(const TensorPtr &in0,
+                                        const TensorPtr &in1,
+                                        PointwiseAttr &attr) {
+    return pointwiseImpl({in0, in1}, attr);
+  }
+  std::shared_ptr<TensorAttr> pointwise(const TensorPtr &in0,
+                                        const TensorPtr &in1,
+                                        const TensorPtr &in2,
+                                        PointwiseAttr &attr) {
+    return pointwiseImpl({in0, in1, in2}, attr);
+  }
+
+  std::shared_ptr<TensorAttr> reduction(const TensorPtr &x,
+                                        ReductionAttr &attr) {
+    nameNode(attr, "reduction");
+    nameTensor(x, attr, "X");
+    attr.setX(x);
+    auto y = outputTensor(attr.getName() + "_Y");
+    attr.setY(y);
+    subNodes_.emplace_back(
+        std::make_shared<ReductionNode>(std::move(attr), context));
+    return y;
+  }
+
+  std::shared_ptr<TensorAttr> sdpa(const TensorPtr &q, const TensorPtr &k,
+                                   const TensorPtr &v, const TensorPtr &mask,
+                                   SdpaAttr &attr) {
+    nameNode(attr, "sdpa");
+    nameTensor(q, attr, "Q");
+    nameTensor(k, attr, "K");
+    nameTensor(v, attr, "V");
+    nameTensor(mask, attr, "MASK");
+    attr.setQ(q).setK(k).setV(v);
+    if (mask)
+      attr.setMASK(mask);
+    auto o = outputTensor(attr.getName() + "_O");
+    attr.setO(o);
+    subNodes_.emplace_back(std::make_shared<SdpaNode>(std::move(attr), context));
+    return o;
+  }
+
+  // Returns {Y, INV_RMS}; INV_RMS is null outside the training phase.
+  std::array<std::shared_ptr<TensorAttr>, 2>
+  rmsnorm(const TensorPtr &x, const TensorPtr &scale, RmsnormAttr &attr) {
+    nameNode(attr, "rmsnorm");
+    nameTensor(x, attr, "X");
+    nameTensor(scale, attr, "SCALE");
+    nameTensor(attr.getEpsilon(), attr, "EPSILON");
+    attr.setX(x);
+    attr.setSCALE(scale);
+    auto y = outputTensor(attr.getName() + "_Y");
+    attr.setY(y);
+    std::shared_ptr<TensorAttr> r;
+    if (attr.getForwardPhase() == NormFwdPhase::TRAINING)
+      r = outputTensor(attr.getName() + "_INV_RMS");
+    attr.setINV_RMS(r);
+    subNodes_.emplace_back(
+        std::make_shared<RmsNormNode>(std::move(attr), context));
+    return {y, r};
+  }
+
+  // Returns {Y, MEAN, INV_VARIANCE}; the statistics are null outside training.
+  std::array<std::shared_ptr<TensorAttr>, 3>
+  layernorm(const TensorPtr &x, const TensorPtr &scale, const TensorPtr &bias,
+            LayernormAttr &attr) {
+    nameNode(attr, "layernorm");
+    nameTensor(x, attr, "X");
+    nameTensor(scale, attr, "SCALE");
+    nameTensor(bias, attr, "BIAS");
+    nameTensor(attr.getEpsilon(), attr, "EPSILON");
+    attr.setX(x);
+    attr.setSCALE(scale);
+    attr.setBIAS(bias);
+    auto y = outputTensor(attr.getName() + "_Y");
+    std::shared_ptr<TensorAttr> m, v;
+    if (attr.getForwardPhase() == NormFwdPhase::TRAINING) {
+      m = outputTensor(attr.getName() + "_MEAN");
+      v = outputTensor(attr.getName() + "_INV_VARIANCE");
+    }
+    attr.setY(y);
+    attr.setMEAN(m);
+    attr.setINV_VARIANCE(v);
+    subNodes_.emplace_back(
+        std::make_shared<LayerNormNode>(std::move(attr), context));
+    return {y, m, v};
+  }
+
+  // Number of kernel launches the loaded plan performs (the analogue of the
+  // dispatch count the reference reads from IREE's compile statistics).
+  std::optional<size_t> getKernelCount() const {
+    if (!loadedPlan_)
+      return std::nullopt;
+    return loadedPlan_->steps.size();
+  }
+
+private:
+  template <typename Attr> void nameNode(Attr &attr, const char *prefix) {
+    if (attr.getName().empty())
+      attr.setName(std::string(prefix) + "_" + std::to_string(subNodes_.size()));
+  }
+  template <typename Attr>
+  static void nameTensor(const TensorPtr &t, const Attr &attr,
+                         const char *suffix) {
+    if (t && t->getName().empty())
+      t->setName(attr.getName() + "_" + suffix);
+  }
+
+  std::shared_ptr<TensorAttr>
+  pointwiseImpl(std::initializer_list<TensorPtr> ins, PointwiseAttr &attr) {
+    nameNode(attr, "pointwise");
+    int i = 0;
+    for (const TensorPtr &t : ins) {
+      nameTensor(t, attr, ("IN_" + std::to_string(i)).c_str());
+      attr.setInput(static_cast<PointwiseAttr::InputNames>(i), t);
+      ++i;
+    }
+    auto out = outputTensor(attr.getName() + "_OUT_0");
+    attr.setOUT_0(out);
+    subNodes_.emplace_back(
+        std::make_shared<PointwiseNode>(std::move(attr), context));
+    return out;
+  }
+
+  // Node outputs start virtual; setOutput(true) makes them graph outputs.
+  std::shared_ptr<TensorAttr> outputTensor(const std::string &name) {
+    auto t = std::make_shared<TensorAttr>();
+    t->setName(name).setIsVirtual(true);
+    fullGraphOutputs_.insert(t);
+    return t;
+  }
+
+  // Input, output and node names share one namespace (graph/graph.h:655-677).
+  ErrorObject preValidateNode() const override final {
+    std::unordered_set<std::string> used;
+    for (const auto *set : {&fullGraphInputs_, &fullGraphOutputs_})
+      for (const auto &t : *set) {
+        FUSILLI_RETURN_ERROR_IF(used.contains(t->getName()),
+                                ErrorCode::InvalidAttribute,
+                                "Symbol name '" + t->getName() +
+                                    "' already in use");
+        used.insert(t->getName());
+      }
+    FUSILLI_CHECK_ERROR(checkNodeNamesAreUnique(used));
+    return ok();
+  }
+
+  ErrorObject inferPropertiesNode() override final {
+    fullGraphInputsSorted_.insert(fullGraphInputs_.begin(),
+                                  fullGraphInputs_.end());
+    fullGraphOutputsSorted_.insert(fullGraphOutputs_.begin(),
+                                   fullGraphOutputs_.end());
+    return ok();
+  }
+
+  void clearRuntimeState() {
+    loadedPlan_.reset();
+    loadedBackend_.reset();
+    workspaceSize_.reset();
+  }
+
+  bool isValidated_ = false;
+  std::optional<plan::Plan> loadedPlan_;
+  std::optional<Backend> loadedBackend_;
+  std::optional<size_t> workspaceSize_;
+
+  std::unordered_set<std::shared_ptr<TensorAttr>> fullGraphInputs_;
+  std::unordered_set<std::shared_ptr<TensorAttr>> fullGraphOutputs_;
+  // Name-sorted views, filled by validate(); they fix the argument order.
+  std::set<std::shared_ptr<TensorAttr>, TensorAttrSortByName>
+      fullGraphInputsSorted_;
+  std::set<std::shared_ptr<TensorAttr>, TensorAttrSortByName>
+      fullGraphOutputsSorted_;
+};
+
+} // namespace fusilli
+
+#endif // FUSILLI_GRAPH_H

@@ -1,0 +1,606 @@
+// End-to-end tests of the graph API on the GPU: the reference samples' known
+// answers (samples/**, tests/test_graph.cpp:551-647) run through
+// Graph::validate -> compile -> execute on Backend::AMDGPU, each executed
+// twice, plus the BASELINE configs at reduced size against plain host loops,
+// and HIP interop (caller-owned stream and device pointers,
+// tests/hip_tests/test_buffer.cpp:132-206).
+#define __HIP_PLATFORM_AMD__ 1
+#include <hip/hip_runtime_api.h>
+
+#include <fusilli.h>
+
+#include <cmath>
+#include <random>
+
+#include "mini_test.h"
+
+using namespace fusilli;
+using Dims = std::vector<int64_t>;
+using Pack = std::unordered_map<std::shared_ptr<TensorAttr>, std::shared_ptr<Buffer>>;
+
+static Dims contig(const Dims &d) {
+  return generateStrideFromDim(d, getContiguousStrideOrder(d.size()));
+}
+static Dims chlast(const Dims &d) {
+  return generateStrideFromDim(d, getChannelsLastStrideOrder(d.size()));
+}
+static TensorAttr mk(const std::string &name, Dims dim, Dims stride, DataType dt) {
+  return TensorAttr().setName(name).setDim(dim).setStride(stride).setDataType(dt);
+}
+static Handle &gpu() {
+  static Handle h = [] {
+    auto e = Handle::create(Backend::AMDGPU);
+    if (isError(e)) {
+      std::printf("no AMDGPU handle: %s\n", ErrorObject(e).getMessage().c_str());
+      std::exit(2);
+    }
+    return std::move(*e);
+  }();
+  return h;
+}
+// Buffer shaped like the tensor's physical dims (tests/utils.h:144-243).
+template <typename T>
+static std::shared_ptr<Buffer> bufOf(const std::shared_ptr<TensorAttr> &t,
+                                     const std::vector<T> &data) {
+  std::vector<size_t> shape;
+  for (int64_t d : t->getPhysicalDim())
+    shape.push_back(static_cast<size_t>(d));
+  auto b = Buffer::allocate(gpu(), shape, data);
+  if (isError(b)) {
+    std::printf("allocate failed: %s\n", ErrorObject(b).getMessage().c_str());
+    std::exit(3);
+  }
+  return std::make_shared<Buffer>(std::move(*b));
+}
+template <typename T>
+static std::shared_ptr<Buffer> fill(const std::shared_ptr<TensorAttr> &t, T v) {
+  size_t n = 1;
+  for (int64_t d : t->getPhysicalDim())
+    n *= static_cast<size_t>(d);
+  return bufOf(t, std::vector<T>(n, v));
+}
+static std::shared_ptr<Buffer> workspaceFor(Graph &g) {
+  auto ws = g.getWorkspaceSize();
+  if (isError(ws) || !ws->has_value() || **ws == 0)
+    return nullptr;
+  auto b = Buffer::allocateRaw(gpu(), **ws);
+  return std::make_shared<Buffer>(std::move(*b));
+}
+template <typename T>
+static std::vector<T> readBack(const std::shared_ptr<Buffer> &b) {
+  std::vector<T> out;
+  auto st = b->read(gpu(), out);
+  if (isError(st))
+    std::printf("read failed: %s\n", st.getMessage().c_str());
+  return out;
+}
+static Graph newGraph(const std::string &name, DataType io,
+                      DataType inter = DataType::Float) {
+  Graph g;
+  g.setName(name).setIODataType(io).setIntermediateDataType(inter)
+      .setComputeDataType(DataType::Float);
+  return g;
+}
+template <typename T> static bool allEqual(const std::vector<T> &v, float x) {
+  for (const T &e : v)
+    if (static_cast<float>(e) != x)
+      return false;
+  return !v.empty();
+}
+
+// ---- convolution samples -----------------------------------------------------
+static void convOnes(bool nhwc, bool bias, bool relu, int64_t r, int64_t pad,
+                     float expectCorner, float expectCentre) {
+  const int64_t n = 4, c = 128, h = 8, w = 8, k = 32;
+  Graph g = newGraph(std::string("conv_") + (nhwc ? "nhwc" : "nchw") +
+                         (bias ? "_b" : "") + (relu ? "_r" : "") + std::to_string(r),
+                     DataType::Half);
+  auto lay = [&](const Dims &d) { return nhwc ? chlast(d) : contig(d); };
+  auto X = g.tensor(mk("x", {n, c, h, w}, lay({n, c, h, w}), DataType::Half));
+  auto W = g.tensor(mk("w", {k, c, r, r}, lay({k, c, r, r}), DataType::Half));
+  ConvFPropAttr ca;
+  ca.setPadding({pad, pad}).setStride({1, 1}).setDilation({1, 1});
+  auto Y = g.convFProp(X, W, ca);
+  std::shared_ptr<TensorAttr> B;
+  if (bias) {
+    B = g.tensor(mk("b", {1, k, 1, 1}, {k, 1, k, k}, DataType::Half));
+    PointwiseAttr add;
+    add.setMode(PointwiseAttr::Mode::ADD);
+    Y = g.pointwise(Y, B, add);
+  }
+  if (relu) {
+    PointwiseAttr rl;
+    rl.setMode(PointwiseAttr::Mode::RELU_FWD);
+    Y = g.pointwise(Y, rl);
+  }
+  Y->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), /*remove=*/true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1)); // fused
+  Pack pack = {{X, fill(X, half(1.0f))}, {W, fill(W, half(1.0f))},
+               {Y, fill(Y, half(0.0f))}};
+  if (bias)
+    pack[B] = fill(B, half(1.0f));
+  auto ws = workspaceFor(g);
+  for (int rep = 0; rep < 2; ++rep) { // samples execute twice
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+    auto out = readBack<half>(pack[Y]);
+    REQUIRE(out.size() == static_cast<size_t>(n * k * h * w));
+    // logical (0,0,0,0) is storage element 0 in both layouts
+    CHECK(static_cast<float>(out[0]) == expectCorner);
+    // logical (0,0,3,3)
+    const size_t centre = nhwc ? static_cast<size_t>((3 * w + 3) * k)
+                               : static_cast<size_t>(3 * w + 3);
+    CHECK(static_cast<float>(out[centre]) == expectCentre);
+    if (r == 1)
+      CHECK(allEqual(out, expectCorner));
+  }
+}
+
+TEST("samples: conv fprop all-ones known answers") {
+  convOnes(false, false, false, 1, 0, 128.f, 128.f); // test_graph.cpp:198-223
+  convOnes(true, false, false, 1, 0, 128.f, 128.f);  // conv_fprop_nhwc_krsc.cpp:95
+  convOnes(true, true, false, 1, 0, 129.f, 129.f);   // conv_fprop_with_bias.cpp:107
+  convOnes(true, true, true, 1, 0, 129.f, 129.f);    // ..._with_relu_and_bias.cpp:112
+  convOnes(true, false, false, 3, 1, 512.f, 1152.f); // ..._with_pad.cpp:94
+  convOnes(false, true, true, 3, 1, 513.f, 1153.f);
+}
+
+// ---- matmul samples ----------------------------------------------------------
+TEST("samples: matmul all-ones, transposed B, bias, batched broadcast") {
+  for (int variant = 0; variant < 3; ++variant) {
+    const int64_t m = 64, k = 128, n = 256;
+    Graph g = newGraph("mm_" + std::to_string(variant), DataType::Half);
+    auto A = g.tensor(mk("a", {m, k}, {k, 1}, DataType::Half));
+    auto B = g.tensor(mk("b", {k, n}, variant == 1 ? Dims{1, k} : Dims{n, 1},
+                         DataType::Half));
+    MatmulAttr ma;
+    auto C = g.matmul(A, B, ma);
+    std::shared_ptr<TensorAttr> bias;
+    if (variant == 2) {
+      bias = g.tensor(mk("bias", {1, n}, {n, 1}, DataType::Half));
+      PointwiseAttr add;
+      add.setMode(PointwiseAttr::Mode::ADD);
+      C = g.pointwise(C, bias, add);
+    }
+    C->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    Pack pack = {{A, fill(A, half(1.f))}, {B, fill(B, half(1.f))},
+                 {C, fill(C, half(0.f))}};
+    if (bias)
+      pack[bias] = fill(bias, half(2.f));
+    auto ws = workspaceFor(g);
+    for (int rep = 0; rep < 2; ++rep) {
+      REQUIRE_OK(g.execute(gpu(), pack, ws));
+      CHECK(allEqual(readBack<half>(pack[C]), variant == 2 ? 130.f : 128.f));
+    }
+  }
+  { // samples/matmul/matmul_batched.cpp: [16,16,M,K] x [1,1,K,N], f32
+    const int64_t m = 16, k = 32, n = 64;
+    Graph g = newGraph("mm_bcast", DataType::Float);
+    auto A = g.tensor(mk("a", {16, 16, m, k}, contig({16, 16, m, k}), DataType::Float));
+    auto B = g.tensor(mk("b", {1, 1, k, n}, contig({1, 1, k, n}), DataType::Float));
+    MatmulAttr ma;
+    auto C = g.matmul(A, B, ma);
+    C->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    Pack pack = {{A, fill(A, 1.f)}, {B, fill(B, 1.f)}, {C, fill(C, 0.f)}};
+    auto ws = workspaceFor(g);
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+    CHECK(allEqual(readBack<float>(pack[C]), 32.f));
+  }
+}
+
+// ---- sdpa samples ------------------------------------------------------------
+TEST("samples: sdpa constant fill equals V") {
+  struct V { bool causal, mask, gqa; int64_t sq, skv; };
+  for (const V &v : {V{false, false, false, 64, 64}, V{true, false, false, 64, 64},
+                     V{false, true, false, 64, 64}, V{false, false, true, 64, 64},
+                     V{false, false, false, 32, 128}}) {
+    const int64_t b = 1, hq = 8, hkv = v.gqa ? 2 : 8, d = 64;
+    Graph g = newGraph("sdpa_" + std::to_string(v.causal) + std::to_string(v.mask) +
+                           std::to_string(v.gqa) + std::to_string(v.skv),
+                       DataType::Half);
+    auto Q = g.tensor(mk("q", {b, hq, v.sq, d}, contig({b, hq, v.sq, d}), DataType::Half));
+    auto K = g.tensor(mk("k", {b, hkv, v.skv, d}, contig({b, hkv, v.skv, d}), DataType::Half));
+    auto Vt = g.tensor(mk("v", {b, hkv, v.skv, d}, contig({b, hkv, v.skv, d}), DataType::Half));
+    std::shared_ptr<TensorAttr> M;
+    if (v.mask)
+      M = g.tensor(mk("m", {b, 1, v.sq, v.skv}, contig({b, 1, v.sq, v.skv}), DataType::Half));
+    SdpaAttr sa;
+    sa.setIsCausal(v.causal).setEnableGqa(v.gqa);
+    auto O = g.sdpa(Q, K, Vt, M, sa);
+    O->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    Pack pack = {{Q, fill(Q, half(0.01f))}, {K, fill(K, half(0.01f))},
+                 {Vt, fill(Vt, half(0.01f))}, {O, fill(O, half(0.f))}};
+    if (M)
+      pack[M] = fill(M, half(-1.0f));
+    auto ws = workspaceFor(g);
+    for (int rep = 0; rep < 2; ++rep) {
+      REQUIRE_OK(g.execute(gpu(), pack, ws));
+      auto out = readBack<half>(pack[O]);
+      bool okAll = !out.empty();
+      for (half e : out)
+        okAll = okAll && std::fabs(static_cast<float>(e) - 0.01f) < 1e-2f;
+      CHECK(okAll); // samples/sdpa_utils.cpp:241-246
+    }
+  }
+}
+
+// ---- norm samples ------------------------------------------------------------
+TEST("samples: rmsnorm and layernorm two-value patterns") {
+  const int64_t n = 2, c = 3, h = 32, w = 32;
+  const size_t inner = static_cast<size_t>(c * h * w);
+  for (bool nhwc : {false, true}) {
+    const float eps = 1e-5f, sc = 2.0f;
+    Graph g = newGraph(std::string("rms_") + (nhwc ? "nhwc" : "nchw"), DataType::Float);
+    auto lay = [&](const Dims &d) { return nhwc ? chlast(d) : contig(d); };
+    auto X = g.tensor(mk("x", {n, c, h, w}, lay({n, c, h, w}), DataType::Float));
+    auto S = g.tensor(mk("s", {1, c, h, w}, lay({1, c, h, w}), DataType::Float));
+    RmsnormAttr ra;
+    ra.setForwardPhase(NormFwdPhase::INFERENCE).setEpsilon(g.tensor(TensorAttr(eps)));
+    auto [Y, R] = g.rmsnorm(X, S, ra);
+    Y->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    std::vector<float> xin(n * inner), expect(n * inner);
+    for (int64_t b = 0; b < n; ++b) { // samples/rmsnorm/rmsnorm_utils.h:26-66
+      const float x0 = 2.f * b + 1.f, x1 = x0 + 2.f;
+      const float rms = std::sqrt((x0 * x0 + x1 * x1) / 2.f + eps);
+      for (size_t i = 0; i < inner; ++i) {
+        const bool first = i < inner / 2;
+        xin[b * inner + i] = first ? x0 : x1;
+        expect[b * inner + i] = sc * (first ? x0 : x1) / rms;
+      }
+    }
+    Pack pack = {{X, bufOf(X, xin)}, {S, fill(S, sc)}, {Y, fill(Y, 0.f)}};
+    auto ws = workspaceFor(g);
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+    auto out = readBack<float>(pack[Y]);
+    bool okAll = out.size() == expect.size();
+    for (size_t i = 0; okAll && i < out.size(); ++i)
+      okAll = std::fabs(out[i] - expect[i]) < 1e-4f;
+    CHECK(okAll);
+  }
+  { // samples/layernorm/layernorm_utils.h:25-82 (training outputs)
+    const float eps = 1e-5f, sc = 2.f, bi = 1.f;
+    Graph g = newGraph("ln_train", DataType::Float);
+    auto X = g.tensor(mk("x", {n, c, h, w}, contig({n, c, h, w}), DataType::Float));
+    auto S = g.tensor(mk("s", {1, c, h, w}, contig({1, c, h, w}), DataType::Float));
+    auto B = g.tensor(mk("b", {1, c, h, w}, contig({1, c, h, w}), DataType::Float));
+    LayernormAttr la;
+    la.setForwardPhase(NormFwdPhase::TRAINING).setEpsilon(g.tensor(TensorAttr(eps)));
+    auto [Y, M, V] = g.layernorm(X, S, B, la);
+    Y->setOutput(true);
+    M->setOutput(true);
+    V->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    std::vector<float> xin(n * inner);
+    for (int64_t b = 0; b < n; ++b)
+      for (size_t i = 0; i < inner; ++i)
+        xin[b * inner + i] = i < inner / 2 ? 2.f * b : 2.f * b + 2.f;
+    Pack pack = {{X, bufOf(X, xin)}, {S, fill(S, sc)}, {B, fill(B, bi)},
+                 {Y, fill(Y, 0.f)}, {M, fill(M, 0.f)}, {V, fill(V, 0.f)}};
+    auto ws = workspaceFor(g);
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+    auto y = readBack<float>(pack[Y]);
+    auto m = readBack<float>(pack[M]);
+    auto v = readBack<float>(pack[V]);
+    const float r = 1.f / std::sqrt(1.f + eps);
+    bool okAll = true;
+    for (int64_t b = 0; b < n; ++b)
+      for (size_t i = 0; i < inner; ++i)
+        okAll = okAll && std::fabs(y[b * inner + i] -
+                                   ((i < inner / 2 ? -sc : sc) * r + bi)) < 1e-4f;
+    CHECK(okAll);
+    CHECK(std::fabs(m[0] - 1.f) < 1e-4f && std::fabs(m[1] - 3.f) < 1e-4f);
+    CHECK(std::fabs(v[0] - r) < 1e-4f && std::fabs(v[1] - r) < 1e-4f);
+  }
+}
+
+// ---- reduction sample --------------------------------------------------------
+TEST("samples: reduction table, element (0,0)") {
+  using M = ReductionAttr::Mode;
+  // samples/reduction/reduction_ops.cpp: [2,16,8,8] -> [2,16,1,1]; inputs
+  // i % 100 - 50; element (0,0) reduces inputs 0..63 = -50..13.
+  struct Row { M mode; float expect; };
+  double sum = 0, sumsq = 0, sumabs = 0;
+  for (int i = 0; i < 64; ++i) {
+    const double x = i - 50;
+    sum += x, sumsq += x * x, sumabs += std::fabs(x);
+  }
+  for (const Row &row : {Row{M::ADD, (float)sum}, Row{M::SUM, (float)sum},
+                         Row{M::MIN, -50.f}, Row{M::MAX, 13.f}, Row{M::AMAX, 50.f},
+                         Row{M::AVG, (float)(sum / 64)}, Row{M::NORM1, (float)sumabs},
+                         Row{M::NORM2, (float)std::sqrt(sumsq)}}) {
+    Graph g = newGraph(std::string("red_") + ReductionAttr::modeName(row.mode),
+                       DataType::Float);
+    auto X = g.tensor(mk("x", {2, 16, 8, 8}, contig({2, 16, 8, 8}), DataType::Float));
+    ReductionAttr ra;
+    ra.setMode(row.mode);
+    auto Y = g.reduction(X, ra);
+    Y->setOutput(true).setDim({2, 16, 1, 1});
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    std::vector<float> xin(2 * 16 * 64);
+    for (size_t i = 0; i < xin.size(); ++i)
+      xin[i] = static_cast<float>(static_cast<int>(i % 100) - 50);
+    Pack pack = {{X, bufOf(X, xin)}, {Y, fill(Y, 0.f)}};
+    REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+    auto out = readBack<float>(pack[Y]);
+    CHECK(std::fabs(out[0] - row.expect) < 0.01f);
+  }
+  { // int32 product with a 2 and a 3 => 6
+    Graph g = newGraph("red_mul_i32", DataType::Int32);
+    auto X = g.tensor(mk("x", {2, 16, 8, 8}, contig({2, 16, 8, 8}), DataType::Int32));
+    ReductionAttr ra;
+    ra.setMode(M::MUL);
+    auto Y = g.reduction(X, ra);
+    Y->setOutput(true).setDim({2, 16, 1, 1});
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    std::vector<int32_t> xin(2 * 16 * 64, 1);
+    xin[0] = 2, xin[1] = 3;
+    Pack pack = {{X, bufOf(X, xin)}, {Y, fill(Y, int32_t(0))}};
+    REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+    CHECK(readBack<int32_t>(pack[Y])[0] == 6);
+  }
+}
+
+// ---- pointwise samples -------------------------------------------------------
+TEST("samples: pointwise transposed add, scalar mul, AOT int32 add") {
+  { // samples/pointwise/pointwise_add_transposed.cpp:22-112
+    Graph g = newGraph("pw_t", DataType::Float);
+    auto A = g.tensor(mk("a", {3, 2}, {2, 1}, DataType::Float));
+    auto B = g.tensor(mk("b", {3, 2}, {1, 3}, DataType::Float));
+    PointwiseAttr add;
+    add.setMode(PointwiseAttr::Mode::ADD);
+    auto O = g.pointwise(A, B, add);
+    O->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    std::vector<float> data = {1, 2, 3, 4, 5, 6};
+    Pack pack = {{A, bufOf(A, data)}, {B, bufOf(B, data)}, {O, fill(O, 0.f)}};
+    REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+    CHECK((readBack<float>(pack[O]) == std::vector<float>{2, 6, 5, 9, 8, 12}));
+  }
+  { // samples/pointwise/pointwise_scalar_mul.cpp:22-78
+    Graph g = newGraph("pw_s", DataType::Float);
+    auto A = g.tensor(mk("a", {2, 16, 8}, contig({2, 16, 8}), DataType::Float));
+    auto two = g.tensor(TensorAttr(2.0f));
+    PointwiseAttr mul;
+    mul.setMode(PointwiseAttr::Mode::MUL);
+    auto O = g.pointwise(A, two, mul);
+    O->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    Pack pack = {{A, fill(A, 3.f)}, {O, fill(O, 0.f)}};
+    REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+    CHECK(allEqual(readBack<float>(pack[O]), 6.f));
+  }
+  { // samples/aot/single_backend.cpp:52-110
+    auto build = [](const std::string &name, std::shared_ptr<TensorAttr> &a,
+                    std::shared_ptr<TensorAttr> &b, std::shared_ptr<TensorAttr> &o) {
+      auto g = std::make_unique<Graph>();
+      g->setName(name).setIODataType(DataType::Int32).setComputeDataType(DataType::Int32);
+      a = g->tensor(mk("a", {4, 8}, {8, 1}, DataType::Int32));
+      b = g->tensor(mk("b", {4, 8}, {8, 1}, DataType::Int32));
+      PointwiseAttr add;
+      add.setMode(PointwiseAttr::Mode::ADD);
+      o = g->pointwise(a, b, add);
+      o->setOutput(true);
+      return g;
+    };
+    std::shared_ptr<TensorAttr> a1, b1, o1, a2, b2, o2;
+    auto producer = build("aot", a1, b1, o1);
+    REQUIRE_OK(producer->validate());
+    REQUIRE_ASSIGN(auto bytes, producer->compileToArtifact(Backend::AMDGPU, true));
+    auto consumer = build("aot", a2, b2, o2);
+    REQUIRE_OK(consumer->validate());
+    REQUIRE_OK(consumer->loadFromArtifact(gpu(), bytes));
+    Pack pack = {{a2, fill(a2, int32_t(2))}, {b2, fill(b2, int32_t(3))},
+                 {o2, fill(o2, int32_t(0))}};
+    REQUIRE_OK(consumer->execute(gpu(), pack, workspaceFor(*consumer)));
+    CHECK(allEqual(readBack<int32_t>(pack[o2]), 5.f));
+  }
+}
+
+// ---- BASELINE configs through the graph API ---------------------------------
+static std::vector<float> randomVec(size_t n, uint32_t seed, float lo, float hi) {
+  std::mt19937 rng(seed);
+  std::vector<float> v(n);
+  for (auto &x : v)
+    x = lo + (hi - lo) * (rng() >> 8) * (1.0f / 16777216.0f);
+  return v;
+}
+
+TEST("config 1: f32 matmul 1x256x512x256 vs host loop, rel 1e-4") {
+  const int64_t m = 256, k = 512, n = 256;
+  Graph g = newGraph("cfg1", DataType::Float);
+  auto A = g.tensor(mk("a", {1, m, k}, contig({1, m, k}), DataType::Float));
+  auto B = g.tensor(mk("b", {1, k, n}, contig({1, k, n}), DataType::Float));
+  MatmulAttr ma;
+  auto C = g.matmul(A, B, ma);
+  C->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  auto a = randomVec(m * k, 1, -1.f, 1.f), b = randomVec(k * n, 2, -1.f, 1.f);
+  Pack pack = {{A, bufOf(A, a)}, {B, bufOf(B, b)}, {C, fill(C, 0.f)}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<float>(pack[C]);
+  double rms = 0, worst = 0;
+  std::vector<double> ref(m * n, 0.0);
+  for (int64_t i = 0; i < m; ++i)
+    for (int64_t kk = 0; kk < k; ++kk)
+      for (int64_t j = 0; j < n; ++j)
+        ref[i * n + j] += (double)a[i * k + kk] * b[kk * n + j];
+  for (double r : ref)
+    rms += r * r;
+  rms = std::sqrt(rms / ref.size());
+  for (size_t i = 0; i < ref.size(); ++i)
+    worst = std::max(worst, std::fabs(out[i] - ref[i]) -
+                                1e-4 * (std::fabs(ref[i]) + rms));
+  CHECK(worst <= 0.0);
+}
+
+TEST("config 3 (reduced): bf16 NHWC conv 3x3 + bias + relu vs host loop") {
+  const int64_t n = 2, c = 64, h = 14, w = 14, k = 128;
+  Graph g = newGraph("cfg3", DataType::BFloat16, DataType::Float);
+  auto X = g.tensor(mk("x", {n, c, h, w}, chlast({n, c, h, w}), DataType::BFloat16));
+  auto W = g.tensor(mk("w", {k, c, 3, 3}, chlast({k, c, 3, 3}), DataType::BFloat16));
+  auto B = g.tensor(mk("b", {1, k, 1, 1}, {k, 1, k, k}, DataType::BFloat16));
+  ConvFPropAttr ca;
+  ca.setPadding({1, 1}).setStride({1, 1}).setDilation({1, 1});
+  auto Y = g.convFProp(X, W, ca);
+  PointwiseAttr add, relu;
+  add.setMode(PointwiseAttr::Mode::ADD);
+  relu.setMode(PointwiseAttr::Mode::RELU_FWD);
+  auto O = g.pointwise(g.pointwise(Y, B, add), relu);
+  O->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  auto xf = randomVec(n * h * w * c, 3, -1.f, 1.f);
+  auto wf = randomVec(k * 9 * c, 4, -0.1f, 0.1f);
+  auto bf = randomVec(k, 5, -1.f, 1.f);
+  std::vector<bf16> xb(xf.size()), wb(wf.size()), bb(bf.size());
+  for (size_t i = 0; i < xf.size(); ++i) xb[i] = (bf16)xf[i], xf[i] = (float)xb[i];
+  for (size_t i = 0; i < wf.size(); ++i) wb[i] = (bf16)wf[i], wf[i] = (float)wb[i];
+  for (size_t i = 0; i < bf.size(); ++i) bb[i] = (bf16)bf[i], bf[i] = (float)bb[i];
+  Pack pack = {{X, bufOf(X, xb)}, {W, bufOf(W, wb)}, {B, bufOf(B, bb)},
+               {O, fill(O, bf16(0.f))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<bf16>(pack[O]);
+  // physical layouts: x [n][h][w][c], w [k][r][s][c], out [n][p][q][k]
+  double worst = 0, rms = 0;
+  std::vector<double> ref(n * h * w * k);
+  for (int64_t in = 0; in < n; ++in)
+    for (int64_t p = 0; p < h; ++p)
+      for (int64_t q = 0; q < w; ++q)
+        for (int64_t kk = 0; kk < k; ++kk) {
+          double acc = 0;
+          for (int64_t r = 0; r < 3; ++r)
+            for (int64_t s = 0; s < 3; ++s) {
+              const int64_t ih = p - 1 + r, iw = q - 1 + s;
+              if (ih < 0 || ih >= h || iw < 0 || iw >= w)
+                continue;
+              for (int64_t cc = 0; cc < c; ++cc)
+                acc += (double)xf[((in * h + ih) * w + iw) * c + cc] *
+                       wf[((kk * 3 + r) * 3 + s) * c + cc];
+            }
+          acc += bf[kk];
+          ref[((in * h + p) * w + q) * k + kk] = acc > 0 ? acc : 0;
+        }
+  for (double r : ref)
+    rms += r * r;
+  rms = std::sqrt(rms / ref.size());
+  for (size_t i = 0; i < ref.size(); ++i)
+    worst = std::max(worst, std::fabs((float)out[i] - ref[i]) -
+                                2e-2 * (std::fabs(ref[i]) + rms));
+  CHECK(worst <= 0.0);
+}
+
+TEST("config 5a (reduced): int8 matmul is bit exact") {
+  const int64_t m = 256, k = 512, n = 384;
+  Graph g = newGraph("cfg5a", DataType::Int8);
+  auto A = g.tensor(mk("a", {m, k}, {k, 1}, DataType::Int8));
+  auto B = g.tensor(mk("b", {k, n}, {n, 1}, DataType::Int8));
+  MatmulAttr ma;
+  auto C = g.matmul(A, B, ma);
+  C->setOutput(true).setDataType(DataType::Int32);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  std::mt19937 rng(5);
+  std::vector<int8_t> a(m * k), b(k * n);
+  for (auto &x : a) x = (int8_t)((int)(rng() % 255) - 127);
+  for (auto &x : b) x = (int8_t)((int)(rng() % 255) - 127);
+  Pack pack = {{A, bufOf(A, a)}, {B, bufOf(B, b)}, {C, fill(C, int32_t(0))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<int32_t>(pack[C]);
+  bool exact = true;
+  for (int64_t i = 0; i < m && exact; ++i)
+    for (int64_t j = 0; j < n && exact; ++j) {
+      int32_t acc = 0;
+      for (int64_t kk = 0; kk < k; ++kk)
+        acc += (int32_t)a[i * k + kk] * (int32_t)b[kk * n + j];
+      exact = out[i * n + j] == acc;
+    }
+  CHECK(exact);
+}
+
+TEST("unfused chain uses the workspace for virtual tensors") {
+  Graph g = newGraph("chain", DataType::Float);
+  auto A = g.tensor(mk("a", {64, 32}, {32, 1}, DataType::Float));
+  PointwiseAttr p1, p2, p3;
+  p1.setMode(PointwiseAttr::Mode::EXP);
+  p2.setMode(PointwiseAttr::Mode::LOG);
+  p3.setMode(PointwiseAttr::Mode::ADD);
+  auto e = g.pointwise(A, p1);
+  auto l = g.pointwise(e, p2);
+  auto O = g.pointwise(l, A, p3);
+  O->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(3));
+  auto ws = workspaceFor(g);
+  REQUIRE(ws != nullptr);
+  auto a = randomVec(64 * 32, 9, -2.f, 2.f);
+  Pack pack = {{A, bufOf(A, a)}, {O, fill(O, 0.f)}};
+  REQUIRE_OK(g.execute(gpu(), pack, ws));
+  auto out = readBack<float>(pack[O]);
+  bool okAll = true;
+  for (size_t i = 0; i < a.size(); ++i)
+    okAll = okAll && std::fabs(out[i] - 2.f * a[i]) < 1e-4f;
+  CHECK(okAll);
+}
+
+// ---- HIP interop -------------------------------------------------------------
+TEST("interop: caller-owned stream and imported device pointers") {
+  hipStream_t stream;
+  REQUIRE(hipStreamCreate(&stream) == hipSuccess);
+  REQUIRE_ASSIGN(Handle h, Handle::create(Backend::AMDGPU, 0,
+                                          reinterpret_cast<uintptr_t>(stream)));
+  const size_t n = 1024;
+  float *a = nullptr, *o = nullptr;
+  REQUIRE(hipMalloc(reinterpret_cast<void **>(&a), n * 4) == hipSuccess);
+  REQUIRE(hipMalloc(reinterpret_cast<void **>(&o), n * 4) == hipSuccess);
+  std::vector<float> host(n, -3.f);
+  REQUIRE(hipMemcpy(a, host.data(), n * 4, hipMemcpyHostToDevice) == hipSuccess);
+  Graph g = newGraph("interop", DataType::Float);
+  auto A = g.tensor(mk("a", {32, 32}, {32, 1}, DataType::Float));
+  PointwiseAttr p;
+  p.setMode(PointwiseAttr::Mode::ABS);
+  auto O = g.pointwise(A, p);
+  O->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(h, true));
+  REQUIRE_ASSIGN(auto wsz, g.getWorkspaceSize());
+  CHECK(wsz.has_value());
+  REQUIRE_ASSIGN(Buffer ab, Buffer::import(a, n * 4, DataType::Float));
+  REQUIRE_ASSIGN(Buffer ob, Buffer::import(o, n * 4, DataType::Float));
+  Pack pack = {{A, std::make_shared<Buffer>(std::move(ab))},
+               {O, std::make_shared<Buffer>(std::move(ob))}};
+  REQUIRE_OK(g.execute(h, pack, nullptr));
+  // stream-ordered: the result is visible after the caller's own sync
+  REQUIRE(hipStreamSynchronize(stream) == hipSuccess);
+  REQUIRE(hipMemcpy(host.data(), o, n * 4, hipMemcpyDeviceToHost) == hipSuccess);
+  CHECK(allEqual(host, 3.f));
+  std::vector<float> viaRead;
+  REQUIRE_OK(pack[O]->read(h, viaRead));
+  CHECK(allEqual(viaRead, 3.f));
+  // a CPU-compiled plan is refused by an AMDGPU handle, and vice versa
+  REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+  CHECK_ERROR(g.execute(cpu, pack, nullptr), ErrorCode::InvalidArgument,
+              "Graph::execute got a handle for backend CPU, but the loaded "
+              "artifact uses backend AMDGPU");
+  (void)hipFree(a);
+  (void)hipFree(o);
+  (void)hipStreamDestroy(stream);
+}
+
+int main(int argc, char **argv) { return mini::run(argc, argv); }

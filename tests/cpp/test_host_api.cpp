@@ -1,0 +1,808 @@
+// Host-only tests of the graph API: layout math against the reference's known
+// answers, per-node validation (codes and messages as in the reference's
+// tests/test_*_node.cpp), the Graph state machine and the artifact contract
+// (tests/test_graph.cpp:373-510), Handle / Buffer rules (tests/test_handle.cpp,
+// tests/test_buffer.cpp).  Needs no GPU.
+#include <fusilli.h>
+
+#include <sstream>
+#include <thread>
+
+#include "mini_test.h"
+
+using namespace fusilli;
+#include "layout_vectors.inc"
+
+using Dims = std::vector<int64_t>;
+
+// ---- layout -----------------------------------------------------------------
+TEST("layout: reference known answers") {
+  TensorAttr t;
+  for (const auto &c : k_physical_dim) {
+    t.setDim(c.dim).setStride(c.stride);
+    CHECK(t.getPhysicalDim() == c.expect);
+  }
+  for (const auto &c : k_logical_to_physical) {
+    t.setDim(c.dim).setStride(c.stride);
+    CHECK(t.getLogicalToPhysicalPermuteOrder() == c.expect);
+  }
+  for (const auto &c : k_physical_to_logical) {
+    t.setDim(c.dim).setStride(c.stride);
+    CHECK(t.getPhysicalToLogicalPermuteOrder() == c.expect);
+  }
+  for (const auto &c : k_valid_representation) {
+    t.setDim(c.dim).setStride(c.stride);
+    CHECK(t.hasValidPhysicalRepresentation() == c.expect);
+  }
+}
+
+TEST("layout: stride orders and generators") {
+  // reference tensor_attributes.h:156-193 examples
+  CHECK((getContiguousStrideOrder(4) == std::vector<size_t>{3, 2, 1, 0}));
+  CHECK((getChannelsLastStrideOrder(4) == std::vector<size_t>{3, 0, 2, 1}));
+  CHECK((getChannelsLastStrideOrder(5) == std::vector<size_t>{4, 0, 3, 2, 1}));
+  CHECK((generateStrideOrderPreservingFormat({10, 30, 20}, 3) ==
+         std::vector<size_t>{0, 2, 1}));
+  CHECK((generateStrideOrderPreservingFormat({10, 30, 20}, 5) ==
+         std::vector<size_t>{0, 2, 1, 3, 4}));
+  // dim (10,3,12,12), order {3,0,2,1} -> stride (432,1,36,3)
+  CHECK((generateStrideFromDim({10, 3, 12, 12}, {3, 0, 2, 1}) ==
+         Dims{432, 1, 36, 3}));
+  // BASELINE config 3 layouts
+  CHECK((generateStrideFromDim({32, 64, 56, 56}, getChannelsLastStrideOrder(4)) ==
+         Dims{200704, 1, 3584, 64}));
+  CHECK((generateStrideFromDim({128, 64, 3, 3}, getChannelsLastStrideOrder(4)) ==
+         Dims{576, 1, 192, 64}));
+  CHECK((getChannelsLastToContiguousPermuteOrder(4) == Dims{0, 3, 1, 2}));
+  CHECK((getContiguousToChannelsLastPermuteOrder(4) == Dims{0, 2, 3, 1}));
+  CHECK((inversePermutation({0, 2, 3, 1}) == Dims{0, 3, 1, 2}));
+  auto nhwc = generateStrideFromLayout({2, 3, 4, 5}, "NHWC");
+  REQUIRE(isOk(nhwc));
+  CHECK((*nhwc == Dims{60, 1, 15, 3}));
+  auto bad = generateStrideFromLayout({2, 3, 4, 5}, "NWHC");
+  CHECK_ERROR(ErrorObject(bad), ErrorCode::InvalidArgument,
+              "Invalid layout string: NWHC");
+  auto rank = generateStrideFromLayout({2, 3, 4}, "NCHW");
+  CHECK_ERROR(ErrorObject(rank), ErrorCode::InvalidArgument,
+              "Invalid input dimensions and layout: they must have the same "
+              "rank");
+}
+
+TEST("layout: broadcast shape") {
+  auto s = computeBroadcastShape({{64, 16, 1, 1}, {1, 32, 1}});
+  REQUIRE(isOk(s));
+  CHECK((*s == Dims{64, 16, 32, 1}));
+  auto e = computeBroadcastShape({{3, 4}, {5, 4}});
+  CHECK_ERROR(ErrorObject(e), ErrorCode::InvalidAttribute,
+              "Cannot broadcast two non unit dimensions");
+  auto empty = computeBroadcastShape({{}, {}});
+  CHECK_ERROR(ErrorObject(empty), ErrorCode::InvalidAttribute,
+              "All input shapes are empty");
+}
+
+TEST("TensorAttr: validate codes and messages") {
+  TensorAttr t;
+  t.setName("x");
+  CHECK_ERROR(t.validate(), ErrorCode::AttributeNotSet, "Tensor 'x' dims not set");
+  t.setDim({2, 3});
+  CHECK_ERROR(t.validate(), ErrorCode::AttributeNotSet,
+              "Tensor 'x' strides not set");
+  t.setStride({3});
+  CHECK_ERROR(t.validate(), ErrorCode::InvalidAttribute,
+              "Tensor 'x' uses dim and stride of different dimensionality");
+  t.setStride({5, 1});
+  CHECK_ERROR(t.validate(), ErrorCode::InvalidAttribute,
+              "Tensor 'x' has invalid physical representation. It must be a "
+              "valid permutation of the logical dimensions");
+  t.setStride({3, 1});
+  CHECK_ERROR(t.validate(), ErrorCode::AttributeNotSet,
+              "Tensor 'x' data type not set");
+  t.setDataType(DataType::Float);
+  CHECK(isOk(t.validate()));
+  t.setIsScalar(true);
+  CHECK_ERROR(t.validate(), ErrorCode::InvalidAttribute,
+              "Tensor 'x' is marked as a scalar but does not have a scalar "
+              "value set");
+  TensorAttr s(2.5f);
+  s.setName("s");
+  CHECK(isOk(s.validate()));
+  CHECK(s.isScalar() && s.getDataType() == DataType::Float &&
+        s.getDim() == Dims{1} && scalarAsDouble(s) == 2.5);
+  s.setIsVirtual(true);
+  CHECK_ERROR(s.validate(), ErrorCode::InvalidAttribute,
+              "Tensor 's' cannot be both virtual (intermediate) and a scalar "
+              "constant");
+  TensorAttr d;
+  d.setName("d").setDim({4, 8}).setStride({8, 1}).setDataType(DataType::Float);
+  d.setDynamicDim(5);
+  CHECK_ERROR(d.validate(), ErrorCode::InvalidAttribute,
+              "Tensor 'd' has dynamic dim index 5 out of range for rank 2");
+}
+
+TEST("TensorAttr: dtype fill, contiguity, volume") {
+  Context ctx;
+  ctx.setIODataType(DataType::Half).setIntermediateDataType(DataType::Float);
+  TensorAttr io, virt;
+  virt.setIsVirtual(true);
+  io.fillFromContext(ctx);
+  virt.fillFromContext(ctx);
+  CHECK(io.getDataType() == DataType::Half);
+  CHECK(virt.getDataType() == DataType::Float);
+  TensorAttr t;
+  t.setDim({2, 3, 4, 5}).setStride({60, 20, 5, 1});
+  CHECK(t.isContiguous() && !t.isChannelsLast() && t.getVolume() == 120);
+  t.setStride({60, 1, 15, 3});
+  CHECK(!t.isContiguous() && t.isChannelsLast());
+  t.setDim({8, 2, 64, 128}).setStride({0, 0, 128, 1});
+  CHECK(t.hasBroadcastDims());
+  CHECK((t.getUnexpandedDim() == Dims{1, 1, 64, 128}));
+}
+
+// ---- helpers ----------------------------------------------------------------
+static TensorAttr mk(const std::string &name, Dims dim, Dims stride,
+                     DataType dt = DataType::Float) {
+  return TensorAttr().setName(name).setDim(dim).setStride(stride).setDataType(dt);
+}
+static Dims contig(const Dims &d) {
+  return generateStrideFromDim(d, getContiguousStrideOrder(d.size()));
+}
+static Dims chlast(const Dims &d) {
+  return generateStrideFromDim(d, getChannelsLastStrideOrder(d.size()));
+}
+static Graph newGraph(const std::string &name, DataType dt = DataType::Float) {
+  Graph g;
+  g.setName(name).setIODataType(dt).setIntermediateDataType(DataType::Float)
+      .setComputeDataType(DataType::Float);
+  return g;
+}
+
+// ---- node validation ----------------------------------------------------------
+TEST("conv node: inference and errors") {
+  {
+    Graph g = newGraph("conv_infer", DataType::BFloat16);
+    auto x = g.tensor(mk("x", {32, 64, 56, 56}, chlast({32, 64, 56, 56}),
+                         DataType::BFloat16));
+    auto w = g.tensor(mk("w", {128, 64, 3, 3}, chlast({128, 64, 3, 3}),
+                         DataType::BFloat16));
+    ConvFPropAttr a;
+    a.setPadding({1, 1}).setStride({1, 1}).setDilation({1, 1});
+    auto y = g.convFProp(x, w, a);
+    y->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK((y->getDim() == Dims{32, 128, 56, 56}));
+    CHECK((y->getStride() == Dims{401408, 1, 7168, 128})); // follows X: NHWC
+    CHECK(y->getName() == "conv_fprop_0_Y");
+    CHECK(y->getDataType() == DataType::BFloat16);
+  }
+  {
+    Graph g = newGraph("conv_shape");
+    auto x = g.tensor(mk("x", {2, 6, 9, 11}, contig({2, 6, 9, 11})));
+    auto w = g.tensor(mk("w", {4, 3, 3, 2}, contig({4, 3, 3, 2})));
+    ConvFPropAttr a;
+    a.setPadding({0, 1}).setStride({2, 1}).setDilation({1, 2});
+    auto y = g.convFProp(x, w, a);
+    y->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK((y->getDim() == Dims{2, 4, 4, 11})); // 1+(9-2-1)/2, 1+(11+2-2-1)/1
+    CHECK(y->isContiguous());
+  }
+  auto build = [](auto &&tweak) {
+    Graph g = newGraph("conv_err");
+    auto x = g.tensor(mk("x", {2, 8, 5, 5}, contig({2, 8, 5, 5})));
+    auto w = g.tensor(mk("w", {4, 8, 1, 1}, contig({4, 8, 1, 1})));
+    ConvFPropAttr a;
+    a.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    tweak(g, x, w, a);
+    auto y = g.convFProp(x, w, a);
+    y->setOutput(true);
+    return g.validate();
+  };
+  CHECK_ERROR(build([](auto &, auto &, auto &, auto &a) { a.setPadding({}); }),
+              ErrorCode::AttributeNotSet, "Conv padding not set");
+  CHECK_ERROR(build([](auto &, auto &, auto &, auto &a) { a.setStride({1}); }),
+              ErrorCode::InvalidAttribute,
+              "Conv stride size does not match number of spatial dimensions");
+  CHECK_ERROR(build([](auto &, auto &x, auto &, auto &) {
+                x->setStride({1, 2, 16, 80});
+              }),
+              ErrorCode::NotImplemented,
+              "Tensor 'x' is neither contiguous nor channels-last as defined "
+              "by its stride");
+  CHECK_ERROR(build([](auto &, auto &, auto &w, auto &) {
+                w->setDim({4, 3, 1, 1}).setStride({3, 1, 1, 1});
+              }),
+              ErrorCode::InvalidAttribute,
+              "Conv input channels must be divisible by the filter channels");
+  CHECK_ERROR(build([](auto &, auto &, auto &w, auto &) {
+                w->setDim({3, 4, 1, 1}).setStride({4, 1, 1, 1});
+              }),
+              ErrorCode::InvalidAttribute,
+              "Conv output channels must be divisible by the group count");
+}
+
+TEST("matmul node: inference and errors") {
+  {
+    Graph g = newGraph("mm");
+    auto a = g.tensor(mk("a", {16, 16, 32, 64}, contig({16, 16, 32, 64})));
+    auto b = g.tensor(mk("b", {1, 1, 64, 128}, contig({1, 1, 64, 128})));
+    MatmulAttr m;
+    auto c = g.matmul(a, b, m);
+    c->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK((c->getDim() == Dims{16, 16, 32, 128}));
+    CHECK(c->isContiguous());
+    CHECK(c->getName() == "matmul_0_C");
+  }
+  auto build = [](Dims ad, Dims as, Dims bd, Dims bs,
+                  DataType bdt = DataType::Float) {
+    Graph g = newGraph("mm_err");
+    auto a = g.tensor(mk("a", ad, as));
+    auto b = g.tensor(mk("b", bd, bs, bdt));
+    MatmulAttr m;
+    auto c = g.matmul(a, b, m);
+    c->setOutput(true);
+    return g.validate();
+  };
+  CHECK_ERROR(build({4}, {1}, {4, 4}, {4, 1}), ErrorCode::InvalidAttribute,
+              "Matmul input tensor A must have a rank of at least 2");
+  CHECK_ERROR(build({2, 4, 4}, {16, 4, 1}, {4, 4}, {4, 1}),
+              ErrorCode::InvalidAttribute,
+              "Matmul input tensors A and B must have the same rank: A has "
+              "rank=3, B has rank=2");
+  CHECK_ERROR(build({4, 8}, {8, 1}, {7, 4}, {4, 1}),
+              ErrorCode::InvalidAttribute,
+              "Matmul input tensors A and B have incompatible inner "
+              "dimensions (K): A has K=8, B has K=7");
+  CHECK_ERROR(build({3, 4, 8}, {32, 8, 1}, {2, 8, 4}, {32, 4, 1}),
+              ErrorCode::InvalidAttribute,
+              "Matmul input tensors A and B have incompatible batch dimensions "
+              "for broadcasting at index 0: A has dim=3, B has dim=2");
+  CHECK_ERROR(build({2, 4, 8}, {8, 16, 1}, {2, 8, 4}, {32, 4, 1}),
+              ErrorCode::InvalidAttribute,
+              "Matmul tensor A has batch dimensions that are not outermost or "
+              "are transposed");
+  CHECK_ERROR(build({4, 8}, {8, 1}, {8, 4}, {4, 1}, DataType::Half),
+              ErrorCode::InvalidAttribute,
+              "Mixed precision matmul is only supported when input tensors A "
+              "and B are of rank 3 (single batch dim): A and B have rank=2");
+}
+
+TEST("pointwise node: inference and errors") {
+  {
+    Graph g = newGraph("pw");
+    auto a = g.tensor(mk("a", {3, 1, 8}, contig({3, 1, 8})));
+    auto b = g.tensor(mk("b", {5, 8}, contig({5, 8})));
+    PointwiseAttr p;
+    p.setMode(PointwiseAttr::Mode::CMP_LT);
+    auto o = g.pointwise(a, b, p);
+    o->setOutput(true).setStride(contig({3, 5, 8}));
+    REQUIRE_OK(g.validate());
+    CHECK((o->getDim() == Dims{3, 5, 8}));
+    CHECK(o->getDataType() == DataType::Boolean); // forced
+    CHECK(o->getName() == "pointwise_0_OUT_0");
+  }
+  {
+    Graph g = newGraph("pw_stride");
+    auto a = g.tensor(mk("a", {2, 3, 4, 5}, chlast({2, 3, 4, 5})));
+    PointwiseAttr p;
+    p.setMode(PointwiseAttr::Mode::RELU_FWD);
+    auto o = g.pointwise(a, p);
+    o->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK((o->getStride() == chlast({2, 3, 4, 5}))); // inherits IN_0
+  }
+  {
+    Graph g = newGraph("pw_err");
+    auto a = g.tensor(mk("a", {4}, {1}));
+    PointwiseAttr p;
+    auto o = g.pointwise(a, p);
+    o->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::AttributeNotSet,
+                "Pointwise mode not set");
+  }
+  {
+    Graph g = newGraph("pw_err2");
+    auto a = g.tensor(mk("a", {4}, {1}));
+    PointwiseAttr p;
+    p.setMode(PointwiseAttr::Mode::ADD);
+    auto o = g.pointwise(a, p);
+    o->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::AttributeNotSet,
+                "ADD mode requires IN_1 input");
+  }
+  {
+    Graph g = newGraph("pw_err3");
+    auto a = g.tensor(mk("a", {4}, {1}));
+    auto b = g.tensor(mk("b", {4}, {1}));
+    PointwiseAttr p;
+    p.setMode(PointwiseAttr::Mode::RELU_FWD);
+    auto o = g.pointwise(a, b, p);
+    o->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::InvalidAttribute,
+                "RELU_FWD mode should not have IN_1 input set");
+  }
+}
+
+TEST("reduction node: inference and errors") {
+  auto build = [](Dims ydim, ReductionAttr::Mode mode, DataType dt) {
+    Graph g = newGraph("red", dt);
+    auto x = g.tensor(mk("x", {2, 16, 8, 8}, contig({2, 16, 8, 8}), dt));
+    ReductionAttr r;
+    r.setMode(mode);
+    auto y = g.reduction(x, r);
+    y->setOutput(true);
+    if (!ydim.empty())
+      y->setDim(ydim);
+    return g.validate();
+  };
+  CHECK(isOk(build({2, 16, 1, 1}, ReductionAttr::Mode::SUM, DataType::Float)));
+  CHECK_ERROR(build({2, 16, 1, 1}, ReductionAttr::Mode::NOT_SET, DataType::Float),
+              ErrorCode::AttributeNotSet, "Reduction mode not set");
+  CHECK_ERROR(build({2, 16, 1}, ReductionAttr::Mode::SUM, DataType::Float),
+              ErrorCode::InvalidAttribute,
+              "Reduction input and output must have the same rank");
+  CHECK_ERROR(build({2, 16, 1, 1}, ReductionAttr::Mode::AVG, DataType::Int32),
+              ErrorCode::InvalidAttribute,
+              "Reduction AVG is not supported for integral or boolean tensors");
+  CHECK_ERROR(build({2, 16, 4, 1}, ReductionAttr::Mode::SUM, DataType::Float),
+              ErrorCode::InvalidAttribute,
+              "Reduction output dimension 2 must be 1 or match input dimension");
+  CHECK_ERROR(build({}, ReductionAttr::Mode::SUM, DataType::Float),
+              ErrorCode::InvalidAttribute,
+              "Reduction requires at least one dimension to reduce (Y[i] == 1 "
+              "where X[i] > 1)");
+}
+
+TEST("sdpa node: inference and errors") {
+  auto build = [](Dims kd, bool gqa, bool causal, bool mask, float dropout,
+                  Dims maskDim = {1, 1, 64, 64}) {
+    Graph g = newGraph("sdpa", DataType::Half);
+    auto q = g.tensor(mk("q", {1, 8, 64, 64}, contig({1, 8, 64, 64}), DataType::Half));
+    auto k = g.tensor(mk("k", kd, contig(kd), DataType::Half));
+    auto v = g.tensor(mk("v", kd, contig(kd), DataType::Half));
+    std::shared_ptr<TensorAttr> m;
+    if (mask)
+      m = g.tensor(mk("m", maskDim, contig(maskDim), DataType::Half));
+    SdpaAttr a;
+    a.setEnableGqa(gqa).setIsCausal(causal).setDropout(dropout);
+    auto o = g.sdpa(q, k, v, m, a);
+    o->setOutput(true);
+    auto st = g.validate();
+    if (isOk(st)) {
+      if (o->getDim() != Dims{1, 8, 64, 64} || !o->isContiguous() ||
+          o->getName() != "sdpa_0_O")
+        return error(ErrorCode::InternalError, "bad inferred output");
+    }
+    return st;
+  };
+  CHECK(isOk(build({1, 8, 64, 64}, false, true, false, 0.f)));
+  CHECK(isOk(build({1, 2, 64, 64}, true, false, true, 0.f)));
+  CHECK_ERROR(build({1, 2, 64, 64}, false, false, false, 0.f),
+              ErrorCode::InvalidAttribute,
+              "SDPA without GQA requires Q heads (8) to equal K heads (2)");
+  CHECK_ERROR(build({1, 3, 64, 64}, true, false, false, 0.f),
+              ErrorCode::InvalidAttribute,
+              "SDPA with GQA requires Q heads (8) to be a multiple of K heads "
+              "(3)");
+  CHECK_ERROR(build({1, 8, 64, 64}, false, true, true, 0.f),
+              ErrorCode::InvalidAttribute,
+              "SDPA attention mask and is_causal are mutually exclusive");
+  CHECK_ERROR(build({1, 8, 64, 64}, false, false, true, 0.f, {1, 1, 32, 64}),
+              ErrorCode::InvalidAttribute,
+              "SDPA attention mask seq_q dim (32) must be 1 or match Q "
+              "sequence length (64)");
+  CHECK_ERROR(build({1, 8, 64, 64}, false, false, false, 1.0f),
+              ErrorCode::InvalidAttribute,
+              "SDPA dropout probability must be in [0, 1)");
+  CHECK_ERROR(build({1, 8, 64, 32}, false, false, false, 0.f),
+              ErrorCode::InvalidAttribute,
+              "SDPA input tensors Q and K must have matching head_dim");
+}
+
+TEST("norm nodes: inference and errors") {
+  {
+    Graph g = newGraph("rms");
+    auto x = g.tensor(mk("x", {2, 3, 32, 32}, chlast({2, 3, 32, 32})));
+    auto s = g.tensor(TensorAttr().setName("s").setDataType(DataType::Float));
+    RmsnormAttr a;
+    a.setForwardPhase(NormFwdPhase::INFERENCE)
+        .setEpsilon(g.tensor(TensorAttr(1e-5f)));
+    auto [y, r] = g.rmsnorm(x, s, a);
+    y->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK(r == nullptr);
+    CHECK((s->getDim() == Dims{1, 3, 32, 32}));
+    CHECK((s->getStride() == chlast({1, 3, 32, 32}))); // follows X's format
+    CHECK((y->getStride() == x->getStride()));
+    CHECK(y->getName() == "rmsnorm_0_Y");
+  }
+  {
+    Graph g = newGraph("rms_train");
+    auto x = g.tensor(mk("x", {2, 8}, {8, 1}));
+    RmsnormAttr a;
+    a.setForwardPhase(NormFwdPhase::TRAINING)
+        .setEpsilon(g.tensor(TensorAttr(1e-5f)));
+    auto [y, r] = g.rmsnorm(x, nullptr, a);
+    y->setOutput(true);
+    r->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::NotImplemented,
+                "RmsNorm training mode is not yet supported: torch-mlir does "
+                "not lower the training variant");
+  }
+  {
+    Graph g = newGraph("rms_err");
+    auto x = g.tensor(mk("x", {2, 8}, {8, 1}));
+    RmsnormAttr a;
+    a.setForwardPhase(NormFwdPhase::INFERENCE);
+    auto [y, r] = g.rmsnorm(x, nullptr, a);
+    y->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::AttributeNotSet,
+                "RmsNorm epsilon not set");
+  }
+  {
+    Graph g = newGraph("ln_train");
+    auto x = g.tensor(mk("x", {4, 3, 8, 8}, contig({4, 3, 8, 8})));
+    auto s = g.tensor(mk("s", {1, 3, 8, 8}, contig({1, 3, 8, 8})));
+    auto b = g.tensor(mk("b", {1, 3, 8, 8}, contig({1, 3, 8, 8})));
+    LayernormAttr a;
+    a.setForwardPhase(NormFwdPhase::TRAINING)
+        .setEpsilon(g.tensor(TensorAttr(1e-5f)));
+    auto [y, m, v] = g.layernorm(x, s, b, a);
+    y->setOutput(true);
+    m->setOutput(true);
+    v->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK((m->getDim() == Dims{4, 1, 1, 1}));
+    CHECK((v->getStride() == Dims{1, 1, 1, 1}));
+    CHECK(m->getName() == "layernorm_0_MEAN" &&
+          v->getName() == "layernorm_0_INV_VARIANCE");
+  }
+  {
+    Graph g = newGraph("ln_err");
+    auto x = g.tensor(mk("x", {4, 3, 8, 8}, contig({4, 3, 8, 8})));
+    auto s = g.tensor(mk("s", {1, 3, 8, 4}, contig({1, 3, 8, 4})));
+    LayernormAttr a;
+    a.setForwardPhase(NormFwdPhase::INFERENCE)
+        .setEpsilon(g.tensor(TensorAttr(1e-5f)));
+    auto [y, m, v] = g.layernorm(x, s, nullptr, a);
+    y->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::InvalidAttribute,
+                "LayerNorm input tensor SCALE must have shape as tensor X with "
+                "single batch");
+  }
+}
+
+// ---- graph state machine ----------------------------------------------------
+struct ConvGraph {
+  std::unique_ptr<Graph> graph;
+  std::shared_ptr<TensorAttr> x, w, y;
+};
+// The reference's executable test graph: all-ones f16 1x1 conv, C = 128
+// (tests/test_graph.cpp:198-223).
+static ConvGraph makeConvGraph(const std::string &name) {
+  ConvGraph c;
+  c.graph = std::make_unique<Graph>();
+  c.graph->setName(name).setIODataType(DataType::Half)
+      .setComputeDataType(DataType::Float);
+  c.x = c.graph->tensor(mk("image", {16, 128, 64, 64},
+                           contig({16, 128, 64, 64}), DataType::Half));
+  c.w = c.graph->tensor(mk("filter", {256, 128, 1, 1},
+                           contig({256, 128, 1, 1}), DataType::Half));
+  ConvFPropAttr a;
+  a.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1}).setName("conv_fprop");
+  c.y = c.graph->convFProp(c.x, c.w, a);
+  c.y->setOutput(true);
+  return c;
+}
+
+TEST("graph: name, symbol uniqueness, broadcast outputs") {
+  {
+    Graph g;
+    CHECK_ERROR(g.validate(), ErrorCode::AttributeNotSet, "Graph name not set");
+  }
+  {
+    Graph g = newGraph("dup");
+    auto a = g.tensor(mk("t", {4}, {1}));
+    auto b = g.tensor(mk("t", {4}, {1}));
+    PointwiseAttr p;
+    p.setMode(PointwiseAttr::Mode::ADD);
+    auto o = g.pointwise(a, b, p);
+    o->setOutput(true);
+    CHECK_ERROR(g.validate(), ErrorCode::InvalidAttribute,
+                "Symbol name 't' already in use");
+  }
+  {
+    Graph g = newGraph("dupnode");
+    auto a = g.tensor(mk("a", {4}, {1}));
+    PointwiseAttr p1, p2;
+    p1.setMode(PointwiseAttr::Mode::RELU_FWD).setName("same");
+    p2.setMode(PointwiseAttr::Mode::RELU_FWD).setName("same");
+    auto m = g.pointwise(a, p1);
+    auto o = g.pointwise(m, p2);
+    o->setOutput(true);
+    auto st = g.validate();
+    CHECK(st.getCode() == ErrorCode::InvalidAttribute);
+  }
+  {
+    Graph g = newGraph("bcast_out");
+    auto a = g.tensor(mk("a", {4, 8}, {8, 1}));
+    PointwiseAttr p;
+    p.setMode(PointwiseAttr::Mode::RELU_FWD);
+    auto o = g.pointwise(a, p);
+    o->setOutput(true).setDim({4, 8}).setStride({0, 1});
+    CHECK_ERROR(g.validate(), ErrorCode::InvalidAttribute,
+                "Tensor 'pointwise_0_OUT_0' has broadcast strides (stride=0) "
+                "on an operation output, which is not yet supported");
+  }
+}
+
+TEST("graph: compile/execute preconditions") {
+  auto c = makeConvGraph("preconditions");
+  auto art = c.graph->compileToArtifact(Backend::AMDGPU);
+  CHECK_ERROR(ErrorObject(art), ErrorCode::NotValidated,
+              "Graph must be validated before being compiled");
+  REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+  CHECK_ERROR(c.graph->loadFromArtifact(cpu, std::vector<uint8_t>{1, 2, 3}),
+              ErrorCode::NotValidated,
+              "Graph must be validated before loading a compiled artifact");
+  REQUIRE_OK(c.graph->validate());
+  REQUIRE_ASSIGN(auto ws0, c.graph->getWorkspaceSize());
+  CHECK(!ws0.has_value()); // nothing loaded yet
+  std::unordered_map<std::shared_ptr<TensorAttr>, std::shared_ptr<Buffer>> pack;
+  auto st = c.graph->execute(cpu, pack, nullptr);
+  CHECK(st.getCode() == ErrorCode::NotCompiled);
+
+  REQUIRE_OK(c.graph->compile(cpu));
+  CHECK(c.graph->getKernelCount() == std::optional<size_t>(1));
+  CHECK_ERROR(c.graph->execute(cpu, pack, nullptr), ErrorCode::InvalidArgument,
+              "Graph::execute requires getWorkspaceSize() to be called before "
+              "workspace allocation and execution");
+  REQUIRE_ASSIGN(auto ws, c.graph->getWorkspaceSize());
+  REQUIRE(ws.has_value());
+  CHECK(*ws == 0);
+  CHECK_ERROR(c.graph->execute(cpu, pack, nullptr), ErrorCode::VariantPackError,
+              "Output tensor missing from variantPack");
+
+  auto bufOf = [&](const std::shared_ptr<TensorAttr> &t) {
+    size_t n = static_cast<size_t>(t->getVolume());
+    auto b = Buffer::allocate(cpu, {n}, std::vector<half>(n, half(1.0f)));
+    return std::make_shared<Buffer>(std::move(*b));
+  };
+  pack[c.y] = bufOf(c.y);
+  CHECK_ERROR(c.graph->execute(cpu, pack, nullptr), ErrorCode::VariantPackError,
+              "Input tensor missing from variantPack");
+  pack[c.x] = bufOf(c.x);
+  pack[c.w] = bufOf(c.w);
+  // Everything is in order; only the missing execution engine stops it.
+  auto run = c.graph->execute(cpu, pack, nullptr);
+  CHECK(run.getCode() == ErrorCode::NotImplemented);
+  // A buffer that is too small is caught before any launch.
+  auto small = Buffer::allocate(cpu, {8}, std::vector<half>(8, half(0.f)));
+  pack[c.y] = std::make_shared<Buffer>(std::move(*small));
+  CHECK(c.graph->execute(cpu, pack, nullptr).getCode() ==
+        ErrorCode::VariantPackError);
+}
+
+TEST("graph: virtual and scalar tensors must stay out of the variant pack") {
+  Graph g = newGraph("pack_rules");
+  auto a = g.tensor(mk("a", {2, 5}, {5, 1}));
+  auto two = g.tensor(TensorAttr(2.0f).setName("two"));
+  PointwiseAttr p1, p2;
+  p1.setMode(PointwiseAttr::Mode::MUL);
+  p2.setMode(PointwiseAttr::Mode::RELU_FWD);
+  auto mid = g.pointwise(a, two, p1); // stays virtual
+  auto out = g.pointwise(mid, p2);
+  out->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+  REQUIRE_OK(g.compile(cpu));
+  REQUIRE_ASSIGN(auto ws, g.getWorkspaceSize());
+  REQUIRE(ws.has_value());
+  CHECK(*ws >= 2 * 5 * 4); // the virtual tensor between the two kernels
+  CHECK(g.getKernelCount() == std::optional<size_t>(2));
+  auto buf = [&] {
+    auto b = Buffer::allocate(cpu, {10}, std::vector<float>(10, 1.f));
+    return std::make_shared<Buffer>(std::move(*b));
+  };
+  auto wsBuf = std::make_shared<Buffer>(std::move(*Buffer::allocateRaw(cpu, *ws)));
+  std::unordered_map<std::shared_ptr<TensorAttr>, std::shared_ptr<Buffer>> pack =
+      {{a, buf()}, {out, buf()}, {mid, buf()}};
+  CHECK_ERROR(g.execute(cpu, pack, wsBuf), ErrorCode::VariantPackError,
+              "Virtual output tensor found in variantPack");
+  pack.erase(mid);
+  pack[two] = buf();
+  CHECK_ERROR(g.execute(cpu, pack, wsBuf), ErrorCode::VariantPackError,
+              "Scalar constant tensor found in variantPack");
+  pack.erase(two);
+  CHECK_ERROR(g.execute(cpu, pack, nullptr), ErrorCode::InvalidArgument,
+              "Workspace buffer required but not provided (size=" +
+                  std::to_string(*ws) + " bytes)");
+  auto tiny = std::make_shared<Buffer>(std::move(*Buffer::allocateRaw(cpu, 8)));
+  CHECK_ERROR(g.execute(cpu, pack, tiny), ErrorCode::InvalidArgument,
+              "Workspace buffer too small: provided 8 bytes, required " +
+                  std::to_string(*ws) + " bytes");
+}
+
+TEST("graph: artifact contract") {
+  REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+  auto consumer = makeConvGraph("aot_consumer");
+  REQUIRE_OK(consumer.graph->validate());
+  std::vector<uint8_t> bytes;
+  {
+    auto producer = makeConvGraph("aot_producer");
+    REQUIRE_OK(producer.graph->validate());
+    REQUIRE_ASSIGN(bytes, producer.graph->compileToArtifact(Backend::CPU));
+  }
+  CHECK(!bytes.empty());
+  // another instance's artifact loads into an identically built graph
+  REQUIRE_OK(consumer.graph->loadFromArtifact(cpu, bytes));
+  REQUIRE_ASSIGN(auto ws, consumer.graph->getWorkspaceSize());
+  CHECK(ws.has_value());
+  // compileToArtifact for another backend leaves the loaded state alone
+  REQUIRE_ASSIGN(auto other, consumer.graph->compileToArtifact(Backend::AMDGPU));
+  CHECK(!other.empty());
+  REQUIRE_ASSIGN(auto ws2, consumer.graph->getWorkspaceSize());
+  CHECK(ws2.has_value());
+  // wrong backend for this handle
+  CHECK(consumer.graph->loadFromArtifact(cpu, other).getCode() ==
+        ErrorCode::RuntimeFailure);
+  REQUIRE_ASSIGN(auto cleared0, consumer.graph->getWorkspaceSize());
+  CHECK(!cleared0.has_value());
+  // garbage bytes fail and clear the loaded state
+  REQUIRE_OK(consumer.graph->loadFromArtifact(cpu, bytes));
+  auto st = consumer.graph->loadFromArtifact(
+      cpu, std::vector<uint8_t>{0xde, 0xad, 0xbe, 0xef});
+  CHECK(isError(st));
+  REQUIRE_ASSIGN(auto cleared, consumer.graph->getWorkspaceSize());
+  CHECK(!cleared.has_value());
+  // a flipped byte is caught by the checksum
+  auto corrupt = bytes;
+  corrupt[corrupt.size() / 2] ^= 0x40;
+  CHECK(isError(consumer.graph->loadFromArtifact(cpu, corrupt)));
+  // an artifact of a different graph is rejected
+  Graph g = newGraph("different");
+  auto a = g.tensor(mk("a", {4, 4}, {4, 1}));
+  PointwiseAttr p;
+  p.setMode(PointwiseAttr::Mode::RELU_FWD);
+  auto o = g.pointwise(a, p);
+  o->setOutput(true);
+  REQUIRE_OK(g.validate());
+  CHECK_ERROR(g.loadFromArtifact(cpu, bytes), ErrorCode::RuntimeFailure,
+              "Artifact does not match this graph (signature mismatch)");
+}
+
+TEST("planner: fusion decisions") {
+  REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+  // conv -> add(bias) -> relu fuses into one kernel, no workspace
+  // (reference lit stats: tests/lit/test_conv_asm_emitter_nhwc_krsc_with_relu.cpp:103-104)
+  {
+    Graph g = newGraph("fuse_conv", DataType::BFloat16);
+    auto x = g.tensor(mk("x", {32, 64, 56, 56}, chlast({32, 64, 56, 56}), DataType::BFloat16));
+    auto w = g.tensor(mk("w", {128, 64, 3, 3}, chlast({128, 64, 3, 3}), DataType::BFloat16));
+    auto b = g.tensor(mk("b", {1, 128, 1, 1}, {128, 1, 128, 128}, DataType::BFloat16));
+    ConvFPropAttr ca;
+    ca.setPadding({1, 1}).setStride({1, 1}).setDilation({1, 1});
+    auto y = g.convFProp(x, w, ca);
+    PointwiseAttr add, relu;
+    add.setMode(PointwiseAttr::Mode::ADD);
+    relu.setMode(PointwiseAttr::Mode::RELU_FWD);
+    auto t = g.pointwise(y, b, add);
+    auto o = g.pointwise(t, relu);
+    o->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(cpu));
+    CHECK(g.getKernelCount() == std::optional<size_t>(1));
+    REQUIRE_ASSIGN(auto ws, g.getWorkspaceSize());
+    CHECK(*ws == 0);
+  }
+  // rmsnorm -> mul(scalar) fuses (BASELINE config 2)
+  {
+    Graph g = newGraph("fuse_rms", DataType::BFloat16);
+    auto x = g.tensor(mk("x", {8192, 4096}, {4096, 1}, DataType::BFloat16));
+    auto s = g.tensor(mk("s", {1, 4096}, {4096, 1}, DataType::BFloat16));
+    RmsnormAttr ra;
+    ra.setForwardPhase(NormFwdPhase::INFERENCE).setEpsilon(g.tensor(TensorAttr(1e-6f)));
+    auto [y, r] = g.rmsnorm(x, s, ra);
+    PointwiseAttr mul;
+    mul.setMode(PointwiseAttr::Mode::MUL);
+    auto o = g.pointwise(y, g.tensor(TensorAttr(0.5f)), mul);
+    o->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(cpu));
+    CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  }
+  // a virtual tensor with two consumers is not fused away
+  {
+    Graph g = newGraph("no_fuse");
+    auto a = g.tensor(mk("a", {256, 128}, {128, 1}));
+    auto b = g.tensor(mk("b", {128, 256}, {256, 1}));
+    MatmulAttr m;
+    auto c = g.matmul(a, b, m);
+    PointwiseAttr p1, p2;
+    p1.setMode(PointwiseAttr::Mode::RELU_FWD);
+    p2.setMode(PointwiseAttr::Mode::ADD);
+    auto r = g.pointwise(c, p1);
+    auto o = g.pointwise(r, c, p2); // c is read twice
+    o->setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(cpu));
+    CHECK(g.getKernelCount() == std::optional<size_t>(3));
+  }
+}
+
+// ---- handle / buffer ----------------------------------------------------------
+TEST("handle: CPU rules and concurrent creation") {
+  auto h = Handle::create(Backend::CPU, /*deviceId=*/0);
+  CHECK_ERROR(ErrorObject(h), ErrorCode::InvalidArgument,
+              "Stream can only be set on AMDGPU backend");
+  auto h2 = Handle::create(Backend::CPU, 0, 0x1234);
+  CHECK_ERROR(ErrorObject(h2), ErrorCode::InvalidArgument,
+              "Stream can only be set on AMDGPU backend");
+  // tests/test_handle.cpp:47-85: many threads create handles at once
+  std::vector<std::thread> threads;
+  std::vector<int> ok_(32, 0);
+  for (int i = 0; i < 32; ++i)
+    threads.emplace_back([&, i] {
+      auto hh = Handle::create(Backend::CPU);
+      ok_[i] = isOk(hh) && hh->getBackend() == Backend::CPU;
+    });
+  for (auto &t : threads)
+    t.join();
+  for (int v : ok_)
+    CHECK(v == 1);
+}
+
+TEST("buffer: allocate / read / move / errors") {
+  REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+  auto zero = Buffer::allocate(cpu, {0}, std::vector<float>{});
+  CHECK_ERROR(ErrorObject(zero), ErrorCode::RuntimeFailure,
+              "Buffer::allocate failed: cannot allocate a buffer with zero "
+              "size");
+  auto mism = Buffer::allocate(cpu, {2, 3}, std::vector<float>(5, 0.f));
+  CHECK_ERROR(ErrorObject(mism), ErrorCode::RuntimeFailure,
+              "Buffer::allocate failed: bufferData size (5) does not match "
+              "product of bufferShape dimensions (6)");
+  auto raw0 = Buffer::allocateRaw(cpu, 0);
+  CHECK_ERROR(ErrorObject(raw0), ErrorCode::RuntimeFailure,
+              "Buffer::allocateRaw failed: cannot allocate zero-size buffer");
+  auto imp = Buffer::import(nullptr, 16);
+  CHECK(ErrorObject(imp).getCode() == ErrorCode::RuntimeFailure);
+
+  std::vector<float> data = {1, 2, 3, 4, 5, 6};
+  REQUIRE_ASSIGN(Buffer b, Buffer::allocate(cpu, {2, 3}, data));
+  CHECK(b != nullptr);
+  std::vector<float> back;
+  REQUIRE_OK(b.read(cpu, back));
+  CHECK(back == data);
+  CHECK_ERROR(b.read(cpu, back), ErrorCode::RuntimeFailure,
+              "Buffer::read failed as outData is NOT empty");
+  Buffer moved = std::move(b);
+  CHECK(b == nullptr);
+  CHECK(moved != nullptr);
+  std::vector<float> again;
+  REQUIRE_OK(moved.read(cpu, again));
+  CHECK(again == data);
+}
+
+TEST("errors: ErrorOr and macros") {
+  auto f = [](bool fail) -> ErrorOr<int> {
+    FUSILLI_RETURN_ERROR_IF(fail, ErrorCode::InvalidArgument, "nope");
+    return ok(7);
+  };
+  auto g = [&](bool fail) -> ErrorObject {
+    FUSILLI_ASSIGN_OR_RETURN(int v, f(fail));
+    FUSILLI_RETURN_ERROR_IF(v != 7, ErrorCode::InternalError, "bad value");
+    return ok();
+  };
+  CHECK(isOk(g(false)));
+  CHECK_ERROR(g(true), ErrorCode::InvalidArgument, "nope");
+  ErrorOr<std::string> s = ok(std::string("hi"));
+  CHECK(*s == "hi" && s->size() == 2);
+  std::ostringstream os;
+  os << error(ErrorCode::VariantPackError, "msg");
+  CHECK(os.str() == "VARIANT_PACK_ERROR: msg");
+  CHECK(dataTypeFromAsm("f8E4M3FN") == DataType::FP8E4M3);
+  CHECK(std::string(dataTypeAsm(DataType::BFloat16)) == "bf16");
+}
+
+int main(int argc, char **argv) { return mini::run(argc, argv); }

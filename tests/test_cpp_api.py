@@ -1,0 +1,30 @@
+"""Runs the C++ graph-API test binaries (tests/cpp).  The host binary needs no
+GPU; the device binary runs the reference samples' known answers end to end on
+Backend::AMDGPU."""
+import os
+import subprocess
+
+import pytest
+
+BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
+
+
+def _run(name, timeout):
+    path = os.path.join(BIN, name)
+    assert os.path.exists(path), \
+        f"{path} missing: run `python -c 'import __graft_entry__ as g; g.build()'`"
+    proc = subprocess.run([path], capture_output=True, text=True, timeout=timeout)
+    tail = "\n".join(proc.stdout.splitlines()[-60:])
+    assert proc.returncode == 0, f"{name} failed:\n{tail}\n{proc.stderr[-2000:]}"
+    assert "0 failed checks" in proc.stdout, tail
+    return proc.stdout
+
+
+def test_cpp_host_api():
+    out = _run("test_host_api", 120)
+    assert "19 cases" in out or "cases, 0 failed" in out
+
+
+@pytest.mark.gpu
+def test_cpp_device_api():
+    _run("test_device_api", 300)
