@@ -1,4 +1,207 @@
+// Convolution forward as implicit GEMM on MFMA.
+//
+// For channels-last tensors (X [N,H,W,C], W [K,R,S,C], OUT [N,P,Q,K]) the
+// convolution is the GEMM  OUT[m, k] = sum_j A[m, j] * Wt[k, j]  with
+// m = (n, p, q) and j = (r, s, c).  A is never built: the GEMM kernel's
+// A-loader gathers each 128-byte run of channels of tap (r, s) straight from
+// X (zeros outside the image), so HBM sees X once per filter tap through L2
+// and the filter once per row tile; bias / activation chains are applied from
+// the accumulators before the single NHWC store.
+//
+// Reference semantics: aten.convolution, groups = 1 here (reference
+// support/asm_emitter.h:690-701, node/conv_node.h:38-56).
 #include "common.h"
 #include "fast_paths.h"
-bool fhip_fast_conv_applicable(const fhip_conv_desc *) { return false; }
-int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *, const void *, const void *, const DevEpilogue &, void *) { return fhip_fail(ctx, "no fast conv"); }
+#include "gemm_kernel.h"
+
+#include <cstdlib>
+
+namespace {
+
+struct ConvPlan {
+  bool ok = false;
+  int kind = 0;
+  int64_t M = 0, N = 0, K = 0;
+  ConvGeom geom{};
+  int bm = 256, bn = 128;
+};
+
+// strides equal the dense channels-last strides of dims (unit dims are free)
+bool is_channels_last(const fhip_tensor_desc &t) {
+  int64_t expect = 1;
+  // order: dim 1 fastest, then spatial dims right to left, dim 0 slowest
+  int order[FHIP_MAX_RANK];
+  int n = 0;
+  order[n++] = 1;
+  for (int i = t.rank - 1; i >= 2; --i)
+    order[n++] = i;
+  order[n++] = 0;
+  for (int i = 0; i < n; ++i) {
+    const int d = order[i];
+    if (t.dim[d] != 1 && t.stride[d] != expect)
+      return false;
+    expect *= t.dim[d];
+  }
+  return true;
+}
+
+// Strides `st` of an operand over the output dims [n, k, spatial...]: do the
+// pixel dims (n, p, q) collapse to one stride `sm` per flattened pixel index?
+bool pixel_stride(const int64_t *st, const int64_t *dim, int sp, int64_t *sm) {
+  const int pix_dims[3] = {1 + sp, sp == 2 ? 2 : -1, 0}; // q, p, n
+  int64_t mult = 1;
+  bool have = false;
+  *sm = 0;
+  for (int i = 0; i < 3; ++i) {
+    const int dd = pix_dims[i];
+    if (dd < 0)
+      continue;
+    if (dim[dd] != 1) {
+      if (!have) {
+        if (st[dd] % mult != 0)
+          return false;
+        *sm = st[dd] / mult;
+        have = true;
+      } else if (st[dd] != *sm * mult) {
+        return false;
+      }
+    }
+    mult *= dim[dd];
+  }
+  return true;
+}
+
+ConvPlan make_plan(const fhip_conv_desc *d) {
+  ConvPlan p;
+  if (d->spatial_rank != 2 && d->spatial_rank != 1)
+    return p;
+  if (d->x.dtype != d->w.dtype)
+    return p;
+  if (d->x.dtype == FHIP_BFLOAT16)
+    p.kind = GK_BF16;
+  else if (d->x.dtype == FHIP_HALF)
+    p.kind = GK_F16;
+  else
+    return p;
+  const int elem = 2;
+  const int sp = d->spatial_rank;
+  const int64_t C = d->x.dim[1];
+  if (d->w.dim[1] != C) // grouped convolutions take the generic kernel
+    return p;
+  if ((C * elem) % kTileKBytes != 0)
+    return p;
+  if (!is_channels_last(d->x) || !is_channels_last(d->w) ||
+      !is_channels_last(d->out))
+    return p;
+  auto f = [](int dt) {
+    return dt == FHIP_FLOAT || dt == FHIP_BFLOAT16 || dt == FHIP_HALF;
+  };
+  if (!f(d->y.dtype) || !f(d->out.dtype) || !fhip_epilogue_is_fast(d->epilogue))
+    return p;
+  ConvGeom &g = p.geom;
+  const int h = sp == 2 ? 0 : -1; // index of the H dim among spatial dims
+  g.H = sp == 2 ? (int32_t)d->x.dim[2] : 1;
+  g.W = (int32_t)d->x.dim[1 + sp];
+  g.C = (int32_t)C;
+  g.P = sp == 2 ? (int32_t)d->y.dim[2] : 1;
+  g.Q = (int32_t)d->y.dim[1 + sp];
+  const int64_t R = sp == 2 ? d->w.dim[2] : 1;
+  g.S = (int32_t)d->w.dim[1 + sp];
+  g.pad_h = h == 0 ? (int32_t)d->padding[0] : 0;
+  g.str_h = h == 0 ? (int32_t)d->stride[0] : 1;
+  g.dil_h = h == 0 ? (int32_t)d->dilation[0] : 1;
+  g.pad_w = (int32_t)d->padding[sp - 1];
+  g.str_w = (int32_t)d->stride[sp - 1];
+  g.dil_w = (int32_t)d->dilation[sp - 1];
+  g.slices_per_tap = (int32_t)(C * elem / kTileKBytes);
+  p.M = d->x.dim[0] * g.P * g.Q;
+  p.N = d->w.dim[0];
+  p.K = R * g.S * C;
+  // 32-bit pixel arithmetic in the gather
+  if (d->x.dim[0] * (int64_t)g.H * g.W >= (1ll << 31) || p.M >= (1ll << 31))
+    return p;
+  // Fused operands must be addressable as base + m * sm + k * sk: either
+  // constant over pixels (a per-channel vector) or laid out like OUT.
+  for (int i = 0; i < d->epilogue.count; ++i) {
+    const fhip_epilogue_op &o = d->epilogue.op[i];
+    if (o.operand_kind != FHIP_OPERAND_TENSOR)
+      continue;
+    if (!f(o.operand.dtype))
+      return p;
+    int64_t st[FHIP_MAX_RANK];
+    if (!fhip_broadcast_strides(o.operand, d->y.rank, d->y.dim, st))
+      return p;
+    int64_t sm;
+    if (!pixel_stride(st, d->y.dim, sp, &sm))
+      return p;
+  }
+  p.bn = p.N > 128 ? 256 : 128;
+  p.bm = p.M >= 256 ? 256 : 128;
+  if (p.bn == 256 && p.bm == 128)
+    p.bn = 128;
+  if (const char *env = getenv("FUSILLI_HIP_CONV_TILE")) {
+    int bm = 0, bn = 0;
+    if (sscanf(env, "%d,%d", &bm, &bn) == 2 && (bm == 128 || bm == 256) &&
+        (bn == 128 || bn == 256) && bm >= bn)
+      p.bm = bm, p.bn = bn;
+  }
+  p.ok = true;
+  return p;
+}
+
+} // namespace
+
+int conv_launch_bf16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
+  return conv_launch_kind<GK_BF16>(ctx, bm, bn, g);
+}
+int conv_launch_f16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
+  return conv_launch_kind<GK_F16>(ctx, bm, bn, g);
+}
+
+bool fhip_fast_conv_applicable(const fhip_conv_desc *d) {
+  return make_plan(d).ok;
+}
+
+int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
+                   const void *w, const DevEpilogue &epi, void *out) {
+  const ConvPlan p = make_plan(d);
+  FHIP_REQUIRE(ctx, p.ok, "conv: descriptor not supported by the MFMA kernel");
+  FHIP_REQUIRE(ctx, ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0,
+               "conv: X and W must be 16-byte aligned");
+  const int sp = d->spatial_rank;
+  GemmArgs g{};
+  g.conv = p.geom;
+  g.a = (const char *)x;
+  g.b = (const char *)w;
+  g.out = (char *)out;
+  g.M = p.M;
+  g.N = p.N;
+  g.K = p.K;
+  g.a_ld = 0;
+  g.b_ld = p.K; // filter rows are R*S*C contiguous elements
+  g.o_sm = p.N; // OUT is dense channels-last: consecutive pixels are N apart
+  g.o_sn = 1;
+  g.o_batch = 0;
+  g.c_dt = d->y.dtype;
+  g.o_dt = d->out.dtype;
+  g.tiles_m = (int)((p.M + p.bm - 1) / p.bm);
+  g.tiles_n = (int)((p.N + p.bn - 1) / p.bn);
+  g.epi = epi;
+  g.epi.rank = 3;
+  for (int i = 0; i < epi.count; ++i) {
+    const DevEpiOp &s = epi.op[i];
+    DevEpiOp &o = g.epi.op[i];
+    int64_t st[FHIP_MAX_RANK], sm = 0;
+    for (int k = 0; k < d->y.rank; ++k)
+      st[k] = s.stride[k];
+    if (s.kind == FHIP_OPERAND_TENSOR)
+      FHIP_REQUIRE(ctx, pixel_stride(st, d->y.dim, sp, &sm),
+                   "conv: fused operand layout not supported");
+    o.stride[0] = 0;
+    o.stride[1] = sm;          // per-pixel step (0 for channel vectors)
+    o.stride[2] = s.stride[1]; // per-channel step
+  }
+  if (p.kind == GK_BF16)
+    return conv_launch_bf16(ctx, p.bm, p.bn, g);
+  return conv_launch_f16(ctx, p.bm, p.bn, g);
+}

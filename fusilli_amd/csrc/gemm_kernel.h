@@ -72,7 +72,21 @@ __device__ __forceinline__ void gemm_static_for(F &&f) {
 constexpr int kTileKBytes = 128; // bytes of K per LDS slice
 constexpr int kThreads = 256;
 
+// Geometry of an implicit-GEMM convolution: A is never materialised; row m of
+// the GEMM is output pixel (n, p, q) and K-slice kt is filter tap (r, s) with a
+// 128-byte run of channels, gathered from the NHWC input (zero outside it).
+struct ConvGeom {
+  int32_t H, W, C;        // input spatial extents and channels
+  int32_t P, Q;           // output spatial extents
+  int32_t S;              // filter width (taps per filter row)
+  int32_t pad_h, pad_w, str_h, str_w, dil_h, dil_w;
+  int32_t slices_per_tap; // C * elem / 128
+};
+
+enum GemmAMode { A_KCONTIG = 0, A_MCONTIG = 1, A_CONV = 2 };
+
 struct GemmArgs {
+  ConvGeom conv;
   const char *a;
   const char *b;
   char *out;
@@ -251,9 +265,10 @@ __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
   }
 }
 
-template <int KIND, int BM, int BN, bool A_KC, bool B_KC>
+template <int KIND, int BM, int BN, int A_MODE, bool B_KC>
 __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   using Acc = typename KindTraits<KIND>::Acc;
+  constexpr bool A_KC = A_MODE != A_MCONTIG;
   constexpr int ELEM = KindTraits<KIND>::kElemBytes;
   constexpr int STEPB = KindTraits<KIND>::kStepBytes;
   constexpr int KSTEPS = kTileKBytes / STEPB;
@@ -308,7 +323,47 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   const int64_t a_ldb = g.a_ld * ELEM, b_ldb = g.b_ld * ELEM;
   const int64_t kt_count = g.K * ELEM / kTileKBytes;
 
-  load_slice<BM, ELEM, A_KC>(a, a_ldb, m0, g.M, 0, ra);
+  // Implicit-GEMM gather state: the rows a thread copies are the same for
+  // every K-slice, so their pixel coordinates are decoded once.
+  constexpr int CONV_ROWS = A_MODE == A_CONV ? GA::kChunks : 1;
+  int32_t cv_pix[CONV_ROWS], cv_ih[CONV_ROWS], cv_iw[CONV_ROWS];
+  if constexpr (A_MODE == A_CONV) {
+#pragma unroll
+    for (int i = 0; i < GA::kChunks; ++i) {
+      const int64_t m = m0 + (threadIdx.x >> 3) + 32 * i;
+      const bool live = m < g.M;
+      const int32_t mm = (int32_t)(live ? m : g.M - 1);
+      const int32_t q = mm % g.conv.Q, pq = mm / g.conv.Q;
+      const int32_t pp = pq % g.conv.P, nn = pq / g.conv.P;
+      cv_pix[i] = nn * g.conv.H * g.conv.W;
+      // rows past M read nothing: park them far outside the image
+      cv_ih[i] = live ? pp * g.conv.str_h - g.conv.pad_h : -(1 << 28);
+      cv_iw[i] = q * g.conv.str_w - g.conv.pad_w;
+    }
+  }
+  auto load_a = [&](int64_t kt) {
+    if constexpr (A_MODE == A_CONV) {
+      const int32_t tap = (int32_t)(kt / g.conv.slices_per_tap);
+      const int32_t cb = (int32_t)(kt % g.conv.slices_per_tap) * kTileKBytes;
+      const int32_t fr = tap / g.conv.S, fs = tap % g.conv.S;
+      const int32_t dh = fr * g.conv.dil_h, dw = fs * g.conv.dil_w;
+      const int col = threadIdx.x & 7;
+#pragma unroll
+      for (int i = 0; i < GA::kChunks; ++i) {
+        const int32_t ih = cv_ih[i] + dh, iw = cv_iw[i] + dw;
+        const bool inside = (uint32_t)ih < (uint32_t)g.conv.H &&
+                            (uint32_t)iw < (uint32_t)g.conv.W;
+        const int64_t pix = (int64_t)cv_pix[i] + ih * g.conv.W + iw;
+        ra[i] = inside ? *reinterpret_cast<const u32x4 *>(
+                             a + pix * ((int64_t)g.conv.C * ELEM) + cb + col * 16)
+                       : u32x4{0, 0, 0, 0};
+      }
+    } else {
+      load_slice<BM, ELEM, A_KC>(a, a_ldb, m0, g.M, kt * kTileKBytes, ra);
+    }
+  };
+
+  load_a(0);
   load_slice<BN, ELEM, B_KC>(b, b_ldb, n0, g.N, 0, rb);
   store_slice<BM, ELEM, A_KC>(lds_a(0), ra);
   store_slice<BN, ELEM, B_KC>(lds_b(0), rb);
@@ -318,7 +373,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
     const int cur = kt & 1;
     const bool more = kt + 1 < kt_count;
     if (more) {
-      load_slice<BM, ELEM, A_KC>(a, a_ldb, m0, g.M, (kt + 1) * kTileKBytes, ra);
+      load_a(kt + 1);
       load_slice<BN, ELEM, B_KC>(b, b_ldb, n0, g.N, (kt + 1) * kTileKBytes, rb);
     }
     const char *sa = lds_a(cur);
@@ -421,12 +476,13 @@ struct GemmPlan {
   int bm = 256, bn = 256;
 };
 
-template <int KIND, int BM, int BN, bool A_KC, bool B_KC>
+template <int KIND, int BM, int BN, int A_MODE, bool B_KC>
 int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
   constexpr int ELEM = KindTraits<KIND>::kElemBytes;
+  constexpr bool A_KC = A_MODE != A_MCONTIG;
   constexpr int lds = 2 * SliceGeom<BM, ELEM, A_KC>::kBytes +
                       2 * SliceGeom<BN, ELEM, B_KC>::kBytes;
-  auto kernel = gemm_kernel<KIND, BM, BN, A_KC, B_KC>;
+  auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC>;
   static bool configured = false;
   if (!configured) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
@@ -443,12 +499,12 @@ int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
 template <int KIND, int BM, int BN>
 int launch_orient(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g) {
   if (p.a_kc && p.b_kc)
-    return launch<KIND, BM, BN, true, true>(ctx, g, p.batch);
+    return launch<KIND, BM, BN, A_KCONTIG, true>(ctx, g, p.batch);
   if (p.a_kc && !p.b_kc)
-    return launch<KIND, BM, BN, true, false>(ctx, g, p.batch);
+    return launch<KIND, BM, BN, A_KCONTIG, false>(ctx, g, p.batch);
   if (!p.a_kc && p.b_kc)
-    return launch<KIND, BM, BN, false, true>(ctx, g, p.batch);
-  return launch<KIND, BM, BN, false, false>(ctx, g, p.batch);
+    return launch<KIND, BM, BN, A_MCONTIG, true>(ctx, g, p.batch);
+  return launch<KIND, BM, BN, A_MCONTIG, false>(ctx, g, p.batch);
 }
 
 template <int KIND>
@@ -460,6 +516,16 @@ int gemm_launch_kind(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g) {
   return launch_orient<KIND, 128, 128>(ctx, p, g);
 }
 
+
+// Implicit-GEMM convolution launchers (A gathered, B = filter, K-contiguous).
+template <int KIND>
+int conv_launch_kind(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
+  if (bm == 256 && bn == 256)
+    return launch<KIND, 256, 256, A_CONV, true>(ctx, g, 1);
+  if (bm == 256 && bn == 128)
+    return launch<KIND, 256, 128, A_CONV, true>(ctx, g, 1);
+  return launch<KIND, 128, 128, A_CONV, true>(ctx, g, 1);
+}
 
 int gemm_launch_bf16(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g);
 int gemm_launch_f16(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g);

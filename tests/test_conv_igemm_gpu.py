@@ -1,0 +1,155 @@
+"""Implicit-GEMM convolution (MFMA kernel) through the C ABI vs the oracle.
+
+Shapes here satisfy the tuned kernel's contract (channels-last bf16/f16,
+C * 2 bytes a multiple of 128, groups = 1); each test asserts that the tuned
+kernel is the one chosen, so a silent fall back to the generic kernel fails.
+"""
+import numpy as np
+import pytest
+
+from fusilli_amd import capi
+from oracle import oracle
+from helpers import HT, assert_close, rand
+
+pytestmark = pytest.mark.gpu
+
+
+def conv_desc(x, w, out, pad, stride, dil, y_dtype, epilogue=()):
+    d = capi.ConvDesc()
+    d.x, d.w = x.desc(), w.desc()
+    d.y = capi.TensorDesc.make(out.dims, out.strides, y_dtype)
+    d.out = out.desc()
+    d.out_dtype = out.dtype
+    d.spatial_rank = len(pad)
+    for i in range(len(pad)):
+        d.padding[i], d.stride[i], d.dilation[i] = pad[i], stride[i], dil[i]
+    d.epilogue = capi.make_epilogue(list(epilogue))
+    return d
+
+
+def run(ctx, x, w, pad, stride, dil, y_dtype, out_dtype=None, epilogue=(),
+        epi_tensors=(), expect_tuned=True):
+    ydims = oracle.conv_output_dims(x.dims, w.dims, pad, stride, dil)
+    out = HT.empty(ydims, y_dtype if out_dtype is None else out_dtype,
+                   oracle.channels_last_strides(ydims))
+    d = conv_desc(x, w, out, pad, stride, dil, y_dtype, epilogue)
+    assert ctx.lib.fhip_conv_fprop_supported(d) == (2 if expect_tuned else 1)
+    bufs = [t.upload(ctx) for t in epi_tensors]
+    dx, dw, dout = x.upload(ctx), w.upload(ctx), out.upload(ctx)
+    ctx.conv_fprop(d, dx, dw, dout, epilogue_operands=bufs)
+    return out.fetch(ctx, dout)
+
+
+def cl(dims, seed, tid, dtype, std=1.0):
+    return HT.from_logical(rand(seed, tid, dims, std=std), dtype,
+                           oracle.channels_last_strides(dims))
+
+
+CASES = [
+    # 3x3 same padding, the shape family of the headline conv config
+    dict(x=[2, 64, 14, 14], w=[128, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    # ragged M (2*7*5 = 70 pixels) and ragged K_out, stride 2
+    dict(x=[2, 64, 13, 9], w=[40, 64, 3, 3], pad=[1, 1], s=[2, 2], d=[1, 1]),
+    # dilation 2 with asymmetric padding / stride, C = 128 (two K slices per tap)
+    dict(x=[1, 128, 17, 12], w=[136, 128, 3, 2], pad=[2, 1], s=[1, 2], d=[2, 2]),
+    # 1x1 (pure GEMM), many pixels, > 256 output channels
+    dict(x=[3, 192, 12, 12], w=[264, 192, 1, 1], pad=[0, 0], s=[1, 1], d=[1, 1]),
+    # 5x5 filter larger than the padded border reach, no padding
+    dict(x=[1, 64, 11, 11], w=[64, 64, 5, 5], pad=[0, 0], s=[1, 1], d=[1, 1]),
+    # padding wider than the filter reach (all-zero taps at the border)
+    dict(x=[1, 64, 6, 6], w=[32, 64, 3, 3], pad=[3, 3], s=[1, 1], d=[1, 1]),
+    # 1-D convolution
+    dict(x=[2, 64, 50], w=[48, 64, 5], pad=[2], s=[2], d=[1]),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_conv_igemm_random_vs_oracle(ctx, case, dtype):
+    x = cl(case["x"], 41, 0, dtype)
+    w = cl(case["w"], 41, 1, dtype, std=0.1)
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], dtype)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"],
+                            case["d"])
+    assert_close(out.logical(), ref, dtype, str(case))
+
+
+@pytest.mark.parametrize("tile", ["128,128", "256,128", "256,256"])
+def test_conv_igemm_every_tile_shape(ctx, tile, monkeypatch):
+    monkeypatch.setenv("FUSILLI_HIP_CONV_TILE", tile)
+    case = dict(x=[2, 64, 15, 17], w=[300, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1])
+    x = cl(case["x"], 42, 0, capi.BFLOAT16)
+    w = cl(case["w"], 42, 1, capi.BFLOAT16, std=0.1)
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"],
+                            case["d"])
+    # f32 result of bf16 inputs: only the accumulation order differs
+    assert_close(out.logical(), ref, capi.FLOAT, tile, rtol=1e-4)
+
+
+def test_conv_igemm_bias_relu_residual(ctx):
+    # conv -> +bias[K] -> relu -> +residual[N,K,P,Q] (channels-last) -> bf16
+    xd, wd = [2, 64, 10, 12], [96, 64, 3, 3]
+    x = cl(xd, 43, 0, capi.BFLOAT16)
+    w = cl(wd, 43, 1, capi.BFLOAT16, std=0.1)
+    yd = oracle.conv_output_dims(xd, wd, [1, 1], [1, 1], [1, 1])
+    bias = HT.from_logical(rand(43, 2, [1, 96, 1, 1]), capi.BFLOAT16,
+                           oracle.channels_last_strides([1, 96, 1, 1]))
+    res = cl(yd, 43, 3, capi.BFLOAT16)
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0,
+                            operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT),
+           capi.epilogue_op(capi.PW["ADD"], capi.BFLOAT16, operand_index=1,
+                            operand=res.desc())]
+    out = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.FLOAT,
+              out_dtype=capi.BFLOAT16, epilogue=epi, epi_tensors=[bias, res])
+    ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
+    ref = np.maximum(ref + bias.logical(), 0.0) + res.logical()
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+
+
+def test_conv_igemm_not_chosen_outside_contract(ctx):
+    # C = 48 (96 bytes per pixel) and grouped filters keep the generic kernel
+    x = cl([1, 48, 8, 8], 44, 0, capi.BFLOAT16)
+    w = cl([16, 48, 3, 3], 44, 1, capi.BFLOAT16, std=0.1)
+    out = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.BFLOAT16, expect_tuned=False)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+    x = cl([1, 128, 8, 8], 44, 2, capi.BFLOAT16)
+    w = cl([16, 64, 3, 3], 44, 3, capi.BFLOAT16, std=0.1)
+    out = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.BFLOAT16, expect_tuned=False)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+
+
+def test_conv_igemm_headline_shape(ctx):
+    """N16 C64 56x56, K128 3x3 pad 1, bf16, + bias + ReLU at full size.
+
+    All-ones input and filter give closed-form answers (64 channels times the
+    number of in-image taps); random data is checked against the oracle on the
+    first and last image (the convolution is independent per image)."""
+    xd, wd = [16, 64, 56, 56], [128, 64, 3, 3]
+    pad, st, dil = [1, 1], [1, 1], [1, 1]
+    bias = HT.from_logical(rand(45, 2, [1, 128, 1, 1]), capi.BFLOAT16,
+                           oracle.channels_last_strides([1, 128, 1, 1]))
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0,
+                            operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.BFLOAT16)]
+    ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
+    ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
+    out = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16)
+    lg = out.logical()
+    taps_h = np.full(56, 3.0); taps_h[[0, -1]] = 2.0
+    expect = 64.0 * taps_h[:, None] * taps_h[None, :]
+    assert np.array_equal(lg, np.broadcast_to(expect, lg.shape))
+
+    x = cl(xd, 45, 0, capi.BFLOAT16)
+    w = cl(wd, 45, 1, capi.BFLOAT16, std=0.05)
+    out = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16,
+              epilogue=epi, epi_tensors=[bias])
+    lg = out.logical()
+    xl = x.logical()
+    for img in (0, 15):
+        ref = oracle.conv_fprop(xl[img:img + 1], w.logical(), pad, st, dil)
+        ref = np.maximum(ref + bias.logical(), 0.0)
+        assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"image {img}")
