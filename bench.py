@@ -138,6 +138,39 @@ def bench_matmul(ctx, steps, warmup, kind, m=4096, n=4096, k=8192):
             "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
 
 
+def bench_conv(ctx, steps, warmup):
+    """C3: conv_fprop bf16 NHWC N16 C64 56x56, K128 3x3 pad 1, + bias + ReLU."""
+    n, c, h, w, k, r = 16, 64, 56, 56, 128, 3
+    cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
+    xd, wd, yd = [n, c, h, w], [k, c, r, r], [n, k, h, w]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.FLOAT)
+    d.out = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
+    bias_desc = capi.TensorDesc.make([1, k, 1, 1], [k, 1, k, k], capi.BFLOAT16)
+    d.epilogue = capi.make_epilogue([
+        capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0,
+                         operand=bias_desc),
+        capi.epilogue_op(capi.PW["RELU_FWD"], capi.BFLOAT16)])
+    assert ctx.lib.fhip_conv_fprop_supported(d) == 2, "MFMA conv not chosen"
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 0, n * c * h * w)))
+    wt = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 1, k * c * r * r, 0.0, 0.05)))
+    bias = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 2, k)))
+    out = ctx.alloc(n * k * h * w * 2)
+    wall_ms, ev_ms = timed_loop(
+        ctx, lambda i: ctx.conv_fprop(d, x, wt, out, epilogue_operands=[bias]),
+        steps, warmup)
+    flop = 2.0 * n * h * w * k * c * r * r
+    return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
+            "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
+
+
 def cpu_baseline_rmsnorm(seconds_budget=12.0):
     """The oracle's bf16 RMSNorm * scalar on the host cores over a row sample."""
     from oracle import oracle
@@ -215,6 +248,8 @@ def main():
             ctx, ksteps, kwarm, "fp8")
         others["matmul_bf16_4096x4096x4096"] = bench_matmul(
             ctx, ksteps, kwarm, "bf16", 4096, 4096, 4096)
+        others["conv_fprop_bf16_n16c64h56w56_k128r3s3_bias_relu"] = bench_conv(
+            ctx, max(20, args.steps // 4), kwarm)
         line["others"] = others
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline_rmsnorm()

@@ -117,9 +117,12 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
   p.M = d->x.dim[0] * g.P * g.Q;
   p.N = d->w.dim[0];
   p.K = R * g.S * C;
-  // 32-bit pixel arithmetic in the gather
-  if (d->x.dim[0] * (int64_t)g.H * g.W >= (1ll << 31) || p.M >= (1ll << 31))
+  // 32-bit byte offsets in the gather; one validity bit per filter tap
+  const int64_t x_bytes = d->x.dim[0] * (int64_t)g.H * g.W * C * elem;
+  if (x_bytes >= (1ll << 31) || p.M >= (1ll << 31) || R * g.S > 32 ||
+      p.K * elem >= (1ll << 23))
     return p;
+  g.x_bytes = (uint32_t)x_bytes;
   // Fused operands must be addressable as base + m * sm + k * sk: either
   // constant over pixels (a per-channel vector) or laid out like OUT.
   for (int i = 0; i < d->epilogue.count; ++i) {
@@ -186,6 +189,8 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   g.o_dt = d->out.dtype;
   g.tiles_m = (int)((p.M + p.bm - 1) / p.bm);
   g.tiles_n = (int)((p.N + p.bn - 1) / p.bn);
+  g.o_vec = (p.N * fhip_dtype_size(d->out.dtype)) % 16 == 0 &&
+            ((uintptr_t)out & 15) == 0;
   g.epi = epi;
   g.epi.rank = 3;
   for (int i = 0; i < epi.count; ++i) {

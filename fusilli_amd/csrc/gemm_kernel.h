@@ -1,5 +1,21 @@
 // MFMA GEMM kernel template and launch helpers; instantiated once per element
 // kind in gemm_<kind>.hip.
+//
+// Data path of one workgroup (256 threads = 2 x 2 wavefronts, each owning a
+// (BM/2) x (BN/2) block of 32x32 MFMA tiles):
+//   * 128-byte K slices of A and B go from global memory straight into LDS
+//     with the LDS-DMA form of the global load (no staging registers), into a
+//     ring of NSTAGE stages, NSTAGE - 1 slices ahead of the MFMAs;
+//   * LDS rows are unpadded; 16-byte chunks are XOR-permuted inside a row so
+//     both the 16-byte fragment reads (K-contiguous operand) and the
+//     transposing 8-byte reads (M/N-contiguous operand) are bank-conflict free;
+//   * MFMA fragments are double buffered in registers: the reads for K-step
+//     s + 1 are in flight during the MFMAs of step s; the single barrier of an
+//     iteration sits before its last K-step, so the first fragments of the
+//     next slice are fetched behind that step's MFMAs;
+//   * accumulators leave through LDS one 32-row band at a time so that every
+//     lane applies the fused epilogue to 8 consecutive columns and stores them
+//     with one or two 16-byte writes.
 #ifndef FUSILLI_AMD_CSRC_GEMM_KERNEL_H
 #define FUSILLI_AMD_CSRC_GEMM_KERNEL_H
 
@@ -81,6 +97,7 @@ struct ConvGeom {
   int32_t S;              // filter width (taps per filter row)
   int32_t pad_h, pad_w, str_h, str_w, dil_h, dil_w;
   int32_t slices_per_tap; // C * elem / 128
+  uint32_t x_bytes;       // bytes of the input tensor (< 2^31)
 };
 
 enum GemmAMode { A_KCONTIG = 0, A_MCONTIG = 1, A_CONV = 2 };
@@ -97,6 +114,7 @@ struct GemmArgs {
   int64_t o_sm, o_sn, o_batch; // output strides in elements
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
+  int32_t o_vec;              // output rows allow aligned 16-byte stores
   DevEpilogue epi;            // strides refer to (batch, m, n)
 };
 
@@ -130,121 +148,184 @@ __device__ __forceinline__ void mfma32(typename KindTraits<KIND>::AccVec &c,
   }
 }
 
-// LDS geometry of one operand slice.
-//   K-contiguous operand: ROWS rows (m or n) of 128 K-bytes, row pitch 144 B
-//   (16-byte reads by 16 lanes of consecutive rows then touch 64 distinct banks).
-//   Other operand: 128/elem K-rows of ROWS*elem bytes; the row pitch is chosen
-//   so the transposing 8-byte reads of a 32-lane half-wavefront are conflict
-//   free (K-rows 16 words apart for 16-bit, 8 words apart for 8-bit elements).
+
+#define GEMM_AS1 __attribute__((address_space(1)))
+#define GEMM_AS3 __attribute__((address_space(3)))
+
+// s_waitcnt immediate: vmcnt <= n, lgkmcnt = 0, expcnt untouched.
+constexpr int gemm_wait_imm(int vm) {
+  return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0x0 << 8);
+}
+
+// LDS geometry of one operand slice (128 K-bytes of ROWS rows).
+//   K-contiguous operand: ROWS rows of 128 bytes; the 16-byte chunk c of row r
+//   sits at chunk position c ^ (r & 7) ^ ((r >> 3) & 1).
+//   Other operand: 128/elem K-rows of ROWS*elem bytes; chunk c of K-row k sits
+//   at position nkc_pos(k, c).
 template <int ROWS, int ELEM, bool KCONTIG> struct SliceGeom {
+  static constexpr int kBytes = ROWS * kTileKBytes;
+  static constexpr int kLoads = kBytes / 4096; // DMA instructions per thread
   static constexpr int kKRows = kTileKBytes / ELEM;
-  static constexpr int kPitch =
-      KCONTIG ? (kTileKBytes + 16)
-              : (ROWS * ELEM + (ELEM == 2 ? 64 : 32));
-  static constexpr int kBytes = KCONTIG ? ROWS * kPitch : kKRows * kPitch;
-  // 16-byte chunks a thread moves per slice
-  static constexpr int kChunks = ROWS * kTileKBytes / 16 / kThreads;
+  static constexpr int kRowBytes = KCONTIG ? kTileKBytes : ROWS * ELEM;
+  static constexpr int kCPR = kRowBytes / 16;        // chunks per LDS row
+  static constexpr int kRowsPerLoad = 1024 / kRowBytes; // LDS rows per wave DMA
 };
 
-// Global -> registers for one slice of one operand.
+__device__ __forceinline__ int kc_swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+
+// Chunk permutation of the M/N-contiguous layout.  A 32-lane half-wavefront
+// of a transposing read covers 4 K-rows x 64 bytes (16-bit) or 8 K-rows x
+// 32 bytes (8-bit); the permutation spreads those over all 64 banks.
+template <int ELEM, int RB> __device__ __forceinline__ int nkc_pos(int k, int c) {
+  if constexpr (ELEM == 2)
+    return c ^ ((k & 3) << 1) ^ ((c & 2) << 2);
+  else if constexpr (RB == 256)
+    return c ^ ((k & 7) << 1);
+  else
+    return c ^ (((k >> 1) & 3) << 1);
+}
+template <int ELEM, int RB> __device__ __forceinline__ int nkc_chunk(int k, int p) {
+  if constexpr (ELEM == 2) {
+    const int t = p ^ ((k & 3) << 1);
+    return t ^ ((t & 2) << 2);
+  } else {
+    return nkc_pos<ELEM, RB>(k, p);
+  }
+}
+
+// Per-thread byte offsets (from the tile's first row / column at K = 0) of the
+// chunks this thread's DMA instructions fetch; the same for every K slice.
 template <int ROWS, int ELEM, bool KCONTIG>
 __device__ __forceinline__ void
-load_slice(const char *base, int64_t ld_bytes, int64_t row0, int64_t rows_total,
-           int64_t k0_bytes, u32x4 (&regs)[SliceGeom<ROWS, ELEM, KCONTIG>::kChunks]) {
+dma_setup(int64_t ld_bytes, int64_t row0, int64_t rows_total,
+          uint32_t (&off)[SliceGeom<ROWS, ELEM, KCONTIG>::kLoads]) {
   using G = SliceGeom<ROWS, ELEM, KCONTIG>;
-  const int t = threadIdx.x;
+  const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
 #pragma unroll
-  for (int i = 0; i < G::kChunks; ++i) {
-    const int c = t + i * kThreads;
+  for (int j = 0; j < G::kLoads; ++j) {
+    const int group = j * 4 + w;
     if constexpr (KCONTIG) {
-      const int row = c >> 3, col = c & 7; // 8 chunks of 16 B per 128-B row
+      const int row = group * 8 + (l >> 3);
+      const int c = (l & 7) ^ kc_swz(row);
       int64_t r = row0 + row;
-      r = r < rows_total ? r : rows_total - 1; // clamp: ragged edge tiles
-      regs[i] = *reinterpret_cast<const u32x4 *>(base + r * ld_bytes + k0_bytes +
-                                                 col * 16);
+      r = r < rows_total ? r : rows_total - 1; // ragged edge tiles
+      off[j] = (uint32_t)((r - row0) * ld_bytes + c * 16);
     } else {
-      constexpr int cpr = ROWS * ELEM / 16; // chunks per K-row
-      const int krow = c / cpr, col = c % cpr;
-      // element index along the row dimension, clamped at the edge
-      int64_t e = row0 + (int64_t)col * (16 / ELEM);
+      const int k = group * G::kRowsPerLoad + l / G::kCPR;
+      const int c = nkc_chunk<ELEM, G::kRowBytes>(k, l % G::kCPR);
+      int64_t e = row0 + (int64_t)c * (16 / ELEM);
       const int64_t last = rows_total - 16 / ELEM;
       e = e < last ? e : last;
-      regs[i] = *reinterpret_cast<const u32x4 *>(
-          base + (k0_bytes / ELEM + krow) * ld_bytes + e * ELEM);
+      off[j] = (uint32_t)(k * ld_bytes + (e - row0) * ELEM);
     }
   }
 }
 
-template <int ROWS, int ELEM, bool KCONTIG>
-__device__ __forceinline__ void
-store_slice(char *lds, const u32x4 (&regs)[SliceGeom<ROWS, ELEM, KCONTIG>::kChunks]) {
-  using G = SliceGeom<ROWS, ELEM, KCONTIG>;
-  const int t = threadIdx.x;
+// One K slice of one operand, global -> LDS: each wavefront instruction moves
+// 64 x 16 bytes to 1024 consecutive LDS bytes.  Buffer addressing (uniform
+// 64-bit base + 32-bit lane offset) keeps these loads on the vector-memory
+// counter only, so waits on LDS reads stay exact while they are in flight;
+// offsets at or past `bytes` read as zero.
+template <int LOADS>
+__device__ __forceinline__ void dma_issue(const char *base, uint32_t bytes,
+                                          const uint32_t (&off)[LOADS],
+                                          uint32_t lds_stage) {
+  const int w = threadIdx.x >> 6;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)base, 0, (int)bytes, 0x00020000);
 #pragma unroll
-  for (int i = 0; i < G::kChunks; ++i) {
-    const int c = t + i * kThreads;
+  for (int j = 0; j < LOADS; ++j) {
+    const uint32_t dst = lds_stage + (uint32_t)(j * 4 + w) * 1024u;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        rsrc, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
+        (int)off[j], 0, 0, 0);
+  }
+}
+
+// Fragment addressing: per-lane LDS byte offsets (within a stage) that stay
+// fixed for the whole kernel; everything that varies is an immediate.
+template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr {
+  static constexpr int ELEM = KindTraits<KIND>::kElemBytes;
+  static constexpr int STEPB = KindTraits<KIND>::kStepBytes;
+  static constexpr int KSTEPS = kTileKBytes / STEPB;
+  static constexpr int CH = STEPB / 16;  // chunks per row per K-step
+  static constexpr int CHH = CH / 2;     // 16-byte reads per fragment
+  static constexpr int RB = ROWS * ELEM; // M/N-contiguous: bytes per K-row
+  static constexpr int N = KCONTIG ? KSTEPS * CHH : NT;
+  uint32_t a[N];
+
+  __device__ __forceinline__ void setup(int tile0) {
+    const int l = threadIdx.x & 63;
     if constexpr (KCONTIG) {
-      const int row = c >> 3, col = c & 7;
-      *reinterpret_cast<u32x4 *>(lds + row * G::kPitch + col * 16) = regs[i];
+      const int r = tile0 * 32 + (l & 31);
+      const int sw = kc_swz(l & 31);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int i = 0; i < CHH; ++i) {
+          const int c = s * CH + (l >> 5) * CHH + i;
+          a[s * CHH + i] = (uint32_t)(r * kTileKBytes + ((c ^ sw) << 4));
+        }
     } else {
-      constexpr int cpr = ROWS * ELEM / 16;
-      const int krow = c / cpr, col = c % cpr;
-      *reinterpret_cast<u32x4 *>(lds + krow * G::kPitch + col * 16) = regs[i];
+      const int L = l & 15, h = (l >> 4) & 1;
+      constexpr int KPL = STEPB / 2 / ELEM; // K values per lane per step
+      const int kq = ELEM == 2 ? (L >> 2) : (L >> 1);
+      const int k = (l >> 5) * KPL + kq;
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int rb = tile0 + i;
+        int c, sub;
+        if constexpr (ELEM == 2) {
+          c = rb * 4 + h * 2 + ((L & 3) >> 1);
+          sub = (L & 1) * 8;
+        } else {
+          c = rb * 2 + h;
+          sub = (L & 1) * 8;
+        }
+        a[i] = (uint32_t)(k * RB + nkc_pos<ELEM, RB>(k, c) * 16 + sub);
+      }
     }
   }
-}
 
-// LDS -> MFMA fragment for rows [rb*32, rb*32+32) at K-step `s` of the slice.
-template <int KIND, int ROWS, bool KCONTIG>
-__device__ __forceinline__ void load_frag(const char *lds, int rb, int s,
-                                          Frag<KIND> &f) {
-  constexpr int ELEM = KindTraits<KIND>::kElemBytes;
-  constexpr int STEPB = KindTraits<KIND>::kStepBytes;
-  using G = SliceGeom<ROWS, ELEM, KCONTIG>;
-  const int l = threadIdx.x & 63;
-  if constexpr (KCONTIG) {
-    const char *p = lds + (rb * 32 + (l & 31)) * G::kPitch + s * STEPB +
-                    (l >> 5) * (STEPB / 2);
+  // Fragments of the NT tiles for K-step S from the stage at LDS address `st`.
+  template <int S>
+  __device__ __forceinline__ void load(uint32_t st, Frag<KIND> (&f)[NT]) const {
+    if constexpr (KCONTIG) {
 #pragma unroll
-    for (int i = 0; i < STEPB / 32; ++i) {
-      const u32x4 v = *reinterpret_cast<const u32x4 *>(p + 16 * i);
-      f.r[4 * i + 0] = v.x;
-      f.r[4 * i + 1] = v.y;
-      f.r[4 * i + 2] = v.z;
-      f.r[4 * i + 3] = v.w;
-    }
-  } else {
-    // Elements of K this lane needs: (STEPB / 2) / ELEM consecutive K-rows.
-    constexpr int KPL = STEPB / 2 / ELEM;
-    const int kbase = s * (STEPB / ELEM) + (l >> 5) * KPL;
-    const int L = l & 15;
-    const int nsub = rb * 32 + ((l >> 4) & 1) * 16;
-    if constexpr (ELEM == 2) {
-      // 16 lanes cover 4 K-rows x 16 columns; a read returns 4 K values.
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int r = 0; r < KPL / 4; ++r) {
-        const int k = kbase + 4 * r + (L >> 2);
-        const int n = nsub + 4 * (L & 3);
-        const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            LDS_PTR(s16x4, lds, k * G::kPitch + n * 2));
-        const u32x2 w = __builtin_bit_cast(u32x2, v);
-        f.r[2 * r + 0] = w.x;
-        f.r[2 * r + 1] = w.y;
-      }
+        for (int i = 0; i < CHH; ++i) {
+          const u32x4 v = *(const GEMM_AS3 u32x4 *)(uintptr_t)(
+              st + a[S * CHH + i] + t * 32 * kTileKBytes);
+          f[t].r[4 * i + 0] = v.x;
+          f[t].r[4 * i + 1] = v.y;
+          f[t].r[4 * i + 2] = v.z;
+          f[t].r[4 * i + 3] = v.w;
+        }
     } else {
-      // 16 lanes cover 8 K-rows x 16 columns; a read returns 8 K values.
+      constexpr int KPL = STEPB / 2 / ELEM;
+      constexpr int RPK = ELEM == 2 ? 4 : 8; // K values per transposing read
 #pragma unroll
-      for (int r = 0; r < KPL / 8; ++r) {
-        const int k = kbase + 8 * r + (L >> 1);
-        const int n = nsub + 8 * (L & 1);
-        const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-            LDS_PTR(i32x2, lds, k * G::kPitch + n));
-        f.r[2 * r + 0] = (uint32_t)v.x;
-        f.r[2 * r + 1] = (uint32_t)v.y;
-      }
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < KPL / RPK; ++r) {
+          const uint32_t ad = st + a[t] + (S * (STEPB / ELEM) + RPK * r) * RB;
+          if constexpr (ELEM == 2) {
+            const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (GEMM_AS3 s16x4 *)(uintptr_t)ad);
+            const u32x2 w = __builtin_bit_cast(u32x2, v);
+            f[t].r[2 * r + 0] = w.x;
+            f[t].r[2 * r + 1] = w.y;
+          } else {
+            const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                (GEMM_AS3 i32x2 *)(uintptr_t)ad);
+            f[t].r[2 * r + 0] = (uint32_t)v.x;
+            f[t].r[2 * r + 1] = (uint32_t)v.y;
+          }
+        }
     }
   }
-}
+};
 
 template <int N>
 __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
@@ -253,36 +334,45 @@ __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
   if (dt == FHIP_FLOAT) {
 #pragma unroll
     for (int i = 0; i < N; ++i)
-      o[i] = ((const float *)p)[off[i]];
+      o[i] = ((const GEMM_AS1 float *)p)[off[i]];
   } else if (dt == FHIP_BFLOAT16) {
 #pragma unroll
     for (int i = 0; i < N; ++i)
-      o[i] = (float)((const __bf16 *)p)[off[i]];
+      o[i] = (float)((const GEMM_AS1 __bf16 *)p)[off[i]];
   } else {
 #pragma unroll
     for (int i = 0; i < N; ++i)
-      o[i] = (float)((const _Float16 *)p)[off[i]];
+      o[i] = (float)((const GEMM_AS1 _Float16 *)p)[off[i]];
   }
 }
 
-template <int KIND, int BM, int BN, int A_MODE, bool B_KC>
+// LDS bytes of the kernel: NSTAGE stages of (A slice + B slice); the epilogue
+// reuses it for four 32-row accumulator bands (one per wavefront).
+template <int BM, int BN, int NSTAGE> struct GemmLds {
+  static constexpr int kStage = (BM + BN) * kTileKBytes;
+  static constexpr int kEpiPitch = (BN / 2) * 4 + 32;
+  static constexpr int kEpiBytes = 4 * 32 * kEpiPitch;
+  static constexpr int kBytes =
+      NSTAGE * kStage > kEpiBytes ? NSTAGE * kStage : kEpiBytes;
+};
+
+template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int NSTAGE>
 __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   using Acc = typename KindTraits<KIND>::Acc;
   constexpr bool A_KC = A_MODE != A_MCONTIG;
   constexpr int ELEM = KindTraits<KIND>::kElemBytes;
   constexpr int STEPB = KindTraits<KIND>::kStepBytes;
   constexpr int KSTEPS = kTileKBytes / STEPB;
+  static_assert(KSTEPS % 2 == 0, "fragment double buffering needs even KSTEPS");
   using GA = SliceGeom<BM, ELEM, A_KC>;
   using GB = SliceGeom<BN, ELEM, B_KC>;
+  using L = GemmLds<BM, BN, NSTAGE>;
   constexpr int WM = BM / 2, WN = BN / 2; // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int LPS = GA::kLoads + GB::kLoads; // DMA instructions per slice
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  // LDS map: A slice 0, A slice 1, B slice 0, B slice 1.
-  auto lds_a = [&](int buf) { return smem + buf * GA::kBytes; };
-  auto lds_b = [&](int buf) {
-    return smem + 2 * GA::kBytes + buf * GB::kBytes;
-  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
   // XCD-aware tile order: hardware deals consecutive workgroup ids to the 8
   // XCDs in turn; give each XCD a contiguous run of logical ids, then walk the
@@ -303,12 +393,101 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   const int64_t batch = blockIdx.y;
 
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-  const char *a = g.a + batch * g.a_batch * ELEM;
-  const char *b = g.b + batch * g.b_batch * ELEM;
+  const int64_t a_ldb = g.a_ld * ELEM, b_ldb = g.b_ld * ELEM;
+  const int kt_count = (int)(g.K * ELEM / kTileKBytes);
 
   const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int l = threadIdx.x & 63;
+
+  // ---- global -> LDS plumbing ---------------------------------------------
+  // A and B tile base pointers at K = 0 and their per-slice advance.
+  const char *a_base;
+  int64_t a_step;
+  uint32_t off_a[GA::kLoads], off_b[GB::kLoads];
+  // implicit-GEMM gather: pixel index of tap (0, 0) and in-image tap mask
+  int32_t cv_pix[A_MODE == A_CONV ? GA::kLoads : 1];
+  uint32_t cv_mask[A_MODE == A_CONV ? GA::kLoads : 1];
+  int cv_chunk = 0;
+  if constexpr (A_MODE == A_CONV) {
+    a_base = g.a;
+    a_step = 0;
+    const int taps = kt_count / g.conv.slices_per_tap;
+#pragma unroll
+    for (int j = 0; j < GA::kLoads; ++j) {
+      const int row = (j * 4 + wave) * 8 + (l >> 3);
+      const int64_t m = m0 + row;
+      const bool live = m < g.M;
+      const int32_t mm = (int32_t)(live ? m : 0);
+      const int32_t q = mm % g.conv.Q, pq = mm / g.conv.Q;
+      const int32_t pp = pq % g.conv.P, nn = pq / g.conv.P;
+      const int32_t ih0 = pp * g.conv.str_h - g.conv.pad_h;
+      const int32_t iw0 = q * g.conv.str_w - g.conv.pad_w;
+      cv_pix[j] = (nn * g.conv.H + ih0) * g.conv.W + iw0;
+      uint32_t mask = 0;
+      for (int t = 0; t < taps; ++t) {
+        const int32_t ih = ih0 + (t / g.conv.S) * g.conv.dil_h;
+        const int32_t iw = iw0 + (t % g.conv.S) * g.conv.dil_w;
+        const bool in = (uint32_t)ih < (uint32_t)g.conv.H &&
+                        (uint32_t)iw < (uint32_t)g.conv.W;
+        mask |= (uint32_t)(in && live) << t;
+      }
+      cv_mask[j] = mask;
+      cv_chunk = ((l & 7) ^ kc_swz(row)) * 16; // same for every j
+    }
+  } else if constexpr (A_KC) {
+    a_base = g.a + batch * g.a_batch * ELEM + m0 * a_ldb;
+    a_step = kTileKBytes;
+    dma_setup<BM, ELEM, true>(a_ldb, m0, g.M, off_a);
+  } else {
+    a_base = g.a + batch * g.a_batch * ELEM + m0 * ELEM;
+    a_step = (int64_t)GA::kKRows * a_ldb;
+    dma_setup<BM, ELEM, false>(a_ldb, m0, g.M, off_a);
+  }
+  const char *b_base;
+  int64_t b_step;
+  if constexpr (B_KC) {
+    b_base = g.b + batch * g.b_batch * ELEM + n0 * b_ldb;
+    b_step = kTileKBytes;
+  } else {
+    b_base = g.b + batch * g.b_batch * ELEM + n0 * ELEM;
+    b_step = (int64_t)GB::kKRows * b_ldb;
+  }
+  dma_setup<BN, ELEM, B_KC>(b_ldb, n0, g.N, off_b);
+
+  auto stage_a = [&](int st) { return lds0 + (uint32_t)st * L::kStage; };
+  auto stage_b = [&](int st) {
+    return lds0 + (uint32_t)st * L::kStage + GA::kBytes;
+  };
+  auto issue = [&](int kt, int st) {
+    if constexpr (A_MODE == A_CONV) {
+      const int32_t tap = kt / g.conv.slices_per_tap;
+      const int32_t cb = (kt % g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
+      const int32_t fr = tap / g.conv.S, fs = tap % g.conv.S;
+      const int32_t dpix = fr * g.conv.dil_h * g.conv.W + fs * g.conv.dil_w;
+      const int32_t cbytes = g.conv.C * ELEM;
+      uint32_t off[GA::kLoads];
+#pragma unroll
+      for (int j = 0; j < GA::kLoads; ++j) {
+        const bool in = (cv_mask[j] >> tap) & 1;
+        // taps outside the image (and rows past M) read past the end: zeros
+        off[j] = in ? (uint32_t)((cv_pix[j] + dpix) * cbytes + cb) : 0x80000000u;
+      }
+      dma_issue<GA::kLoads>(a_base, g.conv.x_bytes, off, stage_a(st));
+    } else {
+      dma_issue<GA::kLoads>(a_base + kt * a_step, 0xffffffffu, off_a,
+                            stage_a(st));
+    }
+    dma_issue<GB::kLoads>(b_base + kt * b_step, 0xffffffffu, off_b,
+                          stage_b(st));
+  };
+
+  // ---- fragments ----------------------------------------------------------
+  FragAddr<KIND, BM, A_KC, TM> fa_addr;
+  FragAddr<KIND, BN, B_KC, TN> fb_addr;
+  fa_addr.setup(wm * TM);
+  fb_addr.setup(wn * TN);
+  Frag<KIND> fa[2][TM], fb[2][TN];
 
   typename KindTraits<KIND>::AccVec acc[TM][TN];
 #pragma unroll
@@ -319,150 +498,190 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
 
-  u32x4 ra[GA::kChunks], rb[GB::kChunks];
-  const int64_t a_ldb = g.a_ld * ELEM, b_ldb = g.b_ld * ELEM;
-  const int64_t kt_count = g.K * ELEM / kTileKBytes;
+  // ---- prologue: fill NSTAGE - 1 stages ------------------------------------
+#pragma unroll
+  for (int p = 0; p < NSTAGE - 1; ++p)
+    if (p < kt_count)
+      issue(p, p);
+  __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  fa_addr.template load<0>(stage_a(0), fa[0]);
+  fb_addr.template load<0>(stage_b(0), fb[0]);
 
-  // Implicit-GEMM gather state: the rows a thread copies are the same for
-  // every K-slice, so their pixel coordinates are decoded once.
-  constexpr int CONV_ROWS = A_MODE == A_CONV ? GA::kChunks : 1;
-  int32_t cv_pix[CONV_ROWS], cv_ih[CONV_ROWS], cv_iw[CONV_ROWS];
-  if constexpr (A_MODE == A_CONV) {
-#pragma unroll
-    for (int i = 0; i < GA::kChunks; ++i) {
-      const int64_t m = m0 + (threadIdx.x >> 3) + 32 * i;
-      const bool live = m < g.M;
-      const int32_t mm = (int32_t)(live ? m : g.M - 1);
-      const int32_t q = mm % g.conv.Q, pq = mm / g.conv.Q;
-      const int32_t pp = pq % g.conv.P, nn = pq / g.conv.P;
-      cv_pix[i] = nn * g.conv.H * g.conv.W;
-      // rows past M read nothing: park them far outside the image
-      cv_ih[i] = live ? pp * g.conv.str_h - g.conv.pad_h : -(1 << 28);
-      cv_iw[i] = q * g.conv.str_w - g.conv.pad_w;
-    }
-  }
-  auto load_a = [&](int64_t kt) {
-    if constexpr (A_MODE == A_CONV) {
-      const int32_t tap = (int32_t)(kt / g.conv.slices_per_tap);
-      const int32_t cb = (int32_t)(kt % g.conv.slices_per_tap) * kTileKBytes;
-      const int32_t fr = tap / g.conv.S, fs = tap % g.conv.S;
-      const int32_t dh = fr * g.conv.dil_h, dw = fs * g.conv.dil_w;
-      const int col = threadIdx.x & 7;
-#pragma unroll
-      for (int i = 0; i < GA::kChunks; ++i) {
-        const int32_t ih = cv_ih[i] + dh, iw = cv_iw[i] + dw;
-        const bool inside = (uint32_t)ih < (uint32_t)g.conv.H &&
-                            (uint32_t)iw < (uint32_t)g.conv.W;
-        const int64_t pix = (int64_t)cv_pix[i] + ih * g.conv.W + iw;
-        ra[i] = inside ? *reinterpret_cast<const u32x4 *>(
-                             a + pix * ((int64_t)g.conv.C * ELEM) + cb + col * 16)
-                       : u32x4{0, 0, 0, 0};
+  int cur = 0;             // stage holding slice kt
+  int fill = NSTAGE - 1;   // stage that slice kt + NSTAGE - 1 goes to
+  for (int kt = 0; kt < kt_count; ++kt) {
+    const bool issued = kt + NSTAGE - 1 < kt_count;
+    if (issued)
+      issue(kt + NSTAGE - 1, fill);
+    __builtin_amdgcn_sched_barrier(0);
+    const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;
+    const uint32_t sa = stage_a(cur), sb = stage_b(cur);
+    gemm_static_for<KSTEPS>([&](auto sc) {
+      constexpr int s = decltype(sc)::value;
+      constexpr int fc = s & 1, fn = fc ^ 1;
+      if constexpr (s + 1 < KSTEPS) {
+        fa_addr.template load<s + 1>(sa, fa[fn]);
+        fb_addr.template load<s + 1>(sb, fb[fn]);
+      } else {
+        // Slice kt + 1 must be in LDS (this thread's DMA, then everyone's),
+        // and every fragment read of this stage must have returned before
+        // another wavefront may refill it.
+        if (issued)
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
+        else
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        if (kt + 1 < kt_count) {
+          fa_addr.template load<0>(stage_a(nxt), fa[fn]);
+          fb_addr.template load<0>(stage_b(nxt), fb[fn]);
+        }
       }
-    } else {
-      load_slice<BM, ELEM, A_KC>(a, a_ldb, m0, g.M, kt * kTileKBytes, ra);
-    }
-  };
-
-  load_a(0);
-  load_slice<BN, ELEM, B_KC>(b, b_ldb, n0, g.N, 0, rb);
-  store_slice<BM, ELEM, A_KC>(lds_a(0), ra);
-  store_slice<BN, ELEM, B_KC>(lds_b(0), rb);
-  __syncthreads();
-
-  for (int64_t kt = 0; kt < kt_count; ++kt) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < kt_count;
-    if (more) {
-      load_a(kt + 1);
-      load_slice<BN, ELEM, B_KC>(b, b_ldb, n0, g.N, (kt + 1) * kTileKBytes, rb);
-    }
-    const char *sa = lds_a(cur);
-    const char *sb = lds_b(cur);
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      Frag<KIND> fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        load_frag<KIND, BM, A_KC>(sa, wm * TM + i, s, fa[i]);
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        load_frag<KIND, BN, B_KC>(sb, wn * TN + j, s, fb[j]);
+      // Keep the fragment reads ahead of this step's MFMAs: the scheduler
+      // would otherwise sink them next to their first use.
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          mfma32<KIND>(acc[i][j], fa[i], fb[j]);
-    }
-    if (more) {
-      store_slice<BM, ELEM, A_KC>(lds_a(cur ^ 1), ra);
-      store_slice<BN, ELEM, B_KC>(lds_b(cur ^ 1), rb);
-    }
-    __syncthreads();
+          mfma32<KIND>(acc[i][j], fa[fc][i], fb[fc][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    cur = nxt;
+    fill = fill + 1 == NSTAGE ? 0 : fill + 1;
   }
 
-  // Epilogue.  Lane l of a 32x32 tile holds column (l & 31) and rows
-  // (r / 4) * 8 + (l >> 5) * 4 + r % 4 for r = 0..15.
+  // ---- epilogue -------------------------------------------------------------
+  // Each wavefront moves its accumulators through a private LDS band of 32
+  // rows x WN columns (row pitch padded by 32 bytes), one tile row at a time,
+  // and reads them back with 8 consecutive columns per lane.
+  constexpr int PITCH = L::kEpiPitch;
+  constexpr int LPR = WN / 8;   // lanes per row
+  constexpr int RPP = 64 / LPR; // rows per pass
+  const uint32_t band = lds0 + (uint32_t)wave * (32 * PITCH);
+  const uint32_t wr = band + (uint32_t)((l >> 5) * 4 * PITCH + (l & 31) * 4);
+  const uint32_t rd = band + (uint32_t)((l / LPR) * PITCH + (l % LPR) * 32);
   const int64_t ob = batch * g.o_batch;
-  gemm_static_for<TM * TN>([&](auto idx) {
-    constexpr int i = decltype(idx)::value / TN;
-    constexpr int j = decltype(idx)::value % TN;
-    const int64_t n = n0 + wn * WN + j * 32 + (l & 31);
-    const int64_t mbase = m0 + wm * WM + i * 32 + (l >> 5) * 4;
-    if (n >= g.N)
-      return;
-    if constexpr (std::is_same<Acc, int>::value) {
+  const int64_t ncol = n0 + wn * WN + (l % LPR) * 8;
+
+#pragma clang loop unroll(disable)
+  for (int i = 0; i < TM; ++i) {
+    gemm_static_for<TM>([&](auto ic) {
+      constexpr int ii = decltype(ic)::value;
+      if (i == ii) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t m = mbase + (r >> 2) * 8 + (r & 3);
-        if (m < g.M)
-          ((int32_t *)g.out)[ob + m * g.o_sm + n * g.o_sn] = acc[i][j][r];
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            *(GEMM_AS3 Acc *)(uintptr_t)(wr + ((r >> 2) * 8 + (r & 3)) * PITCH +
+                                         j * 128) = acc[ii][j][r];
       }
-    } else {
-      float y[16];
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        y[r] = acc[i][j][r];
-      fhip_round_fast_vec<16>(g.c_dt, y);
-      for (int e = 0; e < g.epi.count; ++e) {
-        const DevEpiOp &o = g.epi.op[e];
-        if (o.kind == FHIP_OPERAND_NONE) {
-          fhip_pw_fast_unary_vec<true, 16>(o.mode, y, o.params.swish_beta);
+    });
+#pragma clang loop unroll(disable)
+    for (int p = 0; p < 32 / RPP; ++p) {
+      const int64_t m = m0 + wm * WM + i * 32 + p * RPP + l / LPR;
+      const u32x4 v0 =
+          *(const GEMM_AS3 u32x4 *)(uintptr_t)(rd + p * RPP * PITCH);
+      const u32x4 v1 =
+          *(const GEMM_AS3 u32x4 *)(uintptr_t)(rd + p * RPP * PITCH + 16);
+      if (m >= g.M || ncol >= g.N)
+        continue;
+      const bool full = ncol + 8 <= g.N;
+      const int64_t o0 = ob + m * g.o_sm + ncol * g.o_sn;
+      if constexpr (std::is_same<Acc, int>::value) {
+        GEMM_AS1 int32_t *out = (GEMM_AS1 int32_t *)g.out;
+        if (full && g.o_vec) {
+          *(GEMM_AS1 u32x4 *)(out + o0) = v0;
+          *(GEMM_AS1 u32x4 *)(out + o0 + 4) = v1;
         } else {
-          float other[16];
-          if (o.kind == FHIP_OPERAND_SCALAR) {
+          const uint32_t y[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              other[r] = o.scalar;
-          } else {
-            const int64_t base = batch * o.stride[0] + n * o.stride[2];
-            int64_t off[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              int64_t m = mbase + (r >> 2) * 8 + (r & 3);
-              m = m < g.M ? m : g.M - 1; // edge tiles stay in bounds
-              off[r] = base + m * o.stride[1];
-            }
-            load_operand_vec<16>(o.ptr, o.operand_dtype, off, other);
-          }
-          fhip_pw_fast_binary_vec<16>(o.mode, o.acc_is_in1 != 0, y, other);
+          for (int e = 0; e < 8; ++e)
+            if (ncol + e < g.N)
+              out[o0 + e * g.o_sn] = (int32_t)y[e];
         }
-        fhip_round_fast_vec<16>(o.result_dtype, y);
-      }
+      } else {
+        // (element-wise copies first: bit-casting a vector element directly
+        // reads element 0)
+        const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+        float y[8];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int64_t m = mbase + (r >> 2) * 8 + (r & 3);
-        if (m >= g.M)
-          continue;
-        const int64_t off = ob + m * g.o_sm + n * g.o_sn;
-        if (g.o_dt == FHIP_BFLOAT16)
-          ((__bf16 *)g.out)[off] = (__bf16)y[r];
-        else if (g.o_dt == FHIP_HALF)
-          ((_Float16 *)g.out)[off] = (_Float16)y[r];
-        else
-          ((float *)g.out)[off] = y[r];
+        for (int c = 0; c < 8; ++c)
+          y[c] = __builtin_bit_cast(float, w[c]);
+        fhip_round_fast_vec<8>(g.c_dt, y);
+        for (int e = 0; e < g.epi.count; ++e) {
+          const DevEpiOp &o = g.epi.op[e];
+          if (o.kind == FHIP_OPERAND_NONE) {
+            fhip_pw_fast_unary_vec<true, 8>(o.mode, y, o.params.swish_beta);
+          } else {
+            float other[8];
+            if (o.kind == FHIP_OPERAND_SCALAR) {
+#pragma unroll
+              for (int c = 0; c < 8; ++c)
+                other[c] = o.scalar;
+            } else {
+              const int64_t base = batch * o.stride[0] + m * o.stride[1];
+              int64_t off[8];
+#pragma unroll
+              for (int c = 0; c < 8; ++c) {
+                int64_t n = ncol + c;
+                n = n < g.N ? n : g.N - 1; // edge tiles stay in bounds
+                off[c] = base + n * o.stride[2];
+              }
+              load_operand_vec<8>(o.ptr, o.operand_dtype, off, other);
+            }
+            fhip_pw_fast_binary_vec<8>(o.mode, o.acc_is_in1 != 0, y, other);
+          }
+          fhip_round_fast_vec<8>(o.result_dtype, y);
+        }
+        if (g.o_dt == FHIP_FLOAT) {
+          GEMM_AS1 float *out = (GEMM_AS1 float *)g.out;
+          if (full && g.o_vec) {
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            *(GEMM_AS1 f32x4 *)(out + o0) = f32x4{y[0], y[1], y[2], y[3]};
+            *(GEMM_AS1 f32x4 *)(out + o0 + 4) = f32x4{y[4], y[5], y[6], y[7]};
+          } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+              if (ncol + c < g.N)
+                out[o0 + c * g.o_sn] = y[c];
+          }
+        } else if (g.o_dt == FHIP_BFLOAT16) {
+          GEMM_AS1 __bf16 *out = (GEMM_AS1 __bf16 *)g.out;
+          if (full && g.o_vec) {
+            bf16x8 v;
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+              v[c] = (__bf16)y[c];
+            *(GEMM_AS1 bf16x8 *)(out + o0) = v;
+          } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+              if (ncol + c < g.N)
+                out[o0 + c * g.o_sn] = (__bf16)y[c];
+          }
+        } else {
+          GEMM_AS1 _Float16 *out = (GEMM_AS1 _Float16 *)g.out;
+          if (full && g.o_vec) {
+            f16x8 v;
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+              v[c] = (_Float16)y[c];
+            *(GEMM_AS1 f16x8 *)(out + o0) = v;
+          } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+              if (ncol + c < g.N)
+                out[o0 + c * g.o_sn] = (_Float16)y[c];
+          }
+        }
       }
     }
-  });
+  }
 }
 
 // What the host decided about one matmul call.
@@ -476,13 +695,17 @@ struct GemmPlan {
   int bm = 256, bn = 256;
 };
 
+// Stage count per tile: as many as fit the 160 KB LDS, at most 4.
+template <int BM, int BN> struct GemmStages {
+  static constexpr int kStage = (BM + BN) * kTileKBytes;
+  static constexpr int value = 160 * 1024 / kStage >= 4 ? 4 : 160 * 1024 / kStage;
+};
+
 template <int KIND, int BM, int BN, int A_MODE, bool B_KC>
 int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
-  constexpr int ELEM = KindTraits<KIND>::kElemBytes;
-  constexpr bool A_KC = A_MODE != A_MCONTIG;
-  constexpr int lds = 2 * SliceGeom<BM, ELEM, A_KC>::kBytes +
-                      2 * SliceGeom<BN, ELEM, B_KC>::kBytes;
-  auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC>;
+  constexpr int NSTAGE = GemmStages<BM, BN>::value;
+  constexpr int lds = GemmLds<BM, BN, NSTAGE>::kBytes;
+  auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC, NSTAGE>;
   static bool configured = false;
   if (!configured) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
@@ -515,7 +738,6 @@ int gemm_launch_kind(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g) {
     return launch_orient<KIND, 256, 128>(ctx, p, g);
   return launch_orient<KIND, 128, 128>(ctx, p, g);
 }
-
 
 // Implicit-GEMM convolution launchers (A gathered, B = filter, K-contiguous).
 template <int KIND>

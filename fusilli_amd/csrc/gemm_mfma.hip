@@ -95,6 +95,9 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
     return p;
   if (p.M < 128 || p.N < 128)
     return p;
+  // lane offsets inside a tile's rows are 32-bit
+  if (p.a_ld * elem >= (1ll << 23) || p.b_ld * elem >= (1ll << 23))
+    return p;
   // M/N-contiguous operands are moved in 16-byte column chunks
   if (!p.a_kc && (p.M * elem) % 16 != 0)
     return p;
@@ -180,6 +183,11 @@ int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
   g.o_dt = d->out.dtype;
   g.tiles_m = (int)((p.M + p.bm - 1) / p.bm);
   g.tiles_n = (int)((p.N + p.bn - 1) / p.bn);
+  {
+    const int64_t oe = fhip_dtype_size(d->out.dtype);
+    g.o_vec = p.o_sn == 1 && (p.o_sm * oe) % 16 == 0 &&
+              (p.o_batch * oe) % 16 == 0 && ((uintptr_t)out & 15) == 0;
+  }
   // epilogue strides on (batch, m, n)
   g.epi = epi;
   g.epi.rank = 3;
