@@ -162,9 +162,9 @@ constexpr int gemm_wait_imm(int vm) {
 //   sits at chunk position c ^ (r & 7) ^ ((r >> 3) & 1).
 //   Other operand: 128/elem K-rows of ROWS*elem bytes; chunk c of K-row k sits
 //   at position nkc_pos(k, c).
-template <int ROWS, int ELEM, bool KCONTIG> struct SliceGeom {
+template <int ROWS, int ELEM, bool KCONTIG, int NW = 4> struct SliceGeom {
   static constexpr int kBytes = ROWS * kTileKBytes;
-  static constexpr int kLoads = kBytes / 4096; // DMA instructions per thread
+  static constexpr int kLoads = kBytes / 1024 / NW; // DMA instructions per thread
   static constexpr int kKRows = kTileKBytes / ELEM;
   static constexpr int kRowBytes = KCONTIG ? kTileKBytes : ROWS * ELEM;
   static constexpr int kCPR = kRowBytes / 16;        // chunks per LDS row
@@ -195,15 +195,15 @@ template <int ELEM, int RB> __device__ __forceinline__ int nkc_chunk(int k, int 
 
 // Per-thread byte offsets (from the tile's first row / column at K = 0) of the
 // chunks this thread's DMA instructions fetch; the same for every K slice.
-template <int ROWS, int ELEM, bool KCONTIG>
+template <int ROWS, int ELEM, bool KCONTIG, int NW>
 __device__ __forceinline__ void
 dma_setup(int64_t ld_bytes, int64_t row0, int64_t rows_total,
-          uint32_t (&off)[SliceGeom<ROWS, ELEM, KCONTIG>::kLoads]) {
-  using G = SliceGeom<ROWS, ELEM, KCONTIG>;
+          uint32_t (&off)[SliceGeom<ROWS, ELEM, KCONTIG, NW>::kLoads]) {
+  using G = SliceGeom<ROWS, ELEM, KCONTIG, NW>;
   const int w = threadIdx.x >> 6, l = threadIdx.x & 63;
 #pragma unroll
   for (int j = 0; j < G::kLoads; ++j) {
-    const int group = j * 4 + w;
+    const int group = j * NW + w;
     if constexpr (KCONTIG) {
       const int row = group * 8 + (l >> 3);
       const int c = (l & 7) ^ kc_swz(row);
@@ -226,7 +226,7 @@ dma_setup(int64_t ld_bytes, int64_t row0, int64_t rows_total,
 // 64-bit base + 32-bit lane offset) keeps these loads on the vector-memory
 // counter only, so waits on LDS reads stay exact while they are in flight;
 // offsets at or past `bytes` read as zero.
-template <int LOADS>
+template <int NW, int LOADS, int J0 = 0, int J1 = LOADS>
 __device__ __forceinline__ void dma_issue(const char *base, uint32_t bytes,
                                           const uint32_t (&off)[LOADS],
                                           uint32_t lds_stage) {
@@ -234,8 +234,8 @@ __device__ __forceinline__ void dma_issue(const char *base, uint32_t bytes,
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
       (void *)base, 0, (int)bytes, 0x00020000);
 #pragma unroll
-  for (int j = 0; j < LOADS; ++j) {
-    const uint32_t dst = lds_stage + (uint32_t)(j * 4 + w) * 1024u;
+  for (int j = J0; j < J1; ++j) {
+    const uint32_t dst = lds_stage + (uint32_t)(j * NW + w) * 1024u;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(
         rsrc, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
         (int)off[j], 0, 0, 0);
@@ -327,6 +327,31 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr {
   }
 };
 
+// Scheduling recipe for one K-step: NM MFMAs with NR LDS reads spread over
+// the leading MFMAs and NV global->LDS loads over the trailing quarter (the
+// loads write LDS, so they stay behind the reads that precede them in program
+// order).  Neither memory queue then fills up and stalls the wavefront while
+// the matrix pipe has work.
+template <int NM, int NR, int NV> __device__ __forceinline__ void gemm_interleave() {
+  constexpr int MV0 = NV == 0 ? 0 : (NM / 4 < NV ? NM / 4 : NV);
+  constexpr int MV = (NV + 1) / 2 > MV0 && (NV + 1) / 2 <= NM / 2 ? (NV + 1) / 2 : MV0;
+  constexpr int MR = NM - MV;
+  gemm_static_for<NM>([&](auto mc) {
+    constexpr int m = decltype(mc)::value;
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+    if constexpr (m < MR) {
+      constexpr int nr = ((m + 1) * NR) / MR - (m * NR) / MR;
+      if constexpr (nr > 0)
+        __builtin_amdgcn_sched_group_barrier(0x100, nr, 0); // DS read
+    } else {
+      constexpr int v = m - MR;
+      constexpr int nv = ((v + 1) * NV) / MV - (v * NV) / MV;
+      if constexpr (nv > 0)
+        __builtin_amdgcn_sched_group_barrier(0x020, nv, 0); // VMEM read
+    }
+  });
+}
+
 template <int N>
 __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
                                                  const int64_t (&off)[N],
@@ -348,26 +373,34 @@ __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
 
 // LDS bytes of the kernel: NSTAGE stages of (A slice + B slice); the epilogue
 // reuses it for four 32-row accumulator bands (one per wavefront).
-template <int BM, int BN, int NSTAGE> struct GemmLds {
+template <int BM, int BN, int NSTAGE, int NW> struct GemmLds {
   static constexpr int kStage = (BM + BN) * kTileKBytes;
-  static constexpr int kEpiPitch = (BN / 2) * 4 + 32;
-  static constexpr int kEpiBytes = 4 * 32 * kEpiPitch;
+  static constexpr int kWN = BN / (NW / 2); // wavefront tile columns
+  static constexpr int kEpiPitch = kWN * 4 + 32;
+  static constexpr int kBand = 32 * kEpiPitch; // one wavefront, one tile row
+  static constexpr int kTM = BM / 64;
+  // tile rows that leave together: as many as fit 160 KB
+  static constexpr int kBands =
+      NW * kTM * kBand <= 160 * 1024 ? kTM
+                                     : (NW * 2 * kBand <= 160 * 1024 ? 2 : 1);
+  static constexpr int kEpiBytes = NW * kBands * kBand;
   static constexpr int kBytes =
       NSTAGE * kStage > kEpiBytes ? NSTAGE * kStage : kEpiBytes;
 };
 
-template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int NSTAGE>
-__global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
+template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int NSTAGE, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   using Acc = typename KindTraits<KIND>::Acc;
   constexpr bool A_KC = A_MODE != A_MCONTIG;
   constexpr int ELEM = KindTraits<KIND>::kElemBytes;
   constexpr int STEPB = KindTraits<KIND>::kStepBytes;
   constexpr int KSTEPS = kTileKBytes / STEPB;
   static_assert(KSTEPS % 2 == 0, "fragment double buffering needs even KSTEPS");
-  using GA = SliceGeom<BM, ELEM, A_KC>;
-  using GB = SliceGeom<BN, ELEM, B_KC>;
-  using L = GemmLds<BM, BN, NSTAGE>;
-  constexpr int WM = BM / 2, WN = BN / 2; // wavefront tile
+  using GA = SliceGeom<BM, ELEM, A_KC, NW>;
+  using GB = SliceGeom<BN, ELEM, B_KC, NW>;
+  using L = GemmLds<BM, BN, NSTAGE, NW>;
+  constexpr int WAVES_N = NW / 2;
+  constexpr int WM = BM / 2, WN = BN / WAVES_N; // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int LPS = GA::kLoads + GB::kLoads; // DMA instructions per slice
 
@@ -397,7 +430,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   const int kt_count = (int)(g.K * ELEM / kTileKBytes);
 
   const int wave = threadIdx.x >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int l = threadIdx.x & 63;
 
   // ---- global -> LDS plumbing ---------------------------------------------
@@ -415,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
     const int taps = kt_count / g.conv.slices_per_tap;
 #pragma unroll
     for (int j = 0; j < GA::kLoads; ++j) {
-      const int row = (j * 4 + wave) * 8 + (l >> 3);
+      const int row = (j * NW + wave) * 8 + (l >> 3);
       const int64_t m = m0 + row;
       const bool live = m < g.M;
       const int32_t mm = (int32_t)(live ? m : 0);
@@ -438,11 +471,11 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   } else if constexpr (A_KC) {
     a_base = g.a + batch * g.a_batch * ELEM + m0 * a_ldb;
     a_step = kTileKBytes;
-    dma_setup<BM, ELEM, true>(a_ldb, m0, g.M, off_a);
+    dma_setup<BM, ELEM, true, NW>(a_ldb, m0, g.M, off_a);
   } else {
     a_base = g.a + batch * g.a_batch * ELEM + m0 * ELEM;
     a_step = (int64_t)GA::kKRows * a_ldb;
-    dma_setup<BM, ELEM, false>(a_ldb, m0, g.M, off_a);
+    dma_setup<BM, ELEM, false, NW>(a_ldb, m0, g.M, off_a);
   }
   const char *b_base;
   int64_t b_step;
@@ -453,13 +486,22 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
     b_base = g.b + batch * g.b_batch * ELEM + n0 * ELEM;
     b_step = (int64_t)GB::kKRows * b_ldb;
   }
-  dma_setup<BN, ELEM, B_KC>(b_ldb, n0, g.N, off_b);
+  dma_setup<BN, ELEM, B_KC, NW>(b_ldb, n0, g.N, off_b);
 
   auto stage_a = [&](int st) { return lds0 + (uint32_t)st * L::kStage; };
   auto stage_b = [&](int st) {
     return lds0 + (uint32_t)st * L::kStage + GA::kBytes;
   };
-  auto issue = [&](int kt, int st) {
+  // Part PART of PARTS of slice kt's loads (A and B split alike).
+  // Slices past the end of K are "loaded" with zero-sized buffers: nothing
+  // is fetched and the zeros land in a stage that is never read, which keeps
+  // every iteration identical (no tail variants, exact load counts).
+  auto issue = [&](int kt, int st, auto part_c, auto parts_c) {
+    const uint32_t lim = kt < kt_count ? 0xffffffffu : 0u;
+    constexpr int PART = decltype(part_c)::value;
+    constexpr int PARTS = decltype(parts_c)::value;
+    constexpr int A0 = PART * GA::kLoads / PARTS, A1 = (PART + 1) * GA::kLoads / PARTS;
+    constexpr int B0 = PART * GB::kLoads / PARTS, B1 = (PART + 1) * GB::kLoads / PARTS;
     if constexpr (A_MODE == A_CONV) {
       const int32_t tap = kt / g.conv.slices_per_tap;
       const int32_t cb = (kt % g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
@@ -468,19 +510,22 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
       const int32_t cbytes = g.conv.C * ELEM;
       uint32_t off[GA::kLoads];
 #pragma unroll
-      for (int j = 0; j < GA::kLoads; ++j) {
+      for (int j = A0; j < A1; ++j) {
         const bool in = (cv_mask[j] >> tap) & 1;
         // taps outside the image (and rows past M) read past the end: zeros
         off[j] = in ? (uint32_t)((cv_pix[j] + dpix) * cbytes + cb) : 0x80000000u;
       }
-      dma_issue<GA::kLoads>(a_base, g.conv.x_bytes, off, stage_a(st));
+      dma_issue<NW, GA::kLoads, A0, A1>(a_base, g.conv.x_bytes & lim, off,
+                                    stage_a(st));
     } else {
-      dma_issue<GA::kLoads>(a_base + kt * a_step, 0xffffffffu, off_a,
-                            stage_a(st));
+      dma_issue<NW, GA::kLoads, A0, A1>(a_base + kt * a_step, lim, off_a,
+                                    stage_a(st));
     }
-    dma_issue<GB::kLoads>(b_base + kt * b_step, 0xffffffffu, off_b,
-                          stage_b(st));
+    dma_issue<NW, GB::kLoads, B0, B1>(b_base + kt * b_step, lim, off_b,
+                                  stage_b(st));
   };
+  using One = std::integral_constant<int, 1>;
+  using Zero = std::integral_constant<int, 0>;
 
   // ---- fragments ----------------------------------------------------------
   FragAddr<KIND, BM, A_KC, TM> fa_addr;
@@ -498,11 +543,10 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
       for (int r = 0; r < 16; ++r)
         acc[i][j][r] = 0;
 
-  // ---- prologue: fill NSTAGE - 1 stages ------------------------------------
+  // ---- prologue: fill all NSTAGE stages -------------------------------------
 #pragma unroll
-  for (int p = 0; p < NSTAGE - 1; ++p)
-    if (p < kt_count)
-      issue(p, p);
+  for (int p = 0; p < NSTAGE; ++p)
+    issue(p, p, Zero{}, One{});
   __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_barrier();
@@ -510,84 +554,97 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
   fa_addr.template load<0>(stage_a(0), fa[0]);
   fb_addr.template load<0>(stage_b(0), fb[0]);
 
-  int cur = 0;             // stage holding slice kt
-  int fill = NSTAGE - 1;   // stage that slice kt + NSTAGE - 1 goes to
+  // Reads per fragment set and the loads of a slice spread over the K-steps
+  // that precede the barrier.
+  constexpr int NRA = TM * FragAddr<KIND, BM, A_KC, TM>::CHH *
+                      (A_KC ? 1 : 2);
+  constexpr int NRB = TN * FragAddr<KIND, BN, B_KC, TN>::CHH *
+                      (B_KC ? 1 : 2);
+  using Two = std::integral_constant<int, 2>;
+
+  int cur = 0; // stage holding slice kt
+  // One K slice.  A stage is free again once the barrier of the iteration
+  // that consumes it has passed, and is refilled at once with the slice
+  // NSTAGE ahead: first half of its loads behind the MFMAs of the last
+  // K-step, second half behind K-step 0 of the next iteration.  Every K-step
+  // is one basic block, so the recipe can interleave.
   for (int kt = 0; kt < kt_count; ++kt) {
-    const bool issued = kt + NSTAGE - 1 < kt_count;
-    if (issued)
-      issue(kt + NSTAGE - 1, fill);
-    __builtin_amdgcn_sched_barrier(0);
     const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;
+    const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;
     const uint32_t sa = stage_a(cur), sb = stage_b(cur);
     gemm_static_for<KSTEPS>([&](auto sc) {
       constexpr int s = decltype(sc)::value;
       constexpr int fc = s & 1, fn = fc ^ 1;
-      if constexpr (s + 1 < KSTEPS) {
+      constexpr bool LAST = s + 1 == KSTEPS;
+      if constexpr (!LAST) {
         fa_addr.template load<s + 1>(sa, fa[fn]);
         fb_addr.template load<s + 1>(sb, fb[fn]);
+        if constexpr (s == 0)
+          issue(kt + NSTAGE - 1, prv, One{}, Two{});
       } else {
         // Slice kt + 1 must be in LDS (this thread's DMA, then everyone's),
         // and every fragment read of this stage must have returned before
-        // another wavefront may refill it.
-        if (issued)
-          __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
-        else
-          __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+        // it is refilled.
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        if (kt + 1 < kt_count) {
-          fa_addr.template load<0>(stage_a(nxt), fa[fn]);
-          fb_addr.template load<0>(stage_b(nxt), fb[fn]);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        fa_addr.template load<0>(stage_a(nxt), fa[fn]);
+        fb_addr.template load<0>(stage_b(nxt), fb[fn]);
+        issue(kt + NSTAGE, cur, Zero{}, Two{});
       }
-      // Keep the fragment reads ahead of this step's MFMAs: the scheduler
-      // would otherwise sink them next to their first use.
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           mfma32<KIND>(acc[i][j], fa[fc][i], fb[fc][j]);
+      constexpr int NV = LAST ? LPS / 2 : (s == 0 ? LPS - LPS / 2 : 0);
+      gemm_interleave<TM * TN, NRA + NRB, NV>();
       __builtin_amdgcn_sched_barrier(0);
     });
     cur = nxt;
-    fill = fill + 1 == NSTAGE ? 0 : fill + 1;
   }
+  // zero-sized loads of the last iterations may still be writing LDS
+  __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
   // ---- epilogue -------------------------------------------------------------
-  // Each wavefront moves its accumulators through a private LDS band of 32
-  // rows x WN columns (row pitch padded by 32 bytes), one tile row at a time,
-  // and reads them back with 8 consecutive columns per lane.
+  // Each wavefront moves its accumulators through private LDS bands of 32
+  // rows x WN columns (row pitch padded by 32 bytes), BANDS tile rows at a
+  // time, and reads them back with 8 consecutive columns per lane.
   constexpr int PITCH = L::kEpiPitch;
+  constexpr int BANDS = L::kBands;
   constexpr int LPR = WN / 8;   // lanes per row
   constexpr int RPP = 64 / LPR; // rows per pass
-  const uint32_t band = lds0 + (uint32_t)wave * (32 * PITCH);
+  constexpr int PPB = 32 / RPP; // passes per band
+  const uint32_t band = lds0 + (uint32_t)wave * (BANDS * L::kBand);
   const uint32_t wr = band + (uint32_t)((l >> 5) * 4 * PITCH + (l & 31) * 4);
   const uint32_t rd = band + (uint32_t)((l / LPR) * PITCH + (l % LPR) * 32);
   const int64_t ob = batch * g.o_batch;
   const int64_t ncol = n0 + wn * WN + (l % LPR) * 8;
 
-#pragma clang loop unroll(disable)
-  for (int i = 0; i < TM; ++i) {
-    gemm_static_for<TM>([&](auto ic) {
-      constexpr int ii = decltype(ic)::value;
-      if (i == ii) {
+  gemm_static_for<TM / BANDS>([&](auto rc) {
+    constexpr int round = decltype(rc)::value;
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+    for (int bi = 0; bi < BANDS; ++bi)
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            *(GEMM_AS3 Acc *)(uintptr_t)(wr + ((r >> 2) * 8 + (r & 3)) * PITCH +
-                                         j * 128) = acc[ii][j][r];
-      }
-    });
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          *(GEMM_AS3 Acc *)(uintptr_t)(wr + bi * L::kBand +
+                                       ((r >> 2) * 8 + (r & 3)) * PITCH +
+                                       j * 128) = acc[round * BANDS + bi][j][r];
 #pragma clang loop unroll(disable)
-    for (int p = 0; p < 32 / RPP; ++p) {
-      const int64_t m = m0 + wm * WM + i * 32 + p * RPP + l / LPR;
-      const u32x4 v0 =
-          *(const GEMM_AS3 u32x4 *)(uintptr_t)(rd + p * RPP * PITCH);
-      const u32x4 v1 =
-          *(const GEMM_AS3 u32x4 *)(uintptr_t)(rd + p * RPP * PITCH + 16);
+    for (int p = 0; p < BANDS * PPB; ++p) {
+      const int bi = p / PPB, pp = p % PPB;
+      const int64_t m =
+          m0 + wm * WM + (round * BANDS + bi) * 32 + pp * RPP + l / LPR;
+      const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
+      const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
+      const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
       if (m >= g.M || ncol >= g.N)
         continue;
       const bool full = ncol + 8 <= g.N;
@@ -681,7 +738,7 @@ __global__ __launch_bounds__(kThreads) void gemm_kernel(GemmArgs g) {
         }
       }
     }
-  }
+  });
 }
 
 // What the host decided about one matmul call.
@@ -701,11 +758,19 @@ template <int BM, int BN> struct GemmStages {
   static constexpr int value = 160 * 1024 / kStage >= 4 ? 4 : 160 * 1024 / kStage;
 };
 
+// Wavefronts per workgroup: 8 (two per SIMD, so one can issue MFMAs while
+// the other waits on a memory queue) where each still gets a 2-tile-wide
+// block, else 4.
+template <int BM, int BN> struct GemmWaves {
+  static constexpr int value = BN >= 256 ? 8 : 4;
+};
+
 template <int KIND, int BM, int BN, int A_MODE, bool B_KC>
 int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
   constexpr int NSTAGE = GemmStages<BM, BN>::value;
-  constexpr int lds = GemmLds<BM, BN, NSTAGE>::kBytes;
-  auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC, NSTAGE>;
+  constexpr int NW = GemmWaves<BM, BN>::value;
+  constexpr int lds = GemmLds<BM, BN, NSTAGE, NW>::kBytes;
+  auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC, NSTAGE, NW>;
   static bool configured = false;
   if (!configured) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
@@ -714,7 +779,7 @@ int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
     configured = true;
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
-  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, ctx->stream, g);
+  hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, ctx->stream, g);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }
