@@ -171,6 +171,29 @@ def bench_conv(ctx, steps, warmup):
             "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
 
 
+def bench_sdpa(ctx, steps, warmup):
+    """C4: SDPA forward bf16 causal B4 H32 S2048 D128 ([B,H,S,D] contiguous)."""
+    b, h, sq, d = 4, 32, 2048, 128
+    dims = [b, h, sq, d]
+    strides = [h * sq * d, sq * d, d, 1]
+    desc = capi.SdpaDesc()
+    desc.q = desc.k = desc.v = desc.o = capi.TensorDesc.make(dims, strides, capi.BFLOAT16)
+    desc.is_causal = 1
+    assert ctx.lib.fhip_sdpa_fwd_supported(desc) == 2, "MFMA SDPA not chosen"
+    n = b * h * sq * d
+    q, k, v = (ctx.to_device(synth.f32_to_bf16_bits(synth.normal(9, i, n)))
+               for i in range(3))
+    out = ctx.alloc(n * 2)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.sdpa_fwd(desc, q, k, v, out),
+                                steps, warmup)
+    # causal: only the lower triangle of the S x S score matrix is computed
+    flop = 4.0 * b * h * sq * sq * d / 2
+    return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
+            "kernel_us": round(ev_ms * 1e3, 2), "work": flop,
+            "flop_convention": "4*B*H*S*S*D/2 (causal half)"}
+
+
 def cpu_baseline_rmsnorm(seconds_budget=12.0):
     """The oracle's bf16 RMSNorm * scalar on the host cores over a row sample."""
     from oracle import oracle
@@ -249,6 +272,8 @@ def main():
         others["matmul_bf16_4096x4096x4096"] = bench_matmul(
             ctx, ksteps, kwarm, "bf16", 4096, 4096, 4096)
         others["conv_fprop_bf16_n16c64h56w56_k128r3s3_bias_relu"] = bench_conv(
+            ctx, max(20, args.steps // 4), kwarm)
+        others["sdpa_fwd_bf16_causal_b4h32s2048d128"] = bench_sdpa(
             ctx, max(20, args.steps // 4), kwarm)
         line["others"] = others
     if not args.no_cpu_baseline:

@@ -1,4 +1,466 @@
+// Scaled dot-product attention forward on MFMA (flash-attention style: scores
+// never leave the CU).
+//
+// One workgroup of 8 wavefronts owns 256 query rows of one (batch, head); each
+// wavefront owns 32 of them and walks the keys in tiles of 64:
+//   * K and V tiles go global -> LDS by LDS-DMA into a ring of stages, two
+//     tiles ahead of the math; K rows are read back with 16-byte loads, V with
+//     the transposing 8-byte loads, both conflict-free by chunk permutation;
+//   * scores are computed TRANSPOSED, S^T = K Q^T, so that an MFMA lane holds
+//     32 scores of ONE query: the row maximum and row sum of the online
+//     softmax are in-register reductions plus one exchange between the two
+//     half-wavefronts, and the probabilities, rounded to the input type, are
+//     already laid out as the MFMA operand of O^T += V^T P^T;
+//   * Q fragments stay in registers for the whole kernel; the output
+//     accumulator O^T is rescaled only when some row maximum moved;
+//   * causal workgroups stop at the diagonal, and a wavefront skips tiles that
+//     lie wholly above its own rows.
+//
+// Reference semantics: aten.scaled_dot_product_attention (reference
+// support/asm_emitter.h:2409-2468, node/sdpa_node.h:36-236), GQA by head
+// repetition, causal mask aligned top-left.
 #include "common.h"
 #include "fast_paths.h"
-bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *) { return false; }
-int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *, const void *, const void *, const void *, void *) { return fhip_fail(ctx, "no fast sdpa"); }
+
+#include <type_traits>
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+#define SD_AS1 __attribute__((address_space(1)))
+#define SD_AS3 __attribute__((address_space(3)))
+
+constexpr int kD = 128;         // head dim (Q/K and V)
+constexpr int kRowB = kD * 2;   // bytes per K / V row
+constexpr int kBQ = 256;        // query rows per workgroup
+constexpr int kBKV = 64;        // keys per tile
+constexpr int kWaves = 8;
+constexpr int kStages = 3;
+constexpr int kTileB = kBKV * kRowB;       // one K (or V) tile: 16 KB
+constexpr int kStageB = 2 * kTileB;        // K + V
+constexpr int kLoadsPerTile = kTileB / 1024 / kWaves; // DMA per wave per tile
+constexpr int kOutPitch = kRowB + 16;      // epilogue rows, padded
+constexpr int kLdsB = kStages * kStageB > kWaves * 32 * kOutPitch
+                          ? kStages * kStageB
+                          : kWaves * 32 * kOutPitch;
+constexpr float kNegBig = -1.0e30f;
+
+struct SdpaArgs {
+  const char *q, *k, *v;
+  char *o;
+  int64_t q_sb, q_sh, q_ss; // strides in elements (last dim contiguous)
+  int64_t k_sb, k_sh, k_ss;
+  int64_t v_sb, v_sh, v_ss;
+  int64_t o_sb, o_sh, o_ss;
+  int32_t Sq, Skv, group; // group = Hq / Hkv
+  int32_t causal;
+  float scale_log2e; // softmax scale * log2(e)
+};
+
+template <int N, typename F> __device__ __forceinline__ void sd_static_for(F &&f) {
+  if constexpr (N > 0) {
+    sd_static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x16 sd_mfma(const uint32_t (&a)[4],
+                                          const uint32_t (&b)[4], f32x16 c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+        __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+        __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// two floats -> one register of two 16-bit values (lo = a)
+template <bool BF16> __device__ __forceinline__ uint32_t sd_pack(float a, float b) {
+  if constexpr (BF16) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    bf16x2 v;
+    v[0] = (__bf16)a;
+    v[1] = (__bf16)b;
+    return __builtin_bit_cast(uint32_t, v);
+  } else {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    f16x2 v;
+    v[0] = (_Float16)a;
+    v[1] = (_Float16)b;
+    return __builtin_bit_cast(uint32_t, v);
+  }
+}
+
+// maximum / sum over the two half-wavefronts (lanes l and l ^ 32)
+__device__ __forceinline__ float sd_half_max(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];
+  return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+__device__ __forceinline__ float sd_half_sum(float x) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t r0 = r[0], r1 = r[1];
+  return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+// chunk permutation of the V tile (rows of 256 bytes read by transposing
+// 8-byte loads): spreads the 4 rows x 64 bytes a half-wavefront touches over
+// all 64 banks
+__device__ __forceinline__ int sd_vpos(int row, int c) {
+  return c ^ ((row & 3) << 1) ^ ((c & 2) << 2);
+}
+__device__ __forceinline__ int sd_vchunk(int row, int p) {
+  const int t = p ^ ((row & 3) << 1);
+  return t ^ ((t & 2) << 2);
+}
+
+__device__ __forceinline__ constexpr int sd_wait_imm(int vm) {
+  return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0x0 << 8);
+}
+
+template <bool BF16, bool CAUSAL>
+__global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  const int half = l >> 5, lq = l & 31;
+  // heavy (late) query tiles first: causal tiles near the end do most work
+  const int qtile = CAUSAL ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / g.group;
+  const int q0 = qtile * kBQ;
+  const int qw0 = q0 + wave * 32; // first query row of this wavefront
+  const int qrow = qw0 + lq;      // query this lane's scores belong to
+
+  const char *qp = g.q + (b * g.q_sb + h * g.q_sh) * 2;
+  const char *kp = g.k + (b * g.k_sb + hk * g.k_sh) * 2;
+  const char *vp = g.v + (b * g.v_sb + hk * g.v_sh) * 2;
+  const int64_t k_rowb = g.k_ss * 2, v_rowb = g.v_ss * 2;
+  const int64_t k_bytes = (int64_t)(g.Skv - 1) * k_rowb + kRowB;
+  const int64_t v_bytes = (int64_t)(g.Skv - 1) * v_rowb + kRowB;
+
+  // number of key tiles this workgroup visits
+  int kv_end = g.Skv;
+  if (CAUSAL) {
+    const int last_q = q0 + kBQ - 1 < g.Sq - 1 ? q0 + kBQ - 1 : g.Sq - 1;
+    kv_end = last_q + 1 < g.Skv ? last_q + 1 : g.Skv;
+  }
+  const int tiles = (kv_end + kBKV - 1) / kBKV;
+
+  // ---- Q fragments (B operand of S^T = K Q^T): row lq, 8 d per register quad
+  uint32_t qf[kD / 16][4];
+  {
+    const int qr = qrow < g.Sq ? qrow : g.Sq - 1;
+    const char *src = qp + (int64_t)qr * g.q_ss * 2 + half * 16;
+#pragma unroll
+    for (int ds = 0; ds < kD / 16; ++ds) {
+      const u32x4 v = *(const SD_AS1 u32x4 *)(src + ds * 32);
+      qf[ds][0] = v.x;
+      qf[ds][1] = v.y;
+      qf[ds][2] = v.z;
+      qf[ds][3] = v.w;
+    }
+  }
+
+  // ---- DMA addressing: a wave instruction moves 4 rows x 256 bytes ----------
+  uint32_t koff[kLoadsPerTile], voff[kLoadsPerTile];
+#pragma unroll
+  for (int j = 0; j < kLoadsPerTile; ++j) {
+    const int row = (j * kWaves + wave) * 4 + (l >> 4);
+    const int p = l & 15;
+    koff[j] = (uint32_t)(row * k_rowb + ((p ^ (row & 15)) << 4));
+    voff[j] = (uint32_t)(row * v_rowb + (sd_vchunk(row, p) << 4));
+  }
+  auto issue = [&](int t, int st) {
+    // rows at or past Skv (and tiles past the end) read as zeros
+    const int64_t kv0 = (int64_t)t * kBKV;
+    int64_t kb = k_bytes - kv0 * k_rowb, vb = v_bytes - kv0 * v_rowb;
+    kb = t < tiles && kb > 0 ? kb : 0;
+    vb = t < tiles && vb > 0 ? vb : 0;
+    const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(kp + kv0 * k_rowb), 0, (int)kb, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(vp + kv0 * v_rowb), 0, (int)vb, 0x00020000);
+#pragma unroll
+    for (int j = 0; j < kLoadsPerTile; ++j) {
+      const uint32_t dst = lds0 + (uint32_t)st * kStageB +
+                           (uint32_t)(j * kWaves + wave) * 1024u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          kr, (SD_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
+          (int)koff[j], 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          vr, (SD_AS3 char *)__builtin_amdgcn_readfirstlane(dst + kTileB), 16,
+          (int)voff[j], 0, 0, 0);
+    }
+  };
+
+  // ---- fragment addressing ----------------------------------------------------
+  // K (A operand of S^T): row lq of a 32-key block, 16-byte chunk 2*ds + half
+  uint32_t kaddr[kD / 16];
+#pragma unroll
+  for (int ds = 0; ds < kD / 16; ++ds)
+    kaddr[ds] = (uint32_t)(lq * kRowB + (((ds * 2 + half) ^ (lq & 15)) << 4));
+  // V^T (A operand of O^T += V^T P^T): the keys a lane needs are those whose
+  // probabilities it holds: key = 32*kb + 8*(i/4) + 4*half + i%4 for score
+  // register i; one transposing read returns 4 consecutive keys of one column
+  uint32_t vaddr[kD / 32];
+  {
+    const int L = l & 15, h16 = (l >> 4) & 1;
+    const int row = half * 4 + (L >> 2);
+#pragma unroll
+    for (int dt = 0; dt < kD / 32; ++dt) {
+      const int c = dt * 4 + h16 * 2 + ((L & 3) >> 1);
+      vaddr[dt] = (uint32_t)(row * kRowB + (sd_vpos(row, c) << 4) + (L & 1) * 8);
+    }
+  }
+
+  f32x16 o[kD / 32];
+#pragma unroll
+  for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      o[dt][r] = 0.f;
+  float m_run = kNegBig; // running row maximum (raw scores), same in both halves
+  float l_run = 0.f;     // running row sum, this half's share
+
+  // ---- prologue ---------------------------------------------------------------
+#pragma unroll
+  for (int p = 0; p < kStages - 1; ++p)
+    issue(p, p);
+
+  int st = 0;
+  for (int t = 0; t < tiles; ++t) {
+    // tile t landed (this thread's loads, then everyone's); stage of tile t-1
+    // is free for tile t + kStages - 1
+    __builtin_amdgcn_s_waitcnt(sd_wait_imm((kStages - 2) * 2 * kLoadsPerTile));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    {
+      const int fill = st == 0 ? kStages - 1 : st - 1;
+      issue(t + kStages - 1, fill);
+    }
+    const int kv0 = t * kBKV;
+    const uint32_t sk = lds0 + (uint32_t)st * kStageB, sv = sk + kTileB;
+    st = st + 1 == kStages ? 0 : st + 1;
+    // a wavefront whose rows all lie above this tile has nothing to add
+    if (CAUSAL && kv0 > qw0 + 31)
+      continue;
+
+    // ---- S^T = K Q^T : 2 key blocks of 32 -------------------------------------
+    f32x16 s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        s[kb][r] = 0.f;
+#pragma unroll
+    for (int ds = 0; ds < kD / 16; ++ds)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const u32x4 v =
+            *(const SD_AS3 u32x4 *)(uintptr_t)(sk + kaddr[ds] + kb * 32 * kRowB);
+        const uint32_t kf[4] = {v.x, v.y, v.z, v.w};
+        s[kb] = sd_mfma<BF16>(kf, qf[ds], s[kb]);
+      }
+
+    // ---- mask -----------------------------------------------------------------
+    const bool edge = (CAUSAL && kv0 + kBKV - 1 > qw0) || kv0 + kBKV > g.Skv;
+    if (edge) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kv0 + kb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          const bool dead = key >= g.Skv || (CAUSAL && key > qrow);
+          s[kb][r] = dead ? kNegBig : s[kb][r];
+        }
+    }
+
+    // ---- online softmax -------------------------------------------------------
+    float mx = s[0][0];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        mx = fmaxf(mx, s[kb][r]);
+    mx = sd_half_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float mc = m_new * g.scale_log2e;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * g.scale_log2e);
+    const bool moved = m_new > m_run;
+    m_run = m_new;
+    uint32_t pf[4][4]; // probabilities as B-operand fragments, 16 keys each
+    float psum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * g.scale_log2e - mc);
+        const float p1 = __builtin_amdgcn_exp2f(s[kb][r + 1] * g.scale_log2e - mc);
+        psum += p0 + p1;
+        pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = sd_pack<BF16>(p0, p1);
+      }
+    l_run = l_run * alpha + psum;
+    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+      for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          o[dt][r] *= alpha;
+    }
+
+    // ---- O^T += V^T P^T ---------------------------------------------------------
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int dt = 0; dt < kD / 32; ++dt) {
+        uint32_t vf[4];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const uint32_t ad = sv + vaddr[dt] + (j * 16 + r * 8) * kRowB;
+          const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (SD_AS3 s16x4 *)(uintptr_t)ad);
+          const u32x2 w2 = __builtin_bit_cast(u32x2, v);
+          vf[2 * r + 0] = w2.x;
+          vf[2 * r + 1] = w2.y;
+        }
+        o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
+      }
+  }
+
+  // ---- epilogue: O = O^T / l, through LDS for row-contiguous stores -----------
+  __builtin_amdgcn_s_waitcnt(sd_wait_imm(0));
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  const float inv = 1.0f / sd_half_sum(l_run);
+  const uint32_t band = lds0 + (uint32_t)wave * (32 * kOutPitch);
+  // lane holds query lq, features 32*dt + 8*(r/4) + 4*half + r%4
+#pragma unroll
+  for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      u32x2 w2;
+      w2.x = sd_pack<BF16>(o[dt][r4 * 4 + 0] * inv, o[dt][r4 * 4 + 1] * inv);
+      w2.y = sd_pack<BF16>(o[dt][r4 * 4 + 2] * inv, o[dt][r4 * 4 + 3] * inv);
+      *(SD_AS3 u32x2 *)(uintptr_t)(band + lq * kOutPitch +
+                                   (dt * 32 + r4 * 8 + half * 4) * 2) = w2;
+    }
+  char *op = g.o + (b * g.o_sb + h * g.o_sh) * 2;
+  // 16 lanes cover one 256-byte row; 4 rows per pass
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int row = pass * 4 + (l >> 4);
+    const u32x4 v = *(const SD_AS3 u32x4 *)(uintptr_t)(band + row * kOutPitch +
+                                                       (l & 15) * 16);
+    const int qr = qw0 + row;
+    if (qr < g.Sq)
+      *(SD_AS1 u32x4 *)(op + (int64_t)qr * g.o_ss * 2 + (l & 15) * 16) = v;
+  }
+}
+
+struct SdpaPlan {
+  bool ok = false;
+  bool bf16 = true;
+};
+
+SdpaPlan make_plan(const fhip_sdpa_desc *d) {
+  SdpaPlan p;
+  if (d->mask.rank != 0)
+    return p;
+  const int dt = d->q.dtype;
+  if (dt != FHIP_BFLOAT16 && dt != FHIP_HALF)
+    return p;
+  if (d->k.dtype != dt || d->v.dtype != dt || d->o.dtype != dt)
+    return p;
+  p.bf16 = dt == FHIP_BFLOAT16;
+  if (d->q.rank != 4 || d->q.dim[3] != kD || d->v.dim[3] != kD)
+    return p;
+  const fhip_tensor_desc *ts[4] = {&d->q, &d->k, &d->v, &d->o};
+  for (const fhip_tensor_desc *t : ts) {
+    if (t->stride[3] != 1 && t->dim[3] != 1)
+      return p;
+    for (int i = 0; i < 3; ++i)
+      if (t->dim[i] > 1 && (t->stride[i] < 0 || (t->stride[i] * 2) % 16 != 0))
+        return p;
+  }
+  const int64_t Sq = d->q.dim[2], Skv = d->k.dim[2];
+  if (Sq < 1 || Skv < 1 || Sq >= (1ll << 30) || Skv >= (1ll << 30))
+    return p;
+  // 32-bit lane offsets inside one (batch, head) slab of K / V
+  if (Skv * d->k.stride[2] * 2 >= (1ll << 31) ||
+      Skv * d->v.stride[2] * 2 >= (1ll << 31))
+    return p;
+  if (d->q.dim[1] > 65535 || d->q.dim[0] > 65535)
+    return p;
+  // the running maximum is taken over raw scores: needs a positive scale
+  if (d->has_scale && !(d->scale > 0.f))
+    return p;
+  p.ok = true;
+  return p;
+}
+
+} // namespace
+
+bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d) {
+  return make_plan(d).ok;
+}
+
+int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
+                   const void *k, const void *v, void *o) {
+  const SdpaPlan p = make_plan(d);
+  FHIP_REQUIRE(ctx, p.ok, "sdpa: descriptor not supported by the MFMA kernel");
+  FHIP_REQUIRE(ctx,
+               (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) &
+                15) == 0,
+               "sdpa: Q, K, V, O must be 16-byte aligned");
+  SdpaArgs g{};
+  g.q = (const char *)q;
+  g.k = (const char *)k;
+  g.v = (const char *)v;
+  g.o = (char *)o;
+  auto st = [](const fhip_tensor_desc &t, int i) {
+    return t.dim[i] > 1 ? t.stride[i] : 0;
+  };
+  g.q_sb = st(d->q, 0), g.q_sh = st(d->q, 1), g.q_ss = st(d->q, 2);
+  g.k_sb = st(d->k, 0), g.k_sh = st(d->k, 1), g.k_ss = st(d->k, 2);
+  g.v_sb = st(d->v, 0), g.v_sh = st(d->v, 1), g.v_ss = st(d->v, 2);
+  g.o_sb = st(d->o, 0), g.o_sh = st(d->o, 1), g.o_ss = st(d->o, 2);
+  g.Sq = (int32_t)d->q.dim[2];
+  g.Skv = (int32_t)d->k.dim[2];
+  g.group = (int32_t)(d->q.dim[1] / d->k.dim[1]);
+  g.causal = d->is_causal;
+  const float scale =
+      d->has_scale ? d->scale : 1.0f / sqrtf((float)d->q.dim[3]);
+  g.scale_log2e = scale * 1.4426950408889634f;
+  const dim3 grid((unsigned)((g.Sq + kBQ - 1) / kBQ), (unsigned)d->q.dim[1],
+                  (unsigned)d->q.dim[0]);
+  auto launch = [&](auto kernel) {
+    static bool configured = false;
+    if (!configured) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kLdsB) != hipSuccess)
+        return fhip_fail(ctx, "sdpa: cannot reserve LDS");
+      configured = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(kWaves * 64), kLdsB, ctx->stream, g);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    return 0;
+  };
+  if (p.bf16)
+    return d->is_causal ? launch(sdpa_fwd_kernel<true, true>)
+                        : launch(sdpa_fwd_kernel<true, false>);
+  return d->is_causal ? launch(sdpa_fwd_kernel<false, true>)
+                      : launch(sdpa_fwd_kernel<false, false>);
+}

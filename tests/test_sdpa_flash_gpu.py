@@ -1,0 +1,134 @@
+"""Flash-attention forward (MFMA kernel) through the C ABI vs the oracle.
+
+Every case satisfies the tuned kernel's contract (bf16/f16, head dim 128, no
+mask tensor) and asserts that the tuned kernel is chosen, so a silent fall
+back to the generic kernel fails the test.
+"""
+import numpy as np
+import pytest
+
+from fusilli_amd import capi
+from oracle import oracle
+from helpers import HT, assert_close, rand
+
+pytestmark = pytest.mark.gpu
+
+
+def run(ctx, q, k, v, causal=False, scale=None, o_strides=None, expect_tuned=True):
+    out = HT.empty([q.dims[0], q.dims[1], q.dims[2], v.dims[3]], q.dtype, o_strides)
+    d = capi.SdpaDesc()
+    d.q, d.k, d.v, d.o = q.desc(), k.desc(), v.desc(), out.desc()
+    d.is_causal = int(causal)
+    if scale is not None:
+        d.has_scale, d.scale = 1, scale
+    assert ctx.lib.fhip_sdpa_fwd_supported(d) == (2 if expect_tuned else 1)
+    bufs = [t.upload(ctx) for t in (q, k, v)]
+    dout = out.upload(ctx)
+    ctx.sdpa_fwd(d, bufs[0], bufs[1], bufs[2], dout)
+    return out.fetch(ctx, dout)
+
+
+def bshd_strides(dims):
+    b, h, s, d = dims
+    return [s * h * d, d, h * d, 1]
+
+
+CASES = [
+    dict(B=1, Hq=2, Hkv=2, Sq=256, Skv=256, causal=False),
+    dict(B=1, Hq=2, Hkv=2, Sq=256, Skv=256, causal=True),
+    # ragged: rows past Sq in the last query tile, keys past Skv in the last tile
+    dict(B=2, Hq=3, Hkv=3, Sq=300, Skv=200, causal=False),
+    dict(B=1, Hq=2, Hkv=2, Sq=333, Skv=333, causal=True),
+    # GQA and cross attention; more than one query tile and many key tiles
+    dict(B=1, Hq=4, Hkv=2, Sq=513, Skv=700, causal=False),
+    dict(B=1, Hq=4, Hkv=1, Sq=520, Skv=520, causal=True),
+    # causal with fewer keys than queries, and a single key
+    dict(B=1, Hq=1, Hkv=1, Sq=300, Skv=70, causal=True),
+    dict(B=1, Hq=2, Hkv=2, Sq=40, Skv=1, causal=False),
+    dict(B=1, Hq=1, Hkv=1, Sq=1, Skv=129, causal=False),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_flash_random_vs_oracle(ctx, case, dtype):
+    c = case
+    q = HT.from_logical(rand(51, 0, [c["B"], c["Hq"], c["Sq"], 128]), dtype)
+    k = HT.from_logical(rand(51, 1, [c["B"], c["Hkv"], c["Skv"], 128]), dtype)
+    v = HT.from_logical(rand(51, 2, [c["B"], c["Hkv"], c["Skv"], 128]), dtype)
+    out = run(ctx, q, k, v, causal=c["causal"])
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), is_causal=c["causal"])
+    assert_close(out.logical(), ref, dtype, str(case))
+
+
+def test_flash_bshd_layout_and_scale(ctx):
+    # tensors stored [B, S, H, D] (heads interleaved per position), custom scale
+    dims_q, dims_k = [2, 4, 200, 128], [2, 2, 300, 128]
+    q = HT.from_logical(rand(52, 0, dims_q), capi.BFLOAT16, bshd_strides(dims_q))
+    k = HT.from_logical(rand(52, 1, dims_k), capi.BFLOAT16, bshd_strides(dims_k))
+    v = HT.from_logical(rand(52, 2, dims_k), capi.BFLOAT16, bshd_strides(dims_k))
+    out = run(ctx, q, k, v, scale=0.05, o_strides=bshd_strides(dims_q))
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), scale=0.05)
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+
+
+def test_flash_large_scores_are_stable(ctx):
+    # scores of magnitude ~1e3: the running maximum must keep exp() in range
+    q = HT.from_logical(rand(53, 0, [1, 2, 300, 128]) * 8.0, capi.BFLOAT16)
+    k = HT.from_logical(rand(53, 1, [1, 2, 300, 128]) * 8.0, capi.BFLOAT16)
+    v = HT.from_logical(rand(53, 2, [1, 2, 300, 128]), capi.BFLOAT16)
+    out = run(ctx, q, k, v, causal=True)
+    assert np.all(np.isfinite(out.logical()))
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), is_causal=True)
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_constant_fill_equals_v(ctx, causal):
+    # samples/sdpa_utils.cpp:184-247: q = k = v = 0.01 => output == v (1e-2)
+    q = HT.from_logical(np.full([1, 8, 320, 128], 0.01), capi.HALF)
+    out = run(ctx, q, q, q, causal=causal)
+    assert np.allclose(out.logical(), 0.01, atol=1e-2)
+
+
+def test_flash_uniform_scores_causal_gives_prefix_means(ctx):
+    # q = 0 => uniform attention over the visible prefix: O[i] = mean(V[:i+1])
+    S = 400
+    q = HT.from_logical(np.zeros([1, 1, S, 128]), capi.BFLOAT16)
+    k = HT.from_logical(rand(54, 1, [1, 1, S, 128]), capi.BFLOAT16)
+    v = HT.from_logical(rand(54, 2, [1, 1, S, 128]), capi.BFLOAT16)
+    out = run(ctx, q, k, v, causal=True)
+    vl = v.logical()[0, 0]
+    ref = np.cumsum(vl, axis=0) / np.arange(1, S + 1)[:, None]
+    assert_close(out.logical()[0, 0], ref, capi.BFLOAT16)
+
+
+def test_flash_not_chosen_outside_contract(ctx):
+    # head dim 64 and masked attention keep the generic kernel
+    q = HT.from_logical(rand(55, 0, [1, 2, 70, 64]), capi.BFLOAT16)
+    out = run(ctx, q, q, q, expect_tuned=False)
+    ref = oracle.sdpa(q.logical(), q.logical(), q.logical())
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+
+
+def test_flash_headline_shape(ctx):
+    """B4 H32 S2048 D128 bf16 causal at full size.
+
+    Heads are independent, so the oracle is run on four (batch, head) slices
+    picked across the grid; q = 0 in one further head gives the closed-form
+    prefix means."""
+    B, H, S, D = 4, 32, 2048, 128
+    qv = rand(56, 0, [B, H, S, D])
+    qv[2, 7] = 0.0
+    q = HT.from_logical(qv, capi.BFLOAT16)
+    k = HT.from_logical(rand(56, 1, [B, H, S, D]), capi.BFLOAT16)
+    v = HT.from_logical(rand(56, 2, [B, H, S, D]), capi.BFLOAT16)
+    out = run(ctx, q, k, v, causal=True).logical()
+    assert np.all(np.isfinite(out))
+    ql, kl, vl = q.logical(), k.logical(), v.logical()
+    for b, h in [(0, 0), (1, 13), (3, 31), (2, 20)]:
+        ref = oracle.sdpa(ql[b:b + 1, h:h + 1], kl[b:b + 1, h:h + 1],
+                          vl[b:b + 1, h:h + 1], is_causal=True)
+        assert_close(out[b:b + 1, h:h + 1], ref, capi.BFLOAT16, f"b{b} h{h}")
+    ref = np.cumsum(vl[2, 7], axis=0) / np.arange(1, S + 1)[:, None]
+    assert_close(out[2, 7], ref, capi.BFLOAT16, "uniform head")
