@@ -29,6 +29,11 @@ sys.path.insert(0, ROOT)
 from fusilli_amd import capi, synth  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the headline kernel, measured under rocprofv3
+# (--pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this script, each scaled by
+# what the same counter reads for `--calibrate-copy`): 65 629 KiB fetched +
+# 65 536 KiB written.  Counters cannot be read from inside this process.
+RMSNORM_TRAFFIC_BYTES = (65629 + 65536) * 1024
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}
 
 
@@ -194,6 +199,25 @@ def bench_sdpa(ctx, steps, warmup):
             "flop_convention": "4*B*H*S*S*D/2 (causal half)"}
 
 
+def calibrate_copy(ctx, steps):
+    """Plain copy of known size (pointwise IDENTITY over 64 Mi f32 = 256 MiB
+    read + 256 MiB written): the yardstick that FETCH_SIZE / WRITE_SIZE
+    counter readings of the other kernels are scaled by."""
+    n = 64 * 1024 * 1024
+    d = capi.PointwiseDesc()
+    d.mode, d.num_inputs = capi.PW["IDENTITY"], 1
+    d.in_[0] = capi.TensorDesc.make([n], [1], capi.FLOAT)
+    d.out = capi.TensorDesc.make([n], [1], capi.FLOAT)
+    d.params = capi.PointwiseParams.default()
+    src, dst = ctx.alloc(n * 4), ctx.alloc(n * 4)
+    ctx.memset(src, 0)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.pointwise(d, src, None, None, dst),
+                                steps, 2)
+    return {"bytes_read": n * 4, "bytes_written": n * 4,
+            "kernel_us": round(ev_ms * 1e3, 2),
+            "gbs": round(2 * n * 4 / ev_ms / 1e6, 1)}
+
+
 def cpu_baseline_rmsnorm(seconds_budget=12.0):
     """The oracle's bf16 RMSNorm * scalar on the host cores over a row sample."""
     from oracle import oracle
@@ -224,6 +248,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain copy kernel of known size (counter "
+                         "calibration) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path "
@@ -232,6 +259,10 @@ def main():
         sys.exit(2)
 
     ctx = capi.Context(0)
+    if args.calibrate_copy:
+        print(json.dumps({"calibrate_copy": calibrate_copy(ctx, max(3, args.steps // 20))}))
+        ctx.close()
+        return
     r = bench_rmsnorm(ctx, args.steps, args.warmup, "scalar")
     line = {
         "metric": "GB/s (norms) on 1 MI355X, % roofline",
@@ -253,7 +284,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(r["gbs_kernel"], 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(r["gbs_kernel"] / HBM_PEAK_GBS, 4),
-                     "traffic": None,
+                     "traffic": RMSNORM_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": r["bytes"],
                      "kernel_us": round(r["kernel_ms"] * 1e3, 2)},
     }
