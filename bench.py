@@ -144,8 +144,8 @@ def bench_matmul(ctx, steps, warmup, kind, m=4096, n=4096, k=8192):
 
 
 def bench_conv(ctx, steps, warmup):
-    """C3: conv_fprop bf16 NHWC N16 C64 56x56, K128 3x3 pad 1, + bias + ReLU."""
-    n, c, h, w, k, r = 16, 64, 56, 56, 128, 3
+    """C3: conv_fprop bf16 NHWC N32 C64 56x56, K128 3x3 pad 1, + bias + ReLU."""
+    n, c, h, w, k, r = 32, 64, 56, 56, 128, 3
     cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
     xd, wd, yd = [n, c, h, w], [k, c, r, r], [n, k, h, w]
     d = capi.ConvDesc()
@@ -302,7 +302,7 @@ def main():
             ctx, ksteps, kwarm, "fp8")
         others["matmul_bf16_4096x4096x4096"] = bench_matmul(
             ctx, ksteps, kwarm, "bf16", 4096, 4096, 4096)
-        others["conv_fprop_bf16_n16c64h56w56_k128r3s3_bias_relu"] = bench_conv(
+        others["conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu"] = bench_conv(
             ctx, max(20, args.steps // 4), kwarm)
         others["sdpa_fwd_bf16_causal_b4h32s2048d128"] = bench_sdpa(
             ctx, max(20, args.steps // 4), kwarm)

@@ -123,6 +123,11 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
       p.K * elem >= (1ll << 23))
     return p;
   g.x_bytes = (uint32_t)x_bytes;
+  g.R = (int32_t)R;
+  g.magic_q = conv_magic(g.Q);
+  g.magic_p = conv_magic(g.P);
+  g.magic_s = conv_magic(g.S);
+  g.magic_spt = conv_magic(g.slices_per_tap);
   // Fused operands must be addressable as base + m * sm + k * sk: either
   // constant over pixels (a per-channel vector) or laid out like OUT.
   for (int i = 0; i < d->epilogue.count; ++i) {

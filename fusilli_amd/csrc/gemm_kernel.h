@@ -98,7 +98,24 @@ struct ConvGeom {
   int32_t pad_h, pad_w, str_h, str_w, dil_h, dil_w;
   int32_t slices_per_tap; // C * elem / 128
   uint32_t x_bytes;       // bytes of the input tensor (< 2^31)
+  int32_t R;              // filter height
+  // floor(2^32 / d) for d = Q, P, S, slices_per_tap (see conv_div)
+  uint32_t magic_q, magic_p, magic_s, magic_spt;
 };
+
+// n / d for 0 <= n < 2^31 with magic = floor(2^32 / d): the estimate is at
+// most one too small.
+__host__ __device__ inline uint32_t conv_magic(int32_t d) {
+  return d <= 1 ? 0u : (uint32_t)((1ull << 32) / (uint32_t)d);
+}
+__device__ __forceinline__ int32_t conv_div(int32_t n, int32_t d, uint32_t magic) {
+  if (d == 1)
+    return n;
+  int32_t q = (int32_t)__umulhi((uint32_t)n, magic);
+  if (n - q * d >= d)
+    ++q;
+  return q;
+}
 
 enum GemmAMode { A_KCONTIG = 0, A_MCONTIG = 1, A_CONV = 2 };
 
@@ -445,25 +462,28 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   if constexpr (A_MODE == A_CONV) {
     a_base = g.a;
     a_step = 0;
-    const int taps = kt_count / g.conv.slices_per_tap;
 #pragma unroll
     for (int j = 0; j < GA::kLoads; ++j) {
       const int row = (j * NW + wave) * 8 + (l >> 3);
       const int64_t m = m0 + row;
       const bool live = m < g.M;
       const int32_t mm = (int32_t)(live ? m : 0);
-      const int32_t q = mm % g.conv.Q, pq = mm / g.conv.Q;
-      const int32_t pp = pq % g.conv.P, nn = pq / g.conv.P;
+      const int32_t pq = conv_div(mm, g.conv.Q, g.conv.magic_q);
+      const int32_t q = mm - pq * g.conv.Q;
+      const int32_t nn = conv_div(pq, g.conv.P, g.conv.magic_p);
+      const int32_t pp = pq - nn * g.conv.P;
       const int32_t ih0 = pp * g.conv.str_h - g.conv.pad_h;
       const int32_t iw0 = q * g.conv.str_w - g.conv.pad_w;
       cv_pix[j] = (nn * g.conv.H + ih0) * g.conv.W + iw0;
       uint32_t mask = 0;
-      for (int t = 0; t < taps; ++t) {
-        const int32_t ih = ih0 + (t / g.conv.S) * g.conv.dil_h;
-        const int32_t iw = iw0 + (t % g.conv.S) * g.conv.dil_w;
-        const bool in = (uint32_t)ih < (uint32_t)g.conv.H &&
-                        (uint32_t)iw < (uint32_t)g.conv.W;
-        mask |= (uint32_t)(in && live) << t;
+      int t = 0;
+      for (int fr = 0; fr < g.conv.R; ++fr) {
+        const bool in_h = (uint32_t)(ih0 + fr * g.conv.dil_h) < (uint32_t)g.conv.H;
+        for (int fs = 0; fs < g.conv.S; ++fs, ++t) {
+          const bool in_w =
+              (uint32_t)(iw0 + fs * g.conv.dil_w) < (uint32_t)g.conv.W;
+          mask |= (uint32_t)(in_h && in_w && live) << t;
+        }
       }
       cv_mask[j] = mask;
       cv_chunk = ((l & 7) ^ kc_swz(row)) * 16; // same for every j
@@ -503,9 +523,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
     constexpr int A0 = PART * GA::kLoads / PARTS, A1 = (PART + 1) * GA::kLoads / PARTS;
     constexpr int B0 = PART * GB::kLoads / PARTS, B1 = (PART + 1) * GB::kLoads / PARTS;
     if constexpr (A_MODE == A_CONV) {
-      const int32_t tap = kt / g.conv.slices_per_tap;
-      const int32_t cb = (kt % g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
-      const int32_t fr = tap / g.conv.S, fs = tap % g.conv.S;
+      const int32_t tap = conv_div(kt, g.conv.slices_per_tap, g.conv.magic_spt);
+      const int32_t cb =
+          (kt - tap * g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
+      const int32_t fr = conv_div(tap, g.conv.S, g.conv.magic_s);
+      const int32_t fs = tap - fr * g.conv.S;
       const int32_t dpix = fr * g.conv.dil_h * g.conv.W + fs * g.conv.dil_w;
       const int32_t cbytes = g.conv.C * ELEM;
       uint32_t off[GA::kLoads];

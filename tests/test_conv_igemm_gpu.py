@@ -123,12 +123,12 @@ def test_conv_igemm_not_chosen_outside_contract(ctx):
 
 
 def test_conv_igemm_headline_shape(ctx):
-    """N16 C64 56x56, K128 3x3 pad 1, bf16, + bias + ReLU at full size.
+    """N32 C64 56x56, K128 3x3 pad 1, bf16, + bias + ReLU at full size.
 
     All-ones input and filter give closed-form answers (64 channels times the
     number of in-image taps); random data is checked against the oracle on the
     first and last image (the convolution is independent per image)."""
-    xd, wd = [16, 64, 56, 56], [128, 64, 3, 3]
+    xd, wd = [32, 64, 56, 56], [128, 64, 3, 3]
     pad, st, dil = [1, 1], [1, 1], [1, 1]
     bias = HT.from_logical(rand(45, 2, [1, 128, 1, 1]), capi.BFLOAT16,
                            oracle.channels_last_strides([1, 128, 1, 1]))
@@ -149,7 +149,7 @@ def test_conv_igemm_headline_shape(ctx):
               epilogue=epi, epi_tensors=[bias])
     lg = out.logical()
     xl = x.logical()
-    for img in (0, 15):
+    for img in (0, 31):
         ref = oracle.conv_fprop(xl[img:img + 1], w.logical(), pad, st, dil)
         ref = np.maximum(ref + bias.logical(), 0.0)
         assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"image {img}")
