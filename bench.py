@@ -176,6 +176,53 @@ def bench_conv(ctx, steps, warmup):
             "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
 
 
+def bench_reduce(ctx, steps, warmup, mode="SUM", sets=5):
+    """Row reduction bf16 X[8192,4096] -> f32 Y[8192,1] (reads 64 MiB per launch)."""
+    rows, cols = 8192, 4096
+    d = capi.ReduceDesc()
+    d.x = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.y = capi.TensorDesc.make([rows, 1], [1, 1], capi.FLOAT)
+    d.mode = capi.RED[mode]
+    assert ctx.lib.fhip_reduce_supported(d) == 2, "row-reduction kernel not chosen"
+    xs = [ctx.to_device(synth.f32_to_bf16_bits(synth.normal(10, s, rows * cols)))
+          for s in range(sets)]
+    y = ctx.alloc(rows * 4)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.reduce(d, xs[i % sets], y),
+                                steps, warmup)
+    nbytes = rows * cols * 2 + rows * 4
+    return {"value": round(nbytes / ev_ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "kernel_us": round(ev_ms * 1e3, 2), "bytes": nbytes}
+
+
+def bench_layernorm(ctx, steps, warmup, sets=5):
+    """LayerNorm bf16 X[8192,4096] with scale and bias (inference), bf16 out."""
+    rows, cols = 8192, 4096
+    d = capi.NormDesc()
+    d.x = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.scale = capi.TensorDesc.make([1, cols], [cols, 1], capi.BFLOAT16)
+    d.bias = capi.TensorDesc.make([1, cols], [cols, 1], capi.BFLOAT16)
+    d.y = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.out = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.epsilon = 1e-5
+    d.is_layernorm = 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_norm_fwd_supported(d) == 2, "tuned row kernel not chosen"
+    n = rows * cols
+    scale = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(11, 1, cols, 1.0, 0.02)))
+    bias = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(11, 2, cols, 0.0, 0.02)))
+    xs = [ctx.to_device(synth.f32_to_bf16_bits(synth.normal(11, 10 + s, n))) for s in range(sets)]
+    ys = [ctx.alloc(n * 2) for _ in range(sets)]
+    wall_ms, ev_ms = timed_loop(
+        ctx, lambda i: ctx.norm_fwd(d, xs[i % sets], scale, bias, ys[i % sets]),
+        steps, warmup)
+    nbytes = 2 * n * 2 + 2 * cols * 2
+    return {"value": round(nbytes / ev_ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "kernel_us": round(ev_ms * 1e3, 2), "bytes": nbytes}
+
+
 def bench_sdpa(ctx, steps, warmup):
     """C4: SDPA forward bf16 causal B4 H32 S2048 D128 ([B,H,S,D] contiguous)."""
     b, h, sq, d = 4, 32, 2048, 128
@@ -295,6 +342,12 @@ def main():
             "value": round(r2["gbs_kernel"], 1), "unit": "GB/s",
             "frac_of_hbm_peak": round(r2["gbs_kernel"] / HBM_PEAK_GBS, 4),
             "kernel_us": round(r2["kernel_ms"] * 1e3, 2), "bytes": r2["bytes"]}
+        others["layernorm_bf16_8192x4096_scale_bias"] = bench_layernorm(
+            ctx, args.steps, args.warmup)
+        others["reduce_sum_bf16_8192x4096_rows"] = bench_reduce(
+            ctx, args.steps, args.warmup, "SUM")
+        others["reduce_amax_bf16_8192x4096_rows"] = bench_reduce(
+            ctx, args.steps, args.warmup, "AMAX")
         ksteps, kwarm = max(10, args.steps // 10), max(3, args.warmup // 5)
         others["matmul_int8_4096x8192x4096_i32"] = bench_matmul(
             ctx, ksteps, kwarm, "int8")

@@ -892,7 +892,8 @@ int fhip_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
   (void)workspace;
   (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
-  if (fhip_fast_reduce_applicable(d))
+  // the row kernel moves 16-byte chunks: an unaligned base takes the generic one
+  if (fhip_fast_reduce_applicable(d) && ((uintptr_t)x & 15) == 0)
     return fhip_fast_reduce(ctx, d, x, y);
   ReduceArgs g{};
   g.y = make_dims(d->y);
