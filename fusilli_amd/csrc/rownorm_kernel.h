@@ -156,6 +156,31 @@ __device__ __forceinline__ float row_sum(float v, float *lds, int wave,
   return v;
 }
 
+// Two sums at once (same barriers as one).
+template <int WPR>
+__device__ __forceinline__ void row_sum2(float &a, float &b, float *lds,
+                                         int wave, int lane) {
+  a = wave_sum64(a);
+  b = wave_sum64(b);
+  if constexpr (WPR > 1) {
+    constexpr int W = RowNormGeom<WPR>::kWaves;
+    __syncthreads(); // previous use of lds is complete
+    if (lane == 0) {
+      lds[wave] = a;
+      lds[W + wave] = b;
+    }
+    __syncthreads();
+    const int first = (wave / WPR) * WPR;
+    a = 0.f;
+    b = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i) {
+      a += lds[first + i];
+      b += lds[W + first + i];
+    }
+  }
+}
+
 // One workgroup pass: the whole row is loaded with one 16-byte load per lane
 // per chunk and stays packed in registers (4 VGPRs per chunk) between the
 // statistics pass and the apply pass.
@@ -167,7 +192,7 @@ __global__ __launch_bounds__(RowNormGeom<WPR>::kThreads) void rownorm_kernel(
   constexpr int ROWS_PER_WG = RowNormGeom<WPR>::kRowsPerWg;
   constexpr bool GENERAL = VARIANT == RN_GENERAL;
   constexpr bool LAYERNORM_FIXED = VARIANT == RN_LN_SCALE_BIAS;
-  __shared__ float lds[RowNormGeom<WPR>::kWaves];
+  __shared__ float lds[2 * RowNormGeom<WPR>::kWaves];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -215,37 +240,43 @@ __global__ __launch_bounds__(RowNormGeom<WPR>::kThreads) void rownorm_kernel(
   const bool layernorm = GENERAL ? g.is_layernorm != 0 : LAYERNORM_FIXED;
   const float inv_n = 1.0f / (float)inner;
   float mean = 0.f;
+  float ss = 0.f;
   if (layernorm) {
-    float s = 0.f;
+    // One pass, one reduction: sums of (x - p) and (x - p)^2 about a pivot p
+    // taken from the row itself (its first element, read by every lane from
+    // one cache line), so the variance does not cancel for rows far from 0:
+    //   mean = p + S1/n,  var = S2/n - (S1/n)^2.
+    const float p = row_ok ? (float)xrow[0] : 0.f;
+    float s1 = 0.f, s2 = 0.f;
     static_for<CHUNKS>([&](auto ci) {
       constexpr int c = decltype(ci)::value;
       float v[VEC];
       unpack16<T, VEC>(raw[c], v);
-#pragma unroll
-      for (int i = 0; i < VEC; ++i)
-        s += v[i];
-    });
-    mean = row_sum<WPR>(s, lds, wave, lane) * inv_n;
-  }
-  float ss = 0.f;
-  static_for<CHUNKS>([&](auto ci) {
-    constexpr int c = decltype(ci)::value;
-    float v[VEC];
-    unpack16<T, VEC>(raw[c], v);
-    if (layernorm) {
       const bool live = col0 + c * COL_STEP < inner;
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
-        const float d = live ? v[i] - mean : 0.f;
-        ss += d * d;
+        const float d = live ? v[i] - p : 0.f;
+        s1 += d;
+        s2 += d * d;
       }
-    } else { // padding chunks hold zeros
+    });
+    row_sum2<WPR>(s1, s2, lds, wave, lane);
+    const float m1 = s1 * inv_n;
+    mean = p + m1;
+    const float var = s2 * inv_n - m1 * m1;
+    ss = (var > 0.f ? var : 0.f) * (float)inner;
+  } else {
+    static_for<CHUNKS>([&](auto ci) {
+      constexpr int c = decltype(ci)::value;
+      float v[VEC];
+      unpack16<T, VEC>(raw[c], v);
+      // padding chunks hold zeros
 #pragma unroll
       for (int i = 0; i < VEC; ++i)
         ss += v[i] * v[i];
-    }
-  });
-  ss = row_sum<WPR>(ss, lds, wave, lane);
+    });
+    ss = row_sum<WPR>(ss, lds, wave, lane);
+  }
   const float rstd = 1.0f / sqrtf(ss * inv_n + g.eps);
   if (!row_ok)
     return;
