@@ -248,8 +248,14 @@ __device__ __forceinline__ void dma_issue(const char *base, uint32_t bytes,
                                           const uint32_t (&off)[LOADS],
                                           uint32_t lds_stage) {
   const int w = threadIdx.x >> 6;
+  // the descriptor must sit in scalar registers: say so, or 64-bit pointer
+  // arithmetic done on the vector ALU forces a per-lane loop around each load
+  const uint64_t b64 = (uint64_t)base;
+  const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64);
+  const uint32_t bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      (void *)base, 0, (int)bytes, 0x00020000);
+      (void *)(((uint64_t)bhi << 32) | blo), 0,
+      (int)__builtin_amdgcn_readfirstlane(bytes), 0x00020000);
 #pragma unroll
   for (int j = J0; j < J1; ++j) {
     const uint32_t dst = lds_stage + (uint32_t)(j * NW + w) * 1024u;
@@ -585,6 +591,71 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   using Two = std::integral_constant<int, 2>;
 
   int cur = 0; // stage holding slice kt
+  constexpr bool PINGPONG = NW == 8;
+  if constexpr (PINGPONG) {
+    // Two wavefronts share each SIMD.  Every K-step is split into a memory
+    // phase (fragment reads for the next step, global->LDS loads) and an MFMA
+    // phase, with a barrier after each; wavefronts 4..7 run one phase behind
+    // wavefronts 0..3, so on every SIMD one wavefront feeds the matrix pipe
+    // while the other issues memory instructions.
+    const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
+    if (team)
+      __builtin_amdgcn_s_barrier();
+    for (int kt = 0; kt < kt_count; ++kt) {
+      const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;
+      const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;
+      const uint32_t sa = stage_a(cur), sb = stage_b(cur);
+      gemm_static_for<KSTEPS>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        constexpr int fc = s & 1, fn = fc ^ 1;
+        constexpr bool LAST = s + 1 == KSTEPS;
+        // ---- memory phase
+        if constexpr (!LAST) {
+          fa_addr.template load<s + 1>(sa, fa[fn]);
+          fb_addr.template load<s + 1>(sb, fb[fn]);
+          if constexpr (s == 0 && KSTEPS > 2)
+            issue(kt + NSTAGE - 1, prv, One{}, Two{});
+        } else {
+          // the barrier two phases back made slice kt + 1 visible and retired
+          // this stage (see below)
+          fa_addr.template load<0>(stage_a(nxt), fa[fn]);
+          fb_addr.template load<0>(stage_b(nxt), fb[fn]);
+          if constexpr (KSTEPS > 2)
+            issue(kt + NSTAGE, cur, Zero{}, Two{});
+          else
+            issue(kt + NSTAGE, cur, Zero{}, One{});
+        }
+        if constexpr (s == KSTEPS - 2) {
+          // Both teams wait here, one and two phases ahead of the first read
+          // of slice kt + 1: its loads have landed, and the last fragment
+          // reads of this stage (just issued) have returned before anyone
+          // refills it.
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          __builtin_amdgcn_s_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        } else {
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- MFMA phase
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            mfma32<KIND>(acc[i][j], fa[fc][i], fb[fc][j]);
+        __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      cur = nxt;
+    }
+    if (!team)
+      __builtin_amdgcn_s_barrier();
+  } else {
   // One K slice.  A stage is free again once the barrier of the iteration
   // that consumes it has passed, and is refilled at once with the slice
   // NSTAGE ahead: first half of its loads behind the MFMAs of the last
@@ -626,6 +697,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
       __builtin_amdgcn_sched_barrier(0);
     });
     cur = nxt;
+  }
   }
   // zero-sized loads of the last iterations may still be writing LDS
   __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
