@@ -599,33 +599,43 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
     // wavefronts 0..3, so on every SIMD one wavefront feeds the matrix pipe
     // while the other issues memory instructions.
     const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
+    // PS K-steps per phase: longer phases amortise the two barriers
+    constexpr int PS = KSTEPS >= 4 ? 2 : 1;
+    constexpr int PHASES = KSTEPS / PS;
+    Frag<KIND> pa[2][PS][TM], pb[2][PS][TN];
+    // fragments of the first phase of slice 0 (the prologue's barrier made
+    // the slice visible)
+    gemm_static_for<PS>([&](auto uc) {
+      constexpr int u = decltype(uc)::value;
+      fa_addr.template load<u>(stage_a(0), pa[0][u]);
+      fb_addr.template load<u>(stage_b(0), pb[0][u]);
+    });
     if (team)
       __builtin_amdgcn_s_barrier();
     for (int kt = 0; kt < kt_count; ++kt) {
       const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;
-      const int prv = cur == 0 ? NSTAGE - 1 : cur - 1;
       const uint32_t sa = stage_a(cur), sb = stage_b(cur);
-      gemm_static_for<KSTEPS>([&](auto sc) {
-        constexpr int s = decltype(sc)::value;
-        constexpr int fc = s & 1, fn = fc ^ 1;
-        constexpr bool LAST = s + 1 == KSTEPS;
-        // ---- memory phase
-        if constexpr (!LAST) {
-          fa_addr.template load<s + 1>(sa, fa[fn]);
-          fb_addr.template load<s + 1>(sb, fb[fn]);
-          if constexpr (s == 0 && KSTEPS > 2)
-            issue(kt + NSTAGE - 1, prv, One{}, Two{});
-        } else {
-          // the barrier two phases back made slice kt + 1 visible and retired
-          // this stage (see below)
-          fa_addr.template load<0>(stage_a(nxt), fa[fn]);
-          fb_addr.template load<0>(stage_b(nxt), fb[fn]);
-          if constexpr (KSTEPS > 2)
-            issue(kt + NSTAGE, cur, Zero{}, Two{});
-          else
-            issue(kt + NSTAGE, cur, Zero{}, One{});
-        }
-        if constexpr (s == KSTEPS - 2) {
+      gemm_static_for<PHASES>([&](auto pc) {
+        constexpr int ph = decltype(pc)::value;
+        static_assert(PHASES % 2 == 0, "register sets alternate per phase");
+        constexpr bool LASTP = ph + 1 == PHASES;
+        constexpr int fc = ph & 1, fn = fc ^ 1;
+        // ---- memory phase: fragments of the next phase, loads of a later slice
+        gemm_static_for<PS>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
+          if constexpr (!LASTP) {
+            fa_addr.template load<(ph + 1) * PS + u>(sa, pa[fn][u]);
+            fb_addr.template load<(ph + 1) * PS + u>(sb, pb[fn][u]);
+          } else {
+            fa_addr.template load<u>(stage_a(nxt), pa[fn][u]);
+            fb_addr.template load<u>(stage_b(nxt), pb[fn][u]);
+          }
+        });
+        // the whole next-but-one slice at once: it then has an MFMA phase and
+        // a memory phase of flight time before the wait below
+        if constexpr (LASTP)
+          issue(kt + NSTAGE, cur, Zero{}, One{});
+        if constexpr (ph == PHASES - 2) {
           // Both teams wait here, one and two phases ahead of the first read
           // of slice kt + 1: its loads have landed, and the last fragment
           // reads of this stage (just issued) have returned before anyone
@@ -641,11 +651,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
         // ---- MFMA phase
         __builtin_amdgcn_s_setprio(1);
+        gemm_static_for<PS>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+          for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            mfma32<KIND>(acc[i][j], fa[fc][i], fb[fc][j]);
+            for (int j = 0; j < TN; ++j)
+              mfma32<KIND>(acc[i][j], pa[fc][u][i], pb[fc][u][j]);
+        });
         __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
