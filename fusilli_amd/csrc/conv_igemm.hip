@@ -117,9 +117,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
   p.M = d->x.dim[0] * g.P * g.Q;
   p.N = d->w.dim[0];
   p.K = R * g.S * C;
-  // 32-bit byte offsets in the gather; one validity bit per filter tap
+  // 32-bit byte offsets in the gather; one validity bit per filter row and
+  // one per filter column
   const int64_t x_bytes = d->x.dim[0] * (int64_t)g.H * g.W * C * elem;
-  if (x_bytes >= (1ll << 31) || p.M >= (1ll << 31) || R * g.S > 32 ||
+  if (x_bytes >= (1ll << 31) || p.M >= (1ll << 31) || R > 16 || g.S > 16 ||
       p.K * elem >= (1ll << 23))
     return p;
   g.x_bytes = (uint32_t)x_bytes;
@@ -145,11 +146,14 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
   }
   p.bn = p.N > 128 ? 256 : 128;
   p.bm = p.M >= 256 ? 256 : 128;
-  if (p.bn == 256 && p.bm == 128)
-    p.bn = 128;
+  // 128-wide outputs run as 128 x 128 tiles on two stages: two workgroups
+  // share a compute unit and cover each other's prologue and epilogue
+  if (p.bn == 128 || p.bm == 128)
+    p.bm = p.bn = 128;
   if (const char *env = getenv("FUSILLI_HIP_CONV_TILE")) {
     int bm = 0, bn = 0;
-    if (sscanf(env, "%d,%d", &bm, &bn) == 2 && (bm == 128 || bm == 256) &&
+    if (sscanf(env, "%d,%d", &bm, &bn) == 2 &&
+        (bm == 128 || bm == 256 || (bm == 512 && bn == 128)) &&
         (bn == 128 || bn == 256) && bm >= bn)
       p.bm = bm, p.bn = bn;
   }
@@ -211,6 +215,7 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     o.stride[1] = sm;          // per-pixel step (0 for channel vectors)
     o.stride[2] = s.stride[1]; // per-channel step
   }
+  gemm_fill_linear(d->epilogue, g);
   if (p.kind == GK_BF16)
     return conv_launch_bf16(ctx, p.bm, p.bn, g);
   return conv_launch_f16(ctx, p.bm, p.bn, g);

@@ -132,6 +132,12 @@ struct GemmArgs {
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
   int32_t o_vec;              // output rows allow aligned 16-byte stores
+  // Epilogue applied to the accumulators in registers: every op is one of
+  // ADD / SUB / MUL / RELU / NEG / IDENTITY with a scalar or per-column
+  // operand: v = mul ? v * o : a * v + b * o, then max(v, 0) if relu.
+  int32_t epi_reg;
+  float lin_a[FHIP_MAX_EPILOGUE], lin_b[FHIP_MAX_EPILOGUE];
+  int32_t lin_mul[FHIP_MAX_EPILOGUE], lin_relu[FHIP_MAX_EPILOGUE];
   DevEpilogue epi;            // strides refer to (batch, m, n)
 };
 
@@ -375,6 +381,10 @@ template <int NM, int NR, int NV> __device__ __forceinline__ void gemm_interleav
   });
 }
 
+// Makes the compiler treat `x` as produced here (a value that a pending load
+// delivers must have arrived).
+__device__ __forceinline__ void gemm_pin(float &x) { asm volatile("" : "+v"(x)); }
+
 template <int N>
 __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
                                                  const int64_t (&off)[N],
@@ -396,16 +406,28 @@ __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
 
 // LDS bytes of the kernel: NSTAGE stages of (A slice + B slice); the epilogue
 // reuses it for four 32-row accumulator bands (one per wavefront).
+// Wavefront grid of a tile.  8 wavefronts (two per SIMD, scheduled in
+// alternating memory / MFMA phases) where each still owns 128 x 64 outputs:
+// 256 x 256 as 2 x 4 and 512 x 128 as 4 x 2; otherwise 2 x 2.
+template <int BM, int BN> struct GemmLayout {
+  static constexpr bool kWide = BM == 256 && BN == 256;
+  static constexpr bool kTall = BM == 512 && BN == 128;
+  static constexpr int kWavesM = kTall ? 4 : 2;
+  static constexpr int kWavesN = kWide ? 4 : 2;
+  static constexpr int kWaves = kWavesM * kWavesN;
+};
+
 template <int BM, int BN, int NSTAGE, int NW> struct GemmLds {
   static constexpr int kStage = (BM + BN) * kTileKBytes;
-  static constexpr int kWN = BN / (NW / 2); // wavefront tile columns
+  static constexpr int kWN = BN / GemmLayout<BM, BN>::kWavesN; // wave columns
   static constexpr int kEpiPitch = kWN * 4 + 32;
   static constexpr int kBand = 32 * kEpiPitch; // one wavefront, one tile row
-  static constexpr int kTM = BM / 64;
-  // tile rows that leave together: as many as fit 160 KB
+  static constexpr int kTM = BM / GemmLayout<BM, BN>::kWavesM / 32;
+  // tile rows that leave together: as many as fit 160 KB, or 80 KB where the
+  // stages leave room for two workgroups per compute unit
+  static constexpr int kCap = NSTAGE * kStage <= 80 * 1024 ? 80 * 1024 : 160 * 1024;
   static constexpr int kBands =
-      NW * kTM * kBand <= 160 * 1024 ? kTM
-                                     : (NW * 2 * kBand <= 160 * 1024 ? 2 : 1);
+      NW * kTM * kBand <= kCap ? kTM : (NW * 2 * kBand <= kCap ? 2 : 1);
   static constexpr int kEpiBytes = NW * kBands * kBand;
   static constexpr int kBytes =
       NSTAGE * kStage > kEpiBytes ? NSTAGE * kStage : kEpiBytes;
@@ -422,8 +444,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   using GA = SliceGeom<BM, ELEM, A_KC, NW>;
   using GB = SliceGeom<BN, ELEM, B_KC, NW>;
   using L = GemmLds<BM, BN, NSTAGE, NW>;
-  constexpr int WAVES_N = NW / 2;
-  constexpr int WM = BM / 2, WN = BN / WAVES_N; // wavefront tile
+  constexpr int WAVES_M = GemmLayout<BM, BN>::kWavesM;
+  constexpr int WAVES_N = GemmLayout<BM, BN>::kWavesN;
+  static_assert(WAVES_M * WAVES_N == NW, "wavefront grid");
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N; // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int LPS = GA::kLoads + GB::kLoads; // DMA instructions per slice
 
@@ -461,7 +485,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   const char *a_base;
   int64_t a_step;
   uint32_t off_a[GA::kLoads], off_b[GB::kLoads];
-  // implicit-GEMM gather: pixel index of tap (0, 0) and in-image tap mask
+  // implicit-GEMM gather: pixel index of tap (0, 0) and in-image row / column
+  // masks of the filter
   int32_t cv_pix[A_MODE == A_CONV ? GA::kLoads : 1];
   uint32_t cv_mask[A_MODE == A_CONV ? GA::kLoads : 1];
   int cv_chunk = 0;
@@ -481,16 +506,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
       const int32_t ih0 = pp * g.conv.str_h - g.conv.pad_h;
       const int32_t iw0 = q * g.conv.str_w - g.conv.pad_w;
       cv_pix[j] = (nn * g.conv.H + ih0) * g.conv.W + iw0;
+      // bits 0..15: filter rows inside the image, 16..31: filter columns
       uint32_t mask = 0;
-      int t = 0;
-      for (int fr = 0; fr < g.conv.R; ++fr) {
-        const bool in_h = (uint32_t)(ih0 + fr * g.conv.dil_h) < (uint32_t)g.conv.H;
-        for (int fs = 0; fs < g.conv.S; ++fs, ++t) {
-          const bool in_w =
-              (uint32_t)(iw0 + fs * g.conv.dil_w) < (uint32_t)g.conv.W;
-          mask |= (uint32_t)(in_h && in_w && live) << t;
-        }
-      }
+      for (int fr = 0; fr < g.conv.R; ++fr)
+        mask |= (uint32_t)(live && (uint32_t)(ih0 + fr * g.conv.dil_h) <
+                                       (uint32_t)g.conv.H)
+                << fr;
+      for (int fs = 0; fs < g.conv.S; ++fs)
+        mask |= (uint32_t)((uint32_t)(iw0 + fs * g.conv.dil_w) <
+                           (uint32_t)g.conv.W)
+                << (16 + fs);
       cv_mask[j] = mask;
       cv_chunk = ((l & 7) ^ kc_swz(row)) * 16; // same for every j
     }
@@ -539,7 +564,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
       uint32_t off[GA::kLoads];
 #pragma unroll
       for (int j = A0; j < A1; ++j) {
-        const bool in = (cv_mask[j] >> tap) & 1;
+        const bool in = (cv_mask[j] >> fr) & (cv_mask[j] >> (16 + fs)) & 1;
         // taps outside the image (and rows past M) read past the end: zeros
         off[j] = in ? (uint32_t)((cv_pix[j] + dpix) * cbytes + cb) : 0x80000000u;
       }
@@ -733,6 +758,77 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   const int64_t ob = batch * g.o_batch;
   const int64_t ncol = n0 + wn * WN + (l % LPR) * 8;
 
+  // Lean path: the epilogue is linear with scalar / per-column operands (bias,
+  // scale, ReLU ...), the output rows allow aligned 16-byte stores and this
+  // wavefront has no ragged columns.  A lane's 8 columns are the same in
+  // every pass, so each operand is loaded once, before the passes.
+  const bool lane_full = ncol + 8 <= g.N || ncol >= g.N;
+  const bool lean = g.epi_reg && g.o_vec != 0 &&
+                    __builtin_amdgcn_ballot_w64(!lane_full) == 0;
+  // Per op and column y <- y * S + T: (S, T) = (a, b * operand) for the
+  // additive modes and (operand, -0) for MUL.
+  float S[FHIP_MAX_EPILOGUE][8], T[FHIP_MAX_EPILOGUE][8];
+  if constexpr (!std::is_same<Acc, int>::value) {
+    if (lean) {
+      gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        if (e >= g.epi.count)
+          return;
+        const DevEpiOp &o = g.epi.op[e];
+        float ov[8];
+        if (o.kind == FHIP_OPERAND_TENSOR) {
+          int64_t off[8];
+#pragma unroll
+          for (int c = 0; c < 8; ++c) {
+            int64_t n = ncol + c;
+            n = n < g.N ? n : g.N - 1;
+            off[c] = n * o.stride[2];
+          }
+          load_operand_vec<8>(o.ptr, o.operand_dtype, off, ov);
+        } else {
+#pragma unroll
+          for (int c = 0; c < 8; ++c)
+            ov[c] = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
+        }
+        const bool mul = g.lin_mul[e] != 0;
+        const float a = g.lin_a[e], b = g.lin_b[e];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          S[e][c] = mul ? ov[c] : a;
+          T[e][c] = mul ? -0.f : b * ov[c];
+        }
+      });
+      // The operands are in registers from here on: no pass may wait on the
+      // memory counter, which the stores of earlier passes share.
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+      gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        if (e >= g.epi.count)
+          return;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+{
+          gemm_pin(S[e][c]);
+          gemm_pin(T[e][c]);
+        }
+      });
+    }
+  }
+  const int64_t esz = fhip_dtype_size(g.o_dt);
+  GEMM_AS1 char *lean_ptr =
+      (GEMM_AS1 char *)g.out +
+      (ob + (m0 + wm * WM + l / LPR) * g.o_sm + ncol) * esz;
+  const int64_t lean_m = m0 + wm * WM + l / LPR;
+  const int64_t row_bytes = g.o_sm * esz;
+  const int nops = g.epi.count;
+  const int64_t gM = g.M, gN = g.N;
+  const int o_dt = g.o_dt;
+  int lin_relu[FHIP_MAX_EPILOGUE];
+  gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
+    constexpr int e = decltype(ec)::value;
+    lin_relu[e] = g.lin_relu[e];
+  });
+
   gemm_static_for<TM / BANDS>([&](auto rc) {
     constexpr int round = decltype(rc)::value;
 #pragma unroll
@@ -744,6 +840,82 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
           *(GEMM_AS3 Acc *)(uintptr_t)(wr + bi * L::kBand +
                                        ((r >> 2) * 8 + (r & 3)) * PITCH +
                                        j * 128) = acc[round * BANDS + bi][j][r];
+    if (lean) {
+      // OT: 0 float, 1 bf16, 2 f16 output
+      auto passes = [&](auto ot_c) {
+        constexpr int OT = decltype(ot_c)::value;
+#pragma unroll
+        for (int p = 0; p < BANDS * PPB; ++p) {
+          const int bi = p / PPB, pp = p % PPB;
+          const int rel = (round * BANDS + bi) * 32 + pp * RPP;
+          const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
+          const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
+          const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
+          if (lean_m + rel >= gM || ncol >= gN)
+            continue;
+          GEMM_AS1 char *dst = lean_ptr + rel * row_bytes;
+          if constexpr (std::is_same<Acc, int>::value) {
+            *(GEMM_AS1 u32x4 *)dst = v0;
+            *(GEMM_AS1 u32x4 *)(dst + 16) = v1;
+          } else {
+            const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w,
+                                   v1.x, v1.y, v1.z, v1.w};
+            float y[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+              y[c] = __builtin_bit_cast(float, w[c]);
+            gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
+              constexpr int e = decltype(ec)::value;
+              if (e >= nops)
+                return;
+#pragma unroll
+              for (int c = 0; c < 8; ++c)
+                y[c] = __builtin_fmaf(y[c], S[e][c], T[e][c]);
+              if (lin_relu[e]) {
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                  y[c] = fmaxf(y[c], 0.f);
+              }
+            });
+            if constexpr (OT == 1) {
+              bf16x8 v;
+#pragma unroll
+              for (int c = 0; c < 8; ++c)
+                v[c] = (__bf16)y[c];
+              *(GEMM_AS1 bf16x8 *)dst = v;
+            } else if constexpr (OT == 2) {
+              f16x8 v;
+#pragma unroll
+              for (int c = 0; c < 8; ++c)
+                v[c] = (_Float16)y[c];
+              *(GEMM_AS1 f16x8 *)dst = v;
+            } else {
+              *(GEMM_AS1 u32x4 *)dst =
+                  u32x4{__builtin_bit_cast(uint32_t, y[0]),
+                        __builtin_bit_cast(uint32_t, y[1]),
+                        __builtin_bit_cast(uint32_t, y[2]),
+                        __builtin_bit_cast(uint32_t, y[3])};
+              *(GEMM_AS1 u32x4 *)(dst + 16) =
+                  u32x4{__builtin_bit_cast(uint32_t, y[4]),
+                        __builtin_bit_cast(uint32_t, y[5]),
+                        __builtin_bit_cast(uint32_t, y[6]),
+                        __builtin_bit_cast(uint32_t, y[7])};
+            }
+          }
+        }
+      };
+      if constexpr (std::is_same<Acc, int>::value) {
+        passes(std::integral_constant<int, 0>{});
+      } else {
+        if (o_dt == FHIP_BFLOAT16)
+          passes(std::integral_constant<int, 1>{});
+        else if (o_dt == FHIP_HALF)
+          passes(std::integral_constant<int, 2>{});
+        else
+          passes(std::integral_constant<int, 0>{});
+      }
+      return;
+    }
 #pragma clang loop unroll(disable)
     for (int p = 0; p < BANDS * PPB; ++p) {
       const int bi = p / PPB, pp = p % PPB;
@@ -777,7 +949,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
         for (int c = 0; c < 8; ++c)
           y[c] = __builtin_bit_cast(float, w[c]);
         fhip_round_fast_vec<8>(g.c_dt, y);
-        for (int e = 0; e < g.epi.count; ++e) {
+        for (int e = 0; e < nops; ++e) {
           const DevEpiOp &o = g.epi.op[e];
           if (o.kind == FHIP_OPERAND_NONE) {
             fhip_pw_fast_unary_vec<true, 8>(o.mode, y, o.params.swish_beta);
@@ -848,6 +1020,63 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   });
 }
 
+// Decides whether the epilogue can run on the accumulators in registers and
+// fills its linear form.  `g.epi` must hold the (batch, m, n) strides already.
+inline void gemm_fill_linear(const fhip_epilogue &e, GemmArgs &g) {
+  g.epi_reg = 0;
+  if (e.count == 0) {
+    // the store's conversion is the only rounding
+    g.epi_reg = g.c_dt == FHIP_FLOAT || g.c_dt == g.o_dt;
+    return;
+  }
+  // no rounding between the steps: every intermediate is f32 (the last
+  // result may already have the stored type, which the store's conversion
+  // reproduces)
+  if (g.c_dt != FHIP_FLOAT)
+    return;
+  for (int i = 0; i < e.count; ++i) {
+    const int dt = e.op[i].result_dtype;
+    if (dt != FHIP_FLOAT && !(i + 1 == e.count && dt == g.o_dt))
+      return;
+  }
+  for (int i = 0; i < e.count; ++i) {
+    const fhip_epilogue_op &o = e.op[i];
+    float a = 1.f, b = 0.f;
+    int mul = 0, relu = 0;
+    switch (o.mode) {
+    case FHIP_PW_ADD:
+      b = 1.f;
+      break;
+    case FHIP_PW_SUB: // IN_0 - IN_1
+      a = o.acc_is_in1 ? -1.f : 1.f;
+      b = o.acc_is_in1 ? 1.f : -1.f;
+      break;
+    case FHIP_PW_MUL:
+      mul = 1;
+      break;
+    case FHIP_PW_RELU_FWD:
+      relu = 1;
+      break;
+    case FHIP_PW_NEG:
+      a = -1.f;
+      break;
+    case FHIP_PW_IDENTITY:
+      break;
+    default:
+      return;
+    }
+    // tensor operands must depend on the column only
+    if (o.operand_kind == FHIP_OPERAND_TENSOR &&
+        (g.epi.op[i].stride[0] != 0 || g.epi.op[i].stride[1] != 0))
+      return;
+    g.lin_a[i] = a;
+    g.lin_b[i] = b;
+    g.lin_mul[i] = mul;
+    g.lin_relu[i] = relu;
+  }
+  g.epi_reg = 1;
+}
+
 // What the host decided about one matmul call.
 struct GemmPlan {
   bool ok = false;
@@ -865,16 +1094,13 @@ template <int BM, int BN> struct GemmStages {
   static constexpr int value = 160 * 1024 / kStage >= 4 ? 4 : 160 * 1024 / kStage;
 };
 
-// Wavefronts per workgroup: 8 (two per SIMD, so one can issue MFMAs while
-// the other waits on a memory queue) where each still gets a 2-tile-wide
-// block, else 4.
 template <int BM, int BN> struct GemmWaves {
-  static constexpr int value = BN >= 256 ? 8 : 4;
+  static constexpr int value = GemmLayout<BM, BN>::kWaves;
 };
 
-template <int KIND, int BM, int BN, int A_MODE, bool B_KC>
+template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int STAGES = 0>
 int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
-  constexpr int NSTAGE = GemmStages<BM, BN>::value;
+  constexpr int NSTAGE = STAGES ? STAGES : GemmStages<BM, BN>::value;
   constexpr int NW = GemmWaves<BM, BN>::value;
   constexpr int lds = GemmLds<BM, BN, NSTAGE, NW>::kBytes;
   auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC, NSTAGE, NW>;
@@ -914,11 +1140,15 @@ int gemm_launch_kind(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g) {
 // Implicit-GEMM convolution launchers (A gathered, B = filter, K-contiguous).
 template <int KIND>
 int conv_launch_kind(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
+  if (bm == 512 && bn == 128)
+    return launch<KIND, 512, 128, A_CONV, true>(ctx, g, 1);
   if (bm == 256 && bn == 256)
     return launch<KIND, 256, 256, A_CONV, true>(ctx, g, 1);
   if (bm == 256 && bn == 128)
     return launch<KIND, 256, 128, A_CONV, true>(ctx, g, 1);
-  return launch<KIND, 128, 128, A_CONV, true>(ctx, g, 1);
+  // two stages: two workgroups share a compute unit, and one's prologue and
+  // epilogue hide behind the other's K loop (convolutions have short K)
+  return launch<KIND, 128, 128, A_CONV, true, 2>(ctx, g, 1);
 }
 
 int gemm_launch_bf16(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g);

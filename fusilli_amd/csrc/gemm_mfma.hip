@@ -199,6 +199,7 @@ int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
     o.stride[1] = s.stride[r - 2];
     o.stride[2] = s.stride[r - 1];
   }
+  gemm_fill_linear(d->epilogue, g);
   switch (p.kind) {
   case GK_BF16:
     return gemm_launch_bf16(ctx, p, g);

@@ -74,7 +74,7 @@ def test_conv_igemm_random_vs_oracle(ctx, case, dtype):
     assert_close(out.logical(), ref, dtype, str(case))
 
 
-@pytest.mark.parametrize("tile", ["128,128", "256,128", "256,256"])
+@pytest.mark.parametrize("tile", ["128,128", "256,128", "256,256", "512,128"])
 def test_conv_igemm_every_tile_shape(ctx, tile, monkeypatch):
     monkeypatch.setenv("FUSILLI_HIP_CONV_TILE", tile)
     case = dict(x=[2, 64, 15, 17], w=[300, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1])
