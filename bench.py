@@ -195,6 +195,34 @@ def bench_reduce(ctx, steps, warmup, mode="SUM", sets=5):
             "kernel_us": round(ev_ms * 1e3, 2), "bytes": nbytes}
 
 
+def bench_pointwise(ctx, steps, warmup, mode="ADD", sets=5):
+    """Pointwise bf16 [8192,4096]: ADD of a bias row [1,4096], or unary GELU."""
+    rows, cols = 8192, 4096
+    n = rows * cols
+    d = capi.PointwiseDesc()
+    d.mode = capi.PW[mode]
+    d.params = capi.PointwiseParams.default()
+    d.in_[0] = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.out = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    bias = None
+    if mode == "ADD":
+        d.num_inputs = 2
+        d.in_[1] = capi.TensorDesc.make([1, cols], [cols, 1], capi.BFLOAT16)
+        bias = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(12, 1, cols)))
+    else:
+        d.num_inputs = 1
+    assert ctx.lib.fhip_pointwise_supported(d) == 2, "vector pointwise kernel not chosen"
+    xs = [ctx.to_device(synth.f32_to_bf16_bits(synth.normal(12, 10 + s, n))) for s in range(sets)]
+    ys = [ctx.alloc(n * 2) for _ in range(sets)]
+    wall_ms, ev_ms = timed_loop(
+        ctx, lambda i: ctx.pointwise(d, xs[i % sets], bias, None, ys[i % sets]),
+        steps, warmup)
+    nbytes = 2 * n * 2 + (cols * 2 if bias is not None else 0)
+    return {"value": round(nbytes / ev_ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "kernel_us": round(ev_ms * 1e3, 2), "bytes": nbytes}
+
+
 def bench_layernorm(ctx, steps, warmup, sets=5):
     """LayerNorm bf16 X[8192,4096] with scale and bias (inference), bf16 out."""
     rows, cols = 8192, 4096
@@ -344,6 +372,10 @@ def main():
             "kernel_us": round(r2["kernel_ms"] * 1e3, 2), "bytes": r2["bytes"]}
         others["layernorm_bf16_8192x4096_scale_bias"] = bench_layernorm(
             ctx, args.steps, args.warmup)
+        others["pointwise_add_bf16_8192x4096_bias_row"] = bench_pointwise(
+            ctx, max(5, args.steps // 4), 2, "ADD")
+        others["pointwise_gelu_bf16_8192x4096"] = bench_pointwise(
+            ctx, max(5, args.steps // 4), 2, "GELU_FWD")
         others["reduce_sum_bf16_8192x4096_rows"] = bench_reduce(
             ctx, args.steps, args.warmup, "SUM")
         others["reduce_amax_bf16_8192x4096_rows"] = bench_reduce(

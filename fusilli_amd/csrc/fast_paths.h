@@ -27,4 +27,9 @@ bool fhip_fast_reduce_applicable(const fhip_reduce_desc *d);
 int fhip_fast_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
                      void *y);
 
+bool fhip_fast_pointwise_applicable(const fhip_pointwise_desc *d);
+int fhip_fast_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d,
+                        const void *in0, const void *in1, const void *in2,
+                        void *out);
+
 #endif // FUSILLI_AMD_CSRC_FAST_PATHS_H

@@ -984,7 +984,7 @@ static int pointwise_validate(fhip_ctx *ctx, const fhip_pointwise_desc *d) {
 int fhip_pointwise_supported(const fhip_pointwise_desc *d) {
   if (!d || pointwise_validate(nullptr, d) != 0)
     return 0;
-  return 1;
+  return fhip_fast_pointwise_applicable(d) ? 2 : 1;
 }
 
 int fhip_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d, const void *in0,
@@ -998,6 +998,14 @@ int fhip_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d, const void *in0,
                  "fhip_pointwise: input %d pointer is null", i);
   FHIP_REQUIRE(ctx, out != nullptr, "fhip_pointwise: null output pointer");
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  {
+    // the vector kernel needs 16-byte aligned tensors
+    bool aligned = ((uintptr_t)out & 15) == 0;
+    for (int i = 0; i < d->num_inputs; ++i)
+      aligned = aligned && (d->in_is_scalar[i] || ((uintptr_t)ptr[i] & 15) == 0);
+    if (aligned && fhip_fast_pointwise_applicable(d))
+      return fhip_fast_pointwise(ctx, d, in0, in1, in2, out);
+  }
   PointwiseArgs g{};
   g.out = make_dims(d->out);
   g.os = make_strides(d->out);
