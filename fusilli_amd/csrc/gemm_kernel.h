@@ -882,13 +882,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
 #pragma unroll
               for (int c = 0; c < 8; ++c)
                 v[c] = (__bf16)y[c];
-              *(GEMM_AS1 bf16x8 *)dst = v;
+              __builtin_nontemporal_store(v, (GEMM_AS1 bf16x8 *)dst);
             } else if constexpr (OT == 2) {
               f16x8 v;
 #pragma unroll
               for (int c = 0; c < 8; ++c)
                 v[c] = (_Float16)y[c];
-              *(GEMM_AS1 f16x8 *)dst = v;
+              __builtin_nontemporal_store(v, (GEMM_AS1 f16x8 *)dst);
             } else {
               *(GEMM_AS1 u32x4 *)dst =
                   u32x4{__builtin_bit_cast(uint32_t, y[0]),

@@ -120,26 +120,28 @@ __device__ __forceinline__ void expand(const PwFastArgs &g, int i,
   }
 }
 
+// Streaming (nontemporal) stores: the output is not read again by this
+// kernel, and keeping it out of the caches' way measurably helps the reads.
 template <int DT>
 __device__ __forceinline__ void store8(void *out, int32_t vec,
                                        const float (&v)[8]) {
   if constexpr (DT == 0) {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     f32x4 *p = (f32x4 *)((char *)out + (int64_t)vec * 32);
-    p[0] = f32x4{v[0], v[1], v[2], v[3]};
-    p[1] = f32x4{v[4], v[5], v[6], v[7]};
+    __builtin_nontemporal_store(f32x4{v[0], v[1], v[2], v[3]}, p);
+    __builtin_nontemporal_store(f32x4{v[4], v[5], v[6], v[7]}, p + 1);
   } else if constexpr (DT == 1) {
     bf16x8 a;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       a[i] = (__bf16)v[i];
-    *(bf16x8 *)((char *)out + (int64_t)vec * 16) = a;
+    __builtin_nontemporal_store(a, (bf16x8 *)((char *)out + (int64_t)vec * 16));
   } else {
     f16x8 a;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       a[i] = (_Float16)v[i];
-    *(f16x8 *)((char *)out + (int64_t)vec * 16) = a;
+    __builtin_nontemporal_store(a, (f16x8 *)((char *)out + (int64_t)vec * 16));
   }
 }
 
