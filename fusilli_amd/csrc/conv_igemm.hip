@@ -24,6 +24,7 @@ struct ConvPlan {
   int64_t M = 0, N = 0, K = 0;
   ConvGeom geom{};
   int bm = 256, bn = 128;
+  bool halo = false;
 };
 
 // strides equal the dense channels-last strides of dims (unit dims are free)
@@ -157,6 +158,26 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
         (bn == 128 || bn == 256) && bm >= bn)
       p.bm = bm, p.bn = bn;
   }
+  // Halo mode (the slab of input pixels stays in LDS for all taps): unit
+  // stride, output extent == input extent, and a slab small enough that two
+  // workgroups still share a compute unit.  FUSILLI_HIP_CONV_HALO=0 / 1
+  // overrides the size rule (tests, tuning).
+  p.halo = false;
+  if (g.str_h == 1 && g.str_w == 1 && g.P == g.H && g.Q == g.W) {
+    const int64_t reach = (int64_t)(R - 1) * g.dil_h * g.W +
+                          (int64_t)(g.S - 1) * g.dil_w;
+    const int64_t rows = (128 + reach + 7) / 8 * 8;
+    const int64_t slab = rows * g.slices_per_tap * kTileKBytes + kTileKBytes;
+    const char *env = getenv("FUSILLI_HIP_CONV_HALO");
+    const bool fits = slab + kHaloRingBytes <= 160 * 1024;
+    const bool small = slab + kHaloRingBytes <= 80 * 1024;
+    if (fits && (env ? atoi(env) != 0 : small)) {
+      p.halo = true;
+      p.bm = p.bn = 128;
+      g.halo_rows = (int32_t)rows;
+      g.slab_bytes = (uint32_t)slab;
+    }
+  }
   p.ok = true;
   return p;
 }
@@ -165,6 +186,12 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
 
 int conv_launch_bf16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return conv_launch_kind<GK_BF16>(ctx, bm, bn, g);
+}
+int conv_launch_halo_bf16(fhip_ctx *ctx, const GemmArgs &g) {
+  return conv_launch_halo<GK_BF16>(ctx, g);
+}
+int conv_launch_halo_f16(fhip_ctx *ctx, const GemmArgs &g) {
+  return conv_launch_halo<GK_F16>(ctx, g);
 }
 int conv_launch_f16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return conv_launch_kind<GK_F16>(ctx, bm, bn, g);
@@ -216,6 +243,9 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     o.stride[2] = s.stride[1]; // per-channel step
   }
   gemm_fill_linear(d->epilogue, g);
+  if (p.halo)
+    return p.kind == GK_BF16 ? conv_launch_halo_bf16(ctx, g)
+                             : conv_launch_halo_f16(ctx, g);
   if (p.kind == GK_BF16)
     return conv_launch_bf16(ctx, p.bm, p.bn, g);
   return conv_launch_f16(ctx, p.bm, p.bn, g);

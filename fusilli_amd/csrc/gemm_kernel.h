@@ -101,6 +101,10 @@ struct ConvGeom {
   int32_t R;              // filter height
   // floor(2^32 / d) for d = Q, P, S, slices_per_tap (see conv_div)
   uint32_t magic_q, magic_p, magic_s, magic_spt;
+  // halo mode: rows (input pixels) of the LDS slab, a multiple of 8, and the
+  // slab's bytes including its trailing 128-byte row of zeros
+  int32_t halo_rows;
+  uint32_t slab_bytes;
 };
 
 // n / d for 0 <= n < 2^31 with magic = floor(2^32 / d): the estimate is at
@@ -117,7 +121,11 @@ __device__ __forceinline__ int32_t conv_div(int32_t n, int32_t d, uint32_t magic
   return q;
 }
 
-enum GemmAMode { A_KCONTIG = 0, A_MCONTIG = 1, A_CONV = 2 };
+// A_CONV gathers one filter tap per K slice from global memory.  A_HALO (unit
+// stride, output extent == input extent) loads the tile's input pixels and
+// their halo into LDS once; every tap then reads its fragments from that slab
+// at a shifted row, and only the filter streams through the stage ring.
+enum GemmAMode { A_KCONTIG = 0, A_MCONTIG = 1, A_CONV = 2, A_HALO = 3 };
 
 struct GemmArgs {
   ConvGeom conv;
@@ -449,7 +457,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   static_assert(WAVES_M * WAVES_N == NW, "wavefront grid");
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N; // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int LPS = GA::kLoads + GB::kLoads; // DMA instructions per slice
+  constexpr bool HALO = A_MODE == A_HALO;
+  static_assert(!HALO || (ELEM == 2 && B_KC && NW == 4), "halo mode: 16-bit, 4 waves");
+  // DMA instructions per slice
+  constexpr int LPS = (HALO ? 0 : GA::kLoads) + GB::kLoads;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
@@ -490,7 +501,37 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   int32_t cv_pix[A_MODE == A_CONV ? GA::kLoads : 1];
   uint32_t cv_mask[A_MODE == A_CONV ? GA::kLoads : 1];
   int cv_chunk = 0;
-  if constexpr (A_MODE == A_CONV) {
+  // halo mode: slab row of tap (0, 0) and the validity masks of this lane's
+  // fragment rows
+  int32_t h_row[HALO ? TM : 1];
+  uint32_t h_mask[HALO ? TM : 1];
+  if constexpr (HALO) {
+    a_base = g.a;
+    a_step = 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rt = wm * WM + i * 32 + (l & 31);
+      const int64_t m = m0 + rt;
+      const bool live = m < g.M;
+      const int32_t mm = (int32_t)(live ? m : 0);
+      const int32_t pq = conv_div(mm, g.conv.Q, g.conv.magic_q);
+      const int32_t q = mm - pq * g.conv.Q;
+      const int32_t nn = conv_div(pq, g.conv.P, g.conv.magic_p);
+      const int32_t ih0 = pq - nn * g.conv.P - g.conv.pad_h;
+      const int32_t iw0 = q - g.conv.pad_w;
+      uint32_t mask = 0;
+      for (int fr = 0; fr < g.conv.R; ++fr)
+        mask |= (uint32_t)(live && (uint32_t)(ih0 + fr * g.conv.dil_h) <
+                                       (uint32_t)g.conv.H)
+                << fr;
+      for (int fs = 0; fs < g.conv.S; ++fs)
+        mask |= (uint32_t)((uint32_t)(iw0 + fs * g.conv.dil_w) <
+                           (uint32_t)g.conv.W)
+                << (16 + fs);
+      h_row[i] = rt;
+      h_mask[i] = mask;
+    }
+  } else if constexpr (A_MODE == A_CONV) {
     a_base = g.a;
     a_step = 0;
 #pragma unroll
@@ -539,9 +580,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   }
   dma_setup<BN, ELEM, B_KC, NW>(b_ldb, n0, g.N, off_b);
 
-  auto stage_a = [&](int st) { return lds0 + (uint32_t)st * L::kStage; };
+  // halo mode: [slab | ring of B slices]; otherwise a ring of (A, B) slices
+  constexpr uint32_t STAGE = HALO ? GB::kBytes : L::kStage;
+  const uint32_t ring0 = HALO ? lds0 + g.conv.slab_bytes : lds0;
+  auto stage_a = [&](int st) { return ring0 + (uint32_t)st * STAGE; };
   auto stage_b = [&](int st) {
-    return lds0 + (uint32_t)st * L::kStage + GA::kBytes;
+    return ring0 + (uint32_t)st * STAGE + (HALO ? 0 : GA::kBytes);
   };
   // Part PART of PARTS of slice kt's loads (A and B split alike).
   // Slices past the end of K are "loaded" with zero-sized buffers: nothing
@@ -553,7 +597,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
     constexpr int PARTS = decltype(parts_c)::value;
     constexpr int A0 = PART * GA::kLoads / PARTS, A1 = (PART + 1) * GA::kLoads / PARTS;
     constexpr int B0 = PART * GB::kLoads / PARTS, B1 = (PART + 1) * GB::kLoads / PARTS;
-    if constexpr (A_MODE == A_CONV) {
+    if constexpr (HALO) {
+      // only the filter streams
+    } else if constexpr (A_MODE == A_CONV) {
       const int32_t tap = conv_div(kt, g.conv.slices_per_tap, g.conv.magic_spt);
       const int32_t cb =
           (kt - tap * g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
@@ -597,6 +643,39 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
         acc[i][j][r] = 0;
 
   // ---- prologue: fill all NSTAGE stages -------------------------------------
+  if constexpr (HALO) {
+    // Slab row r holds input pixel pix0 + r in the K-contiguous slice layout
+    // (one 128-byte channel run per slice); pixels before the tensor or past
+    // its end read as zeros, rows of other image lines are masked at use.
+    const int32_t pix0 =
+        (int32_t)m0 - g.conv.pad_h * g.conv.W - g.conv.pad_w;
+    const int32_t cbytes = g.conv.C * ELEM;
+    const int groups = g.conv.halo_rows / 8;
+    const uint64_t b64 = (uint64_t)a_base;
+    const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64);
+    const uint32_t bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(((uint64_t)bhi << 32) | blo), 0,
+        (int)__builtin_amdgcn_readfirstlane(g.conv.x_bytes), 0x00020000);
+    for (int sl = 0; sl < g.conv.slices_per_tap; ++sl)
+      for (int grp = __builtin_amdgcn_readfirstlane(wave); grp < groups;
+           grp += NW) {
+        const int row = grp * 8 + (l >> 3);
+        const int c = (l & 7) ^ kc_swz(row);
+        // modulo 2^32: pixels before the tensor wrap to offsets past its end
+        const uint32_t off = (uint32_t)(pix0 + row) * (uint32_t)cbytes +
+                             (uint32_t)(sl * kTileKBytes + c * 16);
+        const uint32_t dst =
+            lds0 + (uint32_t)(sl * g.conv.halo_rows + row - (l >> 3)) * kTileKBytes;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrc, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
+            (int)off, 0, 0, 0);
+      }
+    // the row of zeros that masked taps read
+    if (threadIdx.x < 8)
+      *(GEMM_AS3 u32x4 *)(uintptr_t)(ring0 - kTileKBytes + threadIdx.x * 16) =
+          u32x4{0, 0, 0, 0};
+  }
 #pragma unroll
   for (int p = 0; p < NSTAGE; ++p)
     issue(p, p, Zero{}, One{});
@@ -604,7 +683,41 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  fa_addr.template load<0>(stage_a(0), fa[0]);
+  // halo mode: per-tap fragment addresses (row base, swizzled chunk bits)
+  uint32_t h_base[HALO ? TM : 1], h_x[HALO ? TM : 1];
+  auto halo_tap = [&](int kt) {
+    const int32_t tap = conv_div(kt, g.conv.slices_per_tap, g.conv.magic_spt);
+    const int32_t sl = kt - tap * g.conv.slices_per_tap;
+    const int32_t fr = conv_div(tap, g.conv.S, g.conv.magic_s);
+    const int32_t fs = tap - fr * g.conv.S;
+    const int32_t dpix = fr * g.conv.dil_h * g.conv.W + fs * g.conv.dil_w;
+    const uint32_t slab = lds0 + (uint32_t)(sl * g.conv.halo_rows) * kTileKBytes;
+#pragma unroll
+    for (int i = 0; i < (HALO ? TM : 1); ++i) {
+      const bool in = (h_mask[i] >> fr) & (h_mask[i] >> (16 + fs)) & 1;
+      const int row = h_row[i] + dpix;
+      h_base[i] = in ? slab + (uint32_t)row * kTileKBytes : ring0 - kTileKBytes;
+      h_x[i] = (uint32_t)(((l >> 5) ^ kc_swz(row)) << 4);
+    }
+  };
+  auto halo_load = [&](auto ks_c, Frag<KIND> (&f)[TM]) {
+    constexpr int ks = decltype(ks_c)::value;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const u32x4 v = *(const GEMM_AS3 u32x4 *)(uintptr_t)(
+          h_base[i] + (h_x[i] ^ (uint32_t)(ks << 5)));
+      f[i].r[0] = v.x;
+      f[i].r[1] = v.y;
+      f[i].r[2] = v.z;
+      f[i].r[3] = v.w;
+    }
+  };
+  if constexpr (HALO) {
+    halo_tap(0);
+    halo_load(Zero{}, fa[0]);
+  } else {
+    fa_addr.template load<0>(stage_a(0), fa[0]);
+  }
   fb_addr.template load<0>(stage_b(0), fb[0]);
 
   // Reads per fragment set and the loads of a slice spread over the K-steps
@@ -708,7 +821,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
       constexpr int fc = s & 1, fn = fc ^ 1;
       constexpr bool LAST = s + 1 == KSTEPS;
       if constexpr (!LAST) {
-        fa_addr.template load<s + 1>(sa, fa[fn]);
+        if constexpr (HALO)
+          halo_load(std::integral_constant<int, s + 1>{}, fa[fn]);
+        else
+          fa_addr.template load<s + 1>(sa, fa[fn]);
         fb_addr.template load<s + 1>(sb, fb[fn]);
         if constexpr (s == 0)
           issue(kt + NSTAGE - 1, prv, One{}, Two{});
@@ -721,7 +837,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         __builtin_amdgcn_sched_barrier(0);
-        fa_addr.template load<0>(stage_a(nxt), fa[fn]);
+        if constexpr (HALO) {
+          halo_tap(kt + 1 < kt_count ? kt + 1 : kt);
+          halo_load(Zero{}, fa[fn]);
+        } else {
+          fa_addr.template load<0>(stage_a(nxt), fa[fn]);
+        }
         fb_addr.template load<0>(stage_b(nxt), fb[fn]);
         issue(kt + NSTAGE, cur, Zero{}, Two{});
       }
@@ -1149,6 +1270,28 @@ int conv_launch_kind(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   // two stages: two workgroups share a compute unit, and one's prologue and
   // epilogue hide behind the other's K loop (convolutions have short K)
   return launch<KIND, 128, 128, A_CONV, true, 2>(ctx, g, 1);
+}
+
+// Halo mode: 128 x 128 tiles, three filter stages behind the slab.
+constexpr int kHaloStages = 3;
+constexpr int kHaloRingBytes = kHaloStages * 128 * kTileKBytes;
+template <int KIND> int conv_launch_halo(fhip_ctx *ctx, const GemmArgs &g) {
+  using L = GemmLds<128, 128, kHaloStages, 4>;
+  const int main_bytes = (int)g.conv.slab_bytes + kHaloRingBytes;
+  const int lds = main_bytes > L::kEpiBytes ? main_bytes : L::kEpiBytes;
+  auto kernel = gemm_kernel<KIND, 128, 128, A_HALO, true, kHaloStages, 4>;
+  static bool configured = false;
+  if (!configured) {
+    FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
+                            reinterpret_cast<const void *>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024));
+    configured = true;
+  }
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1);
+  hipLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, g);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
 }
 
 int gemm_launch_bf16(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g);

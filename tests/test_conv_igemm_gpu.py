@@ -77,6 +77,7 @@ def test_conv_igemm_random_vs_oracle(ctx, case, dtype):
 @pytest.mark.parametrize("tile", ["128,128", "256,128", "256,256", "512,128"])
 def test_conv_igemm_every_tile_shape(ctx, tile, monkeypatch):
     monkeypatch.setenv("FUSILLI_HIP_CONV_TILE", tile)
+    monkeypatch.setenv("FUSILLI_HIP_CONV_HALO", "0")  # the gather kernel's tiles
     case = dict(x=[2, 64, 15, 17], w=[300, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1])
     x = cl(case["x"], 42, 0, capi.BFLOAT16)
     w = cl(case["w"], 42, 1, capi.BFLOAT16, std=0.1)
@@ -85,6 +86,39 @@ def test_conv_igemm_every_tile_shape(ctx, tile, monkeypatch):
                             case["d"])
     # f32 result of bf16 inputs: only the accumulation order differs
     assert_close(out.logical(), ref, capi.FLOAT, tile, rtol=1e-4)
+
+
+SAME_CASES = [
+    # unit stride, output extent == input extent: eligible for the halo kernel
+    dict(x=[2, 64, 14, 14], w=[128, 64, 3, 3], pad=[1, 1], d=[1, 1]),
+    # ragged M (3*9*11 = 297 pixels: 2 full tiles + 41 rows), ragged K_out > 128
+    dict(x=[3, 64, 9, 11], w=[200, 64, 3, 3], pad=[1, 1], d=[1, 1]),
+    # dilation 2 (reach 2 rows + 2 pixels either side)
+    dict(x=[1, 64, 12, 10], w=[64, 64, 3, 3], pad=[2, 2], d=[2, 2]),
+    # 5x5, C = 128 (two K slices per tap)
+    dict(x=[1, 128, 9, 9], w=[48, 128, 5, 5], pad=[2, 2], d=[1, 1]),
+    # asymmetric filter 1x3 and 3x1
+    dict(x=[2, 64, 8, 16], w=[32, 64, 1, 3], pad=[0, 1], d=[1, 1]),
+    dict(x=[2, 64, 16, 8], w=[32, 64, 3, 1], pad=[1, 0], d=[1, 1]),
+    # 1x1 (no halo at all) and 1-D
+    dict(x=[2, 64, 10, 13], w=[136, 64, 1, 1], pad=[0, 0], d=[1, 1]),
+    dict(x=[3, 64, 70], w=[48, 64, 5], pad=[2], d=[1]),
+    # image narrower than the filter reach
+    dict(x=[4, 64, 2, 3], w=[16, 64, 3, 3], pad=[1, 1], d=[1, 1]),
+]
+
+
+@pytest.mark.parametrize("case", SAME_CASES)
+@pytest.mark.parametrize("halo", ["1", "0"])
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_conv_same_geometry_halo_and_gather(ctx, case, halo, dtype, monkeypatch):
+    monkeypatch.setenv("FUSILLI_HIP_CONV_HALO", halo)
+    st = [1] * len(case["pad"])
+    x = cl(case["x"], 46, 0, dtype)
+    w = cl(case["w"], 46, 1, dtype, std=0.1)
+    out = run(ctx, x, w, case["pad"], st, case["d"], capi.FLOAT)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], st, case["d"])
+    assert_close(out.logical(), ref, capi.FLOAT, f"halo={halo} {case}", rtol=1e-4)
 
 
 def test_conv_igemm_bias_relu_residual(ctx):
