@@ -25,6 +25,7 @@ struct ConvPlan {
   ConvGeom geom{};
   int bm = 256, bn = 128;
   bool halo = false;
+  int tile_rows = 0; // halo mode: rows per M tile (<= bm)
 };
 
 // strides equal the dense channels-last strides of dims (unit dims are free)
@@ -166,16 +167,45 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
   if (g.str_h == 1 && g.str_w == 1 && g.P == g.H && g.Q == g.W) {
     const int64_t reach = (int64_t)(R - 1) * g.dil_h * g.W +
                           (int64_t)(g.S - 1) * g.dil_w;
-    const int64_t rows = (128 + reach + 7) / 8 * 8;
-    const int64_t slab = rows * g.slices_per_tap * kTileKBytes + kTileKBytes;
+    auto slab_of = [&](int bm) {
+      const int64_t rows = (bm + reach + 7) / 8 * 8;
+      return rows * g.slices_per_tap * kTileKBytes + kTileKBytes;
+    };
     const char *env = getenv("FUSILLI_HIP_CONV_HALO");
-    const bool fits = slab + kHaloRingBytes <= 160 * 1024;
-    const bool small = slab + kHaloRingBytes <= 80 * 1024;
-    if (fits && (env ? atoi(env) != 0 : small)) {
+    const int want = env ? atoi(env) : -1; // 0 off, 128 / 256 tile, else auto
+    const bool fits128 = slab_of(128) + HaloShape<128>::kRingBytes <= 160 * 1024;
+    const bool small128 = slab_of(128) + HaloShape<128>::kRingBytes <= 80 * 1024;
+    const bool small256 = slab_of(256) + HaloShape<256>::kRingBytes <= 80 * 1024;
+    // 256-row tiles when the output has enough pixels to give every slot
+    // (two workgroups per compute unit) a tile of at least 160 rows
+    const int64_t slots = 2 * 256;
+    const bool big = p.M * ((p.N + 127) / 128) >= 160 * slots;
+    int bm = 0;
+    if (want == 0)
+      bm = 0;
+    else if (want == 256)
+      bm = small256 ? 256 : 0;
+    else if (want > 0)
+      bm = fits128 ? 128 : 0;
+    else
+      bm = small256 && big ? 256 : (small128 ? 128 : 0);
+    if (bm) {
       p.halo = true;
-      p.bm = p.bn = 128;
+      p.bm = bm;
+      p.bn = 128;
+      const int64_t rows = (bm + reach + 7) / 8 * 8;
       g.halo_rows = (int32_t)rows;
-      g.slab_bytes = (uint32_t)slab;
+      g.slab_bytes = (uint32_t)slab_of(bm);
+      // Tile height that spreads the pixels evenly over whole rounds of the
+      // machine's slots (C3: 100352 pixels -> 512 tiles of 196 rows).
+      p.tile_rows = bm;
+      if (bm == 256) {
+        const int64_t tn = (p.N + 127) / 128;
+        const int64_t per_round = slots / tn > 0 ? slots / tn : 1;
+        const int64_t rounds = (p.M + 256 * per_round - 1) / (256 * per_round);
+        const int64_t tiles = rounds * per_round;
+        p.tile_rows = (int)((p.M + tiles - 1) / tiles);
+      }
     }
   }
   p.ok = true;
@@ -187,11 +217,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
 int conv_launch_bf16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return conv_launch_kind<GK_BF16>(ctx, bm, bn, g);
 }
-int conv_launch_halo_bf16(fhip_ctx *ctx, const GemmArgs &g) {
-  return conv_launch_halo<GK_BF16>(ctx, g);
-}
-int conv_launch_halo_f16(fhip_ctx *ctx, const GemmArgs &g) {
-  return conv_launch_halo<GK_F16>(ctx, g);
+template <int KIND>
+int conv_launch_halo_bm(fhip_ctx *ctx, int bm, const GemmArgs &g) {
+  return bm == 256 ? conv_launch_halo<KIND, 256>(ctx, g)
+                   : conv_launch_halo<KIND, 128>(ctx, g);
 }
 int conv_launch_f16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return conv_launch_kind<GK_F16>(ctx, bm, bn, g);
@@ -223,7 +252,8 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   g.o_batch = 0;
   g.c_dt = d->y.dtype;
   g.o_dt = d->out.dtype;
-  g.tiles_m = (int)((p.M + p.bm - 1) / p.bm);
+  g.tile_rows = p.halo ? p.tile_rows : p.bm;
+  g.tiles_m = (int)((p.M + g.tile_rows - 1) / g.tile_rows);
   g.tiles_n = (int)((p.N + p.bn - 1) / p.bn);
   g.o_vec = (p.N * fhip_dtype_size(d->out.dtype)) % 16 == 0 &&
             ((uintptr_t)out & 15) == 0;
@@ -244,8 +274,8 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   }
   gemm_fill_linear(d->epilogue, g);
   if (p.halo)
-    return p.kind == GK_BF16 ? conv_launch_halo_bf16(ctx, g)
-                             : conv_launch_halo_f16(ctx, g);
+    return p.kind == GK_BF16 ? conv_launch_halo_bm<GK_BF16>(ctx, p.bm, g)
+                             : conv_launch_halo_bm<GK_F16>(ctx, p.bm, g);
   if (p.kind == GK_BF16)
     return conv_launch_bf16(ctx, p.bm, p.bn, g);
   return conv_launch_f16(ctx, p.bm, p.bn, g);

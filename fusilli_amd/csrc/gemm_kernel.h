@@ -139,6 +139,9 @@ struct GemmArgs {
   int64_t o_sm, o_sn, o_batch; // output strides in elements
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
+  // rows of an M tile that are computed and stored (0: all BM); a smaller
+  // value lets the host match the tile count to the machine
+  int32_t tile_rows;
   int32_t o_vec;              // output rows allow aligned 16-byte stores
   // Epilogue applied to the accumulators in registers: every op is one of
   // ADD / SUB / MUL / RELU / NEG / IDENTITY with a scalar or per-column
@@ -425,7 +428,7 @@ template <int BM, int BN> struct GemmLayout {
   static constexpr int kWaves = kWavesM * kWavesN;
 };
 
-template <int BM, int BN, int NSTAGE, int NW> struct GemmLds {
+template <int BM, int BN, int NSTAGE, int NW, bool HALO = false> struct GemmLds {
   static constexpr int kStage = (BM + BN) * kTileKBytes;
   static constexpr int kWN = BN / GemmLayout<BM, BN>::kWavesN; // wave columns
   static constexpr int kEpiPitch = kWN * 4 + 32;
@@ -433,7 +436,8 @@ template <int BM, int BN, int NSTAGE, int NW> struct GemmLds {
   static constexpr int kTM = BM / GemmLayout<BM, BN>::kWavesM / 32;
   // tile rows that leave together: as many as fit 160 KB, or 80 KB where the
   // stages leave room for two workgroups per compute unit
-  static constexpr int kCap = NSTAGE * kStage <= 80 * 1024 ? 80 * 1024 : 160 * 1024;
+  static constexpr int kCap =
+      HALO || NSTAGE * kStage <= 80 * 1024 ? 80 * 1024 : 160 * 1024;
   static constexpr int kBands =
       NW * kTM * kBand <= kCap ? kTM : (NW * 2 * kBand <= kCap ? 2 : 1);
   static constexpr int kEpiBytes = NW * kBands * kBand;
@@ -441,8 +445,12 @@ template <int BM, int BN, int NSTAGE, int NW> struct GemmLds {
       NSTAGE * kStage > kEpiBytes ? NSTAGE * kStage : kEpiBytes;
 };
 
+// Halo kernels are laid out for two workgroups per compute unit (two
+// wavefronts per SIMD): at most 256 registers per lane.
 template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int NSTAGE, int NW>
-__global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
+__global__ __launch_bounds__(NW * 64)
+__attribute__((amdgpu_waves_per_eu(A_MODE == A_HALO ? 2 : 1, 8))) void
+gemm_kernel(GemmArgs g) {
   using Acc = typename KindTraits<KIND>::Acc;
   constexpr bool A_KC = A_MODE != A_MCONTIG;
   constexpr int ELEM = KindTraits<KIND>::kElemBytes;
@@ -451,7 +459,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   static_assert(KSTEPS % 2 == 0, "fragment double buffering needs even KSTEPS");
   using GA = SliceGeom<BM, ELEM, A_KC, NW>;
   using GB = SliceGeom<BN, ELEM, B_KC, NW>;
-  using L = GemmLds<BM, BN, NSTAGE, NW>;
+  using L = GemmLds<BM, BN, NSTAGE, NW, A_MODE == A_HALO>;
   constexpr int WAVES_M = GemmLayout<BM, BN>::kWavesM;
   constexpr int WAVES_N = GemmLayout<BM, BN>::kWavesN;
   static_assert(WAVES_M * WAVES_N == NW, "wavefront grid");
@@ -483,7 +491,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   const int tile_n = (pid % per_group) / group_rows;
   const int64_t batch = blockIdx.y;
 
-  const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+  const int tile_rows = g.tile_rows ? g.tile_rows : BM;
+  const int64_t m0 = (int64_t)tile_m * tile_rows, n0 = (int64_t)tile_n * BN;
+  // first row past this tile's share of the output
+  const int64_t m_end = m0 + tile_rows < g.M ? m0 + tile_rows : g.M;
   const int64_t a_ldb = g.a_ld * ELEM, b_ldb = g.b_ld * ELEM;
   const int kt_count = (int)(g.K * ELEM / kTileKBytes);
 
@@ -512,7 +523,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
     for (int i = 0; i < TM; ++i) {
       const int rt = wm * WM + i * 32 + (l & 31);
       const int64_t m = m0 + rt;
-      const bool live = m < g.M;
+      const bool live = m < m_end;
       const int32_t mm = (int32_t)(live ? m : 0);
       const int32_t pq = conv_div(mm, g.conv.Q, g.conv.magic_q);
       const int32_t q = mm - pq * g.conv.Q;
@@ -538,7 +549,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
     for (int j = 0; j < GA::kLoads; ++j) {
       const int row = (j * NW + wave) * 8 + (l >> 3);
       const int64_t m = m0 + row;
-      const bool live = m < g.M;
+      const bool live = m < m_end;
       const int32_t mm = (int32_t)(live ? m : 0);
       const int32_t pq = conv_div(mm, g.conv.Q, g.conv.magic_q);
       const int32_t q = mm - pq * g.conv.Q;
@@ -563,11 +574,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   } else if constexpr (A_KC) {
     a_base = g.a + batch * g.a_batch * ELEM + m0 * a_ldb;
     a_step = kTileKBytes;
-    dma_setup<BM, ELEM, true, NW>(a_ldb, m0, g.M, off_a);
+    dma_setup<BM, ELEM, true, NW>(a_ldb, m0, m_end, off_a);
   } else {
     a_base = g.a + batch * g.a_batch * ELEM + m0 * ELEM;
     a_step = (int64_t)GA::kKRows * a_ldb;
-    dma_setup<BM, ELEM, false, NW>(a_ldb, m0, g.M, off_a);
+    dma_setup<BM, ELEM, false, NW>(a_ldb, m0, m_end, off_a);
   }
   const char *b_base;
   int64_t b_step;
@@ -886,9 +897,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   const bool lane_full = ncol + 8 <= g.N || ncol >= g.N;
   const bool lean = g.epi_reg && g.o_vec != 0 &&
                     __builtin_amdgcn_ballot_w64(!lane_full) == 0;
-  // Per op and column y <- y * S + T: (S, T) = (a, b * operand) for the
-  // additive modes and (operand, -0) for MUL.
-  float S[FHIP_MAX_EPILOGUE][8], T[FHIP_MAX_EPILOGUE][8];
+  // Per op and column: MUL is y <- y * V with V the operand; the additive
+  // modes are y <- a * y + V with V = b * operand.
+  float V[FHIP_MAX_EPILOGUE][8];
   if constexpr (!std::is_same<Acc, int>::value) {
     if (lean) {
       gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
@@ -911,13 +922,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
           for (int c = 0; c < 8; ++c)
             ov[c] = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
         }
-        const bool mul = g.lin_mul[e] != 0;
-        const float a = g.lin_a[e], b = g.lin_b[e];
+        const float b = g.lin_mul[e] ? 1.f : g.lin_b[e];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          S[e][c] = mul ? ov[c] : a;
-          T[e][c] = mul ? -0.f : b * ov[c];
-        }
+        for (int c = 0; c < 8; ++c)
+          V[e][c] = b * ov[c];
       });
       // The operands are in registers from here on: no pass may wait on the
       // memory counter, which the stores of earlier passes share.
@@ -928,10 +936,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
           return;
 #pragma unroll
         for (int c = 0; c < 8; ++c)
-{
-          gemm_pin(S[e][c]);
-          gemm_pin(T[e][c]);
-        }
+          gemm_pin(V[e][c]);
       });
     }
   }
@@ -942,12 +947,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
   const int64_t lean_m = m0 + wm * WM + l / LPR;
   const int64_t row_bytes = g.o_sm * esz;
   const int nops = g.epi.count;
-  const int64_t gM = g.M, gN = g.N;
+  const int64_t gM = m_end, gN = g.N;
   const int o_dt = g.o_dt;
-  int lin_relu[FHIP_MAX_EPILOGUE];
+  int lin_relu[FHIP_MAX_EPILOGUE], lin_mul[FHIP_MAX_EPILOGUE];
+  float lin_a[FHIP_MAX_EPILOGUE];
   gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
     constexpr int e = decltype(ec)::value;
     lin_relu[e] = g.lin_relu[e];
+    lin_mul[e] = g.lin_mul[e];
+    lin_a[e] = g.lin_a[e];
   });
 
   gemm_static_for<TM / BANDS>([&](auto rc) {
@@ -989,9 +997,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
               constexpr int e = decltype(ec)::value;
               if (e >= nops)
                 return;
+              if (lin_mul[e]) {
 #pragma unroll
-              for (int c = 0; c < 8; ++c)
-                y[c] = __builtin_fmaf(y[c], S[e][c], T[e][c]);
+                for (int c = 0; c < 8; ++c)
+                  y[c] *= V[e][c];
+              } else {
+                const float a = lin_a[e];
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+                  y[c] = __builtin_fmaf(a, y[c], V[e][c]);
+              }
               if (lin_relu[e]) {
 #pragma unroll
                 for (int c = 0; c < 8; ++c)
@@ -1045,7 +1060,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_kernel(GemmArgs g) {
       const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
       const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
       const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
-      if (m >= g.M || ncol >= g.N)
+      if (m >= m_end || ncol >= g.N)
         continue;
       const bool full = ncol + 8 <= g.N;
       const int64_t o0 = ob + m * g.o_sm + ncol * g.o_sn;
@@ -1272,14 +1287,21 @@ int conv_launch_kind(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return launch<KIND, 128, 128, A_CONV, true, 2>(ctx, g, 1);
 }
 
-// Halo mode: 128 x 128 tiles, three filter stages behind the slab.
-constexpr int kHaloStages = 3;
-constexpr int kHaloRingBytes = kHaloStages * 128 * kTileKBytes;
-template <int KIND> int conv_launch_halo(fhip_ctx *ctx, const GemmArgs &g) {
-  using L = GemmLds<128, 128, kHaloStages, 4>;
-  const int main_bytes = (int)g.conv.slab_bytes + kHaloRingBytes;
+// Halo mode: 128 x 128 tiles with three filter stages behind the slab, or
+// 256 x 128 tiles with two.
+template <int BM> struct HaloShape {
+  static constexpr int kStages = BM == 256 ? 2 : 3;
+  static constexpr int kRingBytes = kStages * 128 * kTileKBytes;
+};
+template <int KIND, int BM>
+int conv_launch_halo(fhip_ctx *ctx, const GemmArgs &g) {
+  constexpr int STAGES = HaloShape<BM>::kStages;
+  using L = GemmLds<BM, 128, STAGES, 4, true>;
+  const int main_bytes = (int)g.conv.slab_bytes + HaloShape<BM>::kRingBytes;
+  // (the epilogue's bands stay within 80 KB so that two workgroups keep
+  // sharing a compute unit)
   const int lds = main_bytes > L::kEpiBytes ? main_bytes : L::kEpiBytes;
-  auto kernel = gemm_kernel<KIND, 128, 128, A_HALO, true, kHaloStages, 4>;
+  auto kernel = gemm_kernel<KIND, BM, 128, A_HALO, true, STAGES, 4>;
   static bool configured = false;
   if (!configured) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(

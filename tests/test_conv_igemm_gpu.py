@@ -109,7 +109,7 @@ SAME_CASES = [
 
 
 @pytest.mark.parametrize("case", SAME_CASES)
-@pytest.mark.parametrize("halo", ["1", "0"])
+@pytest.mark.parametrize("halo", ["128", "256", "0"])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
 def test_conv_same_geometry_halo_and_gather(ctx, case, halo, dtype, monkeypatch):
     monkeypatch.setenv("FUSILLI_HIP_CONV_HALO", halo)
