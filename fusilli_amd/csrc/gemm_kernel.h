@@ -897,49 +897,6 @@ gemm_kernel(GemmArgs g) {
   const bool lane_full = ncol + 8 <= g.N || ncol >= g.N;
   const bool lean = g.epi_reg && g.o_vec != 0 &&
                     __builtin_amdgcn_ballot_w64(!lane_full) == 0;
-  // Per op and column: MUL is y <- y * V with V the operand; the additive
-  // modes are y <- a * y + V with V = b * operand.
-  float V[FHIP_MAX_EPILOGUE][8];
-  if constexpr (!std::is_same<Acc, int>::value) {
-    if (lean) {
-      gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
-        constexpr int e = decltype(ec)::value;
-        if (e >= g.epi.count)
-          return;
-        const DevEpiOp &o = g.epi.op[e];
-        float ov[8];
-        if (o.kind == FHIP_OPERAND_TENSOR) {
-          int64_t off[8];
-#pragma unroll
-          for (int c = 0; c < 8; ++c) {
-            int64_t n = ncol + c;
-            n = n < g.N ? n : g.N - 1;
-            off[c] = n * o.stride[2];
-          }
-          load_operand_vec<8>(o.ptr, o.operand_dtype, off, ov);
-        } else {
-#pragma unroll
-          for (int c = 0; c < 8; ++c)
-            ov[c] = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
-        }
-        const float b = g.lin_mul[e] ? 1.f : g.lin_b[e];
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-          V[e][c] = b * ov[c];
-      });
-      // The operands are in registers from here on: no pass may wait on the
-      // memory counter, which the stores of earlier passes share.
-      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
-      gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
-        constexpr int e = decltype(ec)::value;
-        if (e >= g.epi.count)
-          return;
-#pragma unroll
-        for (int c = 0; c < 8; ++c)
-          gemm_pin(V[e][c]);
-      });
-    }
-  }
   const int64_t esz = fhip_dtype_size(g.o_dt);
   GEMM_AS1 char *lean_ptr =
       (GEMM_AS1 char *)g.out +
@@ -949,17 +906,140 @@ gemm_kernel(GemmArgs g) {
   const int nops = g.epi.count;
   const int64_t gM = m_end, gN = g.N;
   const int o_dt = g.o_dt;
-  int lin_relu[FHIP_MAX_EPILOGUE], lin_mul[FHIP_MAX_EPILOGUE];
-  float lin_a[FHIP_MAX_EPILOGUE];
-  gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
-    constexpr int e = decltype(ec)::value;
-    lin_relu[e] = g.lin_relu[e];
-    lin_mul[e] = g.lin_mul[e];
-    lin_a[e] = g.lin_a[e];
-  });
+
+  // Lean path, step 1: the chain runs on the accumulators where they are.  A
+  // lane's accumulators of column tile j all belong to one output column, so
+  // an op is y <- y * S + T with one (S, T) pair of registers per (op, j):
+  // (operand, -0) for MUL, (a, b * operand) for the additive modes.
+  if constexpr (!std::is_same<Acc, int>::value) {
+    if (lean && nops > 0) {
+      float S[FHIP_MAX_EPILOGUE][TN], T[FHIP_MAX_EPILOGUE][TN];
+      int lin_relu[FHIP_MAX_EPILOGUE];
+      gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        lin_relu[e] = g.lin_relu[e];
+        if (e >= nops)
+          return;
+        const DevEpiOp &o = g.epi.op[e];
+        const bool mul = g.lin_mul[e] != 0;
+        const float a = g.lin_a[e], b = g.lin_b[e];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          float ov;
+          if (o.kind == FHIP_OPERAND_TENSOR) {
+            int64_t n = n0 + wn * WN + j * 32 + (l & 31);
+            n = n < gN ? n : gN - 1;
+            const int64_t off[1] = {n * o.stride[2]};
+            float one[1];
+            load_operand_vec<1>(o.ptr, o.operand_dtype, off, one);
+            ov = one[0];
+          } else {
+            ov = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
+          }
+          S[e][j] = mul ? ov : a;
+          T[e][j] = mul ? -0.f : b * ov;
+        }
+      });
+      gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
+        constexpr int e = decltype(ec)::value;
+        if (e >= nops)
+          return;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              acc[i][j][r] = __builtin_fmaf(acc[i][j][r], S[e][j], T[e][j]);
+        if (lin_relu[e]) {
+          // one instruction per value (fmaxf would first quiet its input);
+          // NaN -> 0 like fmaxf
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                float y = acc[i][j][r];
+                asm("v_max_f32 %0, 0, %0" : "+v"(y));
+                acc[i][j][r] = y;
+              }
+        }
+      });
+    }
+  }
+  // Step 2, 16-bit outputs: the values are rounded here and leave through LDS
+  // as packed pairs of consecutive rows (half the LDS traffic and passes).
+  const bool packed = !std::is_same<Acc, int>::value && lean &&
+                      (o_dt == FHIP_BFLOAT16 || o_dt == FHIP_HALF);
+  const uint32_t wr2 = band + (uint32_t)((l >> 5) * 2 * PITCH + (l & 31) * 4);
 
   gemm_static_for<TM / BANDS>([&](auto rc) {
     constexpr int round = decltype(rc)::value;
+    if constexpr (!std::is_same<Acc, int>::value) {
+      if (packed) {
+        // pair-row k of a band holds rows 2k and 2k + 1 as (low, high) halves
+        auto run = [&](auto ot_c) {
+          constexpr int OT = decltype(ot_c)::value; // 1 bf16, 2 f16
+#pragma unroll
+          for (int bi = 0; bi < BANDS; ++bi)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+              for (int r = 0; r < 16; r += 2) {
+                const float lo = acc[round * BANDS + bi][j][r];
+                const float hi = acc[round * BANDS + bi][j][r + 1];
+                uint32_t pk;
+                if constexpr (OT == 1) {
+                  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+                  pk = __builtin_bit_cast(uint32_t, b2{(__bf16)lo, (__bf16)hi});
+                } else {
+                  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+                  pk = __builtin_bit_cast(uint32_t,
+                                          h2{(_Float16)lo, (_Float16)hi});
+                }
+                *(GEMM_AS3 uint32_t *)(uintptr_t)(
+                    wr2 + bi * L::kBand +
+                    ((r >> 2) * 4 + ((r & 3) >> 1)) * PITCH + j * 128) = pk;
+              }
+          // a pass covers RPP pair-rows = 2 * RPP rows
+          constexpr int PPB2 = 16 / RPP;
+#pragma unroll
+          for (int p = 0; p < BANDS * PPB2; ++p) {
+            const int bi = p / PPB2, pp = p % PPB2;
+            const int rel = (round * BANDS + bi) * 32 + pp * 2 * RPP;
+            const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
+            const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
+            const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
+            // lane's rows: lean_m' = tile row of pair-row (l / LPR)
+            const int64_t mrow = m0 + wm * WM + rel + 2 * (l / LPR);
+            if (ncol >= gN || mrow >= gM)
+              continue;
+            GEMM_AS1 char *dst =
+                (GEMM_AS1 char *)g.out + (ob + mrow * g.o_sm + ncol) * 2;
+            const u32x4 even = {
+                __builtin_amdgcn_perm(v0.y, v0.x, 0x05040100u),
+                __builtin_amdgcn_perm(v0.w, v0.z, 0x05040100u),
+                __builtin_amdgcn_perm(v1.y, v1.x, 0x05040100u),
+                __builtin_amdgcn_perm(v1.w, v1.z, 0x05040100u)};
+            const u32x4 odd = {
+                __builtin_amdgcn_perm(v0.y, v0.x, 0x07060302u),
+                __builtin_amdgcn_perm(v0.w, v0.z, 0x07060302u),
+                __builtin_amdgcn_perm(v1.y, v1.x, 0x07060302u),
+                __builtin_amdgcn_perm(v1.w, v1.z, 0x07060302u)};
+            __builtin_nontemporal_store(even, (GEMM_AS1 u32x4 *)dst);
+            if (mrow + 1 < gM)
+              __builtin_nontemporal_store(odd,
+                                          (GEMM_AS1 u32x4 *)(dst + row_bytes));
+          }
+        };
+        if (o_dt == FHIP_BFLOAT16)
+          run(std::integral_constant<int, 1>{});
+        else
+          run(std::integral_constant<int, 2>{});
+        return;
+      }
+    }
 #pragma unroll
     for (int bi = 0; bi < BANDS; ++bi)
 #pragma unroll
@@ -970,85 +1050,19 @@ gemm_kernel(GemmArgs g) {
                                        ((r >> 2) * 8 + (r & 3)) * PITCH +
                                        j * 128) = acc[round * BANDS + bi][j][r];
     if (lean) {
-      // OT: 0 float, 1 bf16, 2 f16 output
-      auto passes = [&](auto ot_c) {
-        constexpr int OT = decltype(ot_c)::value;
+      // 4-byte outputs (the chain has already run on the accumulators)
 #pragma unroll
-        for (int p = 0; p < BANDS * PPB; ++p) {
-          const int bi = p / PPB, pp = p % PPB;
-          const int rel = (round * BANDS + bi) * 32 + pp * RPP;
-          const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
-          const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
-          const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
-          if (lean_m + rel >= gM || ncol >= gN)
-            continue;
-          GEMM_AS1 char *dst = lean_ptr + rel * row_bytes;
-          if constexpr (std::is_same<Acc, int>::value) {
-            *(GEMM_AS1 u32x4 *)dst = v0;
-            *(GEMM_AS1 u32x4 *)(dst + 16) = v1;
-          } else {
-            const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w,
-                                   v1.x, v1.y, v1.z, v1.w};
-            float y[8];
-#pragma unroll
-            for (int c = 0; c < 8; ++c)
-              y[c] = __builtin_bit_cast(float, w[c]);
-            gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
-              constexpr int e = decltype(ec)::value;
-              if (e >= nops)
-                return;
-              if (lin_mul[e]) {
-#pragma unroll
-                for (int c = 0; c < 8; ++c)
-                  y[c] *= V[e][c];
-              } else {
-                const float a = lin_a[e];
-#pragma unroll
-                for (int c = 0; c < 8; ++c)
-                  y[c] = __builtin_fmaf(a, y[c], V[e][c]);
-              }
-              if (lin_relu[e]) {
-#pragma unroll
-                for (int c = 0; c < 8; ++c)
-                  y[c] = fmaxf(y[c], 0.f);
-              }
-            });
-            if constexpr (OT == 1) {
-              bf16x8 v;
-#pragma unroll
-              for (int c = 0; c < 8; ++c)
-                v[c] = (__bf16)y[c];
-              __builtin_nontemporal_store(v, (GEMM_AS1 bf16x8 *)dst);
-            } else if constexpr (OT == 2) {
-              f16x8 v;
-#pragma unroll
-              for (int c = 0; c < 8; ++c)
-                v[c] = (_Float16)y[c];
-              __builtin_nontemporal_store(v, (GEMM_AS1 f16x8 *)dst);
-            } else {
-              *(GEMM_AS1 u32x4 *)dst =
-                  u32x4{__builtin_bit_cast(uint32_t, y[0]),
-                        __builtin_bit_cast(uint32_t, y[1]),
-                        __builtin_bit_cast(uint32_t, y[2]),
-                        __builtin_bit_cast(uint32_t, y[3])};
-              *(GEMM_AS1 u32x4 *)(dst + 16) =
-                  u32x4{__builtin_bit_cast(uint32_t, y[4]),
-                        __builtin_bit_cast(uint32_t, y[5]),
-                        __builtin_bit_cast(uint32_t, y[6]),
-                        __builtin_bit_cast(uint32_t, y[7])};
-            }
-          }
-        }
-      };
-      if constexpr (std::is_same<Acc, int>::value) {
-        passes(std::integral_constant<int, 0>{});
-      } else {
-        if (o_dt == FHIP_BFLOAT16)
-          passes(std::integral_constant<int, 1>{});
-        else if (o_dt == FHIP_HALF)
-          passes(std::integral_constant<int, 2>{});
-        else
-          passes(std::integral_constant<int, 0>{});
+      for (int p = 0; p < BANDS * PPB; ++p) {
+        const int bi = p / PPB, pp = p % PPB;
+        const int rel = (round * BANDS + bi) * 32 + pp * RPP;
+        const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
+        const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
+        const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
+        if (lean_m + rel >= gM || ncol >= gN)
+          continue;
+        GEMM_AS1 char *dst = lean_ptr + rel * row_bytes;
+        *(GEMM_AS1 u32x4 *)dst = v0;
+        *(GEMM_AS1 u32x4 *)(dst + 16) = v1;
       }
       return;
     }
