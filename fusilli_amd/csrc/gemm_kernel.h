@@ -519,29 +519,6 @@ gemm_kernel(GemmArgs g) {
   if constexpr (HALO) {
     a_base = g.a;
     a_step = 0;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int rt = wm * WM + i * 32 + (l & 31);
-      const int64_t m = m0 + rt;
-      const bool live = m < m_end;
-      const int32_t mm = (int32_t)(live ? m : 0);
-      const int32_t pq = conv_div(mm, g.conv.Q, g.conv.magic_q);
-      const int32_t q = mm - pq * g.conv.Q;
-      const int32_t nn = conv_div(pq, g.conv.P, g.conv.magic_p);
-      const int32_t ih0 = pq - nn * g.conv.P - g.conv.pad_h;
-      const int32_t iw0 = q - g.conv.pad_w;
-      uint32_t mask = 0;
-      for (int fr = 0; fr < g.conv.R; ++fr)
-        mask |= (uint32_t)(live && (uint32_t)(ih0 + fr * g.conv.dil_h) <
-                                       (uint32_t)g.conv.H)
-                << fr;
-      for (int fs = 0; fs < g.conv.S; ++fs)
-        mask |= (uint32_t)((uint32_t)(iw0 + fs * g.conv.dil_w) <
-                           (uint32_t)g.conv.W)
-                << (16 + fs);
-      h_row[i] = rt;
-      h_mask[i] = mask;
-    }
   } else if constexpr (A_MODE == A_CONV) {
     a_base = g.a;
     a_step = 0;
@@ -690,6 +667,33 @@ gemm_kernel(GemmArgs g) {
 #pragma unroll
   for (int p = 0; p < NSTAGE; ++p)
     issue(p, p, Zero{}, One{});
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (HALO) {
+    // (computed while the prologue's loads are in flight)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int rt = wm * WM + i * 32 + (l & 31);
+      const int64_t m = m0 + rt;
+      const bool live = m < m_end;
+      const int32_t mm = (int32_t)(live ? m : 0);
+      const int32_t pq = conv_div(mm, g.conv.Q, g.conv.magic_q);
+      const int32_t q = mm - pq * g.conv.Q;
+      const int32_t nn = conv_div(pq, g.conv.P, g.conv.magic_p);
+      const int32_t ih0 = pq - nn * g.conv.P - g.conv.pad_h;
+      const int32_t iw0 = q - g.conv.pad_w;
+      uint32_t mask = 0;
+      for (int fr = 0; fr < g.conv.R; ++fr)
+        mask |= (uint32_t)(live && (uint32_t)(ih0 + fr * g.conv.dil_h) <
+                                       (uint32_t)g.conv.H)
+                << fr;
+      for (int fs = 0; fs < g.conv.S; ++fs)
+        mask |= (uint32_t)((uint32_t)(iw0 + fs * g.conv.dil_w) <
+                           (uint32_t)g.conv.W)
+                << (16 + fs);
+      h_row[i] = rt;
+      h_mask[i] = mask;
+    }
+  }
   __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_barrier();
