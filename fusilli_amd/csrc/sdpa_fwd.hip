@@ -14,7 +14,13 @@
 //   * Q fragments stay in registers for the whole kernel; the output
 //     accumulator O^T is rescaled only when some row maximum moved;
 //   * causal workgroups stop at the diagonal, and a wavefront skips tiles that
-//     lie wholly above its own rows.
+//     lie wholly above its own rows;
+//   * the two wavefronts of a SIMD (w and w + 4) alternate: a tile is an MFMA
+//     phase (S^T of tile t and the O^T update of tile t - 1, 32 MFMAs) and a
+//     vector-ALU phase (online softmax of tile t) of about equal length,
+//     separated by workgroup barriers, and wavefronts 4..7 run one phase behind
+//     wavefronts 0..3 -- the matrix pipe works on one wavefront's tile while
+//     the other computes its exponentials.
 //
 // Reference semantics: aten.scaled_dot_product_attention (reference
 // support/asm_emitter.h:2409-2468, node/sdpa_node.h:36-236), GQA by head
@@ -43,7 +49,7 @@ constexpr int kBKV = 64;        // keys per tile
 constexpr int kWaves = 8;
 constexpr int kStages = 3;
 constexpr int kTileB = kBKV * kRowB;       // one K (or V) tile: 16 KB
-constexpr int kStageB = 2 * kTileB;        // K + V
+constexpr int kStageB = 2 * kTileB;        // K ring and V ring, per stage
 constexpr int kLoadsPerTile = kTileB / 1024 / kWaves; // DMA per wave per tile
 constexpr int kOutPitch = kRowB + 16;      // epilogue rows, padded
 constexpr int kLdsB = kStages * kStageB > kWaves * 32 * kOutPitch
@@ -133,9 +139,17 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
   const int half = l >> 5, lq = l & 31;
-  // heavy (late) query tiles first: causal tiles near the end do most work
-  const int qtile = CAUSAL ? (int)gridDim.x - 1 - (int)blockIdx.x : (int)blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z;
+  // Causal masks: a workgroup runs query tile (last - z) and then tile z, a
+  // long and a short one, so all workgroups do the same work (tiles of one
+  // head need 1 .. n key-tile rows).  Otherwise one tile per workgroup.
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
+  const int z = blockIdx.z;
+  const int passes = CAUSAL && n_qtiles - 1 - z != z ? 2 : 1;
+  for (int pass = 0; pass < passes; ++pass) {
+  const int qtile = CAUSAL && pass == 0 ? n_qtiles - 1 - z : z;
+  if (pass) // the first tile's output staging has been read
+    __builtin_amdgcn_s_barrier();
   const int hk = h / g.group;
   const int q0 = qtile * kBQ;
   const int qw0 = q0 + wave * 32; // first query row of this wavefront
@@ -180,28 +194,40 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     koff[j] = (uint32_t)(row * k_rowb + ((p ^ (row & 15)) << 4));
     voff[j] = (uint32_t)(row * v_rowb + (sd_vchunk(row, p) << 4));
   }
-  auto issue = [&](int t, int st) {
-    // rows at or past Skv (and tiles past the end) read as zeros
+  // K tiles live in stages [0, kStages), V tiles in [kStages, 2 kStages).
+  // Rows at or past Skv (and tiles past the end) read as zeros.
+  auto issue_kv = [&](const char *base, int64_t rowb, int64_t bytes,
+                      const uint32_t (&off)[kLoadsPerTile], int t,
+                      uint32_t stage) {
     const int64_t kv0 = (int64_t)t * kBKV;
-    int64_t kb = k_bytes - kv0 * k_rowb, vb = v_bytes - kv0 * v_rowb;
-    kb = t < tiles && kb > 0 ? kb : 0;
-    vb = t < tiles && vb > 0 ? vb : 0;
-    const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(kp + kv0 * k_rowb), 0, (int)kb, 0x00020000);
-    const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(vp + kv0 * v_rowb), 0, (int)vb, 0x00020000);
+    int64_t nb = bytes - kv0 * rowb;
+    nb = t < tiles && nb > 0 ? nb : 0;
+    const uint64_t b64 = (uint64_t)(base + kv0 * rowb);
+    const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64);
+    const uint32_t bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(((uint64_t)bhi << 32) | blo), 0,
+        (int)__builtin_amdgcn_readfirstlane((uint32_t)nb), 0x00020000);
 #pragma unroll
     for (int j = 0; j < kLoadsPerTile; ++j) {
-      const uint32_t dst = lds0 + (uint32_t)st * kStageB +
-                           (uint32_t)(j * kWaves + wave) * 1024u;
+      const uint32_t dst = stage + (uint32_t)(j * kWaves + wave) * 1024u;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          kr, (SD_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
-          (int)koff[j], 0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          vr, (SD_AS3 char *)__builtin_amdgcn_readfirstlane(dst + kTileB), 16,
-          (int)voff[j], 0, 0, 0);
+          r, (SD_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
+          (int)off[j], 0, 0, 0);
     }
   };
+  // ring slot (0 .. kStages - 1) -> LDS address
+  auto k_stage = [&](int slot) { return lds0 + (uint32_t)slot * kTileB; };
+  auto v_stage = [&](int slot) {
+    return lds0 + (uint32_t)(kStages + slot) * kTileB;
+  };
+  auto issue_k = [&](int t, int slot) {
+    issue_kv(kp, k_rowb, k_bytes, koff, t, k_stage(slot));
+  };
+  auto issue_v = [&](int t, int slot) {
+    issue_kv(vp, v_rowb, v_bytes, voff, t, v_stage(slot));
+  };
+  auto next_slot = [](int s) { return s + 1 == kStages ? 0 : s + 1; };
 
   // ---- fragment addressing ----------------------------------------------------
   // K (A operand of S^T): row lq of a 32-key block, 16-byte chunk 2*ds + half
@@ -232,111 +258,162 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   float m_run = kNegBig; // running row maximum (raw scores), same in both halves
   float l_run = 0.f;     // running row sum, this half's share
 
-  // ---- prologue ---------------------------------------------------------------
-#pragma unroll
-  for (int p = 0; p < kStages - 1; ++p)
-    issue(p, p);
-
-  int st = 0;
-  for (int t = 0; t < tiles; ++t) {
-    // tile t landed (this thread's loads, then everyone's); stage of tile t-1
-    // is free for tile t + kStages - 1
-    __builtin_amdgcn_s_waitcnt(sd_wait_imm((kStages - 2) * 2 * kLoadsPerTile));
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  // ---- phases ---------------------------------------------------------------
+  // Global phase p: wavefronts 0..3 run MFMA(t) at p = 2t and VALU(t) at
+  // p = 2t + 1, wavefronts 4..7 one phase later; a barrier ends every phase.
+  //   MFMA(t): S^T of tile t (K stage t) and O^T += V^T P^T of tile t - 1
+  //   VALU(t): loads of K tile t + 2 and V tile t + 1, softmax of tile t
+  // K tile t is read in phases 2t, 2t + 1 and V tile t in 2t + 2, 2t + 3; the
+  // loads issued in VALU(t) reuse the stages of K tile t - 1 and V tile t - 2
+  // (last read in phase 2t - 1) and are first needed in phase 2t + 4.
+  const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
+  issue_k(0, 0);
+  issue_v(0, 0);
+  issue_k(1, 1);
+  // K tile 0 has landed
+  __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if (team)
     __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    {
-      const int fill = st == 0 ? kStages - 1 : st - 1;
-      issue(t + kStages - 1, fill);
-    }
-    const int kv0 = t * kBKV;
-    const uint32_t sk = lds0 + (uint32_t)st * kStageB, sv = sk + kTileB;
-    st = st + 1 == kStages ? 0 : st + 1;
-    // a wavefront whose rows all lie above this tile has nothing to add
-    if (CAUSAL && kv0 > qw0 + 31)
-      continue;
 
-    // ---- S^T = K Q^T : 2 key blocks of 32 -------------------------------------
-    f32x16 s[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        s[kb][r] = 0.f;
-#pragma unroll
-    for (int ds = 0; ds < kD / 16; ++ds)
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const u32x4 v =
-            *(const SD_AS3 u32x4 *)(uintptr_t)(sk + kaddr[ds] + kb * 32 * kRowB);
-        const uint32_t kf[4] = {v.x, v.y, v.z, v.w};
-        s[kb] = sd_mfma<BF16>(kf, qf[ds], s[kb]);
-      }
-
-    // ---- mask -----------------------------------------------------------------
-    const bool edge = (CAUSAL && kv0 + kBKV - 1 > qw0) || kv0 + kBKV > g.Skv;
-    if (edge) {
+  f32x16 s[2];
+  uint32_t pf[4][4]; // probabilities as B-operand fragments, 16 keys each
+  // a wavefront whose rows all lie above a tile has nothing to add
+  auto active = [&](int t) { return !(CAUSAL && t * kBKV > qw0 + 31); };
+  // ring slots of tile t - 1, t, t + 1, t + 2 (slot of t + 2 == slot of t - 1)
+  int sl_prev = kStages - 1, sl_cur = 0, sl_next = 1;
+#pragma clang loop unroll(disable)
+  for (int t = 0; t <= tiles; ++t) {
+    // ---- MFMA phase -----------------------------------------------------------
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_setprio(2);
+    if (t < tiles && active(t)) {
+      const uint32_t sk = k_stage(sl_cur);
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kv0 + kb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-          const bool dead = key >= g.Skv || (CAUSAL && key > qrow);
-          s[kb][r] = dead ? kNegBig : s[kb][r];
+        for (int r = 0; r < 16; ++r)
+          s[kb][r] = 0.f;
+#pragma unroll
+      for (int ds = 0; ds < kD / 16; ++ds)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          const u32x4 v = *(const SD_AS3 u32x4 *)(uintptr_t)(sk + kaddr[ds] +
+                                                             kb * 32 * kRowB);
+          const uint32_t kf[4] = {v.x, v.y, v.z, v.w};
+          s[kb] = sd_mfma<BF16>(kf, qf[ds], s[kb]);
         }
-    }
-
-    // ---- online softmax -------------------------------------------------------
-    float mx = s[0][0];
+      // fragment reads run eight MFMAs ahead, no further (registers)
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        mx = fmaxf(mx, s[kb][r]);
-    mx = sd_half_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float mc = m_new * g.scale_log2e;
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * g.scale_log2e);
-    const bool moved = m_new > m_run;
-    m_run = m_new;
-    uint32_t pf[4][4]; // probabilities as B-operand fragments, 16 keys each
-    float psum = 0.f;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * g.scale_log2e - mc);
-        const float p1 = __builtin_amdgcn_exp2f(s[kb][r + 1] * g.scale_log2e - mc);
-        psum += p0 + p1;
-        pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = sd_pack<BF16>(p0, p1);
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
-    l_run = l_run * alpha + psum;
-    if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    }
+    if (t > 0 && active(t - 1)) {
+      const uint32_t sv = v_stage(sl_prev);
 #pragma unroll
-      for (int dt = 0; dt < kD / 32; ++dt)
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int dt = 0; dt < kD / 32; ++dt) {
+          uint32_t vf[4];
+#pragma unroll
+          for (int r = 0; r < 2; ++r) {
+            const uint32_t ad = sv + vaddr[dt] + (j * 16 + r * 8) * kRowB;
+            const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (SD_AS3 s16x4 *)(uintptr_t)ad);
+            const u32x2 w2 = __builtin_bit_cast(u32x2, v);
+            vf[2 * r + 0] = w2.x;
+            vf[2 * r + 1] = w2.y;
+          }
+          o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
+        }
+      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    }
+    __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_sched_barrier(0);
+    // wavefronts 4..7 issued their newest loads a phase ago and the tiles are
+    // needed after this barrier
+    if (team)
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(0));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (t == tiles)
+      break;
+
+    // ---- vector-ALU phase -------------------------------------------------------
+    issue_k(t + 2, sl_prev);
+    issue_v(t + 1, sl_next);
+    sl_prev = sl_cur;
+    sl_cur = sl_next;
+    sl_next = next_slot(sl_next);
+    if (active(t)) {
+      const int kv0 = t * kBKV;
+      const bool edge = (CAUSAL && kv0 + kBKV - 1 > qw0) || kv0 + kBKV > g.Skv;
+      if (edge) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kv0 + kb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            const bool dead = key >= g.Skv || (CAUSAL && key > qrow);
+            s[kb][r] = dead ? kNegBig : s[kb][r];
+          }
+      }
+      float mx = s[0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          o[dt][r] *= alpha;
-    }
-
-    // ---- O^T += V^T P^T ---------------------------------------------------------
+          mx = fmaxf(mx, s[kb][r]);
+      mx = sd_half_max(mx);
+      const float m_new = fmaxf(m_run, mx);
+      const float mc = m_new * g.scale_log2e;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * g.scale_log2e);
+      const bool moved = m_new > m_run;
+      m_run = m_new;
+      float psum = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int dt = 0; dt < kD / 32; ++dt) {
-        uint32_t vf[4];
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-          const uint32_t ad = sv + vaddr[dt] + (j * 16 + r * 8) * kRowB;
-          const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (SD_AS3 s16x4 *)(uintptr_t)ad);
-          const u32x2 w2 = __builtin_bit_cast(u32x2, v);
-          vf[2 * r + 0] = w2.x;
-          vf[2 * r + 1] = w2.y;
+        for (int r = 0; r < 16; r += 2) {
+          const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * g.scale_log2e - mc);
+          const float p1 =
+              __builtin_amdgcn_exp2f(s[kb][r + 1] * g.scale_log2e - mc);
+          psum += p0 + p1;
+          pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = sd_pack<BF16>(p0, p1);
         }
-        o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
+      l_run = l_run * alpha + psum;
+      // O^T holds tiles 0 .. t - 1 here (their MFMA phases are over)
+      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+        for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            o[dt][r] *= alpha;
       }
+    }
+    // wavefronts 0..3: everything but the loads just issued has landed (the
+    // older batch is needed after the next barrier but one)
+    if (!team)
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   }
+  if (!team)
+    __builtin_amdgcn_s_barrier();
 
   // ---- epilogue: O = O^T / l, through LDS for row-contiguous stores -----------
   __builtin_amdgcn_s_waitcnt(sd_wait_imm(0));
@@ -367,6 +444,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     if (qr < g.Sq)
       *(SD_AS1 u32x4 *)(op + (int64_t)qr * g.o_ss * 2 + (l & 15) * 16) = v;
   }
+  } // pass
 }
 
 struct SdpaPlan {
@@ -401,7 +479,8 @@ SdpaPlan make_plan(const fhip_sdpa_desc *d) {
   if (Skv * d->k.stride[2] * 2 >= (1ll << 31) ||
       Skv * d->v.stride[2] * 2 >= (1ll << 31))
     return p;
-  if (d->q.dim[1] > 65535 || d->q.dim[0] > 65535)
+  // grid: heads x batch x query tiles
+  if (d->q.dim[0] > 65535 || (Sq + kBQ - 1) / kBQ > 65535)
     return p;
   // the running maximum is taken over raw scores: needs a positive scale
   if (d->has_scale && !(d->scale > 0.f))
@@ -443,8 +522,9 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   const float scale =
       d->has_scale ? d->scale : 1.0f / sqrtf((float)d->q.dim[3]);
   g.scale_log2e = scale * 1.4426950408889634f;
-  const dim3 grid((unsigned)((g.Sq + kBQ - 1) / kBQ), (unsigned)d->q.dim[1],
-                  (unsigned)d->q.dim[0]);
+  const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
+  const dim3 grid((unsigned)d->q.dim[1], (unsigned)d->q.dim[0],
+                  (unsigned)(d->is_causal ? (n_qtiles + 1) / 2 : n_qtiles));
   auto launch = [&](auto kernel) {
     static bool configured = false;
     if (!configured) {
