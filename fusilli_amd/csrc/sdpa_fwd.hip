@@ -133,6 +133,17 @@ __device__ __forceinline__ constexpr int sd_wait_imm(int vm) {
   return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0x0 << 8);
 }
 
+// Workgroup barrier without the release fence's "wait for everything": the
+// callers wait for exactly the loads whose data the other wavefronts need
+// (LDS-DMA completion is on the vector-memory counter, LDS reads have been
+// consumed by the MFMAs before every barrier); the empty asm statements keep
+// the compiler from moving memory operations across.
+__device__ __forceinline__ void sd_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 template <bool BF16, bool CAUSAL>
 __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -346,9 +357,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     // needed after this barrier
     if (team)
       __builtin_amdgcn_s_waitcnt(sd_wait_imm(0));
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    sd_barrier();
     if (t == tiles)
       break;
 
@@ -408,9 +417,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     // older batch is needed after the next barrier but one)
     if (!team)
       __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    sd_barrier();
   }
   if (!team)
     __builtin_amdgcn_s_barrier();
