@@ -143,6 +143,30 @@ def bench_matmul(ctx, steps, warmup, kind, m=4096, n=4096, k=8192):
             "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
 
 
+def bench_matmul_f32_c1(ctx, steps, warmup):
+    """BASELINE config 1: f32 A[1,256,512] x B[1,512,256] (the reference's
+    CPU-runnable case).  Runs on the stride-generic f32 MFMA tile kernel
+    (v_mfma_f32_32x32x2_f32, 64 x 64 tiles: 16 workgroups at this size)."""
+    d = capi.MatmulDesc()
+    d.a = capi.TensorDesc.make([1, 256, 512], [256 * 512, 512, 1], capi.FLOAT)
+    d.b = capi.TensorDesc.make([1, 512, 256], [512 * 256, 256, 1], capi.FLOAT)
+    d.c = capi.TensorDesc.make([1, 256, 256], [256 * 256, 256, 1], capi.FLOAT)
+    d.out = capi.TensorDesc.make([1, 256, 256], [256 * 256, 256, 1], capi.FLOAT)
+    d.out_dtype = capi.FLOAT
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_matmul_supported(d) >= 1
+    a = ctx.to_device(synth.uniform(1, 0, 256 * 512).astype(np.float32))
+    b = ctx.to_device(synth.uniform(1, 1, 512 * 256).astype(np.float32))
+    out = ctx.alloc(256 * 256 * 4)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.matmul(d, a, b, out), steps, warmup)
+    flop = 2.0 * 256 * 512 * 256
+    return {"value": round(flop / ev_ms / 1e9, 3), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / 157.3, 5),
+            "kernel_us": round(ev_ms * 1e3, 2), "work": flop,
+            "kernel": "stride-generic f32 MFMA tiles (fhip_matmul_supported == %d)"
+                      % ctx.lib.fhip_matmul_supported(d)}
+
+
 def bench_conv(ctx, steps, warmup):
     """C3: conv_fprop bf16 NHWC N32 C64 56x56, K128 3x3 pad 1, + bias + ReLU."""
     n, c, h, w, k, r = 32, 64, 56, 56, 128, 3
@@ -382,6 +406,8 @@ def main():
             ctx, args.steps, args.warmup, "SUM")
         others["reduce_amax_bf16_8192x4096_rows"] = bench_reduce(
             ctx, args.steps, args.warmup, "AMAX")
+        others["matmul_f32_1x256x512x256"] = bench_matmul_f32_c1(
+            ctx, max(10, args.steps // 4), 3)
         ksteps, kwarm = max(10, args.steps // 10), max(3, args.warmup // 5)
         others["matmul_int8_4096x8192x4096_i32"] = bench_matmul(
             ctx, ksteps, kwarm, "int8")

@@ -93,6 +93,99 @@ __global__ void generic_matmul_kernel(MatmulArgs g, const void *a,
   fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
 }
 
+// f32 x f32 matmul on the f32 matrix instruction (v_mfma_f32_32x32x2_f32), any
+// strides, batch broadcasting and epilogue of the strided kernel above.  A
+// workgroup of 4 wavefronts owns a 64 x 64 output tile of one batch entry and
+// walks K in steps of 16 through LDS (As[k][m], Bs[k][n]); the next step's
+// global loads are in flight while the current one is multiplied.
+constexpr int kF32Tile = 64, kF32K = 16, kF32Pitch = kF32Tile + 4;
+
+__global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
+    MatmulArgs g, const float *a, const float *b, void *out, int tiles_n) {
+  typedef float f32x16 __attribute__((ext_vector_type(16)));
+  __shared__ float As[kF32K][kF32Pitch], Bs[kF32K][kF32Pitch];
+  const int rank = g.out.rank;
+  const int64_t M = g.out.dim[rank - 2], N = g.out.dim[rank - 1];
+  const int64_t m0 = (int64_t)(blockIdx.x / tiles_n) * kF32Tile;
+  const int64_t n0 = (int64_t)(blockIdx.x % tiles_n) * kF32Tile;
+  // batch coordinates of this workgroup
+  int64_t coord[FHIP_MAX_RANK];
+  {
+    int64_t lin = blockIdx.y;
+    for (int r = rank - 3; r >= 0; --r) {
+      coord[r] = lin % g.out.dim[r];
+      lin /= g.out.dim[r];
+    }
+  }
+  int64_t ab = 0, bb = 0;
+  for (int r = 0; r < rank - 2; ++r) {
+    ab += coord[r] * g.a.s[r];
+    bb += coord[r] * g.b.s[r];
+  }
+  const int64_t a_sm = g.a.s[rank - 2], b_sn = g.b.s[rank - 1];
+  const int t = threadIdx.x, wave = t >> 6, l = t & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  // each thread stages 4 elements of A and 4 of B per step; the fastest thread
+  // index runs along whichever dimension is contiguous in memory
+  const bool a_kfast = g.a_k == 1, b_kfast = g.b_k == 1;
+  int a_m[4], a_kk[4], b_n[4], b_kk[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int e = t + i * 256;
+    a_kk[i] = a_kfast ? e % kF32K : e / kF32Tile;
+    a_m[i] = a_kfast ? e / kF32K : e % kF32Tile;
+    b_kk[i] = b_kfast ? e % kF32K : e / kF32Tile;
+    b_n[i] = b_kfast ? e / kF32K : e % kF32Tile;
+  }
+  auto fetch = [&](int64_t k0, float (&ra)[4], float (&rb)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
+      const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
+      ra[i] = m < M && ka < g.K ? a[ab + m * a_sm + ka * g.a_k] : 0.f;
+      rb[i] = n < N && kb < g.K ? b[bb + n * b_sn + kb * g.b_k] : 0.f;
+    }
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.f;
+  float ra[4], rb[4];
+  fetch(0, ra, rb);
+  for (int64_t k0 = 0; k0 < g.K; k0 += kF32K) {
+    __syncthreads(); // the previous step's reads are done
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[a_kk[i]][a_m[i]] = ra[i];
+      Bs[b_kk[i]][b_n[i]] = rb[i];
+    }
+    __syncthreads();
+    if (k0 + kF32K < g.K)
+      fetch(k0 + kF32K, ra, rb);
+#pragma unroll
+    for (int kk = 0; kk < kF32K; kk += 2) {
+      const float av = As[kk + (l >> 5)][wm * 32 + (l & 31)];
+      const float bv = Bs[kk + (l >> 5)][wn * 32 + (l & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+    }
+  }
+  // lane holds column l % 32, rows (r / 4) * 8 + (l / 32) * 4 + r % 4
+  const int64_t n = n0 + wn * 32 + (l & 31);
+  if (n >= N)
+    return;
+  coord[rank - 1] = n;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int64_t m = m0 + wm * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+    if (m >= M)
+      continue;
+    coord[rank - 2] = m;
+    double v = fhip_round_through<double>(g.c_dt, (double)acc[r]);
+    v = fhip_apply_epilogue<double>(g.epi, v, coord);
+    fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
+  }
+}
+
 // --------------------------------------------------------------------------
 // convolution forward (cross-correlation, zero padding, groups = C / fC)
 // --------------------------------------------------------------------------
@@ -534,6 +627,18 @@ int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
   g.o_dt = d->out.dtype;
   g.epi = epi;
   const int64_t total = fhip_desc_volume(d->c);
+  if (d->a.dtype == FHIP_FLOAT && d->b.dtype == FHIP_FLOAT) {
+    const int64_t M = d->c.dim[r - 2], N = d->c.dim[r - 1];
+    const int64_t tm = (M + kF32Tile - 1) / kF32Tile, tn = (N + kF32Tile - 1) / kF32Tile;
+    const int64_t batch = total / (M * N);
+    if (tm * tn < (1ll << 31) && batch <= 65535 && tn < (1ll << 31)) {
+      hipLaunchKernelGGL(tiled_matmul_f32_kernel, dim3((unsigned)(tm * tn), (unsigned)batch),
+                         dim3(256), 0, ctx->stream, g, (const float *)a,
+                         (const float *)b, out, (int)tn);
+      FHIP_HIP_CHECK(ctx, hipGetLastError());
+      return 0;
+    }
+  }
   const bool int_path = fhip_dtype_is_int(d->a.dtype) &&
                         fhip_dtype_is_int(d->b.dtype);
   if (int_path)

@@ -347,14 +347,19 @@ __global__ __launch_bounds__(RowNormGeom<WPR>::kThreads) void rownorm_kernel(
           y[i] += b[i];
       }
     }
-    fhip_round_fast_vec<VEC>(g.y_dt, y);
+    // A value that is stored next is rounded by the store's conversion: rounding
+    // it to the same type first would only repeat the work.
+    constexpr bool Y_IS_LAST = VARIANT == RN_RMS_SCALE || VARIANT == RN_LN_SCALE_BIAS;
+    if (!(Y_IS_LAST && g.y_dt == DT))
+      fhip_round_fast_vec<VEC>(g.y_dt, y);
 
     if constexpr (VARIANT == RN_RMS_SCALE_MULS) {
       const float m = g.epi[0].scalar;
 #pragma unroll
       for (int i = 0; i < VEC; ++i)
         y[i] *= m;
-      fhip_round_fast_vec<VEC>(g.epi[0].result_dtype, y);
+      if (g.epi[0].result_dtype != DT)
+        fhip_round_fast_vec<VEC>(g.epi[0].result_dtype, y);
     } else if constexpr (VARIANT == RN_RMS_SCALE_MULT) {
       float o[VEC];
       if constexpr (PREFETCH)
@@ -364,7 +369,8 @@ __global__ __launch_bounds__(RowNormGeom<WPR>::kThreads) void rownorm_kernel(
 #pragma unroll
       for (int i = 0; i < VEC; ++i)
         y[i] *= o[i];
-      fhip_round_fast_vec<VEC>(g.epi[0].result_dtype, y);
+      if (g.epi[0].result_dtype != DT)
+        fhip_round_fast_vec<VEC>(g.epi[0].result_dtype, y);
     } else if constexpr (GENERAL) {
       for (int e = 0; e < g.epi_count; ++e) {
         const FastEpiOp &o = g.epi[e];
