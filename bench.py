@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): RMSNorm bf16 over X[8192,4096]
+Headline workload (benchmark config 2): RMSNorm bf16 over X[8192,4096]
 (f32 accumulate, eps 1e-6, learned scale) followed by a fused pointwise MUL —
 one `step` is one such launch through the C ABI with inputs resident in HBM.
 Buffer sets are rotated so the 256 MB Infinity Cache cannot serve the reads.
@@ -10,7 +10,7 @@ Prints ONE JSON line.  `value` is algorithmic GB/s over the timed wall-clock
 region; `roofline` prices the kernel's own average duration (HIP events on the
 launch stream) against the 8 TB/s HBM peak; `cpu_baseline` is the CPU oracle's
 restatement of the same op timed on this box's host cores over a bounded
-sample; `others` carries the remaining BASELINE configs (TFLOP/s or GB/s and
+sample; `others` carries the remaining benchmark configs (TFLOP/s or GB/s and
 fraction of their rooflines), measured the same way.
 """
 from __future__ import annotations
@@ -144,7 +144,7 @@ def bench_matmul(ctx, steps, warmup, kind, m=4096, n=4096, k=8192):
 
 
 def bench_matmul_f32_c1(ctx, steps, warmup):
-    """BASELINE config 1: f32 A[1,256,512] x B[1,512,256] (the reference's
+    """benchmark config 1: f32 A[1,256,512] x B[1,512,256] (the reference's
     CPU-runnable case).  Runs on the stride-generic f32 MFMA tile kernel
     (v_mfma_f32_32x32x2_f32, 64 x 64 tiles: 16 workgroups at this size)."""
     d = capi.MatmulDesc()

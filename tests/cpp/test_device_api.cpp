@@ -1,7 +1,7 @@
 // End-to-end tests of the graph API on the GPU: the reference samples' known
 // answers (samples/**, tests/test_graph.cpp:551-647) run through
 // Graph::validate -> compile -> execute on Backend::AMDGPU, each executed
-// twice, plus the BASELINE configs at reduced size against plain host loops,
+// twice, plus the benchmark configs at reduced size against plain host loops,
 // and HIP interop (caller-owned stream and device pointers,
 // tests/hip_tests/test_buffer.cpp:132-206).
 #define __HIP_PLATFORM_AMD__ 1
@@ -410,7 +410,7 @@ TEST("samples: pointwise transposed add, scalar mul, AOT int32 add") {
   }
 }
 
-// ---- BASELINE configs through the graph API ---------------------------------
+// ---- benchmark configs through the graph API ---------------------------------
 static std::vector<float> randomVec(size_t n, uint32_t seed, float lo, float hi) {
   std::mt19937 rng(seed);
   std::vector<float> v(n);

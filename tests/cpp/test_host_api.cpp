@@ -48,7 +48,7 @@ TEST("layout: stride orders and generators") {
   // dim (10,3,12,12), order {3,0,2,1} -> stride (432,1,36,3)
   CHECK((generateStrideFromDim({10, 3, 12, 12}, {3, 0, 2, 1}) ==
          Dims{432, 1, 36, 3}));
-  // BASELINE config 3 layouts
+  // benchmark config 3 layouts
   CHECK((generateStrideFromDim({32, 64, 56, 56}, getChannelsLastStrideOrder(4)) ==
          Dims{200704, 1, 3584, 64}));
   CHECK((generateStrideFromDim({128, 64, 3, 3}, getChannelsLastStrideOrder(4)) ==
@@ -695,7 +695,7 @@ TEST("planner: fusion decisions") {
     REQUIRE_ASSIGN(auto ws, g.getWorkspaceSize());
     CHECK(*ws == 0);
   }
-  // rmsnorm -> mul(scalar) fuses (BASELINE config 2)
+  // rmsnorm -> mul(scalar) fuses (benchmark config 2)
   {
     Graph g = newGraph("fuse_rms", DataType::BFloat16);
     auto x = g.tensor(mk("x", {8192, 4096}, {4096, 1}, DataType::BFloat16));

@@ -1,6 +1,6 @@
 """Graph-API benchmark driver (fusilli_amd/bench): every command of its
 test_commands.txt — the reference's benchmarks/test_commands.txt plus the
-BASELINE configs — must run, plan to a single fused kernel and print one CSV
+benchmark configs — must run, plan to a single fused kernel and print one CSV
 row with the `iter` and `dispatch_count` columns the reference's runner checks
 (benchmarks/test_benchmark_runner.sh:22-43)."""
 import os

@@ -1,6 +1,6 @@
 """MFMA GEMM (bf16 / f16 / int8 / fp8) through the C ABI vs the oracle: every
 operand orientation, ragged edges, batches, fused epilogues, and the full-size
-BASELINE config-5 shapes checked on sampled rows plus a checksum identity."""
+benchmark config-5 shapes checked on sampled rows plus a checksum identity."""
 import numpy as np
 import pytest
 
@@ -103,7 +103,7 @@ def test_gemm_bf16_bias_activation_epilogue(ctx, act):
 
 
 def test_gemm_fp8_per_tensor_scales_bf16_out(ctx):
-    # BASELINE config 5b at reduced size: x ~ U[-1,1], per-tensor scale
+    # benchmark config 5b at reduced size: x ~ U[-1,1], per-tensor scale
     # s = max|x| / 448, saturating RNE cast, C = (A8 B8) * (sa * sb) -> bf16.
     m, n, k = 512, 384, 1024
     xa = rand(73, 0, [m, k], "uniform")

@@ -31,7 +31,7 @@ def run_matmul(ctx, a, b, c_dtype, *, out_dtype=None, epilogue=(),
 
 
 def test_matmul_config1_f32(ctx):
-    # BASELINE config 1: f32 A[1,256,512] x B[1,512,256], U[-1,1], rel 1e-4.
+    # benchmark config 1: f32 A[1,256,512] x B[1,512,256], U[-1,1], rel 1e-4.
     a = HT.from_logical(rand(1, 0, [1, 256, 512], "uniform"), capi.FLOAT)
     b = HT.from_logical(rand(1, 1, [1, 512, 256], "uniform"), capi.FLOAT)
     out = run_matmul(ctx, a, b, capi.FLOAT)

@@ -64,7 +64,7 @@ def test_rmsnorm_rows_vs_oracle(ctx, dtype, rows, cols):
 
 
 def test_rmsnorm_config2_shape_slice_with_scalar_mul(ctx):
-    # BASELINE config 2 at reduced row count: bf16, eps 1e-6, learned scale,
+    # benchmark config 2 at reduced row count: bf16, eps 1e-6, learned scale,
     # followed by a pointwise MUL (scalar operand).
     rows, cols = 256, 4096
     x = HT.from_logical(rand(2, 0, [rows, cols]), capi.BFLOAT16)
