@@ -392,6 +392,15 @@ template <int NM, int NR, int NV> __device__ __forceinline__ void gemm_interleav
   });
 }
 
+// Workgroup barrier with nothing attached: the callers wait for exactly the
+// loads and LDS reads that the hand-over needs; the empty asm statements keep
+// the compiler from moving memory operations across.
+__device__ __forceinline__ void gemm_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // Makes the compiler treat `x` as produced here (a value that a pending load
 // delivers must have arrived).
 __device__ __forceinline__ void gemm_pin(float &x) { asm volatile("" : "+v"(x)); }
@@ -664,9 +673,18 @@ gemm_kernel(GemmArgs g) {
       *(GEMM_AS3 u32x4 *)(uintptr_t)(ring0 - kTileKBytes + threadIdx.x * 16) =
           u32x4{0, 0, 0, 0};
   }
+  constexpr bool PINGPONG = NW == 8;
+  if constexpr (PINGPONG) {
+    // slice 0, and the share of slice 1 that wavefronts 4..7 own (see the loop)
+    static_assert(NSTAGE == 2, "ping-pong tiles alternate two stages");
+    issue(0, 0, Zero{}, One{});
+    if (wave >= 4)
+      issue(1, 1, Zero{}, One{});
+  } else {
 #pragma unroll
-  for (int p = 0; p < NSTAGE; ++p)
-    issue(p, p, Zero{}, One{});
+    for (int p = 0; p < NSTAGE; ++p)
+      issue(p, p, Zero{}, One{});
+  }
   __builtin_amdgcn_sched_barrier(0);
   if constexpr (HALO) {
     // (computed while the prologue's loads are in flight)
@@ -694,10 +712,19 @@ gemm_kernel(GemmArgs g) {
       h_mask[i] = mask;
     }
   }
-  __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  if constexpr (PINGPONG) {
+    // slice 0 has landed (wavefronts 4..7 keep their share of slice 1 in flight)
+    if (wave >= 4)
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(LPS));
+    else
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+    gemm_barrier();
+  } else {
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
   // halo mode: per-tap fragment addresses (row base, swizzled chunk bits)
   uint32_t h_base[HALO ? TM : 1], h_x[HALO ? TM : 1];
   auto halo_tap = [&](int kt) {
@@ -744,83 +771,70 @@ gemm_kernel(GemmArgs g) {
   using Two = std::integral_constant<int, 2>;
 
   int cur = 0; // stage holding slice kt
-  constexpr bool PINGPONG = NW == 8;
   if constexpr (PINGPONG) {
-    // Two wavefronts share each SIMD.  Every K-step is split into a memory
-    // phase (fragment reads for the next step, global->LDS loads) and an MFMA
-    // phase, with a barrier after each; wavefronts 4..7 run one phase behind
-    // wavefronts 0..3, so on every SIMD one wavefront feeds the matrix pipe
-    // while the other issues memory instructions.
+    // Two wavefronts share each SIMD.  A K slice is a memory phase (all of the
+    // slice's fragment reads and this wavefront's share of a later slice's
+    // global -> LDS loads) and an MFMA phase (KSTEPS x TM x TN MFMAs), with a
+    // barrier after each; wavefronts 4..7 (team 1) run one phase behind
+    // wavefronts 0..3 (team 0), so on every SIMD one wavefront feeds the
+    // matrix pipe while the other issues memory instructions.  With g = global
+    // phase number:
+    //   g = 2 kt     : team 0 reads slice kt, loads its share of slice kt + 1
+    //                  into the other stage (team 1 finished reading that
+    //                  stage in phase 2 kt - 1)            | team 1: MFMA(kt-1)
+    //   g = 2 kt + 1 : team 0: MFMA(kt), then waits for its share of slice
+    //                  kt + 1 | team 1 reads slice kt and, once those reads
+    //                  have returned, loads its share of slice kt + 2 into the
+    //                  same stage (team 0 read it in phase 2 kt); it then
+    //                  waits for its share of slice kt + 1
+    // so slice kt + 1 is complete when phase 2 kt + 2 starts, and every load
+    // has two phases to land.
     const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
-    // PS K-steps per phase: longer phases amortise the two barriers
-    constexpr int PS = KSTEPS >= 4 ? 2 : 1;
-    constexpr int PHASES = KSTEPS / PS;
-    Frag<KIND> pa[2][PS][TM], pb[2][PS][TN];
-    // fragments of the first phase of slice 0 (the prologue's barrier made
-    // the slice visible)
-    gemm_static_for<PS>([&](auto uc) {
-      constexpr int u = decltype(uc)::value;
-      fa_addr.template load<u>(stage_a(0), pa[0][u]);
-      fb_addr.template load<u>(stage_b(0), pb[0][u]);
-    });
+    Frag<KIND> pa[KSTEPS][TM], pb[KSTEPS][TN];
     if (team)
-      __builtin_amdgcn_s_barrier();
+      gemm_barrier();
     for (int kt = 0; kt < kt_count; ++kt) {
-      const int nxt = cur + 1 == NSTAGE ? 0 : cur + 1;
+      const int nxt = cur ^ 1;
+      // ---- memory phase
       const uint32_t sa = stage_a(cur), sb = stage_b(cur);
-      gemm_static_for<PHASES>([&](auto pc) {
-        constexpr int ph = decltype(pc)::value;
-        static_assert(PHASES % 2 == 0, "register sets alternate per phase");
-        constexpr bool LASTP = ph + 1 == PHASES;
-        constexpr int fc = ph & 1, fn = fc ^ 1;
-        // ---- memory phase: fragments of the next phase, loads of a later slice
-        gemm_static_for<PS>([&](auto uc) {
-          constexpr int u = decltype(uc)::value;
-          if constexpr (!LASTP) {
-            fa_addr.template load<(ph + 1) * PS + u>(sa, pa[fn][u]);
-            fb_addr.template load<(ph + 1) * PS + u>(sb, pb[fn][u]);
-          } else {
-            fa_addr.template load<u>(stage_a(nxt), pa[fn][u]);
-            fb_addr.template load<u>(stage_b(nxt), pb[fn][u]);
-          }
-        });
-        // the whole next-but-one slice at once: it then has an MFMA phase and
-        // a memory phase of flight time before the wait below
-        if constexpr (LASTP)
-          issue(kt + NSTAGE, cur, Zero{}, One{});
-        if constexpr (ph == PHASES - 2) {
-          // Both teams wait here, one and two phases ahead of the first read
-          // of slice kt + 1: its loads have landed, and the last fragment
-          // reads of this stage (just issued) have returned before anyone
-          // refills it.
-          __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-          __builtin_amdgcn_s_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        } else {
-          __builtin_amdgcn_sched_barrier(0);
-          __builtin_amdgcn_s_barrier();
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // ---- MFMA phase
-        __builtin_amdgcn_s_setprio(1);
-        gemm_static_for<PS>([&](auto uc) {
-          constexpr int u = decltype(uc)::value;
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-              mfma32<KIND>(acc[i][j], pa[fc][u][i], pb[fc][u][j]);
-        });
-        __builtin_amdgcn_s_setprio(0);
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
+      gemm_static_for<KSTEPS>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        fa_addr.template load<u>(sa, pa[u]);
+        fb_addr.template load<u>(sb, pb[u]);
       });
+      if (team) {
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // the reads returned
+        issue(kt + 2, cur, Zero{}, One{});
+        // its share of slice kt + 1 (one batch older) has landed
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(LPS));
+      } else {
+        issue(kt + 1, nxt, Zero{}, One{});
+        // the reads returned: the other team may overwrite the stage next
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      gemm_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      // ---- MFMA phase
+      __builtin_amdgcn_s_setprio(1);
+      gemm_static_for<KSTEPS>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            mfma32<KIND>(acc[i][j], pa[u][i], pb[u][j]);
+      });
+      __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (!team)
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0)); // its share of slice kt + 1
+      gemm_barrier();
+      __builtin_amdgcn_sched_barrier(0);
       cur = nxt;
     }
     if (!team)
-      __builtin_amdgcn_s_barrier();
+      gemm_barrier();
   } else {
   // One K slice.  A stage is free again once the barrier of the iteration
   // that consumes it has passed, and is refilled at once with the slice
