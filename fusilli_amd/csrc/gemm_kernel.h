@@ -1,21 +1,24 @@
 // MFMA GEMM kernel template and launch helpers; instantiated once per element
 // kind in gemm_<kind>.hip.
 //
-// Data path of one workgroup (256 threads = 2 x 2 wavefronts, each owning a
-// (BM/2) x (BN/2) block of 32x32 MFMA tiles):
+// Data path of one workgroup (4 wavefronts as 2 x 2, or 8 as 2 x 4 / 4 x 2, each
+// owning a block of 32x32 MFMA tiles):
 //   * 128-byte K slices of A and B go from global memory straight into LDS
-//     with the LDS-DMA form of the global load (no staging registers), into a
-//     ring of NSTAGE stages, NSTAGE - 1 slices ahead of the MFMAs;
+//     with the LDS-DMA form of the buffer load (no staging registers), into a
+//     ring of NSTAGE stages ahead of the MFMAs; the convolution modes gather A
+//     from the NHWC input per filter tap, or keep the tile's input pixels and
+//     halo resident in LDS for all taps;
 //   * LDS rows are unpadded; 16-byte chunks are XOR-permuted inside a row so
 //     both the 16-byte fragment reads (K-contiguous operand) and the
 //     transposing 8-byte reads (M/N-contiguous operand) are bank-conflict free;
-//   * MFMA fragments are double buffered in registers: the reads for K-step
-//     s + 1 are in flight during the MFMAs of step s; the single barrier of an
-//     iteration sits before its last K-step, so the first fragments of the
-//     next slice are fetched behind that step's MFMAs;
-//   * accumulators leave through LDS one 32-row band at a time so that every
-//     lane applies the fused epilogue to 8 consecutive columns and stores them
-//     with one or two 16-byte writes.
+//   * 4-wave tiles double-buffer MFMA fragments in registers (the reads for
+//     K-step s + 1 are in flight during the MFMAs of step s, one barrier per K
+//     slice); 8-wave tiles alternate a memory phase and an MFMA phase per K
+//     slice between the two wavefronts of each SIMD;
+//   * the fused epilogue runs on the accumulators when it is linear with
+//     per-column operands (16-bit results then leave through LDS as packed
+//     row pairs), otherwise after a trip through LDS in 32-row bands; either
+//     way a lane stores 8 consecutive columns with 16-byte writes.
 #ifndef FUSILLI_AMD_CSRC_GEMM_KERNEL_H
 #define FUSILLI_AMD_CSRC_GEMM_KERNEL_H
 
