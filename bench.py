@@ -145,8 +145,9 @@ def bench_matmul(ctx, steps, warmup, kind, m=4096, n=4096, k=8192):
 
 def bench_matmul_f32_c1(ctx, steps, warmup):
     """benchmark config 1: f32 A[1,256,512] x B[1,512,256] (the reference's
-    CPU-runnable case).  Runs on the stride-generic f32 MFMA tile kernel
-    (v_mfma_f32_32x32x2_f32, 64 x 64 tiles: 16 workgroups at this size)."""
+    CPU-runnable case).  Runs on the stride-generic f32 MFMA kernels
+    (v_mfma_f32_32x32x2_f32; at this size 32 x 32 tiles with K split over the
+    four wavefronts of a workgroup: 64 workgroups)."""
     d = capi.MatmulDesc()
     d.a = capi.TensorDesc.make([1, 256, 512], [256 * 512, 512, 1], capi.FLOAT)
     d.b = capi.TensorDesc.make([1, 512, 256], [512 * 256, 256, 1], capi.FLOAT)

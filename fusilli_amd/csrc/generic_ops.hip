@@ -186,6 +186,102 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
   }
 }
 
+// Small outputs (few 64 x 64 tiles): a workgroup owns a 32 x 32 tile and its 4
+// wavefronts split K four ways (K-steps w, w + 4, ...), each staging its own
+// A / B sub-tiles in a private LDS region (no workgroup barriers in the loop);
+// the partial sums meet in LDS and every wavefront finishes a quarter of the
+// accumulator registers.
+__global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
+    MatmulArgs g, const float *a, const float *b, void *out, int tiles_n) {
+  typedef float f32x16 __attribute__((ext_vector_type(16)));
+  constexpr int T = 32, PITCH = T + 4;
+  __shared__ float As[4][kF32K][PITCH], Bs[4][kF32K][PITCH];
+  __shared__ float part[4][16][64];
+  const int rank = g.out.rank;
+  const int64_t M = g.out.dim[rank - 2], N = g.out.dim[rank - 1];
+  const int64_t m0 = (int64_t)(blockIdx.x / tiles_n) * T;
+  const int64_t n0 = (int64_t)(blockIdx.x % tiles_n) * T;
+  int64_t coord[FHIP_MAX_RANK];
+  {
+    int64_t lin = blockIdx.y;
+    for (int r = rank - 3; r >= 0; --r) {
+      coord[r] = lin % g.out.dim[r];
+      lin /= g.out.dim[r];
+    }
+  }
+  int64_t ab = 0, bb = 0;
+  for (int r = 0; r < rank - 2; ++r) {
+    ab += coord[r] * g.a.s[r];
+    bb += coord[r] * g.b.s[r];
+  }
+  const int64_t a_sm = g.a.s[rank - 2], b_sn = g.b.s[rank - 1];
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  const bool a_kfast = g.a_k == 1, b_kfast = g.b_k == 1;
+  // a lane stages 8 elements of A and 8 of B per step (16 x 32 each)
+  int a_m[8], a_kk[8], b_n[8], b_kk[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = l + i * 64;
+    a_kk[i] = a_kfast ? e % kF32K : e / T;
+    a_m[i] = a_kfast ? e / kF32K : e % T;
+    b_kk[i] = b_kfast ? e % kF32K : e / T;
+    b_n[i] = b_kfast ? e / kF32K : e % T;
+  }
+  auto fetch = [&](int64_t k0, float (&ra)[8], float (&rb)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
+      const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
+      ra[i] = m < M && ka < g.K ? a[ab + m * a_sm + ka * g.a_k] : 0.f;
+      rb[i] = n < N && kb < g.K ? b[bb + n * b_sn + kb * g.b_k] : 0.f;
+    }
+  };
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    acc[r] = 0.f;
+  float ra[8], rb[8];
+  const int64_t stride = 4 * kF32K;
+  fetch((int64_t)wave * kF32K, ra, rb);
+  for (int64_t k0 = (int64_t)wave * kF32K; k0 < g.K; k0 += stride) {
+    // wavefront-private LDS: program order (with the waits the compiler puts
+    // before dependent LDS accesses) is all the synchronisation needed
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      As[wave][a_kk[i]][a_m[i]] = ra[i];
+      Bs[wave][b_kk[i]][b_n[i]] = rb[i];
+    }
+    if (k0 + stride < g.K)
+      fetch(k0 + stride, ra, rb);
+#pragma unroll
+    for (int kk = 0; kk < kF32K; kk += 2) {
+      const float av = As[wave][kk + (l >> 5)][l & 31];
+      const float bv = Bs[wave][kk + (l >> 5)][l & 31];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r)
+    part[wave][r][l] = acc[r];
+  __syncthreads();
+  const int64_t n = n0 + (l & 31);
+  if (n >= N)
+    return;
+  coord[rank - 1] = n;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = wave * 4 + q;
+    const int64_t m = m0 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+    if (m >= M)
+      continue;
+    const float sum = (part[0][r][l] + part[1][r][l]) + (part[2][r][l] + part[3][r][l]);
+    coord[rank - 2] = m;
+    double v = fhip_round_through<double>(g.c_dt, (double)sum);
+    v = fhip_apply_epilogue<double>(g.epi, v, coord);
+    fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
+  }
+}
+
 // --------------------------------------------------------------------------
 // convolution forward (cross-correlation, zero padding, groups = C / fC)
 // --------------------------------------------------------------------------
@@ -631,6 +727,17 @@ int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
     const int64_t M = d->c.dim[r - 2], N = d->c.dim[r - 1];
     const int64_t tm = (M + kF32Tile - 1) / kF32Tile, tn = (N + kF32Tile - 1) / kF32Tile;
     const int64_t batch = total / (M * N);
+    const int64_t sm = (M + 31) / 32, sn = (N + 31) / 32;
+    if (tm * tn * batch < 128 && g.K >= 8 * kF32K && batch <= 65535 &&
+        sm * sn < (1ll << 31)) {
+      // few tiles: 32 x 32 tiles with K split over the wavefronts
+      hipLaunchKernelGGL(splitk_matmul_f32_kernel,
+                         dim3((unsigned)(sm * sn), (unsigned)batch), dim3(256),
+                         0, ctx->stream, g, (const float *)a, (const float *)b,
+                         out, (int)sn);
+      FHIP_HIP_CHECK(ctx, hipGetLastError());
+      return 0;
+    }
     if (tm * tn < (1ll << 31) && batch <= 65535 && tn < (1ll << 31)) {
       hipLaunchKernelGGL(tiled_matmul_f32_kernel, dim3((unsigned)(tm * tn), (unsigned)batch),
                          dim3(256), 0, ctx->stream, g, (const float *)a,

@@ -71,6 +71,25 @@ def test_matmul_batched_and_broadcast(ctx):
     assert_close(out2.logical(), oracle.matmul(a.logical(), b2.logical()), capi.FLOAT)
 
 
+@pytest.mark.parametrize("m,n,k", [(45, 70, 200), (33, 31, 129), (64, 64, 1000),
+                                   (200, 300, 136), (130, 260, 64)])
+@pytest.mark.parametrize("layout", ["nn", "tn", "nt"])
+def test_matmul_f32_mfma_tiles(ctx, m, n, k, layout):
+    # f32 operands run on the f32 matrix instruction: K split over the
+    # wavefronts for small outputs, 64 x 64 tiles otherwise; ragged edges,
+    # both operand orientations, batch broadcast and a fused bias + ReLU
+    a_st = [m * k, 1, m] if layout == "tn" else None
+    a = HT.from_logical(rand(8, 0, [2, m, k]), capi.FLOAT, a_st)
+    bv = rand(8, 1, [1, k, n])
+    b = HT.from_logical(bv, capi.FLOAT, [k * n, 1, k] if layout == "nt" else None)
+    bias = HT.from_logical(rand(8, 2, [1, 1, n]), capi.FLOAT)
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT)]
+    out = run_matmul(ctx, a, b, capi.FLOAT, epilogue=epi, epi_tensors=[bias])
+    ref = np.maximum(oracle.matmul(a.logical(), b.logical()) + bias.logical(), 0.0)
+    assert_close(out.logical(), ref, capi.FLOAT, f"{m}x{n}x{k} {layout}")
+
+
 def test_matmul_strided_operands_and_output(ctx):
     a = HT.from_logical(rand(6, 0, [2, 33, 17]), capi.BFLOAT16, [33 * 17, 1, 33])
     b = HT.from_logical(rand(6, 1, [2, 17, 9]), capi.BFLOAT16, [17 * 9, 1, 17])
