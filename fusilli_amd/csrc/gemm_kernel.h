@@ -494,13 +494,16 @@ gemm_kernel(GemmArgs g) {
   if (tiles % 8 == 0)
     pid = (pid % 8) * (tiles / 8) + pid / 8;
   constexpr int GROUP = 8;
-  const int per_group = GROUP * g.tiles_n;
-  const int group = pid / per_group;
-  const int first_m = group * GROUP;
-  const int group_rows =
-      g.tiles_m - first_m < GROUP ? g.tiles_m - first_m : GROUP;
-  const int tile_m = first_m + (pid % per_group) % group_rows;
-  const int tile_n = (pid % per_group) / group_rows;
+  int tile_m = pid, tile_n = 0;
+  if (g.tiles_n > 1) {
+    const int per_group = GROUP * g.tiles_n;
+    const int group = pid / per_group;
+    const int first_m = group * GROUP;
+    const int group_rows =
+        g.tiles_m - first_m < GROUP ? g.tiles_m - first_m : GROUP;
+    tile_m = first_m + (pid % per_group) % group_rows;
+    tile_n = (pid % per_group) / group_rows;
+  }
   const int64_t batch = blockIdx.y;
 
   const int tile_rows = g.tile_rows ? g.tile_rows : BM;
@@ -626,22 +629,6 @@ gemm_kernel(GemmArgs g) {
   using One = std::integral_constant<int, 1>;
   using Zero = std::integral_constant<int, 0>;
 
-  // ---- fragments ----------------------------------------------------------
-  FragAddr<KIND, BM, A_KC, TM> fa_addr;
-  FragAddr<KIND, BN, B_KC, TN> fb_addr;
-  fa_addr.setup(wm * TM);
-  fb_addr.setup(wn * TN);
-  Frag<KIND> fa[2][TM], fb[2][TN];
-
-  typename KindTraits<KIND>::AccVec acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        acc[i][j][r] = 0;
-
   // ---- prologue: fill all NSTAGE stages -------------------------------------
   if constexpr (HALO) {
     // Slab row r holds input pixel pix0 + r in the K-contiguous slice layout
@@ -689,6 +676,21 @@ gemm_kernel(GemmArgs g) {
       issue(p, p, Zero{}, One{});
   }
   __builtin_amdgcn_sched_barrier(0);
+  // ---- fragments and accumulators (set up while the first loads fly) --------
+  FragAddr<KIND, BM, A_KC, TM> fa_addr;
+  FragAddr<KIND, BN, B_KC, TN> fb_addr;
+  fa_addr.setup(wm * TM);
+  fb_addr.setup(wn * TN);
+  Frag<KIND> fa[2][TM], fb[2][TN];
+
+  typename KindTraits<KIND>::AccVec acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        acc[i][j][r] = 0;
   if constexpr (HALO) {
     // (computed while the prologue's loads are in flight)
 #pragma unroll
