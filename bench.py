@@ -276,9 +276,8 @@ def bench_layernorm(ctx, steps, warmup, sets=5):
             "kernel_us": round(ev_ms * 1e3, 2), "bytes": nbytes}
 
 
-def bench_sdpa(ctx, steps, warmup):
+def bench_sdpa(ctx, steps, warmup, b=4, h=32, sq=2048, d=128):
     """C4: SDPA forward bf16 causal B4 H32 S2048 D128 ([B,H,S,D] contiguous)."""
-    b, h, sq, d = 4, 32, 2048, 128
     dims = [b, h, sq, d]
     strides = [h * sq * d, sq * d, d, 1]
     desc = capi.SdpaDesc()

@@ -22,6 +22,8 @@
 //     wavefronts 0..3 -- the matrix pipe works on one wavefront's tile while
 //     the other computes its exponentials.
 //
+// Head dim 64 or 128 (template parameter); bf16 or f16.
+//
 // Reference semantics: aten.scaled_dot_product_attention (reference
 // support/asm_emitter.h:2409-2468, node/sdpa_node.h:36-236), GQA by head
 // repetition, causal mask aligned top-left.
@@ -42,20 +44,25 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 #define SD_AS1 __attribute__((address_space(1)))
 #define SD_AS3 __attribute__((address_space(3)))
 
-constexpr int kD = 128;         // head dim (Q/K and V)
-constexpr int kRowB = kD * 2;   // bytes per K / V row
 constexpr int kBQ = 256;        // query rows per workgroup
 constexpr int kBKV = 64;        // keys per tile
 constexpr int kWaves = 8;
 constexpr int kStages = 3;
-constexpr int kTileB = kBKV * kRowB;       // one K (or V) tile: 16 KB
-constexpr int kStageB = 2 * kTileB;        // K ring and V ring, per stage
-constexpr int kLoadsPerTile = kTileB / 1024 / kWaves; // DMA per wave per tile
-constexpr int kOutPitch = kRowB + 16;      // epilogue rows, padded
-constexpr int kLdsB = kStages * kStageB > kWaves * 32 * kOutPitch
-                          ? kStages * kStageB
-                          : kWaves * 32 * kOutPitch;
 constexpr float kNegBig = -1.0e30f;
+
+// Sizes that follow from the head dimension HD (Q/K and V), 64 or 128.
+template <int HD> struct SdShape {
+  static constexpr int kRowB = HD * 2;             // bytes per K / V row
+  static constexpr int kChunks = kRowB / 16;       // 16-byte chunks per row
+  static constexpr int kRowsPerLoad = 64 / kChunks; // rows of one wave DMA
+  static constexpr int kTileB = kBKV * kRowB;      // one K (or V) tile
+  static constexpr int kLoadsPerTile = kTileB / 1024 / kWaves; // per wave
+  static constexpr int kOutPitch = kRowB + 16;     // epilogue rows, padded
+  static constexpr int kRingB = 2 * kStages * kTileB; // K ring and V ring
+  static constexpr int kLdsB = kRingB > kWaves * 32 * kOutPitch
+                                   ? kRingB
+                                   : kWaves * 32 * kOutPitch;
+};
 
 struct SdpaArgs {
   const char *q, *k, *v;
@@ -118,15 +125,33 @@ __device__ __forceinline__ float sd_half_sum(float x) {
   return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
 }
 
-// chunk permutation of the V tile (rows of 256 bytes read by transposing
-// 8-byte loads): spreads the 4 rows x 64 bytes a half-wavefront touches over
-// all 64 banks
-__device__ __forceinline__ int sd_vpos(int row, int c) {
-  return c ^ ((row & 3) << 1) ^ ((c & 2) << 2);
+// Chunk permutation of the K tile (16-byte reads, 16 consecutive rows at one
+// chunk index per pass): position of chunk c in row `row` is c ^ sd_kswz(row).
+template <int HD> __device__ __forceinline__ int sd_kswz(int row) {
+  if constexpr (HD == 128)
+    return row & 15;
+  else // 128-byte rows: two rows share the 64 banks
+    return (row & 7) ^ ((row >> 3) & 1);
 }
-__device__ __forceinline__ int sd_vchunk(int row, int p) {
-  const int t = p ^ ((row & 3) << 1);
-  return t ^ ((t & 2) << 2);
+
+// Chunk permutation of the V tile (read by transposing 8-byte loads): spreads
+// the 4 rows x 64 bytes a half-wavefront touches over all 64 banks.  sd_vpos
+// maps a chunk to its position in the row, sd_vchunk is its inverse; both
+// depend on the row only through row % 4, which the fragment walk (steps of 8
+// rows) preserves.
+template <int HD> __device__ __forceinline__ int sd_vpos(int row, int c) {
+  if constexpr (HD == 128)
+    return c ^ ((row & 3) << 1) ^ ((c & 2) << 2);
+  else // rows r and r + 2 start in the same bank: swap the row's halves
+    return c ^ (((row >> 1) & 1) << 2);
+}
+template <int HD> __device__ __forceinline__ int sd_vchunk(int row, int p) {
+  if constexpr (HD == 128) {
+    const int t = p ^ ((row & 3) << 1);
+    return t ^ ((t & 2) << 2);
+  } else {
+    return p ^ (((row >> 1) & 1) << 2);
+  }
 }
 
 __device__ __forceinline__ constexpr int sd_wait_imm(int vm) {
@@ -144,8 +169,12 @@ __device__ __forceinline__ void sd_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <bool BF16, bool CAUSAL>
+template <bool BF16, bool CAUSAL, int HD>
 __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
+  using C = SdShape<HD>;
+  constexpr int kD = HD;
+  constexpr int kRowB = C::kRowB, kTileB = C::kTileB;
+  constexpr int kLoadsPerTile = C::kLoadsPerTile, kOutPitch = C::kOutPitch;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
@@ -196,14 +225,14 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     }
   }
 
-  // ---- DMA addressing: a wave instruction moves 4 rows x 256 bytes ----------
+  // ---- DMA addressing: a wave instruction moves 1 KB, 4 or 8 whole rows ------
   uint32_t koff[kLoadsPerTile], voff[kLoadsPerTile];
 #pragma unroll
   for (int j = 0; j < kLoadsPerTile; ++j) {
-    const int row = (j * kWaves + wave) * 4 + (l >> 4);
-    const int p = l & 15;
-    koff[j] = (uint32_t)(row * k_rowb + ((p ^ (row & 15)) << 4));
-    voff[j] = (uint32_t)(row * v_rowb + (sd_vchunk(row, p) << 4));
+    const int row = (j * kWaves + wave) * C::kRowsPerLoad + l / C::kChunks;
+    const int p = l % C::kChunks;
+    koff[j] = (uint32_t)(row * k_rowb + ((p ^ sd_kswz<HD>(row)) << 4));
+    voff[j] = (uint32_t)(row * v_rowb + (sd_vchunk<HD>(row, p) << 4));
   }
   // K tiles live in stages [0, kStages), V tiles in [kStages, 2 kStages).
   // Rows at or past Skv (and tiles past the end) read as zeros.
@@ -223,7 +252,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     for (int j = 0; j < kLoadsPerTile; ++j) {
       const uint32_t dst = stage + (uint32_t)(j * kWaves + wave) * 1024u;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          r, (SD_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16,
+          r, (SD_AS3 char *)(uintptr_t)__builtin_amdgcn_readfirstlane(dst), 16,
           (int)off[j], 0, 0, 0);
     }
   };
@@ -245,7 +274,8 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   uint32_t kaddr[kD / 16];
 #pragma unroll
   for (int ds = 0; ds < kD / 16; ++ds)
-    kaddr[ds] = (uint32_t)(lq * kRowB + (((ds * 2 + half) ^ (lq & 15)) << 4));
+    kaddr[ds] =
+        (uint32_t)(lq * kRowB + (((ds * 2 + half) ^ sd_kswz<HD>(lq)) << 4));
   // V^T (A operand of O^T += V^T P^T): the keys a lane needs are those whose
   // probabilities it holds: key = 32*kb + 8*(i/4) + 4*half + i%4 for score
   // register i; one transposing read returns 4 consecutive keys of one column
@@ -256,7 +286,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
 #pragma unroll
     for (int dt = 0; dt < kD / 32; ++dt) {
       const int c = dt * 4 + h16 * 2 + ((L & 3) >> 1);
-      vaddr[dt] = (uint32_t)(row * kRowB + (sd_vpos(row, c) << 4) + (L & 1) * 8);
+      vaddr[dt] = (uint32_t)(row * kRowB + (sd_vpos<HD>(row, c) << 4) + (L & 1) * 8);
     }
   }
 
@@ -319,7 +349,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
       // fragment reads run eight MFMAs ahead, no further (registers)
       __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kD / 8 - 8; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
@@ -345,7 +375,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
         }
       __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kD / 8 - 8; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       }
@@ -441,15 +471,16 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
                                    (dt * 32 + r4 * 8 + half * 4) * 2) = w2;
     }
   char *op = g.o + (b * g.o_sb + h * g.o_sh) * 2;
-  // 16 lanes cover one 256-byte row; 4 rows per pass
+  // kChunks lanes cover one output row; 4 or 8 rows per pass
 #pragma unroll
-  for (int pass = 0; pass < 8; ++pass) {
-    const int row = pass * 4 + (l >> 4);
-    const u32x4 v = *(const SD_AS3 u32x4 *)(uintptr_t)(band + row * kOutPitch +
-                                                       (l & 15) * 16);
+  for (int rows = 0; rows < 32; rows += C::kRowsPerLoad) {
+    const int row = rows + l / C::kChunks;
+    const int cb = (l % C::kChunks) * 16;
+    const u32x4 v =
+        *(const SD_AS3 u32x4 *)(uintptr_t)(band + row * kOutPitch + cb);
     const int qr = qw0 + row;
     if (qr < g.Sq)
-      *(SD_AS1 u32x4 *)(op + (int64_t)qr * g.o_ss * 2 + (l & 15) * 16) = v;
+      *(SD_AS1 u32x4 *)(op + (int64_t)qr * g.o_ss * 2 + cb) = v;
   }
   } // pass
 }
@@ -457,6 +488,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
 struct SdpaPlan {
   bool ok = false;
   bool bf16 = true;
+  int hd = 128;
 };
 
 SdpaPlan make_plan(const fhip_sdpa_desc *d) {
@@ -469,8 +501,10 @@ SdpaPlan make_plan(const fhip_sdpa_desc *d) {
   if (d->k.dtype != dt || d->v.dtype != dt || d->o.dtype != dt)
     return p;
   p.bf16 = dt == FHIP_BFLOAT16;
-  if (d->q.rank != 4 || d->q.dim[3] != kD || d->v.dim[3] != kD)
+  if (d->q.rank != 4 || (d->q.dim[3] != 64 && d->q.dim[3] != 128) ||
+      d->k.dim[3] != d->q.dim[3] || d->v.dim[3] != d->q.dim[3])
     return p;
+  p.hd = (int)d->q.dim[3];
   const fhip_tensor_desc *ts[4] = {&d->q, &d->k, &d->v, &d->o};
   for (const fhip_tensor_desc *t : ts) {
     if (t->stride[3] != 1 && t->dim[3] != 1)
@@ -532,22 +566,33 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
   const dim3 grid((unsigned)d->q.dim[1], (unsigned)d->q.dim[0],
                   (unsigned)(d->is_causal ? (n_qtiles + 1) / 2 : n_qtiles));
-  auto launch = [&](auto kernel) {
-    static bool configured = false;
+  auto launch = [&](auto kernel, int lds_bytes, bool &configured) {
     if (!configured) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kLdsB) != hipSuccess)
+                              lds_bytes) != hipSuccess)
         return fhip_fail(ctx, "sdpa: cannot reserve LDS");
       configured = true;
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(kWaves * 64), kLdsB, ctx->stream, g);
+    hipLaunchKernelGGL(kernel, grid, dim3(kWaves * 64), lds_bytes, ctx->stream,
+                       g);
     FHIP_HIP_CHECK(ctx, hipGetLastError());
     return 0;
   };
-  if (p.bf16)
-    return d->is_causal ? launch(sdpa_fwd_kernel<true, true>)
-                        : launch(sdpa_fwd_kernel<true, false>);
-  return d->is_causal ? launch(sdpa_fwd_kernel<false, true>)
-                      : launch(sdpa_fwd_kernel<false, false>);
+  // one flag per kernel instance: [head dim][type][causal]
+  static bool configured[2][2][2] = {};
+  auto pick = [&](auto hd) {
+    constexpr int HD = decltype(hd)::value;
+    bool(&cfg)[2][2] = configured[HD == 128];
+    constexpr int lds = SdShape<HD>::kLdsB;
+    if (p.bf16)
+      return d->is_causal
+                 ? launch(sdpa_fwd_kernel<true, true, HD>, lds, cfg[1][1])
+                 : launch(sdpa_fwd_kernel<true, false, HD>, lds, cfg[1][0]);
+    return d->is_causal
+               ? launch(sdpa_fwd_kernel<false, true, HD>, lds, cfg[0][1])
+               : launch(sdpa_fwd_kernel<false, false, HD>, lds, cfg[0][0]);
+  };
+  return p.hd == 128 ? pick(std::integral_constant<int, 128>{})
+                     : pick(std::integral_constant<int, 64>{});
 }

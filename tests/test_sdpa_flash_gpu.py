@@ -1,7 +1,7 @@
 """Flash-attention forward (MFMA kernel) through the C ABI vs the oracle.
 
-Every case satisfies the tuned kernel's contract (bf16/f16, head dim 128, no
-mask tensor) and asserts that the tuned kernel is chosen, so a silent fall
+Every case satisfies the tuned kernel's contract (bf16/f16, head dim 64 or 128,
+no mask tensor) and asserts that the tuned kernel is chosen, so a silent fall
 back to the generic kernel fails the test.
 """
 import numpy as np
@@ -51,19 +51,21 @@ CASES = [
 
 @pytest.mark.parametrize("case", CASES)
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
-def test_flash_random_vs_oracle(ctx, case, dtype):
+@pytest.mark.parametrize("hd", [128, 64])
+def test_flash_random_vs_oracle(ctx, case, dtype, hd):
     c = case
-    q = HT.from_logical(rand(51, 0, [c["B"], c["Hq"], c["Sq"], 128]), dtype)
-    k = HT.from_logical(rand(51, 1, [c["B"], c["Hkv"], c["Skv"], 128]), dtype)
-    v = HT.from_logical(rand(51, 2, [c["B"], c["Hkv"], c["Skv"], 128]), dtype)
+    q = HT.from_logical(rand(51, 0, [c["B"], c["Hq"], c["Sq"], hd]), dtype)
+    k = HT.from_logical(rand(51, 1, [c["B"], c["Hkv"], c["Skv"], hd]), dtype)
+    v = HT.from_logical(rand(51, 2, [c["B"], c["Hkv"], c["Skv"], hd]), dtype)
     out = run(ctx, q, k, v, causal=c["causal"])
     ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), is_causal=c["causal"])
     assert_close(out.logical(), ref, dtype, str(case))
 
 
-def test_flash_bshd_layout_and_scale(ctx):
+@pytest.mark.parametrize("hd", [128, 64])
+def test_flash_bshd_layout_and_scale(ctx, hd):
     # tensors stored [B, S, H, D] (heads interleaved per position), custom scale
-    dims_q, dims_k = [2, 4, 200, 128], [2, 2, 300, 128]
+    dims_q, dims_k = [2, 4, 200, hd], [2, 2, 300, hd]
     q = HT.from_logical(rand(52, 0, dims_q), capi.BFLOAT16, bshd_strides(dims_q))
     k = HT.from_logical(rand(52, 1, dims_k), capi.BFLOAT16, bshd_strides(dims_k))
     v = HT.from_logical(rand(52, 2, dims_k), capi.BFLOAT16, bshd_strides(dims_k))
@@ -72,11 +74,12 @@ def test_flash_bshd_layout_and_scale(ctx):
     assert_close(out.logical(), ref, capi.BFLOAT16)
 
 
-def test_flash_large_scores_are_stable(ctx):
+@pytest.mark.parametrize("hd", [128, 64])
+def test_flash_large_scores_are_stable(ctx, hd):
     # scores of magnitude ~1e3: the running maximum must keep exp() in range
-    q = HT.from_logical(rand(53, 0, [1, 2, 300, 128]) * 8.0, capi.BFLOAT16)
-    k = HT.from_logical(rand(53, 1, [1, 2, 300, 128]) * 8.0, capi.BFLOAT16)
-    v = HT.from_logical(rand(53, 2, [1, 2, 300, 128]), capi.BFLOAT16)
+    q = HT.from_logical(rand(53, 0, [1, 2, 300, hd]) * 8.0, capi.BFLOAT16)
+    k = HT.from_logical(rand(53, 1, [1, 2, 300, hd]) * 8.0, capi.BFLOAT16)
+    v = HT.from_logical(rand(53, 2, [1, 2, 300, hd]), capi.BFLOAT16)
     out = run(ctx, q, k, v, causal=True)
     assert np.all(np.isfinite(out.logical()))
     ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), is_causal=True)
@@ -84,19 +87,21 @@ def test_flash_large_scores_are_stable(ctx):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-def test_flash_constant_fill_equals_v(ctx, causal):
+@pytest.mark.parametrize("hd", [128, 64])
+def test_flash_constant_fill_equals_v(ctx, causal, hd):
     # samples/sdpa_utils.cpp:184-247: q = k = v = 0.01 => output == v (1e-2)
-    q = HT.from_logical(np.full([1, 8, 320, 128], 0.01), capi.HALF)
+    q = HT.from_logical(np.full([1, 8, 320, hd], 0.01), capi.HALF)
     out = run(ctx, q, q, q, causal=causal)
     assert np.allclose(out.logical(), 0.01, atol=1e-2)
 
 
-def test_flash_uniform_scores_causal_gives_prefix_means(ctx):
+@pytest.mark.parametrize("hd", [128, 64])
+def test_flash_uniform_scores_causal_gives_prefix_means(ctx, hd):
     # q = 0 => uniform attention over the visible prefix: O[i] = mean(V[:i+1])
     S = 400
-    q = HT.from_logical(np.zeros([1, 1, S, 128]), capi.BFLOAT16)
-    k = HT.from_logical(rand(54, 1, [1, 1, S, 128]), capi.BFLOAT16)
-    v = HT.from_logical(rand(54, 2, [1, 1, S, 128]), capi.BFLOAT16)
+    q = HT.from_logical(np.zeros([1, 1, S, hd]), capi.BFLOAT16)
+    k = HT.from_logical(rand(54, 1, [1, 1, S, hd]), capi.BFLOAT16)
+    v = HT.from_logical(rand(54, 2, [1, 1, S, hd]), capi.BFLOAT16)
     out = run(ctx, q, k, v, causal=True)
     vl = v.logical()[0, 0]
     ref = np.cumsum(vl, axis=0) / np.arange(1, S + 1)[:, None]
@@ -104,8 +109,8 @@ def test_flash_uniform_scores_causal_gives_prefix_means(ctx):
 
 
 def test_flash_not_chosen_outside_contract(ctx):
-    # head dim 64 and masked attention keep the generic kernel
-    q = HT.from_logical(rand(55, 0, [1, 2, 70, 64]), capi.BFLOAT16)
+    # other head dims (and f32) keep the generic kernel
+    q = HT.from_logical(rand(55, 0, [1, 2, 70, 96]), capi.BFLOAT16)
     out = run(ctx, q, q, q, expect_tuned=False)
     ref = oracle.sdpa(q.logical(), q.logical(), q.logical())
     assert_close(out.logical(), ref, capi.BFLOAT16)
@@ -132,3 +137,21 @@ def test_flash_headline_shape(ctx):
         assert_close(out[b:b + 1, h:h + 1], ref, capi.BFLOAT16, f"b{b} h{h}")
     ref = np.cumsum(vl[2, 7], axis=0) / np.arange(1, S + 1)[:, None]
     assert_close(out[2, 7], ref, capi.BFLOAT16, "uniform head")
+
+
+def test_flash_head_dim_64_many_tiles(ctx):
+    """Head dim 64, causal, eight query tiles per head: every key-tile count
+    from 1 to 32 occurs, and the paired query tiles (long + short) share one
+    workgroup.  One head has q = 0 for the closed-form prefix means."""
+    B, H, S, D = 1, 3, 2048, 64
+    qv = rand(57, 0, [B, H, S, D])
+    qv[0, 1] = 0.0
+    q = HT.from_logical(qv, capi.BFLOAT16)
+    k = HT.from_logical(rand(57, 1, [B, H, S, D]), capi.BFLOAT16)
+    v = HT.from_logical(rand(57, 2, [B, H, S, D]), capi.BFLOAT16)
+    out = run(ctx, q, k, v, causal=True).logical()
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), is_causal=True)
+    assert_close(out, ref, capi.BFLOAT16)
+    vl = v.logical()[0, 1]
+    assert_close(out[0, 1], np.cumsum(vl, axis=0) / np.arange(1, S + 1)[:, None],
+                 capi.BFLOAT16, "uniform head")
