@@ -196,9 +196,29 @@ def bench_conv(ctx, steps, warmup):
         ctx, lambda i: ctx.conv_fprop(d, x, wt, out, epilogue_operands=[bias]),
         steps, warmup)
     flop = 2.0 * n * h * w * k * c * r * r
+    # launch overhead, reported beside the kernel time: host time to enqueue
+    # one call (descriptor -> plan -> hipLaunchKernel), and the event-to-event
+    # time of a launch on an idle stream (dispatch latency + kernel)
+    launch = lambda: ctx.conv_fprop(d, x, wt, out, epilogue_operands=[bias])
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(50):
+        launch()
+    enqueue_us = (time.perf_counter() - t0) * 1e6 / 50
+    ctx.sync()
+    isolated = []
+    for _ in range(10):
+        e0, e1 = ctx.event(), ctx.event()
+        e0.record()
+        launch()
+        e1.record()
+        ctx.sync()
+        isolated.append(e1.elapsed_ms_since(e0) * 1e3)
     return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
             "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
-            "kernel_us": round(ev_ms * 1e3, 2), "work": flop}
+            "kernel_us": round(ev_ms * 1e3, 2), "work": flop,
+            "launch_overhead": {"host_enqueue_us": round(enqueue_us, 2),
+                                "idle_stream_launch_us": round(min(isolated), 2)}}
 
 
 def bench_reduce(ctx, steps, warmup, mode="SUM", sets=5):

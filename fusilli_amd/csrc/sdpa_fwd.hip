@@ -49,6 +49,7 @@ constexpr int kBKV = 64;        // keys per tile
 constexpr int kWaves = 8;
 constexpr int kStages = 3;
 constexpr float kNegBig = -1.0e30f;
+constexpr float kMaxSlack = 8.0f; // see the softmax phase
 
 // Sizes that follow from the head dimension HD (Q/K and V), 64 or 128.
 template <int HD> struct SdShape {
@@ -156,6 +157,22 @@ template <int HD> __device__ __forceinline__ int sd_vchunk(int row, int p) {
 
 __device__ __forceinline__ constexpr int sd_wait_imm(int vm) {
   return (vm & 0xF) | ((vm >> 4) << 14) | (0x7 << 4) | (0x0 << 8);
+}
+
+// Transposing 8-byte LDS read (4 consecutive rows of one 16-bit column per
+// lane) that the compiler does not see as a memory access, and the wait that
+// goes with it: at most N LDS operations still outstanding, after which the
+// two registers may be used.
+template <int OFFSET>
+__device__ __forceinline__ void sd_read_tr16(u32x2 &dst, uint32_t addr) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "16-bit offset field");
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+               : "=v"(dst)
+               : "v"(addr), "n"(OFFSET));
+}
+template <int N> __device__ __forceinline__ void sd_wait_pin(u32x2 &a, u32x2 &b) {
+  static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit field");
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
 
 // Workgroup barrier without the release fence's "wait for everything": the
@@ -299,14 +316,18 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   float m_run = kNegBig; // running row maximum (raw scores), same in both halves
   float l_run = 0.f;     // running row sum, this half's share
 
-  // ---- phases ---------------------------------------------------------------
-  // Global phase p: wavefronts 0..3 run MFMA(t) at p = 2t and VALU(t) at
-  // p = 2t + 1, wavefronts 4..7 one phase later; a barrier ends every phase.
-  //   MFMA(t): S^T of tile t (K stage t) and O^T += V^T P^T of tile t - 1
-  //   VALU(t): loads of K tile t + 2 and V tile t + 1, softmax of tile t
-  // K tile t is read in phases 2t, 2t + 1 and V tile t in 2t + 2, 2t + 3; the
-  // loads issued in VALU(t) reuse the stages of K tile t - 1 and V tile t - 2
-  // (last read in phase 2t - 1) and are first needed in phase 2t + 4.
+  // ---- rounds ---------------------------------------------------------------
+  // Per key tile t a wavefront runs
+  //   MFMA(t): S^T of tile t (K tile t) and O^T += V^T P^T of tile t - 1
+  //   VALU(t): online softmax of tile t
+  // and one workgroup barrier.  Wavefronts 0..3 place the barrier after
+  // VALU(t), wavefronts 4..7 after MFMA(t): between two barriers one team
+  // runs MFMA(t + 1), VALU(t + 1) and the other VALU(t), MFMA(t + 1), so the
+  // two wavefronts of a SIMD use the matrix pipe and the vector ALU in turn
+  // without waiting for each other in the middle.  Between barrier t and
+  // barrier t + 1 only K tile t + 1 and V tile t are read; the loads issued at
+  // the top of round t (K tile t + 2, V tile t + 1) reuse the stages of K tile
+  // t - 1 and V tile t - 2 and have to land by barrier t + 1.
   const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
   issue_k(0, 0);
   issue_v(0, 0);
@@ -316,8 +337,6 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  if (team)
-    __builtin_amdgcn_s_barrier();
 
   f32x16 s[2];
   uint32_t pf[4][4]; // probabilities as B-operand fragments, 16 keys each
@@ -327,6 +346,8 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   int sl_prev = kStages - 1, sl_cur = 0, sl_next = 1;
 #pragma clang loop unroll(disable)
   for (int t = 0; t <= tiles; ++t) {
+    issue_k(t + 2, sl_prev);
+    issue_v(t + 1, sl_next);
     // ---- MFMA phase -----------------------------------------------------------
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(2);
@@ -356,47 +377,46 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
       __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
     }
     if (t > 0 && active(t - 1)) {
+      // V^T fragments by transposing reads written as asm: the compiler would
+      // make a read it knows to touch LDS wait for every outstanding
+      // global -> LDS load, the tiles fetched ahead included.  Reads run
+      // kAhead MFMAs ahead; sd_wait_pin waits for the oldest pair.
       const uint32_t sv = v_stage(sl_prev);
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int dt = 0; dt < kD / 32; ++dt) {
-          uint32_t vf[4];
-#pragma unroll
-          for (int r = 0; r < 2; ++r) {
-            const uint32_t ad = sv + vaddr[dt] + (j * 16 + r * 8) * kRowB;
-            const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (SD_AS3 s16x4 *)(uintptr_t)ad);
-            const u32x2 w2 = __builtin_bit_cast(u32x2, v);
-            vf[2 * r + 0] = w2.x;
-            vf[2 * r + 1] = w2.y;
-          }
-          o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
-        }
-      __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);
-#pragma unroll
-      for (int i = 0; i < kD / 8 - 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      constexpr int kMfmas = 4 * (kD / 32); // j-major, dt-minor
+      constexpr int kAhead = 8;
+      u32x2 vr[kMfmas][2];
+      auto read = [&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        constexpr int j = m / (kD / 32), dt = m % (kD / 32);
+        const uint32_t ad = sv + vaddr[dt];
+        sd_read_tr16<(j * 16 + 0) * kRowB>(vr[m][0], ad);
+        sd_read_tr16<(j * 16 + 8) * kRowB>(vr[m][1], ad);
+      };
+      sd_static_for<kAhead>(read);
+      sd_static_for<kMfmas>([&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        constexpr int j = m / (kD / 32), dt = m % (kD / 32);
+        constexpr int left = kMfmas - 1 - m < kAhead - 1 ? kMfmas - 1 - m : kAhead - 1;
+        sd_wait_pin<2 * left>(vr[m][0], vr[m][1]);
+        const uint32_t vf[4] = {vr[m][0].x, vr[m][0].y, vr[m][1].x, vr[m][1].y};
+        o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
+        __builtin_amdgcn_sched_barrier(0); // keep the MFMA at its wait
+        if constexpr (m + kAhead < kMfmas)
+          read(std::integral_constant<int, m + kAhead>{});
+      });
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
-    // wavefronts 4..7 issued their newest loads a phase ago and the tiles are
-    // needed after this barrier
-    if (team)
-      __builtin_amdgcn_s_waitcnt(sd_wait_imm(0));
-    sd_barrier();
+    // wavefronts 4..7 end their round here: everything but the loads of this
+    // round has landed
+    if (team) {
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+      sd_barrier();
+    }
     if (t == tiles)
       break;
 
     // ---- vector-ALU phase -------------------------------------------------------
-    issue_k(t + 2, sl_prev);
-    issue_v(t + 1, sl_next);
-    sl_prev = sl_cur;
-    sl_cur = sl_next;
-    sl_next = next_slot(sl_next);
     if (active(t)) {
       const int kv0 = t * kBKV;
       const bool edge = (CAUSAL && kv0 + kBKV - 1 > qw0) || kv0 + kBKV > g.Skv;
@@ -417,10 +437,16 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
         for (int r = 0; r < 16; ++r)
           mx = fmaxf(mx, s[kb][r]);
       mx = sd_half_max(mx);
-      const float m_new = fmaxf(m_run, mx);
+      // The reference point of the exponentials follows the row maximum
+      // lazily: it moves only when the maximum has risen by more than
+      // kMaxSlack (in log2 units of the scaled scores).  Probabilities are
+      // then at most 2^kMaxSlack, sums and outputs stay far inside float
+      // range, and O = sum(p v) / sum(p) does not depend on the reference
+      // point; the rescaling of O^T becomes rare.
+      const bool moved = (mx - m_run) * g.scale_log2e > kMaxSlack;
+      const float m_new = moved ? mx : m_run;
       const float mc = m_new * g.scale_log2e;
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * g.scale_log2e);
-      const bool moved = m_new > m_run;
       m_run = m_new;
       float psum = 0.f;
 #pragma unroll
@@ -443,13 +469,16 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
             o[dt][r] *= alpha;
       }
     }
-    // wavefronts 0..3: everything but the loads just issued has landed (the
-    // older batch is needed after the next barrier but one)
-    if (!team)
+    // wavefronts 0..3 end their round here
+    if (!team) {
       __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
-    sd_barrier();
+      sd_barrier();
+    }
+    sl_prev = sl_cur;
+    sl_cur = sl_next;
+    sl_next = next_slot(sl_next);
   }
-  if (!team)
+  if (!team) // pairs with the last barrier of wavefronts 4..7
     __builtin_amdgcn_s_barrier();
 
   // ---- epilogue: O = O^T / l, through LDS for row-contiguous stores -----------
