@@ -435,12 +435,15 @@ template <typename T, int WPR, int CHUNKS>
 void rownorm_launch_one(int variant, int64_t rows, hipStream_t s,
                         const RowNormArgs &g) {
   constexpr int rpw = RowNormGeom<WPR>::kRowsPerWg;
-  // LayerNorm workgroups walk two or more rows with scale and bias in
-  // registers (measured: 27.2 -> 24.3 us on 8192 x 4096 bf16); the RMSNorm
-  // variants are fastest with one row-block per workgroup.
-  // FUSILLI_HIP_ROWNORM_WGS_PER_CU overrides the workgroups per compute unit.
+  // Workgroups walk the row-blocks with the per-column parameters in
+  // registers.  The grid is capped at a number of workgroups per compute unit
+  // that leaves them UNEVEN shares of a large tensor (1 or 2 row-blocks each on
+  // 8192 rows), which staggers their read and write bursts; measured on
+  // 8192 x 4096 bf16, workgroups per CU -> us: LayerNorm 32: 25.0, 16: 24.3,
+  // 20: 23.95; RMSNorm + MUL 32: 23.5, 20: 23.2, 24: 23.05.
+  // FUSILLI_HIP_ROWNORM_WGS_PER_CU overrides it (0: one row-block each).
   int64_t blocks = (rows + rpw - 1) / rpw;
-  int per_cu = variant == RN_LN_SCALE_BIAS ? 16 : 0;
+  int per_cu = variant == RN_LN_SCALE_BIAS ? 20 : 24;
   if (const char *env = getenv("FUSILLI_HIP_ROWNORM_WGS_PER_CU"))
     per_cu = atoi(env);
   if (per_cu > 0 && blocks > 256ll * per_cu)
