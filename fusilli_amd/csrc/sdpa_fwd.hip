@@ -170,9 +170,34 @@ __device__ __forceinline__ void sd_read_tr16(u32x2 &dst, uint32_t addr) {
                : "=v"(dst)
                : "v"(addr), "n"(OFFSET));
 }
-template <int N> __device__ __forceinline__ void sd_wait_pin(u32x2 &a, u32x2 &b) {
+template <int OFFSET>
+__device__ __forceinline__ void sd_read_b128(u32x4 &dst, uint32_t addr) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "16-bit offset field");
+  asm volatile("ds_read_b128 %0, %1 offset:%2"
+               : "=v"(dst)
+               : "v"(addr), "n"(OFFSET));
+}
+template <int N, typename... R>
+__device__ __forceinline__ void sd_wait_pin(R &...regs) {
   static_assert(N >= 0 && N <= 15, "lgkmcnt is a 4-bit field");
-  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+  if constexpr (sizeof...(R) == 4) {
+    auto f = [](auto &a, auto &b, auto &c, auto &d) {
+      asm volatile("s_waitcnt lgkmcnt(%4)"
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d)
+                   : "n"(N));
+    };
+    f(regs...);
+  } else {
+    static_assert(sizeof...(R) == 8, "four or eight register tuples");
+    auto f = [](auto &a, auto &b, auto &c, auto &d, auto &e, auto &g, auto &h,
+                auto &i) {
+      asm volatile("s_waitcnt lgkmcnt(%8)"
+                   : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(g),
+                     "+v"(h), "+v"(i)
+                   : "n"(N));
+    };
+    f(regs...);
+  }
 }
 
 // Workgroup barrier without the release fence's "wait for everything": the
@@ -351,6 +376,12 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     // ---- MFMA phase -----------------------------------------------------------
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(2);
+    // Fragment reads of both blocks are written as asm: the compiler neither
+    // sees them as LDS accesses (it would make the transposing reads wait for
+    // every outstanding global -> LDS load, the tiles fetched ahead included)
+    // nor waits for them; reads run kAhead MFMAs ahead, and one sd_wait_pin
+    // per kGroup MFMAs waits for that group's fragments.
+    constexpr int kAhead = 8, kGroup = 4;
     if (t < tiles && active(t)) {
       const uint32_t sk = k_stage(sl_cur);
 #pragma unroll
@@ -358,32 +389,35 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           s[kb][r] = 0.f;
+      constexpr int kMfmas = 2 * (kD / 16); // ds-major, kb-minor
+      u32x4 kr[kMfmas];
+      auto read = [&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        sd_read_b128<(m % 2) * 32 * kRowB>(kr[m], sk + kaddr[m / 2]);
+      };
+      sd_static_for<kAhead>(read);
+      sd_static_for<kMfmas / kGroup>([&](auto gc) {
+        constexpr int m0 = decltype(gc)::value * kGroup;
+        constexpr int rest = kMfmas - (m0 + kGroup);
+        constexpr int left = rest < kAhead - kGroup ? rest : kAhead - kGroup;
+        sd_wait_pin<left>(kr[m0], kr[m0 + 1], kr[m0 + 2], kr[m0 + 3]);
 #pragma unroll
-      for (int ds = 0; ds < kD / 16; ++ds)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-          const u32x4 v = *(const SD_AS3 u32x4 *)(uintptr_t)(sk + kaddr[ds] +
-                                                             kb * 32 * kRowB);
-          const uint32_t kf[4] = {v.x, v.y, v.z, v.w};
-          s[kb] = sd_mfma<BF16>(kf, qf[ds], s[kb]);
+        for (int i = 0; i < kGroup; ++i) {
+          const int m = m0 + i;
+          const uint32_t kf[4] = {kr[m].x, kr[m].y, kr[m].z, kr[m].w};
+          s[m % 2] = sd_mfma<BF16>(kf, qf[m / 2], s[m % 2]);
         }
-      // fragment reads run eight MFMAs ahead, no further (registers)
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-      for (int i = 0; i < kD / 8 - 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        __builtin_amdgcn_sched_barrier(0); // keep the MFMAs at their wait
+        sd_static_for<kGroup>([&](auto ic) {
+          constexpr int m = m0 + kAhead + decltype(ic)::value;
+          if constexpr (m < kMfmas)
+            read(std::integral_constant<int, m>{});
+        });
+      });
     }
     if (t > 0 && active(t - 1)) {
-      // V^T fragments by transposing reads written as asm: the compiler would
-      // make a read it knows to touch LDS wait for every outstanding
-      // global -> LDS load, the tiles fetched ahead included.  Reads run
-      // kAhead MFMAs ahead; sd_wait_pin waits for the oldest pair.
       const uint32_t sv = v_stage(sl_prev);
       constexpr int kMfmas = 4 * (kD / 32); // j-major, dt-minor
-      constexpr int kAhead = 8;
       u32x2 vr[kMfmas][2];
       auto read = [&](auto mc) {
         constexpr int m = decltype(mc)::value;
@@ -393,16 +427,26 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
         sd_read_tr16<(j * 16 + 8) * kRowB>(vr[m][1], ad);
       };
       sd_static_for<kAhead>(read);
-      sd_static_for<kMfmas>([&](auto mc) {
-        constexpr int m = decltype(mc)::value;
-        constexpr int j = m / (kD / 32), dt = m % (kD / 32);
-        constexpr int left = kMfmas - 1 - m < kAhead - 1 ? kMfmas - 1 - m : kAhead - 1;
-        sd_wait_pin<2 * left>(vr[m][0], vr[m][1]);
-        const uint32_t vf[4] = {vr[m][0].x, vr[m][0].y, vr[m][1].x, vr[m][1].y};
-        o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
-        __builtin_amdgcn_sched_barrier(0); // keep the MFMA at its wait
-        if constexpr (m + kAhead < kMfmas)
-          read(std::integral_constant<int, m + kAhead>{});
+      sd_static_for<kMfmas / kGroup>([&](auto gc) {
+        constexpr int m0 = decltype(gc)::value * kGroup;
+        constexpr int rest = kMfmas - (m0 + kGroup);
+        constexpr int left = rest < kAhead - kGroup ? rest : kAhead - kGroup;
+        sd_wait_pin<2 * left>(vr[m0][0], vr[m0][1], vr[m0 + 1][0], vr[m0 + 1][1],
+                              vr[m0 + 2][0], vr[m0 + 2][1], vr[m0 + 3][0],
+                              vr[m0 + 3][1]);
+#pragma unroll
+        for (int i = 0; i < kGroup; ++i) {
+          const int m = m0 + i;
+          const int j = m / (kD / 32), dt = m % (kD / 32);
+          const uint32_t vf[4] = {vr[m][0].x, vr[m][0].y, vr[m][1].x, vr[m][1].y};
+          o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        sd_static_for<kGroup>([&](auto ic) {
+          constexpr int m = m0 + kAhead + decltype(ic)::value;
+          if constexpr (m < kMfmas)
+            read(std::integral_constant<int, m>{});
+        });
       });
     }
     __builtin_amdgcn_s_setprio(0);
