@@ -533,6 +533,204 @@ TEST("config 5a (reduced): int8 matmul is bit exact") {
   CHECK(exact);
 }
 
+// worst violation of |got - ref| <= rtol * (|ref| + rms(ref)); <= 0 passes
+template <typename T>
+static double worstViolation(const std::vector<T> &got,
+                             const std::vector<double> &ref, double rtol) {
+  double rms = 0, worst = -1;
+  for (double r : ref)
+    rms += r * r;
+  rms = std::sqrt(rms / (ref.empty() ? 1 : ref.size()));
+  if (got.size() != ref.size())
+    return 1e30;
+  for (size_t i = 0; i < ref.size(); ++i)
+    worst = std::max(worst, std::fabs((double)(float)got[i] - ref[i]) -
+                                rtol * (std::fabs(ref[i]) + rms));
+  return worst;
+}
+
+TEST("config 2 (reduced): bf16 rmsnorm + scalar MUL is one kernel, vs host loop") {
+  const int64_t rows = 96, cols = 4096;
+  const float eps = 1e-6f, mul = 0.5f;
+  Graph g = newGraph("cfg2", DataType::BFloat16, DataType::Float);
+  auto X = g.tensor(mk("x", {rows, cols}, {cols, 1}, DataType::BFloat16));
+  auto S = g.tensor(mk("s", {1, cols}, {cols, 1}, DataType::BFloat16));
+  RmsnormAttr ra;
+  ra.setForwardPhase(NormFwdPhase::INFERENCE).setEpsilon(g.tensor(TensorAttr(eps)));
+  auto [Y, R] = g.rmsnorm(X, S, ra);
+  (void)R;
+  PointwiseAttr pm;
+  pm.setMode(PointwiseAttr::Mode::MUL);
+  auto O = g.pointwise(Y, g.tensor(TensorAttr(mul)), pm);
+  O->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  auto xf = randomVec(rows * cols, 21, -3.f, 3.f), sf = randomVec(cols, 22, 0.9f, 1.1f);
+  std::vector<bf16> xb(xf.size()), sb(sf.size());
+  for (size_t i = 0; i < xf.size(); ++i) xb[i] = (bf16)xf[i], xf[i] = (float)xb[i];
+  for (size_t i = 0; i < sf.size(); ++i) sb[i] = (bf16)sf[i], sf[i] = (float)sb[i];
+  Pack pack = {{X, bufOf(X, xb)}, {S, bufOf(S, sb)}, {O, fill(O, bf16(0.f))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<bf16>(pack[O]);
+  std::vector<double> ref(rows * cols);
+  for (int64_t r = 0; r < rows; ++r) {
+    double ss = 0;
+    for (int64_t c = 0; c < cols; ++c)
+      ss += (double)xf[r * cols + c] * xf[r * cols + c];
+    const double inv = 1.0 / std::sqrt(ss / cols + eps);
+    for (int64_t c = 0; c < cols; ++c)
+      ref[r * cols + c] = xf[r * cols + c] * inv * sf[c] * mul;
+  }
+  CHECK(worstViolation(out, ref, 2e-2) <= 0.0);
+}
+
+TEST("config 4 (reduced): bf16 causal sdpa B1 H2 S320 D128 vs host loop") {
+  const int64_t b = 1, h = 2, s = 320, d = 128;
+  Graph g = newGraph("cfg4", DataType::BFloat16, DataType::Float);
+  const Dims dims = {b, h, s, d};
+  auto Q = g.tensor(mk("q", dims, contig(dims), DataType::BFloat16));
+  auto K = g.tensor(mk("k", dims, contig(dims), DataType::BFloat16));
+  auto V = g.tensor(mk("v", dims, contig(dims), DataType::BFloat16));
+  SdpaAttr sa;
+  sa.setIsCausal(true);
+  auto O = g.sdpa(Q, K, V, nullptr, sa);
+  O->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  const size_t n = b * h * s * d;
+  auto qf = randomVec(n, 31, -1.f, 1.f), kf = randomVec(n, 32, -1.f, 1.f),
+       vf = randomVec(n, 33, -1.f, 1.f);
+  std::vector<bf16> qb(n), kb(n), vb(n);
+  for (size_t i = 0; i < n; ++i) {
+    qb[i] = (bf16)qf[i], qf[i] = (float)qb[i];
+    kb[i] = (bf16)kf[i], kf[i] = (float)kb[i];
+    vb[i] = (bf16)vf[i], vf[i] = (float)vb[i];
+  }
+  Pack pack = {{Q, bufOf(Q, qb)}, {K, bufOf(K, kb)}, {V, bufOf(V, vb)},
+               {O, fill(O, bf16(0.f))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<bf16>(pack[O]);
+  std::vector<double> ref(n, 0.0), p(s);
+  const double scale = 1.0 / std::sqrt((double)d);
+  for (int64_t hh = 0; hh < b * h; ++hh)
+    for (int64_t i = 0; i < s; ++i) { // samples/sdpa_utils.cpp:49-102
+      double mx = -1e300, sum = 0;
+      for (int64_t j = 0; j <= i; ++j) {
+        double acc = 0;
+        for (int64_t c = 0; c < d; ++c)
+          acc += (double)qf[(hh * s + i) * d + c] * kf[(hh * s + j) * d + c];
+        p[j] = acc * scale;
+        mx = std::max(mx, p[j]);
+      }
+      for (int64_t j = 0; j <= i; ++j)
+        p[j] = std::exp(p[j] - mx), sum += p[j];
+      for (int64_t j = 0; j <= i; ++j)
+        for (int64_t c = 0; c < d; ++c)
+          ref[(hh * s + i) * d + c] += p[j] / sum * vf[(hh * s + j) * d + c];
+    }
+  CHECK(worstViolation(out, ref, 2e-2) <= 0.0);
+}
+
+// e4m3fn byte of the nearest representable value (round to nearest even,
+// saturating at 448), by search over the 127 non-negative finite codes
+static uint8_t toE4m3(float x) {
+  auto val = [](int code) {
+    const int e = code >> 3, m = code & 7;
+    return e == 0 ? std::ldexp(m / 8.0, -6) : std::ldexp(1.0 + m / 8.0, e - 7);
+  };
+  const double a = std::fabs((double)x);
+  int best = 0;
+  for (int code = 1; code <= 0x7e; ++code) {
+    const double db = std::fabs(val(best) - a), dc = std::fabs(val(code) - a);
+    if (dc < db || (dc == db && (code & 1) == 0))
+      best = code;
+  }
+  return (uint8_t)(best | (x < 0 ? 0x80 : 0));
+}
+static double fromE4m3(uint8_t bits) {
+  const int code = bits & 0x7f, e = code >> 3, m = code & 7;
+  const double v = e == 0 ? std::ldexp(m / 8.0, -6) : std::ldexp(1.0 + m / 8.0, e - 7);
+  return bits & 0x80 ? -v : v;
+}
+
+TEST("config 5b (reduced): fp8 e4m3 matmul x scale -> bf16 is one kernel, vs host loop") {
+  const int64_t m = 256, k = 512, n = 384;
+  Graph g = newGraph("cfg5b", DataType::FP8E4M3, DataType::Float);
+  auto A = g.tensor(mk("a", {m, k}, {k, 1}, DataType::FP8E4M3));
+  auto B = g.tensor(mk("b", {k, n}, {n, 1}, DataType::FP8E4M3));
+  MatmulAttr ma;
+  auto C = g.matmul(A, B, ma);
+  C->setDataType(DataType::Float);
+  const float sa = 1.5f / 448.f, sb = 0.75f / 448.f;
+  PointwiseAttr pm;
+  pm.setMode(PointwiseAttr::Mode::MUL);
+  auto O = g.pointwise(C, g.tensor(TensorAttr(sa * sb)), pm);
+  O->setOutput(true).setDataType(DataType::BFloat16);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  auto af = randomVec(m * k, 41, -448.f, 448.f), bf = randomVec(k * n, 42, -448.f, 448.f);
+  std::vector<fp8e4m3> a8(af.size()), b8(bf.size());
+  for (size_t i = 0; i < af.size(); ++i) a8[i].bits = toE4m3(af[i]);
+  for (size_t i = 0; i < bf.size(); ++i) b8[i].bits = toE4m3(bf[i]);
+  Pack pack = {{A, bufOf(A, a8)}, {B, bufOf(B, b8)}, {O, fill(O, bf16(0.f))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<bf16>(pack[O]);
+  std::vector<double> ref(m * n, 0.0);
+  for (int64_t i = 0; i < m; ++i)
+    for (int64_t kk = 0; kk < k; ++kk) {
+      const double av = fromE4m3(a8[i * k + kk].bits);
+      for (int64_t j = 0; j < n; ++j)
+        ref[i * n + j] += av * fromE4m3(b8[kk * n + j].bits);
+    }
+  for (double &r : ref)
+    r *= (double)(sa * sb);
+  CHECK(worstViolation(out, ref, 2e-2) <= 0.0);
+}
+
+TEST("fused chain: bf16 matmul -> add bias -> gelu -> mul scalar is one kernel") {
+  const int64_t m = 256, k = 256, n = 384;
+  Graph g = newGraph("chain4", DataType::BFloat16, DataType::Float);
+  auto A = g.tensor(mk("a", {m, k}, {k, 1}, DataType::BFloat16));
+  auto B = g.tensor(mk("b", {k, n}, {n, 1}, DataType::BFloat16));
+  auto Bias = g.tensor(mk("bias", {1, n}, {n, 1}, DataType::BFloat16));
+  MatmulAttr ma;
+  PointwiseAttr add, gelu, mul;
+  add.setMode(PointwiseAttr::Mode::ADD);
+  gelu.setMode(PointwiseAttr::Mode::GELU_FWD);
+  mul.setMode(PointwiseAttr::Mode::MUL);
+  auto C = g.matmul(A, B, ma);
+  auto O = g.pointwise(g.pointwise(g.pointwise(C, Bias, add), gelu),
+                       g.tensor(TensorAttr(0.25f)), mul);
+  O->setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  auto af = randomVec(m * k, 51, -1.f, 1.f), bf = randomVec(k * n, 52, -0.2f, 0.2f),
+       cf = randomVec(n, 53, -1.f, 1.f);
+  std::vector<bf16> ab(af.size()), bb(bf.size()), cb(cf.size());
+  for (size_t i = 0; i < af.size(); ++i) ab[i] = (bf16)af[i], af[i] = (float)ab[i];
+  for (size_t i = 0; i < bf.size(); ++i) bb[i] = (bf16)bf[i], bf[i] = (float)bb[i];
+  for (size_t i = 0; i < cf.size(); ++i) cb[i] = (bf16)cf[i], cf[i] = (float)cb[i];
+  Pack pack = {{A, bufOf(A, ab)}, {B, bufOf(B, bb)}, {Bias, bufOf(Bias, cb)},
+               {O, fill(O, bf16(0.f))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<bf16>(pack[O]);
+  std::vector<double> ref(m * n, 0.0);
+  for (int64_t i = 0; i < m; ++i)
+    for (int64_t kk = 0; kk < k; ++kk)
+      for (int64_t j = 0; j < n; ++j)
+        ref[i * n + j] += (double)af[i * k + kk] * bf[kk * n + j];
+  for (int64_t i = 0; i < m; ++i)
+    for (int64_t j = 0; j < n; ++j) {
+      const double x = ref[i * n + j] + cf[j];
+      ref[i * n + j] = 0.25 * 0.5 * x * (1.0 + std::erf(x / std::sqrt(2.0)));
+    }
+  CHECK(worstViolation(out, ref, 2e-2) <= 0.0);
+}
+
 TEST("unfused chain uses the workspace for virtual tensors") {
   Graph g = newGraph("chain", DataType::Float);
   auto A = g.tensor(mk("a", {64, 32}, {32, 1}, DataType::Float));
