@@ -7,7 +7,8 @@
 //   name,iter,dispatch_count,avg_us,work,unit_per_s
 // `dispatch_count` is the number of kernels the plan launches per execute.
 // Inputs are constant fills like the reference's.  Extras beyond the
-// reference: `rmsnorm` subcommand, `--relu` for conv, int8 / fp8 matmul types.
+// reference: `rmsnorm` subcommand (`--mul s` fuses a scalar multiply), `--relu`
+// for conv, int8 / fp8 matmul types, `--out_scale s` (matmul output x scalar).
 #include <fusilli.h>
 
 #include <cstdio>
@@ -211,6 +212,12 @@ void runConv(const Handle &h, const Args &a, int iter) {
     rl.setMode(PointwiseAttr::Mode::RELU_FWD);
     Y = g.pointwise(Y, rl);
   }
+  if (a.has("--mul")) { // y * scalar fused behind the norm
+    PointwiseAttr mul;
+    mul.setMode(PointwiseAttr::Mode::MUL);
+    Y = g.pointwise(
+        Y, g.tensor(TensorAttr((float)std::atof(a.s("--mul", "", "1").c_str()))), mul);
+  }
   Y->setOutput(true).setDataType(dt);
   OK(g.validate());
   pack[X] = constant(h, X, 1.f);
@@ -246,6 +253,14 @@ void runMatmul(const Handle &h, const Args &a, int iter) {
     PointwiseAttr add;
     add.setMode(PointwiseAttr::Mode::ADD);
     C = g.pointwise(C, bias, add);
+  }
+  if (a.has("--out_scale")) { // C * scalar, as the fp8 configuration dequantises
+    PointwiseAttr mul;
+    mul.setMode(PointwiseAttr::Mode::MUL);
+    C->setDataType(DataType::Float);
+    C = g.pointwise(
+        C, g.tensor(TensorAttr((float)std::atof(a.s("--out_scale", "", "1").c_str()))),
+        mul);
   }
   C->setOutput(true).setDataType(ot);
   OK(g.validate());
@@ -322,6 +337,12 @@ void runNorm(const Handle &h, const Args &a, int iter, bool layer) {
     ra.setEpsilon(eps).setForwardPhase(NormFwdPhase::INFERENCE);
     auto outs = g.rmsnorm(X, S, ra);
     Y = outs[0];
+  }
+  if (a.has("--mul")) { // y * scalar fused behind the norm
+    PointwiseAttr mul;
+    mul.setMode(PointwiseAttr::Mode::MUL);
+    Y = g.pointwise(
+        Y, g.tensor(TensorAttr((float)std::atof(a.s("--mul", "", "1").c_str()))), mul);
   }
   Y->setOutput(true).setDataType(dt);
   OK(g.validate());
