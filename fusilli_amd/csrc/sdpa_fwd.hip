@@ -219,7 +219,9 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   constexpr int kLoadsPerTile = C::kLoadsPerTile, kOutPitch = C::kOutPitch;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
-  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63;
+  // wave index as a scalar: everything derived from it stays in SGPRs
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l = threadIdx.x & 63;
   const int half = l >> 5, lq = l & 31;
   // Causal masks: a workgroup runs query tile (last - z) and then tile z, a
   // long and a short one, so all workgroups do the same work (tiles of one
@@ -277,25 +279,30 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     voff[j] = (uint32_t)(row * v_rowb + (sd_vchunk<HD>(row, p) << 4));
   }
   // K tiles live in stages [0, kStages), V tiles in [kStages, 2 kStages).
-  // Rows at or past Skv (and tiles past the end) read as zeros.
-  auto issue_kv = [&](const char *base, int64_t rowb, int64_t bytes,
-                      const uint32_t (&off)[kLoadsPerTile], int t,
-                      uint32_t stage) {
-    const int64_t kv0 = (int64_t)t * kBKV;
-    int64_t nb = bytes - kv0 * rowb;
-    nb = t < tiles && nb > 0 ? nb : 0;
-    const uint64_t b64 = (uint64_t)(base + kv0 * rowb);
+  // One buffer descriptor per operand covers the whole (batch, head) slab; the
+  // tile's byte offset is added to the lanes' offsets.  Rows at or past Skv
+  // read as zeros (out of the descriptor's range), and so do whole tiles past
+  // the end, whose offset is pushed out of range.
+  auto slab_rsrc = [&](const char *base, int64_t bytes) {
+    const uint64_t b64 = (uint64_t)base;
     const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64);
     const uint32_t bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
-    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+    return __builtin_amdgcn_make_buffer_rsrc(
         (void *)(((uint64_t)bhi << 32) | blo), 0,
-        (int)__builtin_amdgcn_readfirstlane((uint32_t)nb), 0x00020000);
+        (int)__builtin_amdgcn_readfirstlane((uint32_t)bytes), 0x00020000);
+  };
+  const __amdgpu_buffer_rsrc_t k_rsrc = slab_rsrc(kp, k_bytes);
+  const __amdgpu_buffer_rsrc_t v_rsrc = slab_rsrc(vp, v_bytes);
+  auto issue_kv = [&](const __amdgpu_buffer_rsrc_t &r, uint32_t tile_bytes,
+                      const uint32_t (&off)[kLoadsPerTile], int t,
+                      uint32_t stage) {
+    const uint32_t toff = t < tiles ? (uint32_t)t * tile_bytes : 0x80000000u;
 #pragma unroll
     for (int j = 0; j < kLoadsPerTile; ++j) {
       const uint32_t dst = stage + (uint32_t)(j * kWaves + wave) * 1024u;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           r, (SD_AS3 char *)(uintptr_t)__builtin_amdgcn_readfirstlane(dst), 16,
-          (int)off[j], 0, 0, 0);
+          (int)(off[j] + toff), 0, 0, 0);
     }
   };
   // ring slot (0 .. kStages - 1) -> LDS address
@@ -304,10 +311,10 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     return lds0 + (uint32_t)(kStages + slot) * kTileB;
   };
   auto issue_k = [&](int t, int slot) {
-    issue_kv(kp, k_rowb, k_bytes, koff, t, k_stage(slot));
+    issue_kv(k_rsrc, (uint32_t)(kBKV * k_rowb), koff, t, k_stage(slot));
   };
   auto issue_v = [&](int t, int slot) {
-    issue_kv(vp, v_rowb, v_bytes, voff, t, v_stage(slot));
+    issue_kv(v_rsrc, (uint32_t)(kBKV * v_rowb), voff, t, v_stage(slot));
   };
   auto next_slot = [](int s) { return s + 1 == kStages ? 0 : s + 1; };
 
