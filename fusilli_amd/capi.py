@@ -184,6 +184,12 @@ SYMBOLS = {
     "fhip_conv_fprop_workspace_size": (c_int, [POINTER(ConvDesc), POINTER(c_size_t)]),
     "fhip_conv_fprop_supported": (c_int, [POINTER(ConvDesc)]),
     "fhip_conv_fprop": (c_int, [_P, POINTER(ConvDesc), _P, _P, POINTER(_P), _P, _P, c_size_t]),
+    "fhip_conv_dgrad_workspace_size": (c_int, [POINTER(ConvDesc), POINTER(c_size_t)]),
+    "fhip_conv_dgrad_supported": (c_int, [POINTER(ConvDesc)]),
+    "fhip_conv_dgrad": (c_int, [_P, POINTER(ConvDesc), _P, _P, _P, _P, c_size_t]),
+    "fhip_conv_wgrad_workspace_size": (c_int, [POINTER(ConvDesc), POINTER(c_size_t)]),
+    "fhip_conv_wgrad_supported": (c_int, [POINTER(ConvDesc)]),
+    "fhip_conv_wgrad": (c_int, [_P, POINTER(ConvDesc), _P, _P, _P, _P, c_size_t]),
     "fhip_sdpa_fwd_workspace_size": (c_int, [POINTER(SdpaDesc), POINTER(c_size_t)]),
     "fhip_sdpa_fwd_supported": (c_int, [POINTER(SdpaDesc)]),
     "fhip_sdpa_fwd": (c_int, [_P, POINTER(SdpaDesc), _P, _P, _P, _P, _P, _P, c_size_t]),
@@ -360,6 +366,14 @@ class Context:
         self._check(self.lib.fhip_conv_fprop(self.handle, byref(d), _p(x), _p(w),
                                              _epi_ptrs(epilogue_operands),
                                              _p(out), None, 0))
+
+    def conv_dgrad(self, d: ConvDesc, dy, w, dx):
+        self._check(self.lib.fhip_conv_dgrad(self.handle, byref(d), _p(dy),
+                                             _p(w), _p(dx), None, 0))
+
+    def conv_wgrad(self, d: ConvDesc, dy, x, dw):
+        self._check(self.lib.fhip_conv_wgrad(self.handle, byref(d), _p(dy),
+                                             _p(x), _p(dw), None, 0))
 
     def sdpa_fwd(self, d: SdpaDesc, q, k, v, o, mask=None):
         self._check(self.lib.fhip_sdpa_fwd(self.handle, byref(d), _p(q), _p(k),

@@ -361,6 +361,114 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// --------------------------------------------------------------------------
+// convolution backward: data gradient and weight gradient of the forward
+// above (reference node/conv_node.h:255-598; aten.convolution_backward).
+// Both are gathers with f32 accumulation, no atomics.
+// --------------------------------------------------------------------------
+struct ConvBwdArgs {
+  Dims out;          // dgrad: DX [N, C, sp..]; wgrad: DW [K, fC, fsp..]
+  Strides x, w, y;   // strides of X / DX, W / DW, DY
+  int64_t x_dim[FHIP_MAX_RANK];
+  int64_t w_dim[FHIP_MAX_RANK];
+  int64_t y_dim[FHIP_MAX_RANK];
+  int32_t spatial;
+  int64_t pad[3], str[3], dil[3];
+  int64_t groups;
+  int32_t x_dt, w_dt, y_dt;
+};
+
+// DX[n, c, i..] = sum over k of c's group, filter taps f with
+// i + pad - f * dil = o * stride:  DY[n, k, o..] * W[k, c % fC, f..]
+__global__ void generic_conv_dgrad_kernel(ConvBwdArgs g, const void *dy,
+                                          const void *w, void *dx,
+                                          int64_t total) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= total)
+    return;
+  int64_t coord[FHIP_MAX_RANK];
+  unravel(lin, g.out, coord);
+  const int sp = g.spatial;
+  const int64_t n = coord[0], c = coord[1];
+  const int64_t fC = g.w_dim[1];
+  const int64_t kPerGroup = g.w_dim[0] / g.groups;
+  const int64_t grp = c / fC, fc = c - grp * fC;
+  int64_t fvol = 1;
+  for (int i = 0; i < sp; ++i)
+    fvol *= g.w_dim[2 + i];
+  float acc = 0.f;
+  for (int64_t f = 0; f < fvol; ++f) {
+    int64_t rem = f;
+    int64_t yo = n * g.y.s[0];
+    int64_t wo = fc * g.w.s[1];
+    bool hit = true;
+    for (int i = sp - 1; i >= 0; --i) {
+      const int64_t fd = g.w_dim[2 + i];
+      const int64_t fi = rem % fd;
+      rem /= fd;
+      const int64_t t = coord[2 + i] + g.pad[i] - fi * g.dil[i];
+      const int64_t o = t / g.str[i];
+      if (t < 0 || o * g.str[i] != t || o >= g.y_dim[2 + i])
+        hit = false;
+      yo += o * g.y.s[2 + i];
+      wo += fi * g.w.s[2 + i];
+    }
+    if (!hit)
+      continue;
+    for (int64_t kk = 0; kk < kPerGroup; ++kk) {
+      const int64_t k = grp * kPerGroup + kk;
+      acc += fhip_load<float>(dy, g.y_dt, yo + k * g.y.s[1]) *
+             fhip_load<float>(w, g.w_dt, wo + k * g.w.s[0]);
+    }
+  }
+  fhip_store<float>(dx, g.x_dt, dot(coord, g.x, g.out.rank), acc);
+}
+
+// DW[k, fc, f..] = sum over n, o..:  DY[n, k, o..] * X[n, c, o * stride - pad +
+// f * dil] with c = group(k) * fC + fc.  One workgroup per DW element.
+__global__ __launch_bounds__(256) void generic_conv_wgrad_kernel(
+    ConvBwdArgs g, const void *dy, const void *x, void *dw) {
+  __shared__ float part[4];
+  int64_t coord[FHIP_MAX_RANK];
+  unravel((int64_t)blockIdx.x, g.out, coord);
+  const int sp = g.spatial;
+  const int64_t k = coord[0], fc = coord[1];
+  const int64_t kPerGroup = g.w_dim[0] / g.groups;
+  const int64_t c = (k / kPerGroup) * g.w_dim[1] + fc;
+  int64_t ovol = 1;
+  for (int i = 0; i < sp; ++i)
+    ovol *= g.y_dim[2 + i];
+  const int64_t total = g.y_dim[0] * ovol;
+  float acc = 0.f;
+  for (int64_t it = threadIdx.x; it < total; it += blockDim.x) {
+    int64_t rem = it;
+    int64_t yo = k * g.y.s[1];
+    int64_t xo = c * g.x.s[1];
+    bool inside = true;
+    for (int i = sp - 1; i >= 0; --i) {
+      const int64_t od = g.y_dim[2 + i];
+      const int64_t o = rem % od;
+      rem /= od;
+      const int64_t xi = o * g.str[i] - g.pad[i] + coord[2 + i] * g.dil[i];
+      if (xi < 0 || xi >= g.x_dim[2 + i])
+        inside = false;
+      yo += o * g.y.s[2 + i];
+      xo += xi * g.x.s[2 + i];
+    }
+    const int64_t n = rem;
+    if (inside)
+      acc += fhip_load<float>(dy, g.y_dt, yo + n * g.y.s[0]) *
+             fhip_load<float>(x, g.x_dt, xo + n * g.x.s[0]);
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0)
+    part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    fhip_store<float>(dw, g.w_dt, dot(coord, g.w, g.out.rank),
+                      (part[0] + part[1]) + (part[2] + part[3]));
+}
+
 constexpr int kSdpaMaxDvPerLane = 8; // Dv <= 512
 
 __global__ __launch_bounds__(64) void generic_sdpa_kernel(SdpaArgs g,
@@ -856,6 +964,134 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   const int64_t total = fhip_desc_volume(d->y);
   hipLaunchKernelGGL(generic_conv_kernel, dim3(grid_for(total, 256)), dim3(256),
                      0, ctx->stream, g, x, w, out, total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- conv backward (data and weight gradients) -----------------------------
+// The descriptor names the forward problem: x is X (wgrad input) or DX (dgrad
+// output), w is W (dgrad input) or DW (wgrad output), y is DY.
+static int conv_bwd_validate(fhip_ctx *ctx, const fhip_conv_desc *d,
+                             const char *who) {
+  FHIP_REQUIRE(ctx, d != nullptr, "%s: null descriptor", who);
+  if (!fhip_check_desc(ctx, d->x, "conv X/DX") ||
+      !fhip_check_desc(ctx, d->w, "conv W/DW") ||
+      !fhip_check_desc(ctx, d->y, "conv DY"))
+    return 1;
+  const int sp = d->spatial_rank;
+  FHIP_REQUIRE(ctx, sp >= 1 && sp <= 3, "%s: spatial rank %d", who, sp);
+  FHIP_REQUIRE(ctx,
+               d->x.rank == sp + 2 && d->w.rank == sp + 2 && d->y.rank == sp + 2,
+               "%s: tensor ranks must equal spatial rank + 2", who);
+  FHIP_REQUIRE(ctx, d->epilogue.count == 0,
+               "%s: no pointwise chain can be fused into a gradient", who);
+  const int64_t C = d->x.dim[1], fC = d->w.dim[1], K = d->w.dim[0];
+  FHIP_REQUIRE(ctx, fC > 0 && C % fC == 0,
+               "%s: input channels %lld not divisible by filter channels %lld",
+               who, (long long)C, (long long)fC);
+  const int64_t groups = C / fC;
+  FHIP_REQUIRE(ctx, K % groups == 0,
+               "%s: output channels %lld not divisible by groups %lld", who,
+               (long long)K, (long long)groups);
+  FHIP_REQUIRE(ctx, d->y.dim[0] == d->x.dim[0] && d->y.dim[1] == K,
+               "%s: DY batch/channel dims mismatch", who);
+  for (int i = 0; i < sp; ++i) {
+    FHIP_REQUIRE(ctx, d->stride[i] >= 1 && d->dilation[i] >= 1 &&
+                          d->padding[i] >= 0,
+                 "%s: invalid stride/dilation/padding", who);
+    const int64_t expect =
+        1 + (d->x.dim[2 + i] + 2 * d->padding[i] -
+             d->dilation[i] * (d->w.dim[2 + i] - 1) - 1) /
+                d->stride[i];
+    FHIP_REQUIRE(ctx, d->y.dim[2 + i] == expect,
+                 "%s: DY spatial dim %d is %lld, expected %lld", who, i,
+                 (long long)d->y.dim[2 + i], (long long)expect);
+  }
+  return 0;
+}
+
+static ConvBwdArgs conv_bwd_args(const fhip_conv_desc *d, bool dgrad) {
+  ConvBwdArgs g{};
+  g.out = make_dims(dgrad ? d->x : d->w);
+  g.x = make_strides(d->x);
+  g.w = make_strides(d->w);
+  g.y = make_strides(d->y);
+  for (int i = 0; i < d->x.rank; ++i) {
+    g.x_dim[i] = d->x.dim[i];
+    g.w_dim[i] = d->w.dim[i];
+    g.y_dim[i] = d->y.dim[i];
+  }
+  g.spatial = d->spatial_rank;
+  for (int i = 0; i < 3; ++i) {
+    g.pad[i] = d->padding[i];
+    g.str[i] = d->stride[i];
+    g.dil[i] = d->dilation[i];
+  }
+  g.groups = d->x.dim[1] / d->w.dim[1];
+  g.x_dt = d->x.dtype;
+  g.w_dt = d->w.dtype;
+  g.y_dt = d->y.dtype;
+  return g;
+}
+
+int fhip_conv_dgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_conv_dgrad_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_conv_dgrad_supported(const fhip_conv_desc *d) {
+  return d && conv_bwd_validate(nullptr, d, "fhip_conv_dgrad") == 0 ? 1 : 0;
+}
+
+int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
+                    const void *w, void *dx, void *workspace,
+                    size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_conv_dgrad: null context");
+  if (conv_bwd_validate(ctx, d, "fhip_conv_dgrad") != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, dy && w && dx, "fhip_conv_dgrad: null tensor pointer");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  const ConvBwdArgs g = conv_bwd_args(d, true);
+  const int64_t total = fhip_desc_volume(d->x);
+  hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),
+                     dim3(256), 0, ctx->stream, g, dy, w, dx, total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+int fhip_conv_wgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_conv_wgrad_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_conv_wgrad_supported(const fhip_conv_desc *d) {
+  if (!d || conv_bwd_validate(nullptr, d, "fhip_conv_wgrad") != 0)
+    return 0;
+  // one workgroup per DW element
+  return fhip_desc_volume(d->w) < (1ll << 31) ? 1 : 0;
+}
+
+int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
+                    const void *x, void *dw, void *workspace,
+                    size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_conv_wgrad: null context");
+  if (conv_bwd_validate(ctx, d, "fhip_conv_wgrad") != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, dy && x && dw, "fhip_conv_wgrad: null tensor pointer");
+  const int64_t total = fhip_desc_volume(d->w);
+  FHIP_REQUIRE(ctx, total < (1ll << 31),
+               "fhip_conv_wgrad: %lld filter elements exceed the grid limit",
+               (long long)total);
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  const ConvBwdArgs g = conv_bwd_args(d, false);
+  hipLaunchKernelGGL(generic_conv_wgrad_kernel, dim3((unsigned)total), dim3(256),
+                     0, ctx->stream, g, dy, x, dw);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }

@@ -248,6 +248,25 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                     const void *w, const void *const *epilogue_operands,
                     void *out, void *workspace, size_t workspace_bytes);
 
+/* ---- convolution backward: data gradient (node/conv_node.h:428-598,
+ *      ConvDGradNode) and weight gradient (node/conv_node.h:255-426,
+ *      ConvWGradNode); both lower to aten.convolution_backward in the
+ *      reference.  The descriptor names the forward problem: `x` describes DX
+ *      (dgrad output) or X (wgrad input), `w` describes W (dgrad input) or DW
+ *      (wgrad output), `y` describes DY.  `epilogue` must be empty; `out` and
+ *      `out_dtype` are not read.  f32 accumulation, one rounding to the
+ *      gradient's dtype. -------------------------------------------------- */
+int fhip_conv_dgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes);
+int fhip_conv_dgrad_supported(const fhip_conv_desc *d);
+int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
+                    const void *w, void *dx, void *workspace,
+                    size_t workspace_bytes);
+int fhip_conv_wgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes);
+int fhip_conv_wgrad_supported(const fhip_conv_desc *d);
+int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
+                    const void *x, void *dw, void *workspace,
+                    size_t workspace_bytes);
+
 /* ---- scaled dot-product attention forward (node/sdpa_node.h:36-236;
  *      aten.scaled_dot_product_attention, support/asm_emitter.h:2409-2468) */
 typedef struct {

@@ -255,6 +255,103 @@ void oracle_conv_fprop(const float *x, const float *w, double *y, int64_t N,
     }
 }
 
+/* ---- convolution backward (reference node/conv_node.h:255-598; both nodes
+ *      emit aten.convolution_backward): the adjoints of the forward above.
+ *      Written as the forward loop nest run once more, scattering
+ *      dY[n,k,o] into dX (times W) or into dW (times X) -- the same index
+ *      arithmetic as oracle_conv_fprop, so a gather formulation in a kernel
+ *      is checked against a different derivation.  f64 accumulation. ------ */
+void oracle_conv_dgrad(const float *dy, const float *w, double *dx, int64_t N,
+                       int64_t C, int64_t K, int64_t fC, const int64_t *xd,
+                       const int64_t *fd, const int64_t *od, const int64_t *pad,
+                       const int64_t *str, const int64_t *dil) {
+  const int64_t groups = C / fC;
+  const int64_t kpg = K / groups;
+  const int64_t xvol = xd[0] * xd[1] * xd[2];
+  const int64_t fvol = fd[0] * fd[1] * fd[2];
+  const int64_t ovol = od[0] * od[1] * od[2];
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < N; ++n) {
+    for (int64_t i = 0; i < C * xvol; ++i)
+      dx[n * C * xvol + i] = 0.0;
+    for (int64_t k = 0; k < K; ++k) {
+      const int64_t g = k / kpg;
+      for (int64_t o0 = 0; o0 < od[0]; ++o0)
+        for (int64_t o1 = 0; o1 < od[1]; ++o1)
+          for (int64_t o2 = 0; o2 < od[2]; ++o2) {
+            const double gy =
+                dy[(n * K + k) * ovol + (o0 * od[1] + o1) * od[2] + o2];
+            for (int64_t fc = 0; fc < fC; ++fc) {
+              double *xc = dx + (n * C + g * fC + fc) * xvol;
+              const float *wc = w + (k * fC + fc) * fvol;
+              for (int64_t f0 = 0; f0 < fd[0]; ++f0) {
+                const int64_t i0 = o0 * str[0] - pad[0] + f0 * dil[0];
+                if (i0 < 0 || i0 >= xd[0])
+                  continue;
+                for (int64_t f1 = 0; f1 < fd[1]; ++f1) {
+                  const int64_t i1 = o1 * str[1] - pad[1] + f1 * dil[1];
+                  if (i1 < 0 || i1 >= xd[1])
+                    continue;
+                  for (int64_t f2 = 0; f2 < fd[2]; ++f2) {
+                    const int64_t i2 = o2 * str[2] - pad[2] + f2 * dil[2];
+                    if (i2 < 0 || i2 >= xd[2])
+                      continue;
+                    xc[(i0 * xd[1] + i1) * xd[2] + i2] +=
+                        gy * (double)wc[(f0 * fd[1] + f1) * fd[2] + f2];
+                  }
+                }
+              }
+            }
+          }
+    }
+  }
+}
+
+void oracle_conv_wgrad(const float *dy, const float *x, double *dw, int64_t N,
+                       int64_t C, int64_t K, int64_t fC, const int64_t *xd,
+                       const int64_t *fd, const int64_t *od, const int64_t *pad,
+                       const int64_t *str, const int64_t *dil) {
+  const int64_t groups = C / fC;
+  const int64_t kpg = K / groups;
+  const int64_t xvol = xd[0] * xd[1] * xd[2];
+  const int64_t fvol = fd[0] * fd[1] * fd[2];
+  const int64_t ovol = od[0] * od[1] * od[2];
+#pragma omp parallel for schedule(static)
+  for (int64_t k = 0; k < K; ++k) {
+    const int64_t g = k / kpg;
+    for (int64_t i = 0; i < fC * fvol; ++i)
+      dw[k * fC * fvol + i] = 0.0;
+    for (int64_t n = 0; n < N; ++n)
+      for (int64_t o0 = 0; o0 < od[0]; ++o0)
+        for (int64_t o1 = 0; o1 < od[1]; ++o1)
+          for (int64_t o2 = 0; o2 < od[2]; ++o2) {
+            const double gy =
+                dy[(n * K + k) * ovol + (o0 * od[1] + o1) * od[2] + o2];
+            for (int64_t fc = 0; fc < fC; ++fc) {
+              const float *xc = x + (n * C + g * fC + fc) * xvol;
+              double *wc = dw + (k * fC + fc) * fvol;
+              for (int64_t f0 = 0; f0 < fd[0]; ++f0) {
+                const int64_t i0 = o0 * str[0] - pad[0] + f0 * dil[0];
+                if (i0 < 0 || i0 >= xd[0])
+                  continue;
+                for (int64_t f1 = 0; f1 < fd[1]; ++f1) {
+                  const int64_t i1 = o1 * str[1] - pad[1] + f1 * dil[1];
+                  if (i1 < 0 || i1 >= xd[1])
+                    continue;
+                  for (int64_t f2 = 0; f2 < fd[2]; ++f2) {
+                    const int64_t i2 = o2 * str[2] - pad[2] + f2 * dil[2];
+                    if (i2 < 0 || i2 >= xd[2])
+                      continue;
+                    wc[(f0 * fd[1] + f1) * fd[2] + f2] +=
+                        gy * (double)xc[(i0 * xd[1] + i1) * xd[2] + i2];
+                  }
+                }
+              }
+            }
+          }
+  }
+}
+
 /* ---- SDPA: aten.scaled_dot_product_attention (reference
  *      support/asm_emitter.h:2409-2468; CPU formula
  *      samples/sdpa_utils.cpp:49-102):

@@ -58,8 +58,7 @@ _lib = None
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
-            build()
+        build()  # compiles only when the library is missing or stale
         _lib = ctypes.CDLL(_LIB_PATH)
     return _lib
 
@@ -264,6 +263,54 @@ def conv_fprop(x: np.ndarray, w: np.ndarray, padding, stride, dilation) -> np.nd
         pad3(w.shape[2:], 1), pad3(od[2:], 1), pad3(padding, 0),
         pad3(stride, 1), pad3(dilation, 1))
     return y
+
+
+def _conv_backward(fn, dy, other, x_dims, w_dims, padding, stride, dilation,
+                   out_dims):
+    sp = len(x_dims) - 2
+    assert 1 <= sp <= 3
+    n, c = x_dims[:2]
+    k, fc = w_dims[:2]
+    assert c % fc == 0 and k % (c // fc) == 0
+    od = conv_output_dims(x_dims, w_dims, padding, stride, dilation)
+    assert list(dy.shape) == od, (dy.shape, od)
+    lead = 3 - sp
+
+    def pad3(v, fill):
+        return (ctypes.c_int64 * 3)(*([fill] * lead + [int(t) for t in v]))
+
+    gy = np.ascontiguousarray(dy, np.float32)
+    of = np.ascontiguousarray(other, np.float32)
+    out = np.empty(out_dims, np.float64)
+    fn(_ptr(gy), _ptr(of), _ptr(out), ctypes.c_int64(n), ctypes.c_int64(c),
+       ctypes.c_int64(k), ctypes.c_int64(fc), pad3(x_dims[2:], 1),
+       pad3(w_dims[2:], 1), pad3(od[2:], 1), pad3(padding, 0), pad3(stride, 1),
+       pad3(dilation, 1))
+    return out
+
+
+def conv_dgrad(dy: np.ndarray, w: np.ndarray, x_dims, padding, stride,
+               dilation) -> np.ndarray:
+    """Data gradient of conv_fprop (node/conv_node.h:428-598, emitted as
+    aten.convolution_backward).  Pinned by: the reference samples' all-ones
+    answers (1x1 => K, grouped => K / groups), the adjoint identity
+    <conv(x, w), dy> = <x, dgrad(dy, w)> on random inputs, torch autograd
+    (float64) incl. stride/dilation/padding/groups, 1-D and 3-D."""
+    assert dy.ndim == w.ndim == len(x_dims)
+    return _conv_backward(lib().oracle_conv_dgrad, dy, w, list(x_dims),
+                          list(w.shape), padding, stride, dilation,
+                          list(x_dims))
+
+
+def conv_wgrad(dy: np.ndarray, x: np.ndarray, w_dims, padding, stride,
+               dilation) -> np.ndarray:
+    """Weight gradient of conv_fprop (node/conv_node.h:255-426, emitted as
+    aten.convolution_backward).  Pinned by: the reference samples' all-ones
+    answers (1x1 => N*H*W, strided => N*Ho*Wo), the adjoint identity
+    <conv(x, w), dy> = <w, wgrad(dy, x)>, torch autograd (float64)."""
+    return _conv_backward(lib().oracle_conv_wgrad, dy, x, list(x.shape),
+                          list(w_dims), padding, stride, dilation,
+                          list(w_dims))
 
 
 def sdpa(q, k, v, mask=None, is_causal=False, scale=None) -> np.ndarray:

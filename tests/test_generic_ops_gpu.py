@@ -195,6 +195,111 @@ def test_conv_random_vs_oracle(ctx, case, dtype):
     assert_close(out.logical(), ref, dtype, str(case))
 
 
+# ---- conv backward --------------------------------------------------------
+def conv_bwd_desc(x, w, dy, pad, stride, dil):
+    d = capi.ConvDesc()
+    d.x, d.w, d.y = x.desc(), w.desc(), dy.desc()
+    d.spatial_rank = len(pad)
+    for i in range(len(pad)):
+        d.padding[i], d.stride[i], d.dilation[i] = pad[i], stride[i], dil[i]
+    d.epilogue = capi.make_epilogue([])
+    return d
+
+
+def run_conv_dgrad(ctx, dy, w, x_dims, pad, stride, dil, dtype, nhwc=True):
+    dx = HT.empty(x_dims, dtype,
+                  oracle.channels_last_strides(x_dims) if nhwc else None)
+    d = conv_bwd_desc(dx, w, dy, pad, stride, dil)
+    assert ctx.lib.fhip_conv_dgrad_supported(d) == 1
+    bdy, bw, bdx = dy.upload(ctx), w.upload(ctx), dx.upload(ctx)
+    ctx.conv_dgrad(d, bdy, bw, bdx)
+    return dx.fetch(ctx, bdx)
+
+
+def run_conv_wgrad(ctx, dy, x, w_dims, pad, stride, dil, dtype, nhwc=True):
+    dw = HT.empty(w_dims, dtype,
+                  oracle.channels_last_strides(w_dims) if nhwc else None)
+    d = conv_bwd_desc(x, dw, dy, pad, stride, dil)
+    assert ctx.lib.fhip_conv_wgrad_supported(d) == 1
+    bdy, bx, bdw = dy.upload(ctx), x.upload(ctx), dw.upload(ctx)
+    ctx.conv_wgrad(d, bdy, bx, bdw)
+    return dw.fetch(ctx, bdw)
+
+
+@pytest.mark.parametrize("grouped", [False, True])
+def test_conv_dgrad_all_ones_known_answer(ctx, grouped):
+    # samples/convolution/conv_dgrad_nhwc_krsc.cpp:98 (=> K = 16) and
+    # conv_dgrad_nhwc_krsc_grouped.cpp:99 (=> K / groups = 8); NHWC DY, KRSC
+    # (contiguous) W, as the samples lay them out.
+    n, c, k, fc = (4, 16, 32, 4) if grouped else (4, 8, 16, 8)
+    dyd, wd = [n, k, 8, 8], [k, fc, 1, 1]
+    dy = HT.from_logical(np.ones(dyd), capi.HALF, oracle.channels_last_strides(dyd))
+    w = HT.from_logical(np.ones(wd), capi.HALF)
+    dx = run_conv_dgrad(ctx, dy, w, [n, c, 8, 8], [0, 0], [1, 1], [1, 1], capi.HALF)
+    assert np.all(dx.logical() == float(k // (c // fc)))
+
+
+@pytest.mark.parametrize("variant", ["plain", "grouped", "grouped_strided"])
+def test_conv_wgrad_all_ones_known_answer(ctx, variant):
+    # samples/convolution/conv_wgrad_nhwc_krsc.cpp:99 (=> N*H*W = 256),
+    # conv_wgrad_nhwc_krsc_grouped.cpp:99 (=> 256) and
+    # conv_wgrad_nhwc_krsc_grouped_strided.cpp:103 (stride 2 => N*Ho*Wo = 64).
+    n, c, k, fc = (4, 8, 16, 8) if variant == "plain" else (4, 16, 32, 4)
+    st = 2 if variant == "grouped_strided" else 1
+    dyd, xd = [n, k, 8 // st, 8 // st], [n, c, 8, 8]
+    dy = HT.from_logical(np.ones(dyd), capi.HALF, oracle.channels_last_strides(dyd))
+    x = HT.from_logical(np.ones(xd), capi.HALF, oracle.channels_last_strides(xd))
+    dw = run_conv_wgrad(ctx, dy, x, [k, fc, 1, 1], [0, 0], [st, st], [1, 1],
+                        capi.HALF)
+    assert np.all(dw.logical() == float(n * (8 // st) ** 2))
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=[2, 6, 9, 11], w=[4, 6, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    dict(x=[2, 6, 9, 11], w=[4, 3, 3, 2], pad=[0, 1], s=[2, 1], d=[1, 2]),
+    dict(x=[2, 6, 10, 11], w=[6, 2, 3, 3], pad=[1, 2], s=[3, 2], d=[1, 1]),
+    dict(x=[1, 8, 13], w=[8, 2, 4], pad=[2], s=[3], d=[2]),
+    dict(x=[1, 4, 5, 6, 7], w=[2, 4, 2, 3, 3], pad=[1, 0, 1], s=[1, 2, 1], d=[1, 1, 1]),
+    dict(x=[3, 16, 20, 20], w=[24, 16, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+])
+@pytest.mark.parametrize("dtype", [capi.FLOAT, capi.BFLOAT16])
+@pytest.mark.parametrize("nhwc", [False, True])
+def test_conv_backward_random_vs_oracle(ctx, case, dtype, nhwc):
+    lay = oracle.channels_last_strides if nhwc else (lambda dims: None)
+    yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], case["s"],
+                                 case["d"])
+    x = HT.from_logical(rand(32, 0, case["x"]), dtype, lay(case["x"]))
+    w = HT.from_logical(rand(32, 1, case["w"], std=0.2), dtype, lay(case["w"]))
+    dy = HT.from_logical(rand(32, 2, yd), dtype, lay(yd))
+    dx = run_conv_dgrad(ctx, dy, w, case["x"], case["pad"], case["s"],
+                        case["d"], dtype, nhwc)
+    assert_close(dx.logical(),
+                 oracle.conv_dgrad(dy.logical(), w.logical(), case["x"],
+                                   case["pad"], case["s"], case["d"]),
+                 dtype, f"dgrad {case}")
+    dw = run_conv_wgrad(ctx, dy, x, case["w"], case["pad"], case["s"],
+                        case["d"], dtype, nhwc)
+    assert_close(dw.logical(),
+                 oracle.conv_wgrad(dy.logical(), x.logical(), case["w"],
+                                   case["pad"], case["s"], case["d"]),
+                 dtype, f"wgrad {case}")
+
+
+def test_conv_backward_rejects_bad_descriptors(ctx):
+    x = HT.empty([2, 6, 9, 11], capi.FLOAT)
+    w = HT.empty([4, 6, 3, 3], capi.FLOAT)
+    dy = HT.empty([2, 4, 9, 10], capi.FLOAT)  # Q should be 11
+    d = conv_bwd_desc(x, w, dy, [1, 1], [1, 1], [1, 1])
+    assert ctx.lib.fhip_conv_dgrad_supported(d) == 0
+    assert ctx.lib.fhip_conv_wgrad_supported(d) == 0
+    dy = HT.empty([2, 4, 9, 11], capi.FLOAT)
+    d = conv_bwd_desc(x, w, dy, [1, 1], [1, 1], [1, 1])
+    d.epilogue = capi.make_epilogue([capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT)])
+    assert ctx.lib.fhip_conv_dgrad_supported(d) == 0
+    with pytest.raises(Exception, match="gradient"):
+        ctx.conv_dgrad(d, dy.upload(ctx), w.upload(ctx), x.upload(ctx))
+
+
 # ---- sdpa -----------------------------------------------------------------
 def run_sdpa(ctx, q, k, v, *, mask=None, causal=False, scale=None, o_dtype=None):
     o_dtype = q.dtype if o_dtype is None else o_dtype

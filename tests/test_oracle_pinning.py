@@ -154,6 +154,61 @@ def test_conv_matches_torch(case):
     assert np.allclose(got, ref, rtol=1e-9, atol=1e-9)
 
 
+def test_conv_backward_known_answers():
+    # samples/convolution/conv_dgrad_nhwc_krsc.cpp:98: all-ones 1x1 => K
+    dy, w = np.ones([4, 16, 8, 8]), np.ones([16, 8, 1, 1])
+    assert np.all(oracle.conv_dgrad(dy, w, [4, 8, 8, 8], [0, 0], [1, 1], [1, 1]) == 16.0)
+    # conv_dgrad_nhwc_krsc_grouped.cpp:99: grouped => K / groups
+    dy, w = np.ones([4, 32, 8, 8]), np.ones([32, 4, 1, 1])
+    assert np.all(oracle.conv_dgrad(dy, w, [4, 16, 8, 8], [0, 0], [1, 1], [1, 1]) == 8.0)
+    # conv_wgrad_nhwc_krsc.cpp:99: all-ones 1x1 => N*H*W
+    dy, x = np.ones([4, 16, 8, 8]), np.ones([4, 8, 8, 8])
+    assert np.all(oracle.conv_wgrad(dy, x, [16, 8, 1, 1], [0, 0], [1, 1], [1, 1]) == 256.0)
+    # conv_wgrad_nhwc_krsc_grouped.cpp:99 and ..._grouped_strided.cpp:103
+    dy, x = np.ones([4, 32, 8, 8]), np.ones([4, 16, 8, 8])
+    assert np.all(oracle.conv_wgrad(dy, x, [32, 4, 1, 1], [0, 0], [1, 1], [1, 1]) == 256.0)
+    dy = np.ones([4, 32, 4, 4])
+    assert np.all(oracle.conv_wgrad(dy, x, [32, 4, 1, 1], [0, 0], [2, 2], [1, 1]) == 64.0)
+    # a delta gradient picks one filter-shaped window of X (wgrad) and writes
+    # one filter-shaped stamp of W into DX (dgrad), at stride * o - pad
+    x = RNG.normal(size=[1, 1, 7, 9]).astype(np.float32)
+    w = RNG.normal(size=[1, 1, 3, 2]).astype(np.float32)
+    od = oracle.conv_output_dims(x.shape, w.shape, [1, 0], [2, 1], [1, 1])
+    dy = np.zeros(od); dy[0, 0, 2, 3] = 1.0
+    dw = oracle.conv_wgrad(dy, x, w.shape, [1, 0], [2, 1], [1, 1])
+    assert np.array_equal(dw[0, 0], x[0, 0, 3:6, 3:5].astype(np.float64))
+    dx = oracle.conv_dgrad(dy, w, x.shape, [1, 0], [2, 1], [1, 1])
+    want = np.zeros([7, 9]); want[3:6, 3:5] = w[0, 0]
+    assert np.array_equal(dx[0, 0], want)
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=[2, 6, 9, 11], w=[4, 6, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    dict(x=[2, 6, 9, 11], w=[4, 3, 3, 2], pad=[0, 1], s=[2, 1], d=[1, 2]),
+    dict(x=[2, 6, 10, 11], w=[6, 2, 3, 3], pad=[1, 2], s=[3, 2], d=[1, 1]),
+    dict(x=[1, 8, 13], w=[8, 2, 4], pad=[2], s=[3], d=[2]),
+    dict(x=[1, 4, 5, 6, 7], w=[2, 4, 2, 3, 3], pad=[1, 0, 1], s=[1, 2, 1], d=[1, 1, 1]),
+])
+def test_conv_backward_matches_torch_autograd_and_adjoint(case):
+    x = RNG.normal(size=case["x"]).astype(np.float32)
+    w = RNG.normal(size=case["w"]).astype(np.float32)
+    groups = case["x"][1] // case["w"][1]
+    fn = {1: F.conv1d, 2: F.conv2d, 3: F.conv3d}[len(case["pad"])]
+    tx, tw = t64(x).requires_grad_(True), t64(w).requires_grad_(True)
+    y = fn(tx, tw, None, case["s"], case["pad"], case["d"], groups)
+    dy = RNG.normal(size=list(y.shape)).astype(np.float32)
+    y.backward(t64(dy))
+    dx = oracle.conv_dgrad(dy, w, case["x"], case["pad"], case["s"], case["d"])
+    dw = oracle.conv_wgrad(dy, x, case["w"], case["pad"], case["s"], case["d"])
+    assert np.allclose(dx, tx.grad.numpy(), rtol=1e-9, atol=1e-9)
+    assert np.allclose(dw, tw.grad.numpy(), rtol=1e-9, atol=1e-9)
+    # adjoint identities against the (separately pinned) forward
+    fwd = oracle.conv_fprop(x, w, case["pad"], case["s"], case["d"])
+    lhs = float(np.sum(fwd * dy.astype(np.float64)))
+    assert np.isclose(lhs, float(np.sum(dx * x.astype(np.float64))), rtol=1e-9)
+    assert np.isclose(lhs, float(np.sum(dw * w.astype(np.float64))), rtol=1e-9)
+
+
 # ---- attention ------------------------------------------------------------------
 def torch_sdpa(q, k, v, mask=None, causal=False, scale=None):
     rep = q.shape[1] // k.shape[1]
