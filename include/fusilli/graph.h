@@ -271,6 +271,35 @@ public:
     return y;
   }
 
+  // graph.h:795-824 of the reference: DW's dims are set by the caller on the
+  // returned tensor (the filter's channel extent fixes the group count).
+  std::shared_ptr<TensorAttr> convWGrad(const TensorPtr &dy, const TensorPtr &x,
+                                        ConvWGradAttr &attr) {
+    nameNode(attr, "conv_wgrad");
+    nameTensor(dy, attr, "DY");
+    nameTensor(x, attr, "X");
+    attr.setDY(dy).setX(x);
+    auto dw = outputTensor(attr.getName() + "_DW");
+    attr.setDW(dw);
+    subNodes_.emplace_back(
+        std::make_shared<ConvWGradNode>(std::move(attr), context));
+    return dw;
+  }
+
+  // graph.h:826-855 of the reference: DX's dims are set by the caller.
+  std::shared_ptr<TensorAttr> convDGrad(const TensorPtr &dy, const TensorPtr &w,
+                                        ConvDGradAttr &attr) {
+    nameNode(attr, "conv_dgrad");
+    nameTensor(dy, attr, "DY");
+    nameTensor(w, attr, "W");
+    attr.setDY(dy).setW(w);
+    auto dx = outputTensor(attr.getName() + "_DX");
+    attr.setDX(dx);
+    subNodes_.emplace_back(
+        std::make_shared<ConvDGradNode>(std::move(attr), context));
+    return dx;
+  }
+
   std::shared_ptr<TensorAttr> matmul(const TensorPtr &a, const TensorPtr &b,
                                      MatmulAttr &attr) {
     nameNode(attr, "matmul");

@@ -216,6 +216,231 @@ public:
   }
 };
 
+// ---- convolution weight gradient (node/conv_node.h:255-426) --------------------
+class ConvWGradNode : public NodeCRTP<ConvWGradNode> {
+public:
+  ConvWGradAttr convWGradAttr;
+  ConvWGradNode(ConvWGradAttr &&attr, const Context &ctx)
+      : NodeCRTP(ctx), convWGradAttr(std::move(attr)) {}
+  const std::string &getName() const override final {
+    return convWGradAttr.getName();
+  }
+  Type getType() const override final { return Type::WGrad; }
+
+  ErrorObject preValidateNode() const override final {
+    FUSILLI_LOG_LABEL_ENDL("INFO: Pre-Validating ConvWGradNode '" << getName()
+                                                                  << "'");
+    const auto &pad = convWGradAttr.getPadding();
+    const auto &str = convWGradAttr.getStride();
+    const auto &dil = convWGradAttr.getDilation();
+    FUSILLI_RETURN_ERROR_IF(pad.empty(), ErrorCode::AttributeNotSet,
+                            "ConvWGrad padding not set");
+    FUSILLI_RETURN_ERROR_IF(str.empty(), ErrorCode::AttributeNotSet,
+                            "ConvWGrad stride not set");
+    FUSILLI_RETURN_ERROR_IF(dil.empty(), ErrorCode::AttributeNotSet,
+                            "ConvWGrad dilation not set");
+    const TensorPtr dy = convWGradAttr.getDY(), x = convWGradAttr.getX(),
+                    dw = convWGradAttr.getDW();
+    FUSILLI_RETURN_ERROR_IF(!dy, ErrorCode::AttributeNotSet,
+                            "ConvWGrad gradient tensor DY not set");
+    FUSILLI_RETURN_ERROR_IF(!x, ErrorCode::AttributeNotSet,
+                            "ConvWGrad input tensor X not set");
+    FUSILLI_RETURN_ERROR_IF(!dw, ErrorCode::AttributeNotSet,
+                            "ConvWGrad output tensor DW not set");
+    const size_t dyRank = dy->getDim().size(), xRank = x->getDim().size();
+    FUSILLI_RETURN_ERROR_IF(
+        dyRank < 3 || xRank < 3, ErrorCode::InvalidAttribute,
+        "ConvWGrad input tensors DY/X must have a rank of at least 3");
+    FUSILLI_RETURN_ERROR_IF(dyRank != xRank, ErrorCode::InvalidAttribute,
+                            "ConvWGrad tensors DY and X have different ranks");
+    const size_t spatial = dyRank - 2;
+    FUSILLI_RETURN_ERROR_IF(
+        pad.size() != spatial, ErrorCode::InvalidAttribute,
+        "ConvWGrad padding size does not match number of spatial dimensions");
+    FUSILLI_RETURN_ERROR_IF(
+        str.size() != spatial, ErrorCode::InvalidAttribute,
+        "ConvWGrad stride size does not match number of spatial dimensions");
+    FUSILLI_RETURN_ERROR_IF(
+        dil.size() != spatial, ErrorCode::InvalidAttribute,
+        "ConvWGrad dilation size does not match number of spatial dimensions");
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(dy),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(dy));
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(x),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(x));
+    // The filter's channel extent gives the group count, so DW's dims are the
+    // caller's to set (conv_node.h:372-375).
+    FUSILLI_RETURN_ERROR_IF(dw->getDim().size() < 2,
+                            ErrorCode::InvalidAttribute,
+                            "ConvWGrad weight gradient tensor DW must have a "
+                            "rank of at least 3");
+    const int64_t inC = x->getDim()[1], outC = dy->getDim()[1],
+                  filterC = dw->getDim()[1];
+    FUSILLI_RETURN_ERROR_IF(filterC <= 0 || inC % filterC != 0,
+                            ErrorCode::InvalidAttribute,
+                            "ConvWGrad input (X) channels must be divisible by "
+                            "the filter (W) channels");
+    const int64_t groups = inC / filterC;
+    FUSILLI_RETURN_ERROR_IF(
+        groups <= 0 || groups > inC || groups > outC,
+        ErrorCode::InvalidAttribute,
+        "ConvWGrad group count must be greater than 0 and less than or equal "
+        "to the numbers of input and outputs channels");
+    FUSILLI_RETURN_ERROR_IF(
+        outC % groups != 0, ErrorCode::InvalidAttribute,
+        "ConvWGrad output (DY) channels must be divisible by the group count");
+    return ok();
+  }
+
+  ErrorObject inferPropertiesNode() override final {
+    convWGradAttr.fillFromContext(context);
+    const TensorPtr dy = convWGradAttr.getDY(), dw = convWGradAttr.getDW();
+    if (dw->getStride().empty()) {
+      // follows the gradient's layout (conv_node.h:376-386)
+      const size_t rank = dw->getDim().size();
+      dw->setStride(generateStrideFromDim(
+          dw->getDim(), dy->isContiguous() ? getContiguousStrideOrder(rank)
+                                           : getChannelsLastStrideOrder(rank)));
+    }
+    return ok();
+  }
+
+  ErrorObject postValidateNode() const override final {
+    const TensorPtr dy = convWGradAttr.getDY(), x = convWGradAttr.getX(),
+                    dw = convWGradAttr.getDW();
+    FUSILLI_RETURN_ERROR_IF(
+        dw->getDim().size() < 3, ErrorCode::InvalidAttribute,
+        "ConvWGrad weight gradient tensor DW must have a rank of at least 3");
+    FUSILLI_RETURN_ERROR_IF(
+        dw->getDim().size() != x->getDim().size() ||
+            dy->getDim() != getConvInferredOutputShape(
+                                x->getDim(), dw->getDim(),
+                                convWGradAttr.getDilation(),
+                                convWGradAttr.getPadding(),
+                                convWGradAttr.getStride()),
+        ErrorCode::InvalidAttribute,
+        "ConvWGrad output DW dimensions do not match the expected shapes "
+        "inferred based on input dimensions");
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(dw),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(dw));
+    return ok();
+  }
+};
+
+// ---- convolution data gradient (node/conv_node.h:428-598) ----------------------
+class ConvDGradNode : public NodeCRTP<ConvDGradNode> {
+public:
+  ConvDGradAttr convDGradAttr;
+  ConvDGradNode(ConvDGradAttr &&attr, const Context &ctx)
+      : NodeCRTP(ctx), convDGradAttr(std::move(attr)) {}
+  const std::string &getName() const override final {
+    return convDGradAttr.getName();
+  }
+  Type getType() const override final { return Type::DGrad; }
+
+  ErrorObject preValidateNode() const override final {
+    FUSILLI_LOG_LABEL_ENDL("INFO: Pre-Validating ConvDGradNode '" << getName()
+                                                                  << "'");
+    const auto &pad = convDGradAttr.getPadding();
+    const auto &str = convDGradAttr.getStride();
+    const auto &dil = convDGradAttr.getDilation();
+    FUSILLI_RETURN_ERROR_IF(pad.empty(), ErrorCode::AttributeNotSet,
+                            "ConvDGrad padding not set");
+    FUSILLI_RETURN_ERROR_IF(str.empty(), ErrorCode::AttributeNotSet,
+                            "ConvDGrad stride not set");
+    FUSILLI_RETURN_ERROR_IF(dil.empty(), ErrorCode::AttributeNotSet,
+                            "ConvDGrad dilation not set");
+    const TensorPtr dy = convDGradAttr.getDY(), w = convDGradAttr.getW(),
+                    dx = convDGradAttr.getDX();
+    FUSILLI_RETURN_ERROR_IF(!dy, ErrorCode::AttributeNotSet,
+                            "ConvDGrad gradient tensor DY not set");
+    FUSILLI_RETURN_ERROR_IF(!w, ErrorCode::AttributeNotSet,
+                            "ConvDGrad input tensor W not set");
+    FUSILLI_RETURN_ERROR_IF(!dx, ErrorCode::AttributeNotSet,
+                            "ConvDGrad output tensor DX not set");
+    const size_t dyRank = dy->getDim().size(), wRank = w->getDim().size();
+    FUSILLI_RETURN_ERROR_IF(
+        dyRank < 3 || wRank < 3, ErrorCode::InvalidAttribute,
+        "ConvDGrad input tensors DY/W must have a rank of at least 3");
+    const size_t spatial = dyRank - 2;
+    FUSILLI_RETURN_ERROR_IF(
+        pad.size() != spatial, ErrorCode::InvalidAttribute,
+        "ConvDGrad padding size does not match number of spatial dimensions");
+    FUSILLI_RETURN_ERROR_IF(
+        str.size() != spatial, ErrorCode::InvalidAttribute,
+        "ConvDGrad stride size does not match number of spatial dimensions");
+    FUSILLI_RETURN_ERROR_IF(
+        dil.size() != spatial, ErrorCode::InvalidAttribute,
+        "ConvDGrad dilation size does not match number of spatial dimensions");
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(dy),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(dy));
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(w),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(w));
+    // DX's dims are the caller's to set: padding and stride do not determine
+    // the input extent uniquely.
+    FUSILLI_RETURN_ERROR_IF(
+        dx->getDim().size() < 2, ErrorCode::InvalidAttribute,
+        "ConvDGrad input gradient DX must have a rank of at least 3");
+    const int64_t inC = dx->getDim()[1], outC = w->getDim()[0],
+                  filterC = w->getDim()[1];
+    FUSILLI_RETURN_ERROR_IF(filterC <= 0 || inC % filterC != 0,
+                            ErrorCode::InvalidAttribute,
+                            "ConvDGrad input (DX) channels must be divisible "
+                            "by the filter (W) channels");
+    const int64_t groups = inC / filterC;
+    FUSILLI_RETURN_ERROR_IF(
+        groups <= 0 || groups > inC || groups > outC,
+        ErrorCode::InvalidAttribute,
+        "ConvDGrad group count must be greater than 0 and less than or equal "
+        "to the numbers of input and outputs channels");
+    FUSILLI_RETURN_ERROR_IF(
+        outC % groups != 0, ErrorCode::InvalidAttribute,
+        "ConvDGrad output (DY) channels must be divisible by the group count");
+    return ok();
+  }
+
+  ErrorObject inferPropertiesNode() override final {
+    convDGradAttr.fillFromContext(context);
+    const TensorPtr dy = convDGradAttr.getDY(), dx = convDGradAttr.getDX();
+    if (dx->getStride().empty()) {
+      const size_t rank = dx->getDim().size();
+      dx->setStride(generateStrideFromDim(
+          dx->getDim(), dy->isContiguous() ? getContiguousStrideOrder(rank)
+                                           : getChannelsLastStrideOrder(rank)));
+    }
+    return ok();
+  }
+
+  ErrorObject postValidateNode() const override final {
+    const TensorPtr dy = convDGradAttr.getDY(), w = convDGradAttr.getW(),
+                    dx = convDGradAttr.getDX();
+    FUSILLI_RETURN_ERROR_IF(
+        dx->getDim().size() < 3, ErrorCode::InvalidAttribute,
+        "ConvDGrad input gradient DX must have a rank of at least 3");
+    FUSILLI_RETURN_ERROR_IF(dy->getDim().size() != dx->getDim().size(),
+                            ErrorCode::InvalidAttribute,
+                            "ConvDGrad tensors DY and DX have different ranks");
+    FUSILLI_RETURN_ERROR_IF(
+        w->getDim().size() != dx->getDim().size() ||
+            dy->getDim() != getConvInferredOutputShape(
+                                dx->getDim(), w->getDim(),
+                                convDGradAttr.getDilation(),
+                                convDGradAttr.getPadding(),
+                                convDGradAttr.getStride()),
+        ErrorCode::InvalidAttribute,
+        "ConvDGrad DY dimensions do not match the expected shapes inferred "
+        "based on DX and W");
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(dx),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(dx));
+    return ok();
+  }
+};
+
 // ---- matmul -------------------------------------------------------------------
 // Batch dims take the larger extent; last two dims are M x N
 // (node/matmul_node.h:40-66).

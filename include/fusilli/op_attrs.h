@@ -84,7 +84,44 @@ private:
 
 enum class NormFwdPhase : uint8_t { NOT_SET, TRAINING, INFERENCE };
 
-// ---- convolution forward (attributes/conv_attributes.h) ---------------------
+// ---- convolution (attributes/conv_attributes.h) -------------------------------
+// Padding / stride / dilation setters and getters shared by the three
+// convolution attribute classes.
+#define FUSILLI_CONV_GEOMETRY(CLASS)                                           \
+  CLASS &setPadding(const std::vector<int64_t> &v) {                           \
+    padding_ = v;                                                              \
+    return *this;                                                              \
+  }                                                                            \
+  CLASS &setStride(const std::vector<int64_t> &v) {                            \
+    stride_ = v;                                                               \
+    return *this;                                                              \
+  }                                                                            \
+  CLASS &setDilation(const std::vector<int64_t> &v) {                          \
+    dilation_ = v;                                                             \
+    return *this;                                                              \
+  }                                                                            \
+  template <Int64Range R> CLASS &setPadding(R &&v) {                           \
+    padding_.assign(v.begin(), v.end());                                       \
+    return *this;                                                              \
+  }                                                                            \
+  template <Int64Range R> CLASS &setStride(R &&v) {                            \
+    stride_.assign(v.begin(), v.end());                                        \
+    return *this;                                                              \
+  }                                                                            \
+  template <Int64Range R> CLASS &setDilation(R &&v) {                          \
+    dilation_.assign(v.begin(), v.end());                                      \
+    return *this;                                                              \
+  }                                                                            \
+  const std::vector<int64_t> &getPadding() const { return padding_; }          \
+  const std::vector<int64_t> &getStride() const { return stride_; }            \
+  const std::vector<int64_t> &getDilation() const { return dilation_; }        \
+                                                                               \
+private:                                                                       \
+  std::vector<int64_t> padding_, stride_, dilation_;                           \
+                                                                               \
+public:
+
+// forward (conv_attributes.h:20-84)
 class ConvFPropAttr : public AttributesCRTP<ConvFPropAttr> {
 public:
   enum class InputNames : uint8_t { X, W };
@@ -93,37 +130,31 @@ public:
   FUSILLI_IN_SLOT(ConvFPropAttr, X)
   FUSILLI_IN_SLOT(ConvFPropAttr, W)
   FUSILLI_OUT_SLOT(ConvFPropAttr, Y)
+  FUSILLI_CONV_GEOMETRY(ConvFPropAttr)
+};
 
-  ConvFPropAttr &setPadding(const std::vector<int64_t> &v) {
-    padding_ = v;
-    return *this;
-  }
-  ConvFPropAttr &setStride(const std::vector<int64_t> &v) {
-    stride_ = v;
-    return *this;
-  }
-  ConvFPropAttr &setDilation(const std::vector<int64_t> &v) {
-    dilation_ = v;
-    return *this;
-  }
-  template <Int64Range R> ConvFPropAttr &setPadding(R &&v) {
-    padding_.assign(v.begin(), v.end());
-    return *this;
-  }
-  template <Int64Range R> ConvFPropAttr &setStride(R &&v) {
-    stride_.assign(v.begin(), v.end());
-    return *this;
-  }
-  template <Int64Range R> ConvFPropAttr &setDilation(R &&v) {
-    dilation_.assign(v.begin(), v.end());
-    return *this;
-  }
-  const std::vector<int64_t> &getPadding() const { return padding_; }
-  const std::vector<int64_t> &getStride() const { return stride_; }
-  const std::vector<int64_t> &getDilation() const { return dilation_; }
+// weight gradient (conv_attributes.h:86-139)
+class ConvWGradAttr : public AttributesCRTP<ConvWGradAttr> {
+public:
+  enum class InputNames : uint8_t { DY, X };
+  enum class OutputNames : uint8_t { DW };
+  FUSILLI_SLOT_MAPS
+  FUSILLI_IN_SLOT(ConvWGradAttr, DY)
+  FUSILLI_IN_SLOT(ConvWGradAttr, X)
+  FUSILLI_OUT_SLOT(ConvWGradAttr, DW)
+  FUSILLI_CONV_GEOMETRY(ConvWGradAttr)
+};
 
-private:
-  std::vector<int64_t> padding_, stride_, dilation_;
+// data gradient (conv_attributes.h:141-191)
+class ConvDGradAttr : public AttributesCRTP<ConvDGradAttr> {
+public:
+  enum class InputNames : uint8_t { DY, W };
+  enum class OutputNames : uint8_t { DX };
+  FUSILLI_SLOT_MAPS
+  FUSILLI_IN_SLOT(ConvDGradAttr, DY)
+  FUSILLI_IN_SLOT(ConvDGradAttr, W)
+  FUSILLI_OUT_SLOT(ConvDGradAttr, DX)
+  FUSILLI_CONV_GEOMETRY(ConvDGradAttr)
 };
 
 // ---- matmul (attributes/matmul_attributes.h) --------------------------------

@@ -39,6 +39,8 @@ enum class StepKind : uint32_t {
   Norm = 4,
   Reduce = 5,
   Pointwise = 6,
+  ConvDGrad = 7,
+  ConvWGrad = 8,
 };
 
 constexpr int kMaxSlots = 12;
@@ -80,6 +82,7 @@ struct Step {
 // Slot positions per step kind.
 enum : int { kMmA = 0, kMmB = 1, kMmOut = 2, kMmEpi = 3 };
 enum : int { kCvX = 0, kCvW = 1, kCvOut = 2, kCvEpi = 3 };
+enum : int { kCbDY = 0, kCbIn = 1, kCbOut = 2 }; // conv gradients
 enum : int { kSdQ = 0, kSdK = 1, kSdV = 2, kSdMask = 3, kSdO = 4 };
 enum : int {
   kNmX = 0,
@@ -272,6 +275,11 @@ public:
         i = next;
         break;
       }
+      case INode::Type::WGrad:
+      case INode::Type::DGrad:
+        FUSILLI_CHECK_ERROR(planConvBackward(i));
+        ++i;
+        break;
       case INode::Type::RmsNorm:
       case INode::Type::LayerNorm: {
         FUSILLI_ASSIGN_OR_RETURN(size_t next, planNorm(i));
@@ -321,6 +329,12 @@ private:
     switch (n.getType()) {
     case INode::Type::Convolution:
       each(static_cast<const ConvFPropNode &>(n).convFPropAttr);
+      break;
+    case INode::Type::WGrad:
+      each(static_cast<const ConvWGradNode &>(n).convWGradAttr);
+      break;
+    case INode::Type::DGrad:
+      each(static_cast<const ConvDGradNode &>(n).convDGradAttr);
       break;
     case INode::Type::Matmul:
       each(static_cast<const MatmulNode &>(n).matmulAttr);
@@ -737,6 +751,50 @@ private:
 
   const std::vector<std::shared_ptr<INode>> &nodes_;
   Plan plan_;
+  // Conv gradients: one step each, nothing fused (the descriptor names the
+  // forward problem: x = X / DX, w = W / DW, y = DY).
+  ErrorObject planConvBackward(size_t i) {
+    const bool dgrad = nodes_[i]->getType() == INode::Type::DGrad;
+    TensorPtr x, w, dy;
+    const std::vector<int64_t> *pad, *str, *dil;
+    if (dgrad) {
+      const auto &a = static_cast<const ConvDGradNode &>(*nodes_[i]).convDGradAttr;
+      x = a.getDX(), w = a.getW(), dy = a.getDY();
+      pad = &a.getPadding(), str = &a.getStride(), dil = &a.getDilation();
+    } else {
+      const auto &a = static_cast<const ConvWGradNode &>(*nodes_[i]).convWGradAttr;
+      x = a.getX(), w = a.getDW(), dy = a.getDY();
+      pad = &a.getPadding(), str = &a.getStride(), dil = &a.getDilation();
+    }
+    Step s;
+    s.kind = static_cast<uint32_t>(dgrad ? StepKind::ConvDGrad
+                                         : StepKind::ConvWGrad);
+    fhip_conv_desc &d = s.desc.conv;
+    FUSILLI_ASSIGN_OR_RETURN(d.x, toDesc(x));
+    FUSILLI_ASSIGN_OR_RETURN(d.w, toDesc(w));
+    FUSILLI_ASSIGN_OR_RETURN(d.y, toDesc(dy));
+    d.spatial_rank = static_cast<int32_t>(pad->size());
+    FUSILLI_RETURN_ERROR_IF(d.spatial_rank > 3, ErrorCode::NotImplemented,
+                            "Convolutions above 3 spatial dims are not "
+                            "supported");
+    for (int k = 0; k < d.spatial_rank; ++k) {
+      d.padding[k] = (*pad)[k];
+      d.stride[k] = (*str)[k];
+      d.dilation[k] = (*dil)[k];
+    }
+    const int supported =
+        dgrad ? fhip_conv_dgrad_supported(&d) : fhip_conv_wgrad_supported(&d);
+    FUSILLI_RETURN_ERROR_IF(supported == 0, ErrorCode::NotImplemented,
+                            "Conv gradient node '" + nodes_[i]->getName() +
+                                "' is not executable by this backend: " +
+                                fhip_last_error(nullptr));
+    FUSILLI_ASSIGN_OR_RETURN(s.slot[kCbDY], readSlot(dy));
+    FUSILLI_ASSIGN_OR_RETURN(s.slot[kCbIn], readSlot(dgrad ? w : x));
+    FUSILLI_ASSIGN_OR_RETURN(s.slot[kCbOut], writeSlot(dgrad ? x : w));
+    plan_.steps.push_back(s);
+    return ok();
+  }
+
   std::unordered_map<const TensorAttr *, int32_t> argIndex_;
   std::vector<TensorPtr> argTensors_;
   std::unordered_map<const TensorAttr *, size_t> workspaceIndex_;
@@ -774,6 +832,14 @@ inline ErrorObject execute(fhip_ctx *ctx, const Plan &p,
       rc = fhip_conv_fprop(ctx, &s.desc.conv, ptr(s.slot[kCvX]),
                            ptr(s.slot[kCvW]), epi, ptr(s.slot[kCvOut]), nullptr,
                            0);
+      break;
+    case StepKind::ConvDGrad:
+      rc = fhip_conv_dgrad(ctx, &s.desc.conv, ptr(s.slot[kCbDY]),
+                           ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]), nullptr, 0);
+      break;
+    case StepKind::ConvWGrad:
+      rc = fhip_conv_wgrad(ctx, &s.desc.conv, ptr(s.slot[kCbDY]),
+                           ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]), nullptr, 0);
       break;
     case StepKind::Sdpa:
       rc = fhip_sdpa_fwd(ctx, &s.desc.sdpa, ptr(s.slot[kSdQ]),

@@ -88,6 +88,14 @@ template <typename T> static bool allEqual(const std::vector<T> &v, float x) {
   return !v.empty();
 }
 
+static std::vector<float> randomVec(size_t n, uint32_t seed, float lo, float hi) {
+  std::mt19937 rng(seed);
+  std::vector<float> v(n);
+  for (auto &x : v)
+    x = lo + (hi - lo) * (rng() >> 8) * (1.0f / 16777216.0f);
+  return v;
+}
+
 // ---- convolution samples -----------------------------------------------------
 static void convOnes(bool nhwc, bool bias, bool relu, int64_t r, int64_t pad,
                      float expectCorner, float expectCentre) {
@@ -144,6 +152,121 @@ TEST("samples: conv fprop all-ones known answers") {
   convOnes(true, true, true, 1, 0, 129.f, 129.f);    // ..._with_relu_and_bias.cpp:112
   convOnes(true, false, false, 3, 1, 512.f, 1152.f); // ..._with_pad.cpp:94
   convOnes(false, true, true, 3, 1, 513.f, 1153.f);
+}
+
+// ---- convolution gradient samples ----------------------------------------------
+// samples/convolution/conv_dgrad_nhwc_krsc{,_grouped}.cpp and
+// conv_wgrad_nhwc_krsc{,_grouped,_grouped_strided}.cpp: all-ones f16, 1x1
+// filters, NHWC activations and gradients, KRSC filters; each run twice.
+static void convGradOnes(bool dgrad, int64_t c, int64_t k, int64_t fc,
+                         int64_t st, bool biasGrad, float expect) {
+  const int64_t n = 4, h = 8, w = 8, ho = h / st, wo = w / st;
+  Graph g = newGraph(std::string(dgrad ? "dgrad_" : "wgrad_") + std::to_string(c) +
+                         "_" + std::to_string(fc) + "_" + std::to_string(st) +
+                         (biasGrad ? "_db" : ""),
+                     DataType::Half);
+  auto DY = g.tensor(mk("dy", {n, k, ho, wo}, chlast({n, k, ho, wo}), DataType::Half));
+  std::shared_ptr<TensorAttr> IN, OUT, DB;
+  if (dgrad) {
+    IN = g.tensor(mk("w", {k, fc, 1, 1}, contig({k, fc, 1, 1}), DataType::Half));
+    ConvDGradAttr a;
+    a.setPadding({0, 0}).setStride({st, st}).setDilation({1, 1});
+    OUT = g.convDGrad(DY, IN, a);
+    OUT->setDim({n, c, h, w}).setOutput(true);
+  } else {
+    IN = g.tensor(mk("x", {n, c, h, w}, chlast({n, c, h, w}), DataType::Half));
+    ConvWGradAttr a;
+    a.setPadding({0, 0}).setStride({st, st}).setDilation({1, 1});
+    OUT = g.convWGrad(DY, IN, a);
+    OUT->setDim({k, fc, 1, 1}).setOutput(true);
+  }
+  if (biasGrad) { // bias gradient: DY summed over batch and space
+    ReductionAttr ra;
+    ra.setMode(ReductionAttr::Mode::SUM).setName("bias_reduction");
+    DB = g.reduction(DY, ra);
+    DB->setDim({1, k, 1, 1}).setStride({1, 1, 1, 1}).setOutput(true);
+  }
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), /*remove=*/true));
+  Pack pack = {{DY, fill(DY, half(1.0f))}, {IN, fill(IN, half(1.0f))},
+               {OUT, fill(OUT, half(0.0f))}};
+  if (biasGrad)
+    pack[DB] = fill(DB, half(0.0f));
+  auto ws = workspaceFor(g);
+  for (int rep = 0; rep < 2; ++rep) {
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+    auto out = readBack<half>(pack[OUT]);
+    REQUIRE(out.size() ==
+            static_cast<size_t>(dgrad ? n * c * h * w : k * fc));
+    CHECK(allEqual(out, expect));
+    if (biasGrad)
+      CHECK(allEqual(readBack<half>(pack[DB]), static_cast<float>(n * ho * wo)));
+  }
+}
+
+TEST("samples: conv dgrad / wgrad all-ones known answers") {
+  convGradOnes(true, 8, 16, 8, 1, false, 16.f);  // conv_dgrad_nhwc_krsc.cpp:98: K
+  convGradOnes(true, 8, 16, 8, 1, true, 16.f);   // ...:207-217 with the bias gradient
+  convGradOnes(true, 16, 32, 4, 1, false, 8.f);  // ..._grouped.cpp:99: K / groups
+  convGradOnes(false, 8, 16, 8, 1, false, 256.f); // conv_wgrad_nhwc_krsc.cpp:99: N*H*W
+  convGradOnes(false, 8, 16, 8, 1, true, 256.f);  // ...:208-217
+  convGradOnes(false, 16, 32, 4, 1, false, 256.f); // ..._grouped.cpp:99
+  convGradOnes(false, 16, 32, 4, 2, false, 64.f);  // ..._grouped_strided.cpp:103
+}
+
+TEST("conv gradients: f32 3x3 stride 2 pad 1 against host loops") {
+  const int64_t n = 2, c = 6, h = 9, w = 10, k = 4, r = 3, st = 2, pad = 1;
+  const int64_t ho = 1 + (h + 2 * pad - r) / st, wo = 1 + (w + 2 * pad - r) / st;
+  auto xf = randomVec(n * c * h * w, 21, -1.f, 1.f);
+  auto wf = randomVec(k * c * r * r, 22, -1.f, 1.f);
+  auto gf = randomVec(n * k * ho * wo, 23, -1.f, 1.f);
+  // contiguous NCHW / KCRS throughout
+  std::vector<double> dxRef(xf.size(), 0.0), dwRef(wf.size(), 0.0);
+  for (int64_t in = 0; in < n; ++in)
+    for (int64_t kk = 0; kk < k; ++kk)
+      for (int64_t p = 0; p < ho; ++p)
+        for (int64_t q = 0; q < wo; ++q) {
+          const double gy = gf[((in * k + kk) * ho + p) * wo + q];
+          for (int64_t cc = 0; cc < c; ++cc)
+            for (int64_t fr = 0; fr < r; ++fr)
+              for (int64_t fs = 0; fs < r; ++fs) {
+                const int64_t ih = p * st - pad + fr, iw = q * st - pad + fs;
+                if (ih < 0 || ih >= h || iw < 0 || iw >= w)
+                  continue;
+                const size_t xi = ((in * c + cc) * h + ih) * w + iw;
+                const size_t wi = ((kk * c + cc) * r + fr) * r + fs;
+                dxRef[xi] += gy * wf[wi];
+                dwRef[wi] += gy * xf[xi];
+              }
+        }
+  Graph g = newGraph("conv_grads_f32", DataType::Float);
+  auto DY = g.tensor(mk("dy", {n, k, ho, wo}, contig({n, k, ho, wo}), DataType::Float));
+  auto X = g.tensor(mk("x", {n, c, h, w}, contig({n, c, h, w}), DataType::Float));
+  auto W = g.tensor(mk("w", {k, c, r, r}, contig({k, c, r, r}), DataType::Float));
+  ConvDGradAttr da;
+  da.setPadding({pad, pad}).setStride({st, st}).setDilation({1, 1});
+  auto DX = g.convDGrad(DY, W, da);
+  DX->setDim({n, c, h, w}).setOutput(true);
+  ConvWGradAttr wa;
+  wa.setPadding({pad, pad}).setStride({st, st}).setDilation({1, 1});
+  auto DW = g.convWGrad(DY, X, wa);
+  DW->setDim({k, c, r, r}).setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(2));
+  Pack pack = {{DY, bufOf(DY, gf)}, {X, bufOf(X, xf)}, {W, bufOf(W, wf)},
+               {DX, fill(DX, 0.f)}, {DW, fill(DW, 0.f)}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto dx = readBack<float>(pack[DX]);
+  auto dw = readBack<float>(pack[DW]);
+  REQUIRE(dx.size() == dxRef.size());
+  REQUIRE(dw.size() == dwRef.size());
+  double worst = 0;
+  for (size_t i = 0; i < dx.size(); ++i)
+    worst = std::max(worst, std::fabs(dx[i] - dxRef[i]) - 1e-4 * (std::fabs(dxRef[i]) + 1.0));
+  for (size_t i = 0; i < dw.size(); ++i)
+    worst = std::max(worst, std::fabs(dw[i] - dwRef[i]) - 1e-4 * (std::fabs(dwRef[i]) + 1.0));
+  CHECK(worst <= 0.0);
 }
 
 // ---- matmul samples ----------------------------------------------------------
@@ -411,13 +534,6 @@ TEST("samples: pointwise transposed add, scalar mul, AOT int32 add") {
 }
 
 // ---- benchmark configs through the graph API ---------------------------------
-static std::vector<float> randomVec(size_t n, uint32_t seed, float lo, float hi) {
-  std::mt19937 rng(seed);
-  std::vector<float> v(n);
-  for (auto &x : v)
-    x = lo + (hi - lo) * (rng() >> 8) * (1.0f / 16777216.0f);
-  return v;
-}
 
 TEST("config 1: f32 matmul 1x256x512x256 vs host loop, rel 1e-4") {
   const int64_t m = 256, k = 512, n = 256;

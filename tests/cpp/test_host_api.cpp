@@ -220,6 +220,180 @@ TEST("conv node: inference and errors") {
               "Conv output channels must be divisible by the group count");
 }
 
+TEST("conv gradient nodes: inference and errors") {
+  // tests/test_conv_node.cpp:503-1333 of the reference
+  const int64_t n = 16, c = 256, h = 64, w = 32, k = 128;
+  {
+    // wgrad: DW keeps the caller's dims and takes DY's layout (NHWC here)
+    Graph g = newGraph("wgrad_infer", DataType::Half);
+    auto dy = g.tensor(mk("dy", {n, k, h, w}, chlast({n, k, h, w}), DataType::Half));
+    auto x = g.tensor(mk("x", {n, c, h, w}, chlast({n, c, h, w}), DataType::Half));
+    ConvWGradAttr a;
+    a.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    auto dw = g.convWGrad(dy, x, a);
+    dw->setDim({k, c, 1, 1}).setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK(dw->getName() == "conv_wgrad_0_DW");
+    CHECK((dw->getStride() == chlast({k, c, 1, 1})));
+    CHECK(dw->getDataType() == DataType::Half);
+  }
+  {
+    // dgrad: DX keeps the caller's dims and takes DY's layout (contiguous)
+    Graph g = newGraph("dgrad_infer", DataType::Half);
+    auto dy = g.tensor(mk("dy", {n, k, h, w}, contig({n, k, h, w}), DataType::Half));
+    auto wt = g.tensor(mk("w", {k, c, 1, 1}, contig({k, c, 1, 1}), DataType::Half));
+    ConvDGradAttr a;
+    a.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    auto dx = g.convDGrad(dy, wt, a);
+    dx->setDim({n, c, h, w}).setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK(dx->getName() == "conv_dgrad_0_DX");
+    CHECK(dx->isContiguous());
+  }
+  Context ctx;
+  auto T = [](const char *name, Dims d, Dims st) {
+    return std::make_shared<TensorAttr>(mk(name, d, st));
+  };
+  auto wnode = [&](auto &&tweak) {
+    ConvWGradAttr a;
+    a.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    a.setDY(T("DY", {n, k, h, w}, chlast({n, k, h, w})))
+        .setX(T("X", {n, c, h, w}, chlast({n, c, h, w})))
+        .setDW(T("DW", {k, c, 1, 1}, contig({k, c, 1, 1})));
+    tweak(a);
+    return ConvWGradNode(std::move(a), ctx);
+  };
+  auto dnode = [&](auto &&tweak) {
+    ConvDGradAttr a;
+    a.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    a.setDY(T("DY", {n, k, h, w}, chlast({n, k, h, w})))
+        .setW(T("W", {k, c, 1, 1}, contig({k, c, 1, 1})))
+        .setDX(T("DX", {n, c, h, w}, chlast({n, c, h, w})));
+    tweak(a);
+    return ConvDGradNode(std::move(a), ctx);
+  };
+  REQUIRE_OK(wnode([](auto &) {}).preValidateNode());
+  REQUIRE_OK(dnode([](auto &) {}).preValidateNode());
+  CHECK_ERROR(wnode([](auto &a) { a.setPadding(Dims{}); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvWGrad padding not set");
+  CHECK_ERROR(wnode([](auto &a) { a.setStride(Dims{}); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvWGrad stride not set");
+  CHECK_ERROR(wnode([](auto &a) { a.setDilation(Dims{}); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvWGrad dilation not set");
+  CHECK_ERROR(wnode([](auto &a) { a.setDY(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvWGrad gradient tensor DY not set");
+  CHECK_ERROR(wnode([](auto &a) { a.setX(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvWGrad input tensor X not set");
+  CHECK_ERROR(wnode([](auto &a) { a.setDW(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvWGrad output tensor DW not set");
+  CHECK_ERROR(dnode([](auto &a) { a.setPadding(Dims{}); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvDGrad padding not set");
+  CHECK_ERROR(dnode([](auto &a) { a.setDY(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvDGrad gradient tensor DY not set");
+  CHECK_ERROR(dnode([](auto &a) { a.setW(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvDGrad input tensor W not set");
+  CHECK_ERROR(dnode([](auto &a) { a.setDX(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "ConvDGrad output tensor DX not set");
+  // ranks
+  CHECK_ERROR(wnode([&](auto &a) {
+                a.setDY(std::make_shared<TensorAttr>(mk("DY", {n, k}, {k, 1})));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvWGrad input tensors DY/X must have a rank of at least 3");
+  CHECK_ERROR(wnode([&](auto &a) {
+                a.setX(std::make_shared<TensorAttr>(
+                    mk("X", {n, c, 2, h, w}, contig({n, c, 2, h, w}))));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvWGrad tensors DY and X have different ranks");
+  CHECK_ERROR(wnode([](auto &a) { a.setStride({1}); }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvWGrad stride size does not match number of spatial dimensions");
+  CHECK_ERROR(dnode([](auto &a) { a.setDilation({1, 1, 1}); }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvDGrad dilation size does not match number of spatial "
+              "dimensions");
+  CHECK_ERROR(dnode([&](auto &a) {
+                a.setW(std::make_shared<TensorAttr>(mk("W", {k, c}, {c, 1})));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvDGrad input tensors DY/W must have a rank of at least 3");
+  // layouts
+  CHECK_ERROR(wnode([&](auto &a) {
+                a.setX(std::make_shared<TensorAttr>(
+                    mk("X", {n, c, h, w}, {c * h * w, w, 1, h})));
+              }).preValidateNode(),
+              ErrorCode::NotImplemented,
+              "Tensor 'X' is neither contiguous nor channels-last as defined "
+              "by its stride");
+  // group counts
+  CHECK_ERROR(wnode([&](auto &a) {
+                a.setDW(std::make_shared<TensorAttr>(
+                    mk("DW", {k, 7, 1, 1}, contig({k, 7, 1, 1}))));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvWGrad input (X) channels must be divisible by the filter "
+              "(W) channels");
+  CHECK_ERROR(dnode([&](auto &a) {
+                a.setW(std::make_shared<TensorAttr>(
+                    mk("W", {k, 7, 1, 1}, contig({k, 7, 1, 1}))));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvDGrad input (DX) channels must be divisible by the filter "
+              "(W) channels");
+  CHECK_ERROR(dnode([&](auto &a) {
+                // 256 / 1 = 256 groups > 128 output channels
+                a.setW(std::make_shared<TensorAttr>(
+                    mk("W", {k, 1, 1, 1}, contig({k, 1, 1, 1}))));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "ConvDGrad group count must be greater than 0 and less than or "
+              "equal to the numbers of input and outputs channels");
+  // post-validation: rank and shape agreement
+  {
+    auto node = wnode([&](auto &a) {
+      a.setDW(std::make_shared<TensorAttr>(mk("DW", {k, c}, {c, 1})));
+    });
+    REQUIRE_OK(node.preValidateNode());
+    REQUIRE_OK(node.inferPropertiesNode());
+    CHECK_ERROR(node.postValidateNode(), ErrorCode::InvalidAttribute,
+                "ConvWGrad weight gradient tensor DW must have a rank of at "
+                "least 3");
+  }
+  {
+    auto node = wnode([&](auto &a) { // {c, k, r, s} instead of {k, c, r, s}
+      a.setDW(std::make_shared<TensorAttr>(
+          mk("DW", {c, k, 1, 1}, contig({c, k, 1, 1}))));
+    });
+    REQUIRE_OK(node.preValidateNode());
+    REQUIRE_OK(node.inferPropertiesNode());
+    CHECK_ERROR(node.postValidateNode(), ErrorCode::InvalidAttribute,
+                "ConvWGrad output DW dimensions do not match the expected "
+                "shapes inferred based on input dimensions");
+  }
+  {
+    auto node = dnode([&](auto &a) {
+      a.setW(std::make_shared<TensorAttr>(
+          mk("W", {c, k, 1, 1}, contig({c, k, 1, 1}))));
+    });
+    REQUIRE_OK(node.preValidateNode());
+    REQUIRE_OK(node.inferPropertiesNode());
+    CHECK_ERROR(node.postValidateNode(), ErrorCode::InvalidAttribute,
+                "ConvDGrad DY dimensions do not match the expected shapes "
+                "inferred based on DX and W");
+  }
+  {
+    auto node = dnode([&](auto &a) {
+      a.setPadding({0, 0, 0}).setStride({1, 1, 1}).setDilation({1, 1, 1});
+      a.setDY(std::make_shared<TensorAttr>(
+          mk("DY", {n, k, 2, h, w}, contig({n, k, 2, h, w}))));
+    });
+    REQUIRE_OK(node.preValidateNode());
+    CHECK_ERROR(node.postValidateNode(), ErrorCode::InvalidAttribute,
+                "ConvDGrad tensors DY and DX have different ranks");
+  }
+}
+
 TEST("matmul node: inference and errors") {
   {
     Graph g = newGraph("mm");
