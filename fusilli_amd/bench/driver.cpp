@@ -185,12 +185,46 @@ void runConv(const Handle &h, const Args &a, int iter) {
                 q = a.i("-q", "--pad_w", 0), u = a.i("-u", "--conv_stride_h", 1),
                 v = a.i("-v", "--conv_stride_w", 1), l = a.i("-l", "--dilation_h", 1),
                 j = a.i("-j", "--dilation_w", 1), gcount = a.i("-g", "--group_count", 1);
-  if (a.i("-F", "--mode", 1) != 1)
-    die("conv: only -F 1 (forward) is supported");
+  // MIOpen's direction flag, as in the reference driver (driver.cpp:1159-1167):
+  // 1 forward, 2 data gradient, 4 weight gradient
+  const int64_t mode = a.i("-F", "--mode", 1);
+  if (mode != 1 && mode != 2 && mode != 4)
+    die("conv: -F must be 1 (forward), 2 (data gradient) or 4 (weight gradient)");
   const DataType dt = a.has("--bf16") ? DataType::BFloat16
                       : a.has("--fp16") ? DataType::Half : DataType::Float;
   const bool nhwc = a.s("--in_layout", "", "NCHW") == "NHWC";
   auto lay = [&](const Dims &d) { return nhwc ? chlast(d) : contig(d); };
+  if (mode != 1) {
+    const Dims xd = {n, c, H, W}, wd = {k, c / gcount, y, x};
+    const Dims yd = getConvInferredOutputShape(xd, wd, {l, j}, {p, q}, {u, v});
+    Graph g;
+    g.setName(mode == 2 ? "benchmark_conv_dgrad" : "benchmark_conv_wgrad")
+        .setIODataType(dt).setIntermediateDataType(DataType::Float)
+        .setComputeDataType(DataType::Float);
+    auto DY = g.tensor(mk("dy", yd, lay(yd), dt));
+    TensorPtr IN, OUT;
+    if (mode == 2) {
+      IN = g.tensor(mk("w", wd, lay(wd), dt));
+      ConvDGradAttr da;
+      da.setPadding({p, q}).setStride({u, v}).setDilation({l, j});
+      OUT = g.convDGrad(DY, IN, da);
+      OUT->setDim(xd);
+    } else {
+      IN = g.tensor(mk("x", xd, lay(xd), dt));
+      ConvWGradAttr wa;
+      wa.setPadding({p, q}).setStride({u, v}).setDilation({l, j});
+      OUT = g.convWGrad(DY, IN, wa);
+      OUT->setDim(wd);
+    }
+    OUT->setOutput(true).setDataType(dt);
+    OK(g.validate());
+    Pack pack = {{DY, constant(h, DY, 1.f)}, {IN, constant(h, IN, 1.f)},
+                 {OUT, constant(h, OUT, 0.f)}};
+    Run r{mode == 2 ? "conv_dgrad" : "conv_wgrad",
+          2.0 * n * yd[2] * yd[3] * k * (c / gcount) * y * x};
+    timeGraph(h, g, pack, r, iter);
+    return;
+  }
   Graph g;
   g.setName("benchmark_conv_fprop").setIODataType(dt)
       .setIntermediateDataType(DataType::Float).setComputeDataType(DataType::Float);

@@ -367,9 +367,22 @@ class Context:
                                              _epi_ptrs(epilogue_operands),
                                              _p(out), None, 0))
 
-    def conv_dgrad(self, d: ConvDesc, dy, w, dx):
+    def conv_dgrad(self, d: ConvDesc, dy, w, dx, workspace=None):
+        """`workspace`: a DeviceBuffer of at least conv_dgrad_workspace(d)
+        bytes; allocated here when omitted."""
+        need = self.conv_dgrad_workspace(d)
+        if need and workspace is None:
+            workspace = self.alloc(need)
         self._check(self.lib.fhip_conv_dgrad(self.handle, byref(d), _p(dy),
-                                             _p(w), _p(dx), None, 0))
+                                             _p(w), _p(dx), _p(workspace),
+                                             need))
+
+    def conv_dgrad_workspace(self, d: ConvDesc) -> int:
+        n = c_size_t(0)
+        if self.lib.fhip_conv_dgrad_workspace_size(byref(d), byref(n)) != 0:
+            # a query without a context reports through the process-wide slot
+            raise FusilliHipError(self.lib.fhip_last_error(None).decode())
+        return n.value
 
     def conv_wgrad(self, d: ConvDesc, dy, x, dw):
         self._check(self.lib.fhip_conv_wgrad(self.handle, byref(d), _p(dy),

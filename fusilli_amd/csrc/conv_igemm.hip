@@ -187,8 +187,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
       bm = small256 ? 256 : 0;
     else if (want > 0)
       bm = fits128 ? 128 : 0;
-    else
-      bm = small256 && big ? 256 : (small128 ? 128 : 0);
+    else // a slab past 80 KB (one workgroup per compute unit) still beats
+         // the gather on large outputs: 55.6 vs 74 us for C = K = 128, 56 x 56
+      bm = small256 && big ? 256
+                           : (small128 || (fits128 && big) ? 128 : 0);
     if (bm) {
       p.halo = true;
       p.bm = bm;
@@ -279,4 +281,126 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   if (p.kind == GK_BF16)
     return conv_launch_bf16(ctx, p.bm, p.bn, g);
   return conv_launch_f16(ctx, p.bm, p.bn, g);
+}
+
+// ---------------------------------------------------------------------------
+// Data gradient on the same kernels.  With unit strides and one group
+//   DX[n, c, i] = sum_{k, f} DY[n, k, i + pad - f * dil] * W[k, c, f]
+// is the forward convolution of DY (K channels) with the filter
+//   W'[c, k, f'] = W[k, c, F - 1 - f']   (taps mirrored, channel roles swapped)
+// under padding' = dil * (F - 1) - pad.  W' is small (the filter's size); it is
+// rebuilt in the caller's workspace on every call, channels-last, by a
+// transposing copy, and the forward kernel does the rest.
+// (Reference node/conv_node.h:428-598; aten.convolution_backward, input
+// gradient.)
+// ---------------------------------------------------------------------------
+namespace {
+
+struct DgradPlan {
+  bool ok = false;
+  fhip_conv_desc fwd; // the equivalent forward problem
+  size_t filter_bytes = 0;
+};
+
+DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
+  DgradPlan p;
+  const int sp = d->spatial_rank;
+  if (sp != 1 && sp != 2)
+    return p;
+  if (d->w.dim[1] != d->x.dim[1]) // groups
+    return p;
+  if (d->y.dtype != d->w.dtype)
+    return p;
+  fhip_conv_desc &f = p.fwd;
+  std::memset(&f, 0, sizeof(f));
+  f.spatial_rank = sp;
+  for (int i = 0; i < sp; ++i) {
+    if (d->stride[i] != 1)
+      return p;
+    const int64_t pad = d->dilation[i] * (d->w.dim[2 + i] - 1) - d->padding[i];
+    if (pad < 0)
+      return p;
+    f.padding[i] = pad;
+    f.stride[i] = 1;
+    f.dilation[i] = d->dilation[i];
+  }
+  f.x = d->y; // DY plays the input
+  f.y = d->x; // DX plays the output
+  f.out = d->x;
+  f.out_dtype = d->x.dtype;
+  // W' [C, K, F...], dense channels-last
+  f.w.rank = d->w.rank;
+  f.w.dtype = d->w.dtype;
+  f.w.dim[0] = d->w.dim[1];
+  f.w.dim[1] = d->w.dim[0];
+  int64_t st = f.w.dim[1];
+  f.w.stride[1] = 1;
+  for (int i = sp - 1; i >= 0; --i) {
+    f.w.dim[2 + i] = d->w.dim[2 + i];
+    f.w.stride[2 + i] = st;
+    st *= f.w.dim[2 + i];
+  }
+  f.w.stride[0] = st;
+  if (!fhip_fast_conv_applicable(&f))
+    return p;
+  p.filter_bytes = (size_t)(st * f.w.dim[0]) * fhip_dtype_size(f.w.dtype);
+  p.ok = true;
+  return p;
+}
+
+struct FlipArgs {
+  int64_t K, C, R, S;         // R = 1 for one spatial dim
+  int64_t sk, sc, sr, ss;     // element strides of W [K, C, R, S]
+};
+
+// dst[c][r'][s'][k] = src[k][c][R - 1 - r'][S - 1 - s'], 16-bit elements
+__global__ void conv_flip_filter_kernel(FlipArgs a, const uint16_t *src,
+                                        uint16_t *dst, int64_t total) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= total)
+    return;
+  const int64_t k = lin % a.K;
+  int64_t rem = lin / a.K;
+  const int64_t s2 = rem % a.S;
+  rem /= a.S;
+  const int64_t r2 = rem % a.R;
+  const int64_t c = rem / a.R;
+  dst[lin] = src[k * a.sk + c * a.sc + (a.R - 1 - r2) * a.sr +
+                 (a.S - 1 - s2) * a.ss];
+}
+
+} // namespace
+
+bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
+                                     size_t *workspace_bytes) {
+  const DgradPlan p = make_dgrad_plan(d);
+  if (workspace_bytes)
+    *workspace_bytes = p.ok ? p.filter_bytes : 0;
+  return p.ok;
+}
+
+int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
+                         const void *w, void *dx, void *workspace) {
+  const DgradPlan p = make_dgrad_plan(d);
+  FHIP_REQUIRE(ctx, p.ok, "conv dgrad: descriptor not supported by the MFMA kernel");
+  FHIP_REQUIRE(ctx, ((uintptr_t)workspace & 15) == 0,
+               "conv dgrad: workspace must be 16-byte aligned");
+  const int sp = d->spatial_rank;
+  FlipArgs a;
+  a.K = d->w.dim[0];
+  a.C = d->w.dim[1];
+  a.R = sp == 2 ? d->w.dim[2] : 1;
+  a.S = d->w.dim[1 + sp];
+  a.sk = d->w.dim[0] == 1 ? 0 : d->w.stride[0];
+  a.sc = d->w.dim[1] == 1 ? 0 : d->w.stride[1];
+  a.sr = sp == 2 ? d->w.stride[2] : 0;
+  a.ss = d->w.stride[1 + sp];
+  const int64_t total = a.K * a.C * a.R * a.S;
+  hipLaunchKernelGGL(conv_flip_filter_kernel,
+                     dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     ctx->stream, a, (const uint16_t *)w, (uint16_t *)workspace,
+                     total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  DevEpilogue epi{};
+  return fhip_fast_conv(ctx, &p.fwd, dy, workspace, epi, dx);
 }

@@ -14,6 +14,13 @@ bool fhip_fast_conv_applicable(const fhip_conv_desc *d);
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                    const void *w, const DevEpilogue &epi, void *out);
 
+// Data gradient through the forward kernel (unit strides, one group); needs
+// `*workspace_bytes` of 16-byte aligned workspace for the mirrored filter.
+bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
+                                     size_t *workspace_bytes);
+int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
+                         const void *w, void *dx, void *workspace);
+
 bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d);
 int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
                    const void *k, const void *v, void *o);

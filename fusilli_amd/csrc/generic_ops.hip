@@ -1037,11 +1037,16 @@ static ConvBwdArgs conv_bwd_args(const fhip_conv_desc *d, bool dgrad) {
 int fhip_conv_dgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
   FHIP_REQUIRE(nullptr, d && bytes, "fhip_conv_dgrad_workspace_size: null");
   *bytes = 0;
+  if (conv_bwd_validate(nullptr, d, "fhip_conv_dgrad") != 0)
+    return 1;
+  fhip_fast_conv_dgrad_applicable(d, bytes);
   return 0;
 }
 
 int fhip_conv_dgrad_supported(const fhip_conv_desc *d) {
-  return d && conv_bwd_validate(nullptr, d, "fhip_conv_dgrad") == 0 ? 1 : 0;
+  if (!d || conv_bwd_validate(nullptr, d, "fhip_conv_dgrad") != 0)
+    return 0;
+  return fhip_fast_conv_dgrad_applicable(d, nullptr) ? 2 : 1;
 }
 
 int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
@@ -1051,9 +1056,15 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   if (conv_bwd_validate(ctx, d, "fhip_conv_dgrad") != 0)
     return 1;
   FHIP_REQUIRE(ctx, dy && w && dx, "fhip_conv_dgrad: null tensor pointer");
-  (void)workspace;
-  (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  size_t need = 0;
+  if (fhip_fast_conv_dgrad_applicable(d, &need)) {
+    FHIP_REQUIRE(ctx, workspace && workspace_bytes >= need,
+                 "fhip_conv_dgrad: this descriptor needs %zu bytes of workspace "
+                 "(fhip_conv_dgrad_workspace_size), got %zu",
+                 need, workspace ? workspace_bytes : (size_t)0);
+    return fhip_fast_conv_dgrad(ctx, d, dy, w, dx, workspace);
+  }
   const ConvBwdArgs g = conv_bwd_args(d, true);
   const int64_t total = fhip_desc_volume(d->x);
   hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),

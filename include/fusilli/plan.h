@@ -82,7 +82,7 @@ struct Step {
 // Slot positions per step kind.
 enum : int { kMmA = 0, kMmB = 1, kMmOut = 2, kMmEpi = 3 };
 enum : int { kCvX = 0, kCvW = 1, kCvOut = 2, kCvEpi = 3 };
-enum : int { kCbDY = 0, kCbIn = 1, kCbOut = 2 }; // conv gradients
+enum : int { kCbDY = 0, kCbIn = 1, kCbOut = 2, kCbScratch = 3 }; // conv gradients
 enum : int { kSdQ = 0, kSdK = 1, kSdV = 2, kSdMask = 3, kSdO = 4 };
 enum : int {
   kNmX = 0,
@@ -791,6 +791,21 @@ private:
     FUSILLI_ASSIGN_OR_RETURN(s.slot[kCbDY], readSlot(dy));
     FUSILLI_ASSIGN_OR_RETURN(s.slot[kCbIn], readSlot(dgrad ? w : x));
     FUSILLI_ASSIGN_OR_RETURN(s.slot[kCbOut], writeSlot(dgrad ? x : w));
+    // kernel scratch (the data gradient's mirrored filter): a workspace
+    // region of its own, like a virtual tensor
+    size_t scratch = 0;
+    const int rc = dgrad ? fhip_conv_dgrad_workspace_size(&d, &scratch)
+                         : fhip_conv_wgrad_workspace_size(&d, &scratch);
+    FUSILLI_RETURN_ERROR_IF(rc != 0, ErrorCode::InternalError,
+                            std::string(fhip_last_error(nullptr)));
+    if (scratch > 0) {
+      WorkspaceTensor t;
+      t.offset = workspaceCursor_;
+      t.bytes = scratch;
+      workspaceCursor_ += (t.bytes + 255) / 256 * 256;
+      plan_.workspaceTensors.push_back(t);
+      s.slot[kCbScratch] = workspaceSlot(plan_.workspaceTensors.size() - 1);
+    }
     plan_.steps.push_back(s);
     return ok();
   }
@@ -816,6 +831,11 @@ inline ErrorObject execute(fhip_ctx *ctx, const Plan &p,
         p.workspaceTensors[static_cast<size_t>(-slot - 2)];
     return static_cast<char *>(workspace) + w.offset;
   };
+  auto bytesOf = [&](int32_t slot) -> size_t { // of a workspace region
+    return slot <= -2
+               ? p.workspaceTensors[static_cast<size_t>(-slot - 2)].bytes
+               : 0;
+  };
   for (const Step &s : p.steps) {
     int rc = 0;
     const void *epi[FHIP_MAX_EPILOGUE] = {nullptr, nullptr, nullptr, nullptr};
@@ -835,11 +855,13 @@ inline ErrorObject execute(fhip_ctx *ctx, const Plan &p,
       break;
     case StepKind::ConvDGrad:
       rc = fhip_conv_dgrad(ctx, &s.desc.conv, ptr(s.slot[kCbDY]),
-                           ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]), nullptr, 0);
+                           ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]),
+                           ptr(s.slot[kCbScratch]), bytesOf(s.slot[kCbScratch]));
       break;
     case StepKind::ConvWGrad:
       rc = fhip_conv_wgrad(ctx, &s.desc.conv, ptr(s.slot[kCbDY]),
-                           ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]), nullptr, 0);
+                           ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]),
+                           ptr(s.slot[kCbScratch]), bytesOf(s.slot[kCbScratch]));
       break;
     case StepKind::Sdpa:
       rc = fhip_sdpa_fwd(ctx, &s.desc.sdpa, ptr(s.slot[kSdQ]),

@@ -255,7 +255,11 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
  *      (dgrad output) or X (wgrad input), `w` describes W (dgrad input) or DW
  *      (wgrad output), `y` describes DY.  `epilogue` must be empty; `out` and
  *      `out_dtype` are not read.  f32 accumulation, one rounding to the
- *      gradient's dtype. -------------------------------------------------- */
+ *      gradient's dtype.  fhip_conv_dgrad_supported returns 2 where the MFMA
+ *      kernel takes the problem (16-bit channels-last tensors, unit strides,
+ *      one group): it then needs fhip_conv_dgrad_workspace_size bytes of
+ *      16-byte aligned workspace (a mirrored copy of the filter) and fails
+ *      without them. ------------------------------------------------------ */
 int fhip_conv_dgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes);
 int fhip_conv_dgrad_supported(const fhip_conv_desc *d);
 int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,

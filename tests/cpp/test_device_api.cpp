@@ -621,6 +621,56 @@ TEST("config 3 (reduced): bf16 NHWC conv 3x3 + bias + relu vs host loop") {
   CHECK(worst <= 0.0);
 }
 
+TEST("config 3 data gradient (reduced): bf16 NHWC on the MFMA kernel, scratch from the plan's workspace") {
+  const int64_t n = 2, c = 64, h = 14, w = 14, k = 128;
+  Graph g = newGraph("cfg3_dgrad", DataType::BFloat16, DataType::Float);
+  auto DY = g.tensor(mk("dy", {n, k, h, w}, chlast({n, k, h, w}), DataType::BFloat16));
+  auto W = g.tensor(mk("w", {k, c, 3, 3}, chlast({k, c, 3, 3}), DataType::BFloat16));
+  ConvDGradAttr da;
+  da.setPadding({1, 1}).setStride({1, 1}).setDilation({1, 1});
+  auto DX = g.convDGrad(DY, W, da);
+  DX->setDim({n, c, h, w}).setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  auto wsSize = g.getWorkspaceSize();
+  REQUIRE(!isError(wsSize) && wsSize->has_value());
+  CHECK(**wsSize >= static_cast<size_t>(k * c * 9 * 2)); // the mirrored filter
+  auto gf = randomVec(n * h * w * k, 31, -1.f, 1.f);
+  auto wf = randomVec(k * 9 * c, 32, -0.1f, 0.1f);
+  std::vector<bf16> gb(gf.size()), wb(wf.size());
+  for (size_t i = 0; i < gf.size(); ++i) gb[i] = (bf16)gf[i], gf[i] = (float)gb[i];
+  for (size_t i = 0; i < wf.size(); ++i) wb[i] = (bf16)wf[i], wf[i] = (float)wb[i];
+  Pack pack = {{DY, bufOf(DY, gb)}, {W, bufOf(W, wb)}, {DX, fill(DX, bf16(0.f))}};
+  REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+  auto out = readBack<bf16>(pack[DX]);
+  // physical layouts: dy [n][p][q][k], w [k][r][s][c], dx [n][h][w][c]
+  std::vector<double> ref(n * h * w * c, 0.0);
+  for (int64_t in = 0; in < n; ++in)
+    for (int64_t p = 0; p < h; ++p)
+      for (int64_t q = 0; q < w; ++q)
+        for (int64_t r = 0; r < 3; ++r)
+          for (int64_t s = 0; s < 3; ++s) {
+            const int64_t ih = p - 1 + r, iw = q - 1 + s;
+            if (ih < 0 || ih >= h || iw < 0 || iw >= w)
+              continue;
+            for (int64_t kk = 0; kk < k; ++kk) {
+              const double gy = gf[((in * h + p) * w + q) * k + kk];
+              for (int64_t cc = 0; cc < c; ++cc)
+                ref[((in * h + ih) * w + iw) * c + cc] +=
+                    gy * wf[((kk * 3 + r) * 3 + s) * c + cc];
+            }
+          }
+  REQUIRE(out.size() == ref.size());
+  double worst = 0, rms = 0;
+  for (double r : ref)
+    rms += r * r;
+  rms = std::sqrt(rms / ref.size());
+  for (size_t i = 0; i < ref.size(); ++i)
+    worst = std::max(worst, std::fabs((float)out[i] - ref[i]) -
+                                2e-2 * (std::fabs(ref[i]) + rms));
+  CHECK(worst <= 0.0);
+}
+
 TEST("config 5a (reduced): int8 matmul is bit exact") {
   const int64_t m = 256, k = 512, n = 384;
   Graph g = newGraph("cfg5a", DataType::Int8);

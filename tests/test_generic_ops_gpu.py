@@ -206,11 +206,13 @@ def conv_bwd_desc(x, w, dy, pad, stride, dil):
     return d
 
 
-def run_conv_dgrad(ctx, dy, w, x_dims, pad, stride, dil, dtype, nhwc=True):
+def run_conv_dgrad(ctx, dy, w, x_dims, pad, stride, dil, dtype, nhwc=True,
+                   tuned=False):
     dx = HT.empty(x_dims, dtype,
                   oracle.channels_last_strides(x_dims) if nhwc else None)
     d = conv_bwd_desc(dx, w, dy, pad, stride, dil)
-    assert ctx.lib.fhip_conv_dgrad_supported(d) == 1
+    assert ctx.lib.fhip_conv_dgrad_supported(d) == (2 if tuned else 1)
+    assert (ctx.conv_dgrad_workspace(d) > 0) == tuned
     bdy, bw, bdx = dy.upload(ctx), w.upload(ctx), dx.upload(ctx)
     ctx.conv_dgrad(d, bdy, bw, bdx)
     return dx.fetch(ctx, bdx)
@@ -283,6 +285,71 @@ def test_conv_backward_random_vs_oracle(ctx, case, dtype, nhwc):
                  oracle.conv_wgrad(dy.logical(), x.logical(), case["w"],
                                    case["pad"], case["s"], case["d"]),
                  dtype, f"wgrad {case}")
+
+
+@pytest.mark.parametrize("case", [
+    # C % 64 == 0 is not needed: the reduction runs over K
+    dict(x=[2, 24, 20, 20], w=[64, 24, 3, 3], pad=[1, 1], d=[1, 1]),
+    dict(x=[3, 64, 17, 13], w=[128, 64, 3, 3], pad=[1, 1], d=[1, 1]),
+    dict(x=[2, 40, 19, 23], w=[64, 40, 3, 2], pad=[2, 0], d=[2, 1]),
+    dict(x=[1, 16, 30, 9], w=[192, 16, 1, 1], pad=[0, 0], d=[1, 1]),
+    dict(x=[2, 72, 11, 11], w=[64, 72, 5, 5], pad=[0, 3], d=[1, 1]),
+    dict(x=[4, 32, 150], w=[64, 32, 4], pad=[2], d=[3]),
+])
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("w_nhwc", [True, False])
+def test_conv_dgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
+    # unit strides, one group, 16-bit channels-last gradients: the forward
+    # MFMA kernel on the mirrored filter (any filter layout)
+    sp = len(case["pad"])
+    ones = [1] * sp
+    yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], ones, case["d"])
+    w = HT.from_logical(rand(33, 1, case["w"], std=0.2), dtype,
+                        oracle.channels_last_strides(case["w"]) if w_nhwc else None)
+    dy = HT.from_logical(rand(33, 2, yd), dtype, oracle.channels_last_strides(yd))
+    dx = run_conv_dgrad(ctx, dy, w, case["x"], case["pad"], ones, case["d"],
+                        dtype, tuned=True)
+    assert_close(dx.logical(),
+                 oracle.conv_dgrad(dy.logical(), w.logical(), case["x"],
+                                   case["pad"], ones, case["d"]),
+                 dtype, f"dgrad {case}")
+
+
+def test_conv_dgrad_config3_shape_closed_form_and_oracle(ctx):
+    # the data gradient of benchmark config 3 (N32 C64 56x56, K128 3x3 pad 1).
+    # All-ones: DX = K * (taps whose output pixel exists) = 128 * {9, 6, 4}.
+    xd, wd = [32, 64, 56, 56], [128, 64, 3, 3]
+    yd = oracle.conv_output_dims(xd, wd, [1, 1], [1, 1], [1, 1])
+    cl = oracle.channels_last_strides
+    dy = HT.from_logical(np.ones(yd), capi.BFLOAT16, cl(yd))
+    w = HT.from_logical(np.ones(wd), capi.BFLOAT16, cl(wd))
+    dx = run_conv_dgrad(ctx, dy, w, xd, [1, 1], [1, 1], [1, 1], capi.BFLOAT16,
+                        tuned=True).logical()
+    edge = np.full(56, 3.0); edge[0] = edge[-1] = 2.0
+    want = 128.0 * np.outer(edge, edge)
+    assert np.array_equal(dx, np.broadcast_to(want, xd))
+    # random values: the first two images against the oracle
+    dy = HT.from_logical(rand(34, 0, yd), capi.BFLOAT16, cl(yd))
+    w = HT.from_logical(rand(34, 1, wd, std=0.05), capi.BFLOAT16, cl(wd))
+    dx = run_conv_dgrad(ctx, dy, w, xd, [1, 1], [1, 1], [1, 1], capi.BFLOAT16,
+                        tuned=True).logical()
+    ref = oracle.conv_dgrad(dy.logical()[:2], w.logical(), [2] + xd[1:],
+                            [1, 1], [1, 1], [1, 1])
+    assert_close(dx[:2], ref, capi.BFLOAT16, "config 3 dgrad")
+
+
+def test_conv_dgrad_needs_its_workspace(ctx):
+    xd, wd = [2, 24, 20, 20], [64, 24, 3, 3]
+    cl = oracle.channels_last_strides
+    dx = HT.empty(xd, capi.BFLOAT16, cl(xd))
+    w = HT.empty(wd, capi.BFLOAT16, cl(wd))
+    dy = HT.empty([2, 64, 20, 20], capi.BFLOAT16, cl([2, 64, 20, 20]))
+    d = conv_bwd_desc(dx, w, dy, [1, 1], [1, 1], [1, 1])
+    assert ctx.conv_dgrad_workspace(d) == 64 * 24 * 9 * 2
+    with pytest.raises(Exception, match="workspace"):
+        ctx._check(ctx.lib.fhip_conv_dgrad(ctx.handle, d, dy.upload(ctx).ptr,
+                                           w.upload(ctx).ptr, dx.upload(ctx).ptr,
+                                           None, 0))
 
 
 def test_conv_backward_rejects_bad_descriptors(ctx):
