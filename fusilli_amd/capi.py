@@ -113,6 +113,14 @@ class NormDesc(Structure):
                 ("out_dtype", c_int32), ("out", TensorDesc)]
 
 
+class BatchNormDesc(Structure):
+    _fields_ = [("x", TensorDesc), ("y", TensorDesc), ("training", c_int32),
+                ("has_scale", c_int32), ("has_bias", c_int32),
+                ("scale_dtype", c_int32), ("bias_dtype", c_int32),
+                ("running_dtype", c_int32), ("stats_dtype", c_int32),
+                ("epsilon", c_float)]
+
+
 class ReduceDesc(Structure):
     _fields_ = [("x", TensorDesc), ("y", TensorDesc), ("mode", c_int32)]
 
@@ -196,6 +204,10 @@ SYMBOLS = {
     "fhip_norm_fwd_workspace_size": (c_int, [POINTER(NormDesc), POINTER(c_size_t)]),
     "fhip_norm_fwd_supported": (c_int, [POINTER(NormDesc)]),
     "fhip_norm_fwd": (c_int, [_P, POINTER(NormDesc), _P, _P, _P, POINTER(_P), _P, _P, _P, _P, c_size_t]),
+    "fhip_batchnorm_fwd_workspace_size": (c_int, [POINTER(BatchNormDesc), POINTER(c_size_t)]),
+    "fhip_batchnorm_fwd_supported": (c_int, [POINTER(BatchNormDesc)]),
+    "fhip_batchnorm_fwd": (c_int, [_P, POINTER(BatchNormDesc), _P, _P, _P, _P, _P,
+                                   _P, _P, _P, _P, c_size_t]),
     "fhip_reduce_workspace_size": (c_int, [POINTER(ReduceDesc), POINTER(c_size_t)]),
     "fhip_reduce_supported": (c_int, [POINTER(ReduceDesc)]),
     "fhip_reduce": (c_int, [_P, POINTER(ReduceDesc), _P, _P, _P, c_size_t]),
@@ -387,6 +399,14 @@ class Context:
     def conv_wgrad(self, d: ConvDesc, dy, x, dw):
         self._check(self.lib.fhip_conv_wgrad(self.handle, byref(d), _p(dy),
                                              _p(x), _p(dw), None, 0))
+
+    def batchnorm_fwd(self, d: BatchNormDesc, x, y, scale=None, bias=None,
+                      running_mean=None, running_var=None, saved_mean=None,
+                      saved_inv_variance=None):
+        self._check(self.lib.fhip_batchnorm_fwd(
+            self.handle, byref(d), _p(x), _p(scale), _p(bias), _p(running_mean),
+            _p(running_var), _p(y), _p(saved_mean), _p(saved_inv_variance),
+            None, 0))
 
     def sdpa_fwd(self, d: SdpaDesc, q, k, v, o, mask=None):
         self._check(self.lib.fhip_sdpa_fwd(self.handle, byref(d), _p(q), _p(k),

@@ -693,6 +693,83 @@ __global__ __launch_bounds__(256) void generic_reduce_kernel(ReduceArgs g,
 }
 
 // --------------------------------------------------------------------------
+// batch normalisation forward (reference node/batchnorm_node.h:33-245;
+// aten.native_batch_norm, support/asm_emitter.h:1066-1290): per channel c
+//   inference: y = (x - mean[c]) / sqrt(var[c] + eps) * scale[c] + bias[c]
+//   training:  mean and biased variance of x over batch and space, y from
+//              them, and the two saved statistics (mean, 1 / sqrt(var + eps))
+// --------------------------------------------------------------------------
+struct BatchNormArgs {
+  Dims x;        // [N, C, spatial...]
+  Strides xs, ys;
+  int32_t x_dt, y_dt, scale_dt, bias_dt, mean_dt, stats_dt;
+  float eps;
+};
+
+__global__ void generic_batchnorm_infer_kernel(BatchNormArgs g, const void *x,
+                                               const void *scale,
+                                               const void *bias,
+                                               const void *mean, const void *var,
+                                               void *y, int64_t total) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= total)
+    return;
+  int64_t coord[FHIP_MAX_RANK];
+  unravel(lin, g.x, coord);
+  const int64_t c = coord[1];
+  const float m = fhip_load<float>(mean, g.mean_dt, c);
+  const float v = fhip_load<float>(var, g.mean_dt, c);
+  const float sc = scale ? fhip_load<float>(scale, g.scale_dt, c) : 1.f;
+  const float b = bias ? fhip_load<float>(bias, g.bias_dt, c) : 0.f;
+  const float xv = fhip_load<float>(x, g.x_dt, dot(coord, g.xs, g.x.rank));
+  const float r = (xv - m) * (1.0f / sqrtf(v + g.eps)) * sc + b;
+  fhip_store<float>(y, g.y_dt, dot(coord, g.ys, g.x.rank), r);
+}
+
+// One workgroup per channel, three walks over the channel's N x spatial
+// elements: mean, centred second moment, output.
+__global__ __launch_bounds__(256) void generic_batchnorm_train_kernel(
+    BatchNormArgs g, const void *x, const void *scale, const void *bias,
+    void *y, void *saved_mean, void *saved_inv_var) {
+  __shared__ float part[4];
+  const int64_t c = blockIdx.x;
+  const int rank = g.x.rank;
+  int64_t inner = 1; // spatial volume
+  for (int i = 2; i < rank; ++i)
+    inner *= g.x.dim[i];
+  const int64_t count = g.x.dim[0] * inner;
+  auto offset = [&](int64_t it, const Strides &st) {
+    int64_t rem = it, off = c * st.s[1];
+    for (int i = rank - 1; i >= 2; --i) {
+      off += (rem % g.x.dim[i]) * st.s[i];
+      rem /= g.x.dim[i];
+    }
+    return off + rem * st.s[0];
+  };
+  float acc = 0.f;
+  for (int64_t it = threadIdx.x; it < count; it += blockDim.x)
+    acc += fhip_load<float>(x, g.x_dt, offset(it, g.xs));
+  const float mean = block_sum_256(acc, part) / (float)count;
+  acc = 0.f;
+  for (int64_t it = threadIdx.x; it < count; it += blockDim.x) {
+    const float dv = fhip_load<float>(x, g.x_dt, offset(it, g.xs)) - mean;
+    acc += dv * dv;
+  }
+  const float var = block_sum_256(acc, part) / (float)count;
+  const float inv = 1.0f / sqrtf(var + g.eps);
+  const float sc = scale ? fhip_load<float>(scale, g.scale_dt, c) : 1.f;
+  const float b = bias ? fhip_load<float>(bias, g.bias_dt, c) : 0.f;
+  for (int64_t it = threadIdx.x; it < count; it += blockDim.x) {
+    const float xv = fhip_load<float>(x, g.x_dt, offset(it, g.xs));
+    fhip_store<float>(y, g.y_dt, offset(it, g.ys), (xv - mean) * inv * sc + b);
+  }
+  if (threadIdx.x == 0) {
+    fhip_store<float>(saved_mean, g.stats_dt, c, mean);
+    fhip_store<float>(saved_inv_var, g.stats_dt, c, inv);
+  }
+}
+
+// --------------------------------------------------------------------------
 // pointwise
 // --------------------------------------------------------------------------
 struct PointwiseArgs {
@@ -1308,6 +1385,99 @@ int fhip_norm_fwd(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
   hipLaunchKernelGGL(generic_norm_kernel, dim3((unsigned)d->x.dim[0]),
                      dim3(256), 0, ctx->stream, g, x, scale, bias, out, mean,
                      inv_variance);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+// ---- batch norm -----------------------------------------------------------
+static int batchnorm_validate(fhip_ctx *ctx, const fhip_batchnorm_desc *d) {
+  FHIP_REQUIRE(ctx, d != nullptr, "fhip_batchnorm_fwd: null descriptor");
+  if (!fhip_check_desc(ctx, d->x, "batchnorm X") ||
+      !fhip_check_desc(ctx, d->y, "batchnorm Y"))
+    return 1;
+  FHIP_REQUIRE(ctx, d->x.rank >= 2, "fhip_batchnorm_fwd: X rank %d < 2",
+               d->x.rank);
+  FHIP_REQUIRE(ctx, dims_equal(d->y, d->x.rank, d->x.dim),
+               "fhip_batchnorm_fwd: Y dims differ from X dims");
+  auto fl = [](int dt) {
+    return dt == FHIP_FLOAT || dt == FHIP_HALF || dt == FHIP_BFLOAT16 ||
+           dt == FHIP_DOUBLE;
+  };
+  FHIP_REQUIRE(ctx, fl(d->x.dtype) && fl(d->y.dtype),
+               "fhip_batchnorm_fwd: X and Y must be floating point");
+  FHIP_REQUIRE(ctx, !d->has_scale || fl(d->scale_dtype),
+               "fhip_batchnorm_fwd: SCALE must be floating point");
+  FHIP_REQUIRE(ctx, !d->has_bias || fl(d->bias_dtype),
+               "fhip_batchnorm_fwd: BIAS must be floating point");
+  if (d->training)
+    FHIP_REQUIRE(ctx, fl(d->stats_dtype),
+                 "fhip_batchnorm_fwd: saved statistics must be floating point");
+  else
+    FHIP_REQUIRE(ctx, fl(d->running_dtype),
+                 "fhip_batchnorm_fwd: running statistics must be floating "
+                 "point");
+  FHIP_REQUIRE(ctx, d->epsilon >= 0.f, "fhip_batchnorm_fwd: negative epsilon");
+  FHIP_REQUIRE(ctx, !d->training || d->x.dim[1] < (1ll << 31),
+               "fhip_batchnorm_fwd: channel count exceeds the grid limit");
+  return 0;
+}
+
+int fhip_batchnorm_fwd_workspace_size(const fhip_batchnorm_desc *d,
+                                      size_t *bytes) {
+  FHIP_REQUIRE(nullptr, d && bytes, "fhip_batchnorm_fwd_workspace_size: null");
+  *bytes = 0;
+  return 0;
+}
+
+int fhip_batchnorm_fwd_supported(const fhip_batchnorm_desc *d) {
+  return d && batchnorm_validate(nullptr, d) == 0 ? 1 : 0;
+}
+
+int fhip_batchnorm_fwd(fhip_ctx *ctx, const fhip_batchnorm_desc *d,
+                       const void *x, const void *scale, const void *bias,
+                       const void *running_mean, const void *running_var,
+                       void *y, void *saved_mean, void *saved_inv_variance,
+                       void *workspace, size_t workspace_bytes) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_batchnorm_fwd: null context");
+  if (batchnorm_validate(ctx, d) != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, x && y, "fhip_batchnorm_fwd: null tensor pointer");
+  FHIP_REQUIRE(ctx, !d->has_scale == !scale && !d->has_bias == !bias,
+               "fhip_batchnorm_fwd: SCALE / BIAS pointers disagree with the "
+               "descriptor");
+  if (d->training)
+    FHIP_REQUIRE(ctx, saved_mean && saved_inv_variance,
+                 "fhip_batchnorm_fwd: training needs the saved statistics' "
+                 "buffers");
+  else
+    FHIP_REQUIRE(ctx, running_mean && running_var,
+                 "fhip_batchnorm_fwd: inference needs running mean and "
+                 "variance");
+  (void)workspace;
+  (void)workspace_bytes;
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  BatchNormArgs g{};
+  g.x = make_dims(d->x);
+  g.xs = make_strides(d->x);
+  g.ys = make_strides(d->y);
+  g.x_dt = d->x.dtype;
+  g.y_dt = d->y.dtype;
+  g.scale_dt = d->scale_dtype;
+  g.bias_dt = d->bias_dtype;
+  g.mean_dt = d->running_dtype;
+  g.stats_dt = d->stats_dtype;
+  g.eps = d->epsilon;
+  const int64_t total = fhip_desc_volume(d->x);
+  if (total == 0)
+    return 0;
+  if (d->training)
+    hipLaunchKernelGGL(generic_batchnorm_train_kernel,
+                       dim3((unsigned)d->x.dim[1]), dim3(256), 0, ctx->stream, g,
+                       x, scale, bias, y, saved_mean, saved_inv_variance);
+  else
+    hipLaunchKernelGGL(generic_batchnorm_infer_kernel,
+                       dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream, g,
+                       x, scale, bias, running_mean, running_var, y, total);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }

@@ -318,6 +318,35 @@ int fhip_norm_fwd(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
                   const void *const *epilogue_operands, void *out, void *mean,
                   void *inv_variance, void *workspace, size_t workspace_bytes);
 
+/* ---- batch normalisation forward (node/batchnorm_node.h:33-245;
+ *      aten.native_batch_norm, support/asm_emitter.h:1066-1290).  Statistics
+ *      are per channel (dim 1) over batch and space.  SCALE, BIAS, the
+ *      running statistics and the saved statistics are dense vectors of C
+ *      elements.  Inference (training = 0) normalises with the running mean
+ *      and variance; training computes the batch mean and biased variance,
+ *      normalises with them and stores mean and 1 / sqrt(var + eps).  The
+ *      reference's MOMENTUM operand does not influence any of these outputs
+ *      (the op returns no updated running statistics) and has no field. --- */
+typedef struct {
+  fhip_tensor_desc x; /* [N, C, spatial...] */
+  fhip_tensor_desc y; /* same dims */
+  int32_t training;
+  int32_t has_scale, has_bias;
+  int32_t scale_dtype, bias_dtype;
+  int32_t running_dtype; /* MEAN and VAR (inference) */
+  int32_t stats_dtype;   /* SAVED_MEAN and SAVED_INV_VARIANCE (training) */
+  float epsilon;
+} fhip_batchnorm_desc;
+
+int fhip_batchnorm_fwd_workspace_size(const fhip_batchnorm_desc *d,
+                                      size_t *bytes);
+int fhip_batchnorm_fwd_supported(const fhip_batchnorm_desc *d);
+int fhip_batchnorm_fwd(fhip_ctx *ctx, const fhip_batchnorm_desc *d,
+                       const void *x, const void *scale, const void *bias,
+                       const void *running_mean, const void *running_var,
+                       void *y, void *saved_mean, void *saved_inv_variance,
+                       void *workspace, size_t workspace_bytes);
+
 /* ---- reduction (node/reduction_node.h:31-146;
  *      support/asm_emitter.h:2165-2322).  Keep-dim: y has x's rank; a dim is
  *      reduced where y.dim == 1 and x.dim > 1. --------------------------- */

@@ -381,6 +381,36 @@ RED_ADD, RED_SUM, RED_MUL, RED_MIN, RED_MAX, RED_AMAX, RED_AVG, RED_NORM1, \
     RED_NORM2, RED_MUL_NO_ZEROS = range(1, 11)
 
 
+def batchnorm(x, scale, bias, running_mean, running_var, eps, training):
+    """aten.native_batch_norm (asm_emitter.h:1066-1290, node/batchnorm_node.h):
+    statistics per channel (dim 1) over batch and space.  Inference uses the
+    running mean / variance; training the batch mean and BIASED variance, and
+    also returns (mean, 1 / sqrt(var + eps)).  Returns (y, saved_mean,
+    saved_inv_variance); the last two are None for inference.
+    Pinned by: the reference samples' answers (samples/batchnorm/
+    batchnorm_utils.h:22-107: x = c + 1 under mean 0 / var 1; a +-1 half / half
+    pattern => mean 0, inv_variance 1/sqrt(1 + eps)), torch.native_batch_norm
+    in float64, and the invariants mean_c(y) = bias, var_c(y) =
+    scale^2 var / (var + eps)."""
+    x = np.asarray(x, np.float32).astype(np.float64)
+    c = x.shape[1]
+    shape = [1, c] + [1] * (x.ndim - 2)
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    if training:
+        mean = x.mean(axis=axes)
+        var = ((x - mean.reshape(shape)) ** 2).mean(axis=axes)
+    else:
+        mean = np.asarray(running_mean, np.float32).astype(np.float64)
+        var = np.asarray(running_var, np.float32).astype(np.float64)
+    inv = 1.0 / np.sqrt(var + float(eps))
+    y = (x - mean.reshape(shape)) * inv.reshape(shape)
+    if scale is not None:
+        y = y * np.asarray(scale, np.float32).astype(np.float64).reshape(shape)
+    if bias is not None:
+        y = y + np.asarray(bias, np.float32).astype(np.float64).reshape(shape)
+    return (y, mean, inv) if training else (y, None, None)
+
+
 def reduction(x: np.ndarray, out_dims, mode: int) -> np.ndarray:
     """Keep-dim reductions over dims where out == 1 < x
     (node/reduction_node.h:47-56; asm_emitter.h:2165-2322).  Pinned by the

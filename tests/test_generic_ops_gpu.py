@@ -367,6 +367,113 @@ def test_conv_backward_rejects_bad_descriptors(ctx):
         ctx.conv_dgrad(d, dy.upload(ctx), w.upload(ctx), x.upload(ctx))
 
 
+# ---- batch norm -----------------------------------------------------------
+def run_batchnorm(ctx, x, *, training, eps, scale=None, bias=None, mean=None,
+                  var=None, y_dtype=None, stats_dtype=capi.FLOAT):
+    """Returns (y, saved_mean, saved_inv_variance) as logical arrays."""
+    c = x.dims[1]
+    y = HT.empty(x.dims, x.dtype if y_dtype is None else y_dtype, x.strides)
+    d = capi.BatchNormDesc()
+    d.x, d.y = x.desc(), y.desc()
+    d.training = int(training)
+    d.has_scale, d.has_bias = int(scale is not None), int(bias is not None)
+    d.scale_dtype = scale.dtype if scale is not None else capi.FLOAT
+    d.bias_dtype = bias.dtype if bias is not None else capi.FLOAT
+    d.running_dtype = mean.dtype if mean is not None else capi.FLOAT
+    d.stats_dtype = stats_dtype
+    d.epsilon = eps
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 1
+    up = lambda t: None if t is None else t.upload(ctx)
+    sm, sv = HT.empty([c], stats_dtype), HT.empty([c], stats_dtype)
+    by, bsm, bsv = y.upload(ctx), sm.upload(ctx), sv.upload(ctx)
+    ctx.batchnorm_fwd(d, x.upload(ctx), by, up(scale), up(bias), up(mean), up(var),
+                      bsm if training else None, bsv if training else None)
+    y.fetch(ctx, by)
+    if not training:
+        return y.logical(), None, None
+    return y.logical(), sm.fetch(ctx, bsm).logical(), sv.fetch(ctx, bsv).logical()
+
+
+@pytest.mark.parametrize("nhwc", [False, True])
+@pytest.mark.parametrize("affine", [False, True])
+def test_batchnorm_inference_known_answer(ctx, nhwc, affine):
+    # samples/batchnorm/batchnorm_infer_{nchw,nchw_scale_bias,nhwc_scale_bias}.cpp
+    # with batchnorm_utils.h:22-47: x = c + 1, mean 0, var 1.
+    n, c, h, w, eps = 2, 4, 8, 8, 1e-5
+    xd = [n, c, h, w]
+    xv = np.broadcast_to(np.arange(1, c + 1, dtype=np.float64).reshape(1, c, 1, 1), xd)
+    x = HT.from_logical(xv, capi.FLOAT, oracle.channels_last_strides(xd) if nhwc else None)
+    vec = lambda v: HT.from_logical(np.full([c], v), capi.FLOAT)
+    y, _, _ = run_batchnorm(ctx, x, training=False, eps=eps,
+                            scale=vec(2.0) if affine else None,
+                            bias=vec(0.5) if affine else None,
+                            mean=vec(0.0), var=vec(1.0))
+    want = xv / np.sqrt(np.float32(1 + eps))
+    want = 2.0 * want + 0.5 if affine else want
+    assert np.max(np.abs(y - want)) < 1e-4  # the samples' tolerance
+
+
+@pytest.mark.parametrize("affine", [False, True])
+def test_batchnorm_training_known_answer(ctx, affine):
+    # samples/batchnorm/batchnorm_train_nchw{,_scale_bias}.cpp with
+    # batchnorm_utils.h:60-104: +-1 halves => mean 0, inv_variance 1/sqrt(1+eps).
+    n, c, h, w, eps = 2, 4, 8, 8, 1e-5
+    flat = np.where(np.arange(n * h * w) < n * h * w // 2, -1.0, 1.0)
+    xv = np.broadcast_to(flat.reshape(n, 1, h, w), [n, c, h, w])
+    x = HT.from_logical(xv, capi.FLOAT)
+    vec = lambda v: HT.from_logical(np.full([c], v), capi.FLOAT)
+    y, m, v = run_batchnorm(ctx, x, training=True, eps=eps,
+                            scale=vec(2.0) if affine else None,
+                            bias=vec(0.5) if affine else None)
+    inv = 1.0 / np.sqrt(1.0 + eps)
+    want = xv * inv
+    want = 2.0 * want + 0.5 if affine else want
+    assert np.max(np.abs(y - want)) < 1e-4
+    assert np.max(np.abs(m)) < 1e-4 and np.max(np.abs(v - inv)) < 1e-4
+
+
+@pytest.mark.parametrize("dims", [[3, 5, 7, 6], [4, 3, 9], [2, 6], [2, 3, 4, 5, 2],
+                                  [8, 64, 28, 28]])
+@pytest.mark.parametrize("training", [False, True])
+@pytest.mark.parametrize("dtype", [capi.FLOAT, capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("nhwc", [False, True])
+def test_batchnorm_random_vs_oracle(ctx, dims, training, dtype, nhwc):
+    if nhwc and len(dims) < 3:
+        pytest.skip("no spatial dims")
+    c, eps = dims[1], 1e-3
+    x = HT.from_logical(rand(41, 0, dims, std=2.0, mean=1.0), dtype,
+                        oracle.channels_last_strides(dims) if nhwc else None)
+    sc = HT.from_logical(rand(41, 1, [c], mean=1.0, std=0.3), dtype)
+    b = HT.from_logical(rand(41, 2, [c]), dtype)
+    rm = HT.from_logical(rand(41, 3, [c]), capi.FLOAT)
+    rv = HT.from_logical(rand(41, 4, [c], "uniform", lo=0.5, hi=1.5), capi.FLOAT)
+    y, m, v = run_batchnorm(ctx, x, training=training, eps=eps, scale=sc, bias=b,
+                            mean=None if training else rm,
+                            var=None if training else rv)
+    ry, rmean, rinv = oracle.batchnorm(x.logical(), sc.logical(), b.logical(),
+                                       rm.logical(), rv.logical(), eps, training)
+    assert_close(y, ry, dtype, f"batchnorm {dims}")
+    if training:
+        assert_close(m, rmean, capi.FLOAT, "saved mean")
+        assert_close(v, rinv, capi.FLOAT, "saved inv variance")
+
+
+def test_batchnorm_rejects_bad_descriptors(ctx):
+    d = capi.BatchNormDesc()
+    d.x = capi.TensorDesc.make([2, 4, 8, 8], [256, 64, 8, 1], capi.FLOAT)
+    d.y = capi.TensorDesc.make([2, 4, 8, 7], [224, 56, 7, 1], capi.FLOAT)
+    d.running_dtype = d.stats_dtype = d.scale_dtype = d.bias_dtype = capi.FLOAT
+    d.epsilon = 1e-5
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 0
+    d.y = d.x
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 1
+    d.x = capi.TensorDesc.make([8], [1], capi.FLOAT)
+    d.y = d.x
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 0
+    d.x = d.y = capi.TensorDesc.make([2, 4, 8, 8], [256, 64, 8, 1], capi.INT32)
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 0
+
+
 # ---- sdpa -----------------------------------------------------------------
 def run_sdpa(ctx, q, k, v, *, mask=None, causal=False, scale=None, o_dtype=None):
     o_dtype = q.dtype if o_dtype is None else o_dtype

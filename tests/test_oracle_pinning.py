@@ -209,6 +209,55 @@ def test_conv_backward_matches_torch_autograd_and_adjoint(case):
     assert np.isclose(lhs, float(np.sum(dw * w.astype(np.float64))), rtol=1e-9)
 
 
+# ---- batch norm -----------------------------------------------------------------
+def test_batchnorm_known_answers():
+    # samples/batchnorm/batchnorm_utils.h:22-47 (inference): x = c + 1, mean 0,
+    # var 1 => scale * (c + 1) / sqrt(1 + eps) + bias
+    n, c, h, w, eps = 2, 4, 8, 8, 1e-5
+    x = np.broadcast_to(np.arange(1, c + 1, dtype=np.float64).reshape(1, c, 1, 1),
+                        [n, c, h, w])
+    y, m, v = oracle.batchnorm(x, None, None, np.zeros(c), np.ones(c), eps, False)
+    assert m is None and v is None
+    assert np.allclose(y, x / np.sqrt(1 + eps), rtol=1e-12)
+    y, _, _ = oracle.batchnorm(x, np.full(c, 2.0), np.full(c, 0.5), np.zeros(c),
+                               np.ones(c), eps, False)
+    assert np.allclose(y, 2.0 * x / np.sqrt(1 + eps) + 0.5, rtol=1e-12)
+    # batchnorm_utils.h:60-104 (training): -1 on the first half of (n, h, w),
+    # +1 on the second => mean 0, biased var 1
+    flat = np.where(np.arange(n * h * w) < n * h * w // 2, -1.0, 1.0)
+    x = np.broadcast_to(flat.reshape(n, 1, h, w), [n, c, h, w])
+    y, m, v = oracle.batchnorm(x, np.full(c, 2.0), np.full(c, 0.5), None, None,
+                               eps, True)
+    assert np.allclose(m, 0.0) and np.allclose(v, 1 / np.sqrt(1 + eps), rtol=1e-12)
+    assert np.allclose(y, 2.0 * x / np.sqrt(1 + eps) + 0.5, rtol=1e-12)
+
+
+@pytest.mark.parametrize("dims", [[3, 5, 7, 6], [4, 3, 9], [2, 6], [2, 3, 4, 5, 2]])
+@pytest.mark.parametrize("training", [False, True])
+@pytest.mark.parametrize("affine", [False, True])
+def test_batchnorm_matches_torch_and_invariants(dims, training, affine):
+    c, eps = dims[1], 1e-3
+    x = (RNG.normal(size=dims) * 2 + 1).astype(np.float32)
+    sc = RNG.normal(size=c).astype(np.float32) if affine else None
+    b = RNG.normal(size=c).astype(np.float32) if affine else None
+    rm = RNG.normal(size=c).astype(np.float32)
+    rv = (RNG.uniform(size=c) + 0.5).astype(np.float32)
+    ty, tm, tv = torch.native_batch_norm(
+        t64(x), None if sc is None else t64(sc), None if b is None else t64(b),
+        t64(rm), t64(rv), training, 0.1, eps)
+    y, m, v = oracle.batchnorm(x, sc, b, rm, rv, eps, training)
+    assert np.allclose(y, ty.numpy(), rtol=1e-9, atol=1e-9)
+    if training:
+        assert np.allclose(m, tm.numpy(), rtol=1e-9, atol=1e-12)
+        assert np.allclose(v, tv.numpy(), rtol=1e-9)
+        axes = tuple(i for i in range(len(dims)) if i != 1)
+        var = x.astype(np.float64).var(axis=axes)
+        s64 = np.ones(c) if sc is None else sc.astype(np.float64)
+        b64 = np.zeros(c) if b is None else b.astype(np.float64)
+        assert np.allclose(y.mean(axis=axes), b64, atol=1e-9)
+        assert np.allclose(y.var(axis=axes), s64 ** 2 * var / (var + eps), rtol=1e-9)
+
+
 # ---- attention ------------------------------------------------------------------
 def torch_sdpa(q, k, v, mask=None, causal=False, scale=None):
     rep = q.shape[1] // k.shape[1]
