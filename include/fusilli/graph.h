@@ -404,6 +404,38 @@ public:
     return {y, m, v};
   }
 
+  // graph.h:860-913 of the reference.  SAVED_MEAN and SAVED_INV_VARIANCE are
+  // null outside the training phase.
+  std::array<std::shared_ptr<TensorAttr>, 3>
+  batchnorm(const TensorPtr &x, const TensorPtr &scale, const TensorPtr &bias,
+            const TensorPtr &mean, const TensorPtr &var, BatchnormAttr &attr) {
+    nameNode(attr, "batchnorm");
+    nameTensor(x, attr, "X");
+    nameTensor(scale, attr, "SCALE");
+    nameTensor(bias, attr, "BIAS");
+    nameTensor(mean, attr, "MEAN");
+    nameTensor(var, attr, "VAR");
+    nameTensor(attr.getEpsilon(), attr, "EPSILON");
+    nameTensor(attr.getMomentum(), attr, "MOMENTUM");
+    attr.setX(x);
+    attr.setSCALE(scale);
+    attr.setBIAS(bias);
+    attr.setMEAN(mean);
+    attr.setVAR(var);
+    auto y = outputTensor(attr.getName() + "_Y");
+    std::shared_ptr<TensorAttr> m, v;
+    if (attr.getForwardPhase() == NormFwdPhase::TRAINING) {
+      m = outputTensor(attr.getName() + "_SAVED_MEAN");
+      v = outputTensor(attr.getName() + "_SAVED_INV_VARIANCE");
+    }
+    attr.setY(y);
+    attr.setSAVED_MEAN(m);
+    attr.setSAVED_INV_VARIANCE(v);
+    subNodes_.emplace_back(
+        std::make_shared<BatchNormNode>(std::move(attr), context));
+    return {y, m, v};
+  }
+
   // Number of kernel launches the loaded plan performs (the analogue of the
   // dispatch count the reference reads from IREE's compile statistics).
   std::optional<size_t> getKernelCount() const {

@@ -1094,6 +1094,137 @@ private:
   }
 };
 
+// ---- batch norm (node/batchnorm_node.h:33-245) -----------------------------------
+class BatchNormNode : public NodeCRTP<BatchNormNode> {
+public:
+  BatchnormAttr batchnormAttr;
+  BatchNormNode(BatchnormAttr &&attr, const Context &ctx)
+      : NodeCRTP(ctx), batchnormAttr(std::move(attr)) {}
+  const std::string &getName() const override final {
+    return batchnormAttr.getName();
+  }
+  Type getType() const override final { return Type::BatchNorm; }
+
+  ErrorObject preValidateNode() const override final {
+    FUSILLI_LOG_LABEL_ENDL("INFO: Pre-Validating BatchNormNode '" << getName()
+                                                                  << "'");
+    FUSILLI_RETURN_ERROR_IF(batchnormAttr.getForwardPhase() ==
+                                NormFwdPhase::NOT_SET,
+                            ErrorCode::AttributeNotSet,
+                            "BatchNorm forward phase not set");
+    const TensorPtr x = batchnormAttr.getX(), y = batchnormAttr.getY();
+    FUSILLI_RETURN_ERROR_IF(!x, ErrorCode::AttributeNotSet,
+                            "BatchNorm input tensor X not set");
+    FUSILLI_RETURN_ERROR_IF(!y, ErrorCode::AttributeNotSet,
+                            "BatchNorm output tensor Y not set");
+    FUSILLI_RETURN_ERROR_IF(
+        x->getDim().size() < 2, ErrorCode::InvalidAttribute,
+        "BatchNorm input tensor X must have a rank of at least 2");
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(x),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(x));
+    if (!training()) {
+      FUSILLI_RETURN_ERROR_IF(!batchnormAttr.getMEAN(),
+                              ErrorCode::AttributeNotSet,
+                              "BatchNorm inference requires running MEAN");
+      FUSILLI_RETURN_ERROR_IF(!batchnormAttr.getVAR(),
+                              ErrorCode::AttributeNotSet,
+                              "BatchNorm inference requires running VAR");
+      FUSILLI_RETURN_ERROR_IF(
+          batchnormAttr.getSAVED_MEAN() != nullptr, ErrorCode::InvalidAttribute,
+          "BatchNorm SAVED_MEAN should not be set in inference mode");
+      FUSILLI_RETURN_ERROR_IF(
+          batchnormAttr.getSAVED_INV_VARIANCE() != nullptr,
+          ErrorCode::InvalidAttribute,
+          "BatchNorm SAVED_INV_VARIANCE should not be set in inference mode");
+    } else {
+      FUSILLI_RETURN_ERROR_IF(!batchnormAttr.getSAVED_MEAN(),
+                              ErrorCode::AttributeNotSet,
+                              "BatchNorm training requires SAVED_MEAN output");
+      FUSILLI_RETURN_ERROR_IF(
+          !batchnormAttr.getSAVED_INV_VARIANCE(), ErrorCode::AttributeNotSet,
+          "BatchNorm training requires SAVED_INV_VARIANCE output");
+    }
+    const TensorPtr eps = batchnormAttr.getEpsilon();
+    FUSILLI_RETURN_ERROR_IF(!eps, ErrorCode::AttributeNotSet,
+                            "BatchNorm epsilon not set");
+    FUSILLI_RETURN_ERROR_IF(!eps->isScalar(), ErrorCode::InvalidAttribute,
+                            "BatchNorm epsilon must be a scalar constant");
+    const TensorPtr mom = batchnormAttr.getMomentum();
+    FUSILLI_RETURN_ERROR_IF(!mom, ErrorCode::AttributeNotSet,
+                            "BatchNorm momentum not set");
+    FUSILLI_RETURN_ERROR_IF(!mom->isScalar(), ErrorCode::InvalidAttribute,
+                            "BatchNorm momentum must be a scalar constant");
+    return ok();
+  }
+
+  ErrorObject inferPropertiesNode() override final {
+    batchnormAttr.fillFromContext(context);
+    const TensorPtr x = batchnormAttr.getX(), y = batchnormAttr.getY();
+    const std::vector<int64_t> cDim = {x->getDim()[1]};
+    auto infer1D = [&](const TensorPtr &t) {
+      if (!t)
+        return;
+      if (t->getDim().empty())
+        t->setDim(cDim);
+      if (t->getStride().empty())
+        t->setStride(std::vector<int64_t>{1});
+    };
+    infer1D(batchnormAttr.getSCALE());
+    infer1D(batchnormAttr.getBIAS());
+    infer1D(batchnormAttr.getMEAN());
+    infer1D(batchnormAttr.getVAR());
+    if (y->getDim().empty())
+      y->setDim(x->getDim());
+    if (y->getStride().empty())
+      y->setStride(x->getStride());
+    if (training()) {
+      infer1D(batchnormAttr.getSAVED_MEAN());
+      infer1D(batchnormAttr.getSAVED_INV_VARIANCE());
+    }
+    return ok();
+  }
+
+  ErrorObject postValidateNode() const override final {
+    const TensorPtr x = batchnormAttr.getX(), y = batchnormAttr.getY();
+    const std::vector<int64_t> cDim = {x->getDim()[1]};
+    FUSILLI_RETURN_ERROR_IF(
+        x->getDim() != y->getDim(), ErrorCode::InvalidAttribute,
+        "BatchNorm output Y tensor must have the same shape as input X tensor");
+    FUSILLI_RETURN_ERROR_IF(!detail::contiguousOrChannelsLast(y),
+                            ErrorCode::NotImplemented,
+                            detail::layoutMessage(y));
+    auto check1D = [&](const TensorPtr &t, const std::string &name) {
+      if (!t)
+        return ok();
+      FUSILLI_RETURN_ERROR_IF(
+          t->getDim() != cDim, ErrorCode::InvalidAttribute,
+          "BatchNorm tensor " + name +
+              " must be 1D with size equal to channel dimension C");
+      FUSILLI_RETURN_ERROR_IF(t->getStride() != std::vector<int64_t>{1},
+                              ErrorCode::InvalidAttribute,
+                              "BatchNorm tensor " + name +
+                                  " must have unit stride");
+      return ok();
+    };
+    FUSILLI_CHECK_ERROR(check1D(batchnormAttr.getSCALE(), "SCALE"));
+    FUSILLI_CHECK_ERROR(check1D(batchnormAttr.getBIAS(), "BIAS"));
+    FUSILLI_CHECK_ERROR(check1D(batchnormAttr.getMEAN(), "MEAN"));
+    FUSILLI_CHECK_ERROR(check1D(batchnormAttr.getVAR(), "VAR"));
+    if (training()) {
+      FUSILLI_CHECK_ERROR(check1D(batchnormAttr.getSAVED_MEAN(), "SAVED_MEAN"));
+      FUSILLI_CHECK_ERROR(check1D(batchnormAttr.getSAVED_INV_VARIANCE(),
+                                  "SAVED_INV_VARIANCE"));
+    }
+    return ok();
+  }
+
+private:
+  bool training() const {
+    return batchnormAttr.getForwardPhase() == NormFwdPhase::TRAINING;
+  }
+};
+
 } // namespace fusilli
 
 #endif // FUSILLI_NODES_H

@@ -456,6 +456,39 @@ private:
   NormFwdPhase phase_ = NormFwdPhase::NOT_SET;
 };
 
+// ---- batch norm (attributes/batchnorm_attributes.h) ------------------------------
+class BatchnormAttr : public AttributesCRTP<BatchnormAttr> {
+public:
+  enum class InputNames : uint8_t { X, SCALE, BIAS, MEAN, VAR, EPSILON, MOMENTUM };
+  enum class OutputNames : uint8_t { Y, SAVED_MEAN, SAVED_INV_VARIANCE };
+  FUSILLI_SLOT_MAPS
+  FUSILLI_IN_SLOT(BatchnormAttr, X)
+  FUSILLI_IN_SLOT(BatchnormAttr, SCALE)
+  FUSILLI_IN_SLOT(BatchnormAttr, BIAS)
+  FUSILLI_IN_SLOT(BatchnormAttr, MEAN)
+  FUSILLI_IN_SLOT(BatchnormAttr, VAR)
+  FUSILLI_OUT_SLOT(BatchnormAttr, Y)
+  FUSILLI_OUT_SLOT(BatchnormAttr, SAVED_MEAN)
+  FUSILLI_OUT_SLOT(BatchnormAttr, SAVED_INV_VARIANCE)
+
+  BatchnormAttr &setEpsilon(const TensorPtr &eps) {
+    return setInput(InputNames::EPSILON, eps);
+  }
+  TensorPtr getEpsilon() const { return getInput(InputNames::EPSILON); }
+  BatchnormAttr &setMomentum(const TensorPtr &m) {
+    return setInput(InputNames::MOMENTUM, m);
+  }
+  TensorPtr getMomentum() const { return getInput(InputNames::MOMENTUM); }
+  BatchnormAttr &setForwardPhase(NormFwdPhase p) {
+    phase_ = p;
+    return *this;
+  }
+  NormFwdPhase getForwardPhase() const { return phase_; }
+
+private:
+  NormFwdPhase phase_ = NormFwdPhase::NOT_SET;
+};
+
 #undef FUSILLI_IN_SLOT
 #undef FUSILLI_OUT_SLOT
 #undef FUSILLI_SLOT_MAPS

@@ -41,6 +41,7 @@ enum class StepKind : uint32_t {
   Pointwise = 6,
   ConvDGrad = 7,
   ConvWGrad = 8,
+  BatchNorm = 9,
 };
 
 constexpr int kMaxSlots = 12;
@@ -59,6 +60,7 @@ union StepDesc {
   fhip_norm_desc norm;
   fhip_reduce_desc reduce;
   fhip_pointwise_desc pointwise;
+  fhip_batchnorm_desc batchnorm;
 };
 
 struct Step {
@@ -92,6 +94,16 @@ enum : int {
   kNmMean = 4,
   kNmRstd = 5,
   kNmEpi = 6
+};
+enum : int {
+  kBnX = 0,
+  kBnScale = 1,
+  kBnBias = 2,
+  kBnMean = 3,
+  kBnVar = 4,
+  kBnY = 5,
+  kBnSavedMean = 6,
+  kBnSavedInvVar = 7
 };
 enum : int { kRdX = 0, kRdY = 1 };
 enum : int { kPwIn0 = 0, kPwIn1 = 1, kPwIn2 = 2, kPwOut = 3 };
@@ -280,6 +292,10 @@ public:
         FUSILLI_CHECK_ERROR(planConvBackward(i));
         ++i;
         break;
+      case INode::Type::BatchNorm:
+        FUSILLI_CHECK_ERROR(planBatchNorm(i));
+        ++i;
+        break;
       case INode::Type::RmsNorm:
       case INode::Type::LayerNorm: {
         FUSILLI_ASSIGN_OR_RETURN(size_t next, planNorm(i));
@@ -329,6 +345,9 @@ private:
     switch (n.getType()) {
     case INode::Type::Convolution:
       each(static_cast<const ConvFPropNode &>(n).convFPropAttr);
+      break;
+    case INode::Type::BatchNorm:
+      each(static_cast<const BatchNormNode &>(n).batchnormAttr);
       break;
     case INode::Type::WGrad:
       each(static_cast<const ConvWGradNode &>(n).convWGradAttr);
@@ -751,6 +770,64 @@ private:
 
   const std::vector<std::shared_ptr<INode>> &nodes_;
   Plan plan_;
+  // Batch norm: one step, nothing fused.  MOMENTUM is validated by the node
+  // and has no effect on the outputs.
+  ErrorObject planBatchNorm(size_t i) {
+    const auto &a = static_cast<const BatchNormNode &>(*nodes_[i]).batchnormAttr;
+    const bool training = a.getForwardPhase() == NormFwdPhase::TRAINING;
+    Step s;
+    s.kind = static_cast<uint32_t>(StepKind::BatchNorm);
+    fhip_batchnorm_desc &d = s.desc.batchnorm;
+    FUSILLI_ASSIGN_OR_RETURN(d.x, toDesc(a.getX()));
+    FUSILLI_ASSIGN_OR_RETURN(d.y, toDesc(a.getY()));
+    d.training = training ? 1 : 0;
+    d.epsilon = static_cast<float>(scalarAsDouble(*a.getEpsilon()));
+    const int32_t f32 = static_cast<int32_t>(DataType::Float);
+    d.scale_dtype = d.bias_dtype = d.running_dtype = d.stats_dtype = f32;
+    if (const TensorPtr t = a.getSCALE()) {
+      d.has_scale = 1;
+      d.scale_dtype = static_cast<int32_t>(t->getDataType());
+      FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnScale], readSlot(t));
+    }
+    if (const TensorPtr t = a.getBIAS()) {
+      d.has_bias = 1;
+      d.bias_dtype = static_cast<int32_t>(t->getDataType());
+      FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnBias], readSlot(t));
+    }
+    if (!training) {
+      const TensorPtr m = a.getMEAN(), v = a.getVAR();
+      FUSILLI_RETURN_ERROR_IF(m->getDataType() != v->getDataType(),
+                              ErrorCode::NotImplemented,
+                              "BatchNorm MEAN and VAR must share an element "
+                              "type");
+      d.running_dtype = static_cast<int32_t>(m->getDataType());
+      FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnMean], readSlot(m));
+      FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnVar], readSlot(v));
+    } else {
+      const TensorPtr m = a.getSAVED_MEAN(), v = a.getSAVED_INV_VARIANCE();
+      FUSILLI_RETURN_ERROR_IF(m->getDataType() != v->getDataType(),
+                              ErrorCode::NotImplemented,
+                              "BatchNorm SAVED_MEAN and SAVED_INV_VARIANCE must "
+                              "share an element type");
+      d.stats_dtype = static_cast<int32_t>(m->getDataType());
+    }
+    FUSILLI_RETURN_ERROR_IF(fhip_batchnorm_fwd_supported(&d) == 0,
+                            ErrorCode::NotImplemented,
+                            "BatchNorm node '" + a.getName() +
+                                "' is not executable by this backend: " +
+                                fhip_last_error(nullptr));
+    FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnX], readSlot(a.getX()));
+    FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnY], writeSlot(a.getY()));
+    if (training) {
+      FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnSavedMean],
+                               writeSlot(a.getSAVED_MEAN()));
+      FUSILLI_ASSIGN_OR_RETURN(s.slot[kBnSavedInvVar],
+                               writeSlot(a.getSAVED_INV_VARIANCE()));
+    }
+    plan_.steps.push_back(s);
+    return ok();
+  }
+
   // Conv gradients: one step each, nothing fused (the descriptor names the
   // forward problem: x = X / DX, w = W / DW, y = DY).
   ErrorObject planConvBackward(size_t i) {
@@ -862,6 +939,13 @@ inline ErrorObject execute(fhip_ctx *ctx, const Plan &p,
       rc = fhip_conv_wgrad(ctx, &s.desc.conv, ptr(s.slot[kCbDY]),
                            ptr(s.slot[kCbIn]), ptr(s.slot[kCbOut]),
                            ptr(s.slot[kCbScratch]), bytesOf(s.slot[kCbScratch]));
+      break;
+    case StepKind::BatchNorm:
+      rc = fhip_batchnorm_fwd(ctx, &s.desc.batchnorm, ptr(s.slot[kBnX]),
+                              ptr(s.slot[kBnScale]), ptr(s.slot[kBnBias]),
+                              ptr(s.slot[kBnMean]), ptr(s.slot[kBnVar]),
+                              ptr(s.slot[kBnY]), ptr(s.slot[kBnSavedMean]),
+                              ptr(s.slot[kBnSavedInvVar]), nullptr, 0);
       break;
     case StepKind::Sdpa:
       rc = fhip_sdpa_fwd(ctx, &s.desc.sdpa, ptr(s.slot[kSdQ]),

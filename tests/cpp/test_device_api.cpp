@@ -269,6 +269,97 @@ TEST("conv gradients: f32 3x3 stride 2 pad 1 against host loops") {
   CHECK(worst <= 0.0);
 }
 
+// ---- batch norm samples ----------------------------------------------------------
+// samples/batchnorm/*.cpp with the generators of batchnorm_utils.h:22-107.
+static void batchnormSample(bool training, bool nhwc, bool affine) {
+  const int64_t n = 2, c = 4, h = 8, w = 8;
+  const float eps = 1e-5f, scale = 2.0f, bias = 0.5f;
+  Graph g = newGraph(std::string("bn_") + (training ? "train" : "infer") +
+                         (nhwc ? "_nhwc" : "_nchw") + (affine ? "_sb" : ""),
+                     DataType::Float);
+  const Dims xd = {n, c, h, w};
+  auto X = g.tensor(mk("x", xd, nhwc ? chlast(xd) : contig(xd), DataType::Float));
+  std::shared_ptr<TensorAttr> SC, BI, MEAN, VAR;
+  if (affine) {
+    SC = g.tensor(mk("scale", {c}, {1}, DataType::Float));
+    BI = g.tensor(mk("bias", {c}, {1}, DataType::Float));
+  }
+  if (!training) {
+    MEAN = g.tensor(mk("mean", {c}, {1}, DataType::Float));
+    VAR = g.tensor(mk("var", {c}, {1}, DataType::Float));
+  }
+  BatchnormAttr a;
+  a.setForwardPhase(training ? NormFwdPhase::TRAINING : NormFwdPhase::INFERENCE)
+      .setEpsilon(g.tensor(TensorAttr(eps).setName("epsilon")))
+      .setMomentum(g.tensor(TensorAttr(0.1f).setName("momentum")))
+      .setName("batchnorm");
+  auto [Y, SM, SV] = g.batchnorm(X, SC, BI, MEAN, VAR, a);
+  Y->setName("y").setDataType(DataType::Float).setOutput(true);
+  if (training) {
+    SM->setName("saved_mean").setDataType(DataType::Float).setOutput(true);
+    SV->setName("saved_inv_var").setDataType(DataType::Float).setOutput(true);
+  }
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), /*remove=*/true));
+  CHECK(g.getKernelCount() == std::optional<size_t>(1));
+  // logical NCHW values, written through X's strides
+  const float invStd = 1.0f / std::sqrt(1.0f + eps);
+  std::vector<float> xin(n * c * h * w), want(xin.size());
+  for (int64_t ni = 0; ni < n; ++ni)
+    for (int64_t ci = 0; ci < c; ++ci)
+      for (int64_t hi = 0; hi < h; ++hi)
+        for (int64_t wi = 0; wi < w; ++wi) {
+          const float xv = training
+                               ? (ni * h * w + hi * w + wi < n * h * w / 2 ? -1.f : 1.f)
+                               : static_cast<float>(ci + 1);
+          const size_t idx = nhwc ? ((ni * h + hi) * w + wi) * c + ci
+                                  : ((ni * c + ci) * h + hi) * w + wi;
+          xin[idx] = xv;
+          want[idx] = (affine ? scale : 1.f) * xv * invStd + (affine ? bias : 0.f);
+        }
+  Pack pack = {{X, bufOf(X, xin)}, {Y, fill(Y, 0.f)}};
+  if (affine) {
+    pack[SC] = fill(SC, scale);
+    pack[BI] = fill(BI, bias);
+  }
+  if (training) {
+    pack[SM] = fill(SM, 7.f);
+    pack[SV] = fill(SV, 7.f);
+  } else {
+    pack[MEAN] = fill(MEAN, 0.f);
+    pack[VAR] = fill(VAR, 1.f);
+  }
+  auto ws = workspaceFor(g);
+  for (int rep = 0; rep < 2; ++rep) {
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+    auto out = readBack<float>(pack[Y]);
+    REQUIRE(out.size() == want.size());
+    float worst = 0;
+    for (size_t i = 0; i < out.size(); ++i)
+      worst = std::max(worst, std::fabs(out[i] - want[i]));
+    CHECK(worst < 1e-4f); // the samples' tolerance
+    if (training) {
+      auto sm = readBack<float>(pack[SM]);
+      auto sv = readBack<float>(pack[SV]);
+      REQUIRE(sm.size() == static_cast<size_t>(c));
+      REQUIRE(sv.size() == static_cast<size_t>(c));
+      for (int64_t ci = 0; ci < c; ++ci) {
+        CHECK(std::fabs(sm[ci]) < 1e-4f);
+        CHECK(std::fabs(sv[ci] - invStd) < 1e-4f);
+      }
+    }
+  }
+}
+
+TEST("samples: batchnorm inference and training known answers") {
+  batchnormSample(false, false, false); // batchnorm_infer_nchw.cpp
+  batchnormSample(false, false, true);  // batchnorm_infer_nchw_scale_bias.cpp
+  batchnormSample(false, true, true);   // batchnorm_infer_nhwc_scale_bias.cpp
+  batchnormSample(true, false, false);  // batchnorm_train_nchw.cpp
+  batchnormSample(true, false, true);   // batchnorm_train_nchw_scale_bias.cpp
+  batchnormSample(true, true, true);
+}
+
 // ---- matmul samples ----------------------------------------------------------
 TEST("samples: matmul all-ones, transposed B, bias, batched broadcast") {
   for (int variant = 0; variant < 3; ++variant) {

@@ -669,6 +669,158 @@ static ConvGraph makeConvGraph(const std::string &name) {
   return c;
 }
 
+TEST("batchnorm node: inference and errors") {
+  // tests/test_batchnorm_node.cpp of the reference
+  const Dims xd = {2, 4, 8, 8};
+  {
+    Graph g = newGraph("bn_train");
+    auto x = g.tensor(mk("x", xd, chlast(xd)));
+    BatchnormAttr a;
+    a.setForwardPhase(NormFwdPhase::TRAINING)
+        .setEpsilon(g.tensor(TensorAttr(1e-5f)))
+        .setMomentum(g.tensor(TensorAttr(0.1f)));
+    auto scale = g.tensor(TensorAttr().setName("scale").setDataType(DataType::Float));
+    auto [y, m, v] = g.batchnorm(x, scale, nullptr, nullptr, nullptr, a);
+    y->setOutput(true);
+    m->setOutput(true);
+    v->setOutput(true);
+    REQUIRE_OK(g.validate());
+    CHECK(y->getName() == "batchnorm_0_Y");
+    CHECK(m->getName() == "batchnorm_0_SAVED_MEAN");
+    CHECK(v->getName() == "batchnorm_0_SAVED_INV_VARIANCE");
+    CHECK((y->getDim() == xd));
+    CHECK((y->getStride() == chlast(xd))); // follows X
+    CHECK((scale->getDim() == Dims{4}));
+    CHECK((scale->getStride() == Dims{1}));
+    CHECK((m->getDim() == Dims{4}));
+    CHECK((v->getStride() == Dims{1}));
+  }
+  {
+    Graph g = newGraph("bn_infer");
+    auto x = g.tensor(mk("x", xd, contig(xd)));
+    auto mean = g.tensor(mk("mean", {4}, {1}));
+    auto var = g.tensor(mk("var", {4}, {1}));
+    BatchnormAttr a;
+    a.setForwardPhase(NormFwdPhase::INFERENCE)
+        .setEpsilon(g.tensor(TensorAttr(1e-5f)))
+        .setMomentum(g.tensor(TensorAttr(0.1f)));
+    auto [y, m, v] = g.batchnorm(x, nullptr, nullptr, mean, var, a);
+    y->setOutput(true);
+    CHECK(m == nullptr);
+    CHECK(v == nullptr);
+    REQUIRE_OK(g.validate());
+    CHECK(y->isContiguous());
+  }
+  Context ctx;
+  auto T = [](const char *name, Dims d, Dims st) {
+    return std::make_shared<TensorAttr>(mk(name, d, st));
+  };
+  auto S = [](float v) { return std::make_shared<TensorAttr>(TensorAttr(v)); };
+  auto node = [&](bool training, auto &&tweak) {
+    BatchnormAttr a;
+    a.setForwardPhase(training ? NormFwdPhase::TRAINING : NormFwdPhase::INFERENCE)
+        .setEpsilon(S(1e-5f)).setMomentum(S(0.1f));
+    a.setX(T("X", xd, contig(xd))).setY(T("Y", xd, contig(xd)));
+    if (training)
+      a.setSAVED_MEAN(T("SM", {4}, {1})).setSAVED_INV_VARIANCE(T("SV", {4}, {1}));
+    else
+      a.setMEAN(T("MEAN", {4}, {1})).setVAR(T("VAR", {4}, {1}));
+    tweak(a);
+    return BatchNormNode(std::move(a), ctx);
+  };
+  REQUIRE_OK(node(false, [](auto &) {}).preValidateNode());
+  REQUIRE_OK(node(true, [](auto &) {}).preValidateNode());
+  CHECK_ERROR(node(false, [](auto &a) {
+                a.setForwardPhase(NormFwdPhase::NOT_SET);
+              }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "BatchNorm forward phase not set");
+  CHECK_ERROR(node(false, [](auto &a) { a.setX(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "BatchNorm input tensor X not set");
+  CHECK_ERROR(node(false, [](auto &a) { a.setY(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "BatchNorm output tensor Y not set");
+  CHECK_ERROR(node(false, [](auto &a) { a.setEpsilon(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "BatchNorm epsilon not set");
+  CHECK_ERROR(node(false, [](auto &a) { a.setMomentum(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet, "BatchNorm momentum not set");
+  CHECK_ERROR(node(false, [&](auto &a) {
+                a.setEpsilon(T("eps", {1}, {1}));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm epsilon must be a scalar constant");
+  CHECK_ERROR(node(false, [&](auto &a) {
+                a.setMomentum(T("mom", {1}, {1}));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm momentum must be a scalar constant");
+  CHECK_ERROR(node(false, [&](auto &a) { a.setX(T("X", {8}, {1})); }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm input tensor X must have a rank of at least 2");
+  CHECK_ERROR(node(false, [&](auto &a) {
+                a.setX(T("X", xd, {256, 8, 1, 64}));
+              }).preValidateNode(),
+              ErrorCode::NotImplemented,
+              "Tensor 'X' is neither contiguous nor channels-last as defined "
+              "by its stride");
+  CHECK_ERROR(node(false, [](auto &a) { a.setMEAN(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet,
+              "BatchNorm inference requires running MEAN");
+  CHECK_ERROR(node(false, [](auto &a) { a.setVAR(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet,
+              "BatchNorm inference requires running VAR");
+  CHECK_ERROR(node(false, [&](auto &a) {
+                a.setSAVED_MEAN(T("SM", {4}, {1}));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm SAVED_MEAN should not be set in inference mode");
+  CHECK_ERROR(node(false, [&](auto &a) {
+                a.setSAVED_INV_VARIANCE(T("SV", {4}, {1}));
+              }).preValidateNode(),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm SAVED_INV_VARIANCE should not be set in inference mode");
+  CHECK_ERROR(node(true, [](auto &a) { a.setSAVED_MEAN(nullptr); }).preValidateNode(),
+              ErrorCode::AttributeNotSet,
+              "BatchNorm training requires SAVED_MEAN output");
+  CHECK_ERROR(node(true, [](auto &a) {
+                a.setSAVED_INV_VARIANCE(nullptr);
+              }).preValidateNode(),
+              ErrorCode::AttributeNotSet,
+              "BatchNorm training requires SAVED_INV_VARIANCE output");
+  // post-validation
+  auto post = [&](bool training, auto &&tweak) {
+    auto n = node(training, tweak);
+    ErrorObject e = n.preValidateNode();
+    if (isOk(e))
+      e = n.inferPropertiesNode();
+    return isOk(e) ? n.postValidateNode() : e;
+  };
+  REQUIRE_OK(post(false, [](auto &) {}));
+  CHECK_ERROR(post(false, [&](auto &a) {
+                a.setY(T("Y", {2, 4, 8, 7}, contig({2, 4, 8, 7})));
+              }),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm output Y tensor must have the same shape as input X "
+              "tensor");
+  CHECK_ERROR(post(false, [&](auto &a) { a.setY(T("Y", xd, {256, 8, 1, 64})); }),
+              ErrorCode::NotImplemented,
+              "Tensor 'Y' is neither contiguous nor channels-last as defined "
+              "by its stride");
+  CHECK_ERROR(post(false, [&](auto &a) { a.setSCALE(T("S", {5}, {1})); }),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm tensor SCALE must be 1D with size equal to channel "
+              "dimension C");
+  CHECK_ERROR(post(false, [&](auto &a) { a.setBIAS(T("B", {1, 4}, {4, 1})); }),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm tensor BIAS must be 1D with size equal to channel "
+              "dimension C");
+  CHECK_ERROR(post(false, [&](auto &a) { a.setVAR(T("VAR", {4}, {2})); }),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm tensor VAR must have unit stride");
+  CHECK_ERROR(post(true, [&](auto &a) { a.setSAVED_MEAN(T("SM", {8}, {1})); }),
+              ErrorCode::InvalidAttribute,
+              "BatchNorm tensor SAVED_MEAN must be 1D with size equal to "
+              "channel dimension C");
+}
+
 TEST("graph: name, symbol uniqueness, broadcast outputs") {
   {
     Graph g;
