@@ -10,6 +10,7 @@
 #define FUSILLI_GRAPH_H
 
 #include <array>
+#include <map>
 #include <optional>
 #include <set>
 #include <span>
@@ -166,15 +167,20 @@ public:
         "Graph::execute requires getWorkspaceSize() to be called before "
         "workspace allocation and execution");
 
+    // Tensors with dynamic dims take their extents from the buffers: a plan
+    // specialised to those extents replaces the loaded one.
+    FUSILLI_ASSIGN_OR_RETURN(const plan::Plan *planPtr,
+                             planForBuffers(handle, variantPack));
+    const plan::Plan &activePlan = *planPtr;
     std::vector<void *> args;
-    args.reserve(loadedPlan_->args.size());
+    args.reserve(activePlan.args.size());
     auto push = [&](const std::shared_ptr<TensorAttr> &t) -> ErrorObject {
       const std::shared_ptr<Buffer> &buf = variantPack.at(t);
       FUSILLI_RETURN_ERROR_IF(!buf || buf->data() == nullptr,
                               ErrorCode::VariantPackError,
                               "Tensor '" + t->getName() +
                                   "' has a null buffer in variantPack");
-      const plan::ArgInfo &info = loadedPlan_->args[args.size()];
+      const plan::ArgInfo &info = activePlan.args[args.size()];
       FUSILLI_RETURN_ERROR_IF(
           buf->sizeInBytes() < info.minBytes, ErrorCode::VariantPackError,
           "Buffer for tensor '" + t->getName() + "' holds " +
@@ -246,7 +252,13 @@ public:
                               "Tensor '" + kv.first->getName() +
                                   "' is backed by host memory; AMDGPU "
                                   "execution needs device buffers");
-    return plan::execute(handle.getContext(), *loadedPlan_, args, workspacePtr);
+    FUSILLI_RETURN_ERROR_IF(
+        activePlan.workspaceBytes > *workspaceSize_, ErrorCode::InvalidArgument,
+        "The buffers' extents need " +
+            std::to_string(activePlan.workspaceBytes) +
+            " bytes of workspace, more than getWorkspaceSize() reported (" +
+            std::to_string(*workspaceSize_) + ")");
+    return plan::execute(handle.getContext(), activePlan, args, workspacePtr);
   }
 
   // ---- builders ---------------------------------------------------------------
@@ -507,12 +519,124 @@ private:
     loadedPlan_.reset();
     loadedBackend_.reset();
     workspaceSize_.reset();
+    dynamicPlans_.clear();
+  }
+
+  // ---- dynamic dims (reference samples/dynamic_shapes/*.cpp) --------------------
+  // A tensor marked with setDynamicDims() is declared at the extents compile()
+  // plans for; execute() may be given buffers whose shape differs in those
+  // dims.  The plan for a new set of extents is built on first use and kept.
+  // Every tensor whose extents change must be in the variant pack (a virtual
+  // tensor's extents cannot be read from a buffer).
+
+  // Puts back the dims, strides and dynamic-dim marks it replaced.
+  class ShapeOverride {
+  public:
+    ShapeOverride() = default;
+    ShapeOverride(const ShapeOverride &) = delete;
+    ShapeOverride &operator=(const ShapeOverride &) = delete;
+    void set(const std::shared_ptr<TensorAttr> &t, std::vector<int64_t> dims) {
+      saved_.push_back({t, t->getDim(), t->getStride()});
+      // dense strides in the tensor's own dim order; broadcast dims stay 0
+      const auto perm = t->getLogicalToPhysicalPermuteOrder();
+      const std::vector<int64_t> oldDim = t->getDim(), oldStride = t->getStride();
+      std::vector<int64_t> stride(dims.size(), 1);
+      int64_t run = 1;
+      for (size_t i = dims.size(); i-- > 0;) {
+        const size_t src = static_cast<size_t>(perm[i]);
+        if (oldDim[src] > 1 && oldStride[src] == 0) {
+          stride[src] = 0;
+        } else {
+          stride[src] = run;
+          run *= dims[src];
+        }
+      }
+      t->setDim(dims).setStride(stride);
+    }
+    ~ShapeOverride() {
+      for (auto it = saved_.rbegin(); it != saved_.rend(); ++it)
+        it->t->setDim(it->dim).setStride(it->stride);
+    }
+
+  private:
+    struct Saved {
+      std::shared_ptr<TensorAttr> t;
+      std::vector<int64_t> dim, stride;
+    };
+    std::vector<Saved> saved_;
+  };
+
+  // The loaded plan, or the plan specialised to the extents of the buffers
+  // bound to tensors with dynamic dims.
+  ErrorOr<const plan::Plan *> planForBuffers(
+      const Handle &handle,
+      const std::unordered_map<std::shared_ptr<TensorAttr>,
+                               std::shared_ptr<Buffer>> &variantPack) const {
+    std::vector<int64_t> key;
+    std::vector<std::pair<std::shared_ptr<TensorAttr>, std::vector<int64_t>>>
+        changed;
+    auto visit = [&](const std::shared_ptr<TensorAttr> &t) -> ErrorObject {
+      if (!t->hasDynamicDims())
+        return ok();
+      auto it = variantPack.find(t);
+      if (it == variantPack.end() || !it->second)
+        return ok(); // reported by the variant-pack checks
+      const std::vector<size_t> &shape = it->second->getShape();
+      const std::vector<int64_t> &dim = t->getDim();
+      if (shape.size() != dim.size())
+        return ok(); // an untyped / imported buffer carries no extents
+      const auto perm = t->getLogicalToPhysicalPermuteOrder();
+      std::vector<int64_t> now = dim;
+      for (size_t i = 0; i < dim.size(); ++i) {
+        const size_t src = static_cast<size_t>(perm[i]);
+        if (dim[src] > 1 && t->getStride()[src] == 0)
+          continue; // broadcast dims occupy one element
+        now[src] = static_cast<int64_t>(shape[i]);
+      }
+      const auto &dyn = t->getDynamicDims();
+      for (size_t i = 0; i < dim.size(); ++i)
+        FUSILLI_RETURN_ERROR_IF(
+            now[i] != dim[i] &&
+                std::find(dyn.begin(), dyn.end(), i) == dyn.end(),
+            ErrorCode::VariantPackError,
+            "Buffer for tensor '" + t->getName() + "' has extent " +
+                std::to_string(now[i]) + " in dim " + std::to_string(i) +
+                ", which is not a dynamic dim (expected " +
+                std::to_string(dim[i]) + ")");
+      for (size_t i = 0; i < dim.size(); ++i)
+        FUSILLI_RETURN_ERROR_IF(now[i] < 1, ErrorCode::VariantPackError,
+                                "Buffer for tensor '" + t->getName() +
+                                    "' has an empty dynamic dim");
+      key.insert(key.end(), now.begin(), now.end());
+      if (now != dim)
+        changed.emplace_back(t, std::move(now));
+      return ok();
+    };
+    for (const auto &out : fullGraphOutputsSorted_)
+      if (!out->isVirtual())
+        FUSILLI_CHECK_ERROR(visit(out));
+    for (const auto &in : fullGraphInputsSorted_)
+      if (!in->isScalar())
+        FUSILLI_CHECK_ERROR(visit(in));
+    if (changed.empty())
+      return ok(&*loadedPlan_);
+    if (auto it = dynamicPlans_.find(key); it != dynamicPlans_.end())
+      return ok(&it->second);
+    ShapeOverride scope;
+    for (auto &[t, dims] : changed)
+      scope.set(t, dims);
+    plan::Planner planner(subNodes_, fullGraphInputsSorted_,
+                          fullGraphOutputsSorted_, handle.getBackend());
+    FUSILLI_ASSIGN_OR_RETURN(plan::Plan p, planner.run());
+    return ok(&dynamicPlans_.emplace(std::move(key), std::move(p)).first->second);
   }
 
   bool isValidated_ = false;
   std::optional<plan::Plan> loadedPlan_;
   std::optional<Backend> loadedBackend_;
   std::optional<size_t> workspaceSize_;
+  // plans for buffer extents that differ from the declared ones
+  mutable std::map<std::vector<int64_t>, plan::Plan> dynamicPlans_;
 
   std::unordered_set<std::shared_ptr<TensorAttr>> fullGraphInputs_;
   std::unordered_set<std::shared_ptr<TensorAttr>> fullGraphOutputs_;

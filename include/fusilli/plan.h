@@ -227,10 +227,8 @@ inline ErrorOr<fhip_tensor_desc> toDesc(const TensorPtr &t) {
                           ErrorCode::NotImplemented,
                           "Tensor '" + t->getName() + "' has rank above " +
                               std::to_string(FHIP_MAX_RANK));
-  FUSILLI_RETURN_ERROR_IF(t->hasDynamicDims(), ErrorCode::NotImplemented,
-                          "Tensor '" + t->getName() +
-                              "' has dynamic dims; this backend plans static "
-                              "shapes only");
+  // Dynamic dims are planned at the extents the TensorAttr holds: the graph
+  // re-plans with the buffers' extents when they differ (Graph::execute).
   FUSILLI_RETURN_ERROR_IF(dataTypeSize(t->getDataType()) == 0,
                           ErrorCode::NotImplemented,
                           "Tensor '" + t->getName() + "' has element type " +

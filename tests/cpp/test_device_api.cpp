@@ -360,6 +360,143 @@ TEST("samples: batchnorm inference and training known answers") {
   batchnormSample(true, true, true);
 }
 
+// ---- dynamic dims --------------------------------------------------------------
+// samples/dynamic_shapes/conv_fprop_dynamic_batch.cpp,
+// reduction_min_max_dynamic_batch.cpp, sdpa_basic_dynamic_sequence.cpp: one
+// compiled graph, buffers of several extents in the dynamic dim.
+template <typename T>
+static std::shared_ptr<Buffer> shaped(const Dims &shape, T v) {
+  std::vector<size_t> sh(shape.begin(), shape.end());
+  size_t n = 1;
+  for (size_t d : sh)
+    n *= d;
+  auto b = Buffer::allocate(gpu(), sh, std::vector<T>(n, v));
+  if (isError(b)) {
+    std::printf("allocate failed: %s\n", ErrorObject(b).getMessage().c_str());
+    std::exit(3);
+  }
+  return std::make_shared<Buffer>(std::move(*b));
+}
+
+TEST("dynamic dims: conv batch, reduction batch and sdpa sequence from one compiled graph each") {
+  {
+    const int64_t n = 4, c = 4, h = 4, w = 4, k = 4;
+    Graph g = newGraph("dynamic_conv_fprop", DataType::Half);
+    auto X = g.tensor(mk("image", {n, c, h, w}, contig({n, c, h, w}), DataType::Half)
+                          .setDynamicDims({0}));
+    auto W = g.tensor(mk("filter", {k, c, 1, 1}, contig({k, c, 1, 1}), DataType::Half));
+    ConvFPropAttr ca;
+    ca.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    auto Y = g.convFProp(X, W, ca);
+    Y->setDynamicDims({0}).setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    auto ws = g.getWorkspaceSize();
+    REQUIRE(!isError(ws) && ws->has_value());
+    CHECK(**ws == 0);
+    auto wBuf = fill(W, half(1.f));
+    for (int64_t rn : {int64_t{1}, int64_t{2}, n, int64_t{2}}) {
+      Pack pack = {{X, shaped<half>({rn, c, h, w}, half(1.f))}, {W, wBuf},
+                   {Y, shaped<half>({rn, k, h, w}, half(0.f))}};
+      REQUIRE_OK(g.execute(gpu(), pack, nullptr));
+      auto out = readBack<half>(pack[Y]);
+      REQUIRE(out.size() == static_cast<size_t>(rn * k * h * w));
+      CHECK(allEqual(out, 4.f)); // conv_fprop_dynamic_batch.cpp:110
+    }
+    // a non-dynamic dim must keep its extent
+    Pack bad = {{X, shaped<half>({2, c, h, w + 1}, half(1.f))}, {W, wBuf},
+                {Y, shaped<half>({2, k, h, w}, half(0.f))}};
+    CHECK_ERROR(g.execute(gpu(), bad, nullptr), ErrorCode::VariantPackError,
+                "Buffer for tensor 'image' has extent 5 in dim 3, which is not "
+                "a dynamic dim (expected 4)");
+  }
+  {
+    // NHWC activations: the buffer's shape is in physical order
+    const int64_t n = 4, c = 8, h = 3, w = 5, k = 16;
+    Graph g = newGraph("dynamic_conv_nhwc", DataType::Half);
+    auto X = g.tensor(mk("image", {n, c, h, w}, chlast({n, c, h, w}), DataType::Half)
+                          .setDynamicDims({0}));
+    auto W = g.tensor(mk("filter", {k, c, 1, 1}, chlast({k, c, 1, 1}), DataType::Half));
+    ConvFPropAttr ca;
+    ca.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    auto Y = g.convFProp(X, W, ca);
+    Y->setDynamicDims({0}).setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    REQUIRE(!isError(g.getWorkspaceSize()));
+    auto wBuf = fill(W, half(1.f));
+    for (int64_t rn : {int64_t{3}, n}) {
+      Pack pack = {{X, shaped<half>({rn, h, w, c}, half(1.f))}, {W, wBuf},
+                   {Y, shaped<half>({rn, h, w, k}, half(0.f))}};
+      REQUIRE_OK(g.execute(gpu(), pack, nullptr));
+      auto out = readBack<half>(pack[Y]);
+      REQUIRE(out.size() == static_cast<size_t>(rn * k * h * w));
+      CHECK(allEqual(out, 8.f));
+    }
+  }
+  {
+    const int64_t n = 4, c = 6, l = 10;
+    Graph g = newGraph("dynamic_reduction", DataType::Float);
+    auto X = g.tensor(mk("x", {n, c, l}, contig({n, c, l}), DataType::Float)
+                          .setDynamicDims({0}));
+    ReductionAttr ra;
+    ra.setMode(ReductionAttr::Mode::MAX);
+    auto Y = g.reduction(X, ra);
+    Y->setDim({n, c, 1}).setStride({c, 1, 1}).setDynamicDims({0}).setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    REQUIRE(!isError(g.getWorkspaceSize()));
+    for (int64_t rn : {int64_t{1}, int64_t{3}, n}) {
+      std::vector<float> xin(rn * c * l);
+      for (size_t i = 0; i < xin.size(); ++i)
+        xin[i] = static_cast<float>((i * 7) % 23) - 11.f;
+      std::vector<size_t> sh = {static_cast<size_t>(rn), static_cast<size_t>(c),
+                                static_cast<size_t>(l)};
+      auto xb = Buffer::allocate(gpu(), sh, xin);
+      REQUIRE(!isError(xb));
+      Pack pack = {{X, std::make_shared<Buffer>(std::move(*xb))},
+                   {Y, shaped<float>({rn, c, 1}, 0.f)}};
+      REQUIRE_OK(g.execute(gpu(), pack, nullptr));
+      auto out = readBack<float>(pack[Y]);
+      REQUIRE(out.size() == static_cast<size_t>(rn * c));
+      bool same = true;
+      for (int64_t r = 0; r < rn * c; ++r) {
+        float mx = xin[r * l];
+        for (int64_t i = 1; i < l; ++i)
+          mx = std::max(mx, xin[r * l + i]);
+        same = same && out[r] == mx;
+      }
+      CHECK(same);
+    }
+  }
+  {
+    const int64_t b = 1, hh = 8, sq = 64, d = 64;
+    Graph g = newGraph("dynamic_sdpa", DataType::Half);
+    const Dims dims = {b, hh, sq, d};
+    auto Q = g.tensor(mk("q", dims, contig(dims), DataType::Half).setDynamicDims({2}));
+    auto K = g.tensor(mk("k", dims, contig(dims), DataType::Half).setDynamicDims({2}));
+    auto V = g.tensor(mk("v", dims, contig(dims), DataType::Half).setDynamicDims({2}));
+    SdpaAttr sa;
+    auto O = g.sdpa(Q, K, V, nullptr, sa);
+    O->setDynamicDims({2}).setOutput(true);
+    REQUIRE_OK(g.validate());
+    REQUIRE_OK(g.compile(gpu(), true));
+    REQUIRE(!isError(g.getWorkspaceSize()));
+    for (int64_t rs : {int64_t{16}, int64_t{32}, sq}) {
+      const Dims rd = {b, hh, rs, d};
+      Pack pack = {{Q, shaped<half>(rd, half(0.01f))}, {K, shaped<half>(rd, half(0.01f))},
+                   {V, shaped<half>(rd, half(0.01f))}, {O, shaped<half>(rd, half(0.f))}};
+      REQUIRE_OK(g.execute(gpu(), pack, workspaceFor(g)));
+      auto out = readBack<half>(pack[O]);
+      REQUIRE(out.size() == static_cast<size_t>(b * hh * rs * d));
+      float worst = 0;
+      for (half v : out) // constant V => O = V (sdpa_basic_dynamic_sequence.cpp)
+        worst = std::max(worst, std::fabs(static_cast<float>(v) - 0.01f));
+      CHECK(worst < 1e-3f);
+    }
+  }
+}
+
 // ---- matmul samples ----------------------------------------------------------
 TEST("samples: matmul all-ones, transposed B, bias, batched broadcast") {
   for (int variant = 0; variant < 3; ++variant) {
