@@ -173,9 +173,14 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
     };
     const char *env = getenv("FUSILLI_HIP_CONV_HALO");
     const int want = env ? atoi(env) : -1; // 0 off, 128 / 256 tile, else auto
-    const bool fits128 = slab_of(128) + HaloShape<128>::kRingBytes <= 160 * 1024;
-    const bool small128 = slab_of(128) + HaloShape<128>::kRingBytes <= 80 * 1024;
-    const bool small256 = slab_of(256) + HaloShape<256>::kRingBytes <= 80 * 1024;
+    const bool narrow = p.N <= 64; // 64-wide column tiles: half the filter ring
+    const int ring128 = narrow ? HaloShape<128, 64>::kRingBytes
+                               : HaloShape<128>::kRingBytes;
+    const int ring256 = narrow ? HaloShape<256, 64>::kRingBytes
+                               : HaloShape<256>::kRingBytes;
+    const bool fits128 = slab_of(128) + ring128 <= 160 * 1024;
+    const bool small128 = slab_of(128) + ring128 <= 80 * 1024;
+    const bool small256 = slab_of(256) + ring256 <= 80 * 1024;
     // 256-row tiles when the output has enough pixels to give every slot
     // (two workgroups per compute unit) a tile of at least 160 rows
     const int64_t slots = 2 * 256;
@@ -194,7 +199,7 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
     if (bm) {
       p.halo = true;
       p.bm = bm;
-      p.bn = 128;
+      p.bn = narrow ? 64 : 128;
       const int64_t rows = (bm + reach + 7) / 8 * 8;
       g.halo_rows = (int32_t)rows;
       g.slab_bytes = (uint32_t)slab_of(bm);
@@ -220,7 +225,10 @@ int conv_launch_bf16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return conv_launch_kind<GK_BF16>(ctx, bm, bn, g);
 }
 template <int KIND>
-int conv_launch_halo_bm(fhip_ctx *ctx, int bm, const GemmArgs &g) {
+int conv_launch_halo_bm(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
+  if (bn == 64)
+    return bm == 256 ? conv_launch_halo<KIND, 256, 64>(ctx, g)
+                     : conv_launch_halo<KIND, 128, 64>(ctx, g);
   return bm == 256 ? conv_launch_halo<KIND, 256>(ctx, g)
                    : conv_launch_halo<KIND, 128>(ctx, g);
 }
@@ -276,8 +284,8 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   }
   gemm_fill_linear(d->epilogue, g);
   if (p.halo)
-    return p.kind == GK_BF16 ? conv_launch_halo_bm<GK_BF16>(ctx, p.bm, g)
-                             : conv_launch_halo_bm<GK_F16>(ctx, p.bm, g);
+    return p.kind == GK_BF16 ? conv_launch_halo_bm<GK_BF16>(ctx, p.bm, p.bn, g)
+                             : conv_launch_halo_bm<GK_F16>(ctx, p.bm, p.bn, g);
   if (p.kind == GK_BF16)
     return conv_launch_bf16(ctx, p.bm, p.bn, g);
   return conv_launch_f16(ctx, p.bm, p.bn, g);

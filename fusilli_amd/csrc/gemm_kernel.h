@@ -1326,19 +1326,21 @@ int conv_launch_kind(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
 
 // Halo mode: 128 x 128 tiles with three filter stages behind the slab, or
 // 256 x 128 tiles with two.
-template <int BM> struct HaloShape {
-  static constexpr int kStages = BM == 256 ? 2 : 3;
-  static constexpr int kRingBytes = kStages * 128 * kTileKBytes;
+// Outputs of at most 64 channels take 64-wide column tiles (no padded MFMA
+// columns).
+template <int BM, int BN = 128> struct HaloShape {
+  static constexpr int kStages = BM == 256 || BN == 64 ? 2 : 3;
+  static constexpr int kRingBytes = kStages * BN * kTileKBytes;
 };
-template <int KIND, int BM>
+template <int KIND, int BM, int BN = 128>
 int conv_launch_halo(fhip_ctx *ctx, const GemmArgs &g) {
-  constexpr int STAGES = HaloShape<BM>::kStages;
-  using L = GemmLds<BM, 128, STAGES, 4, true>;
-  const int main_bytes = (int)g.conv.slab_bytes + HaloShape<BM>::kRingBytes;
+  constexpr int STAGES = HaloShape<BM, BN>::kStages;
+  using L = GemmLds<BM, BN, STAGES, 4, true>;
+  const int main_bytes = (int)g.conv.slab_bytes + HaloShape<BM, BN>::kRingBytes;
   // (the epilogue's bands stay within 80 KB so that two workgroups keep
   // sharing a compute unit)
   const int lds = main_bytes > L::kEpiBytes ? main_bytes : L::kEpiBytes;
-  auto kernel = gemm_kernel<KIND, BM, 128, A_HALO, true, STAGES, 4>;
+  auto kernel = gemm_kernel<KIND, BM, BN, A_HALO, true, STAGES, 4>;
   static bool configured = false;
   if (!configured) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
