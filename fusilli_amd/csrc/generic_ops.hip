@@ -425,48 +425,98 @@ __global__ void generic_conv_dgrad_kernel(ConvBwdArgs g, const void *dy,
 }
 
 // DW[k, fc, f..] = sum over n, o..:  DY[n, k, o..] * X[n, c, o * stride - pad +
-// f * dil] with c = group(k) * fC + fc.  One workgroup per DW element.
+// f * dil] with c = group(k) * fC + fc.  A workgroup owns one (k, filter tap)
+// and 64 filter channels: lane = channel (channels-last X is read in
+// contiguous runs, the DY value is the same for the whole wavefront), the four
+// wavefronts split the pixels and their sums meet in LDS.  The pixel
+// decomposition is wavefront-uniform.
 __global__ __launch_bounds__(256) void generic_conv_wgrad_kernel(
     ConvBwdArgs g, const void *dy, const void *x, void *dw) {
-  __shared__ float part[4];
-  int64_t coord[FHIP_MAX_RANK];
-  unravel((int64_t)blockIdx.x, g.out, coord);
+  __shared__ float part[4][64];
   const int sp = g.spatial;
-  const int64_t k = coord[0], fc = coord[1];
+  int64_t fvol = 1;
+  for (int i = 0; i < sp; ++i)
+    fvol *= g.w_dim[2 + i];
+  const int64_t k = blockIdx.x / fvol;
+  int64_t tap = blockIdx.x - k * fvol;
+  int64_t f[3] = {0, 0, 0};
+  for (int i = sp - 1; i >= 0; --i) {
+    f[i] = tap % g.w_dim[2 + i];
+    tap /= g.w_dim[2 + i];
+  }
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t fC = g.w_dim[1];
+  const int64_t fc = (int64_t)blockIdx.y * 64 + lane;
   const int64_t kPerGroup = g.w_dim[0] / g.groups;
-  const int64_t c = (k / kPerGroup) * g.w_dim[1] + fc;
+  const int64_t c = (k / kPerGroup) * fC + (fc < fC ? fc : 0);
   int64_t ovol = 1;
   for (int i = 0; i < sp; ++i)
     ovol *= g.y_dim[2 + i];
   const int64_t total = g.y_dim[0] * ovol;
-  float acc = 0.f;
-  for (int64_t it = threadIdx.x; it < total; it += blockDim.x) {
-    int64_t rem = it;
-    int64_t yo = k * g.y.s[1];
-    int64_t xo = c * g.x.s[1];
-    bool inside = true;
+  const int64_t y_k = k * g.y.s[1], x_c = c * g.x.s[1];
+  // This wavefront's pixels are wave, wave + 4, ...: coordinates advance by
+  // carries (no division in the loop), and eight pixels' loads are in flight
+  // together.
+  int64_t o[3] = {0, 0, 0}, n = 0;
+  {
+    int64_t rem = wave;
     for (int i = sp - 1; i >= 0; --i) {
-      const int64_t od = g.y_dim[2 + i];
-      const int64_t o = rem % od;
-      rem /= od;
-      const int64_t xi = o * g.str[i] - g.pad[i] + coord[2 + i] * g.dil[i];
-      if (xi < 0 || xi >= g.x_dim[2 + i])
-        inside = false;
-      yo += o * g.y.s[2 + i];
-      xo += xi * g.x.s[2 + i];
+      o[i] = rem % g.y_dim[2 + i];
+      rem /= g.y_dim[2 + i];
     }
-    const int64_t n = rem;
-    if (inside)
-      acc += fhip_load<float>(dy, g.y_dt, yo + n * g.y.s[0]) *
-             fhip_load<float>(x, g.x_dt, xo + n * g.x.s[0]);
+    n = rem;
   }
-  acc = wave_sum(acc);
-  if ((threadIdx.x & 63) == 0)
-    part[threadIdx.x >> 6] = acc;
+  constexpr int U = 8;
+  float acc = 0.f;
+  for (int64_t it = wave; it < total; it += 4 * U) {
+    int64_t yo[U], xo[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      bool inside = it + 4 * u < total;
+      int64_t yy = y_k + n * g.y.s[0], xx = x_c + n * g.x.s[0];
+      for (int i = 0; i < sp; ++i) {
+        const int64_t xi = o[i] * g.str[i] - g.pad[i] + f[i] * g.dil[i];
+        if (xi < 0 || xi >= g.x_dim[2 + i])
+          inside = false;
+        yy += o[i] * g.y.s[2 + i];
+        xx += xi * g.x.s[2 + i];
+      }
+      ok[u] = inside;
+      yo[u] = inside ? yy : y_k; // a valid address either way
+      xo[u] = inside ? xx : x_c;
+      // next pixel of this wavefront
+      o[sp - 1] += 4;
+      for (int i = sp - 1; i > 0; --i)
+        while (o[i] >= g.y_dim[2 + i]) {
+          o[i] -= g.y_dim[2 + i];
+          ++o[i - 1];
+        }
+      while (o[0] >= g.y_dim[2]) {
+        o[0] -= g.y_dim[2];
+        ++n;
+      }
+    }
+    float gy[U], xv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      gy[u] = fhip_load<float>(dy, g.y_dt, yo[u]);
+      xv[u] = fhip_load<float>(x, g.x_dt, xo[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      acc += ok[u] ? gy[u] * xv[u] : 0.f;
+  }
+  part[wave][lane] = acc;
   __syncthreads();
-  if (threadIdx.x == 0)
-    fhip_store<float>(dw, g.w_dt, dot(coord, g.w, g.out.rank),
-                      (part[0] + part[1]) + (part[2] + part[3]));
+  if (wave == 0 && fc < fC) {
+    const float sum = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+    int64_t off = k * g.w.s[0] + fc * g.w.s[1];
+    for (int i = 0; i < sp; ++i)
+      off += f[i] * g.w.s[2 + i];
+    fhip_store<float>(dw, g.w_dt, off, sum);
+  }
 }
 
 constexpr int kSdpaMaxDvPerLane = 8; // Dv <= 512
@@ -1156,11 +1206,24 @@ int fhip_conv_wgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
   return 0;
 }
 
+// grid of the weight-gradient kernel: x = K * filter taps, y = blocks of 64
+// filter channels
+static bool conv_wgrad_grid(const fhip_conv_desc *d, dim3 *grid) {
+  int64_t fvol = 1;
+  for (int i = 0; i < d->spatial_rank; ++i)
+    fvol *= d->w.dim[2 + i];
+  const int64_t gx = d->w.dim[0] * fvol, gy = (d->w.dim[1] + 63) / 64;
+  if (gx >= (1ll << 31) || gy > 65535)
+    return false;
+  *grid = dim3((unsigned)gx, (unsigned)gy);
+  return true;
+}
+
 int fhip_conv_wgrad_supported(const fhip_conv_desc *d) {
   if (!d || conv_bwd_validate(nullptr, d, "fhip_conv_wgrad") != 0)
     return 0;
-  // one workgroup per DW element
-  return fhip_desc_volume(d->w) < (1ll << 31) ? 1 : 0;
+  dim3 grid;
+  return conv_wgrad_grid(d, &grid) ? 1 : 0;
 }
 
 int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
@@ -1170,16 +1233,17 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   if (conv_bwd_validate(ctx, d, "fhip_conv_wgrad") != 0)
     return 1;
   FHIP_REQUIRE(ctx, dy && x && dw, "fhip_conv_wgrad: null tensor pointer");
-  const int64_t total = fhip_desc_volume(d->w);
-  FHIP_REQUIRE(ctx, total < (1ll << 31),
-               "fhip_conv_wgrad: %lld filter elements exceed the grid limit",
-               (long long)total);
+  dim3 grid;
+  FHIP_REQUIRE(ctx, conv_wgrad_grid(d, &grid),
+               "fhip_conv_wgrad: the filter exceeds the grid limits");
   (void)workspace;
   (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
   const ConvBwdArgs g = conv_bwd_args(d, false);
-  hipLaunchKernelGGL(generic_conv_wgrad_kernel, dim3((unsigned)total), dim3(256),
-                     0, ctx->stream, g, dy, x, dw);
+  if (fhip_desc_volume(d->w) == 0)
+    return 0;
+  hipLaunchKernelGGL(generic_conv_wgrad_kernel, grid, dim3(256), 0, ctx->stream,
+                     g, dy, x, dw);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }
