@@ -173,7 +173,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
     };
     const char *env = getenv("FUSILLI_HIP_CONV_HALO");
     const int want = env ? atoi(env) : -1; // 0 off, 128 / 256 tile, else auto
-    const bool narrow = p.N <= 64; // 64-wide column tiles: half the filter ring
+    // 64-wide column tiles: half the filter ring (FUSILLI_HIP_CONV_BN=64
+    // forces them for wider outputs: tuning)
+    const char *bn_env = getenv("FUSILLI_HIP_CONV_BN");
+    const bool narrow = p.N <= 64 || (bn_env && atoi(bn_env) == 64);
     const int ring128 = narrow ? HaloShape<128, 64>::kRingBytes
                                : HaloShape<128>::kRingBytes;
     const int ring256 = narrow ? HaloShape<256, 64>::kRingBytes
