@@ -267,6 +267,35 @@ def bench_conv_dgrad(ctx, steps, warmup):
             "kernels_per_call": 2}
 
 
+def bench_conv_wgrad(ctx, steps, warmup):
+    """Weight gradient of C3: DY bf16 NHWC [32,128,56,56], X [32,64,56,56] ->
+    DW KRSC [128,64,3,3]; zero-padded copies of both operands, one batched
+    MFMA GEMM per filter row, a sum over the batch (6 kernels per call)."""
+    n, c, h, w, k, r = 32, 64, 56, 56, 128, 3
+    cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
+    xd, wd, yd = [n, c, h, w], [k, c, r, r], [n, k, h, w]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_conv_wgrad_supported(d) == 2, "MFMA wgrad not chosen"
+    dy = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(10, 0, n * k * h * w)))
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(10, 1, n * c * h * w)))
+    dw = ctx.alloc(k * c * r * r * 2)
+    ws = ctx.alloc(ctx.conv_wgrad_workspace(d))
+    wall_ms, ev_ms = timed_loop(
+        ctx, lambda i: ctx.conv_wgrad(d, dy, x, dw, workspace=ws), steps, warmup)
+    flop = 2.0 * n * h * w * k * c * r * r
+    return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
+            "call_us": round(ev_ms * 1e3, 2), "work": flop,
+            "kernels_per_call": 6}
+
+
 def bench_reduce(ctx, steps, warmup, mode="SUM", sets=5):
     """Row reduction bf16 X[8192,4096] -> f32 Y[8192,1] (reads 64 MiB per launch)."""
     rows, cols = 8192, 4096
@@ -492,6 +521,8 @@ def main():
               bench_conv(ctx, max(20, args.steps // 4), kwarm))
         other("conv_dgrad_bf16_n32c64h56w56_k128r3s3",
               bench_conv_dgrad(ctx, max(20, args.steps // 4), kwarm))
+        other("conv_wgrad_bf16_n32c64h56w56_k128r3s3",
+              bench_conv_wgrad(ctx, max(20, args.steps // 10), kwarm))
         other("sdpa_fwd_bf16_causal_b4h32s2048d128",
               bench_sdpa(ctx, max(20, args.steps // 4), kwarm))
         line["others"] = others

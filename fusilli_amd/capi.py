@@ -396,9 +396,21 @@ class Context:
             raise FusilliHipError(self.lib.fhip_last_error(None).decode())
         return n.value
 
-    def conv_wgrad(self, d: ConvDesc, dy, x, dw):
+    def conv_wgrad(self, d: ConvDesc, dy, x, dw, workspace=None):
+        """`workspace`: a DeviceBuffer of at least conv_wgrad_workspace(d)
+        bytes; allocated here when omitted."""
+        need = self.conv_wgrad_workspace(d)
+        if need and workspace is None:
+            workspace = self.alloc(need)
         self._check(self.lib.fhip_conv_wgrad(self.handle, byref(d), _p(dy),
-                                             _p(x), _p(dw), None, 0))
+                                             _p(x), _p(dw), _p(workspace),
+                                             need))
+
+    def conv_wgrad_workspace(self, d: ConvDesc) -> int:
+        n = c_size_t(0)
+        if self.lib.fhip_conv_wgrad_workspace_size(byref(d), byref(n)) != 0:
+            raise FusilliHipError(self.lib.fhip_last_error(None).decode())
+        return n.value
 
     def batchnorm_fwd(self, d: BatchNormDesc, x, y, scale=None, bias=None,
                       running_mean=None, running_var=None, saved_mean=None,

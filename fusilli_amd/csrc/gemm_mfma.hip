@@ -91,7 +91,9 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
     return p;
   if (p.a_kc ? p.a_ld < p.K : p.a_ld < p.M)
     return p;
-  if (p.b_kc ? p.b_ld < p.K : p.b_ld < p.N)
+  // (rows of an N-contiguous B may overlap, b_ld < N: the weight gradient
+  // reads the filter taps of one row as one run of S * C elements per pixel)
+  if (p.b_kc && p.b_ld < p.K)
     return p;
   if (p.M < 128 || p.N < 128)
     return p;

@@ -1203,6 +1203,9 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
 int fhip_conv_wgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
   FHIP_REQUIRE(nullptr, d && bytes, "fhip_conv_wgrad_workspace_size: null");
   *bytes = 0;
+  if (conv_bwd_validate(nullptr, d, "fhip_conv_wgrad") != 0)
+    return 1;
+  fhip_fast_conv_wgrad_applicable(d, bytes);
   return 0;
 }
 
@@ -1222,6 +1225,8 @@ static bool conv_wgrad_grid(const fhip_conv_desc *d, dim3 *grid) {
 int fhip_conv_wgrad_supported(const fhip_conv_desc *d) {
   if (!d || conv_bwd_validate(nullptr, d, "fhip_conv_wgrad") != 0)
     return 0;
+  if (fhip_fast_conv_wgrad_applicable(d, nullptr))
+    return 2;
   dim3 grid;
   return conv_wgrad_grid(d, &grid) ? 1 : 0;
 }
@@ -1233,6 +1238,15 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   if (conv_bwd_validate(ctx, d, "fhip_conv_wgrad") != 0)
     return 1;
   FHIP_REQUIRE(ctx, dy && x && dw, "fhip_conv_wgrad: null tensor pointer");
+  size_t need = 0;
+  if (fhip_fast_conv_wgrad_applicable(d, &need)) {
+    FHIP_REQUIRE(ctx, workspace && workspace_bytes >= need,
+                 "fhip_conv_wgrad: this descriptor needs %zu bytes of workspace "
+                 "(fhip_conv_wgrad_workspace_size), got %zu",
+                 need, workspace ? workspace_bytes : (size_t)0);
+    FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+    return fhip_fast_conv_wgrad(ctx, d, dy, x, dw, workspace);
+  }
   dim3 grid;
   FHIP_REQUIRE(ctx, conv_wgrad_grid(d, &grid),
                "fhip_conv_wgrad: the filter exceeds the grid limits");

@@ -218,11 +218,13 @@ def run_conv_dgrad(ctx, dy, w, x_dims, pad, stride, dil, dtype, nhwc=True,
     return dx.fetch(ctx, bdx)
 
 
-def run_conv_wgrad(ctx, dy, x, w_dims, pad, stride, dil, dtype, nhwc=True):
-    dw = HT.empty(w_dims, dtype,
+def run_conv_wgrad(ctx, dy, x, w_dims, pad, stride, dil, dtype, nhwc=True,
+                   tuned=False, w_dtype=None):
+    dw = HT.empty(w_dims, dtype if w_dtype is None else w_dtype,
                   oracle.channels_last_strides(w_dims) if nhwc else None)
     d = conv_bwd_desc(x, dw, dy, pad, stride, dil)
-    assert ctx.lib.fhip_conv_wgrad_supported(d) == 1
+    assert ctx.lib.fhip_conv_wgrad_supported(d) == (2 if tuned else 1)
+    assert (ctx.conv_wgrad_workspace(d) > 0) == tuned
     bdy, bx, bdw = dy.upload(ctx), x.upload(ctx), dw.upload(ctx)
     ctx.conv_wgrad(d, bdy, bx, bdw)
     return dw.fetch(ctx, bdw)
@@ -336,6 +338,50 @@ def test_conv_dgrad_config3_shape_closed_form_and_oracle(ctx):
     ref = oracle.conv_dgrad(dy.logical()[:2], w.logical(), [2] + xd[1:],
                             [1, 1], [1, 1], [1, 1])
     assert_close(dx[:2], ref, capi.BFLOAT16, "config 3 dgrad")
+
+
+@pytest.mark.parametrize("case", [
+    dict(x=[2, 64, 12, 12], w=[128, 64, 3, 3], pad=[1, 1], d=[1, 1]),
+    dict(x=[3, 32, 9, 21], w=[136, 32, 2, 5], pad=[0, 2], d=[1, 1]),
+    dict(x=[1, 128, 7, 70], w=[192, 128, 3, 1], pad=[2, 0], d=[2, 1]),
+    dict(x=[5, 24, 16, 16], w=[128, 24, 1, 7], pad=[0, 3], d=[1, 1]),
+])
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("w_nhwc", [True, False])
+def test_conv_wgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
+    # unit strides, one group, 16-bit channels-last X and DY, K >= 128 and
+    # S * C >= 128: batched MFMA GEMMs over zero-padded grids
+    yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], [1, 1], case["d"])
+    cl = oracle.channels_last_strides
+    x = HT.from_logical(rand(35, 0, case["x"]), dtype, cl(case["x"]))
+    dy = HT.from_logical(rand(35, 2, yd), dtype, cl(yd))
+    dw = run_conv_wgrad(ctx, dy, x, case["w"], case["pad"], [1, 1], case["d"],
+                        dtype, nhwc=w_nhwc, tuned=True, w_dtype=capi.FLOAT)
+    ref = oracle.conv_wgrad(dy.logical(), x.logical(), case["w"], case["pad"],
+                            [1, 1], case["d"])
+    assert_close(dw.logical(), ref, dtype, f"wgrad {case}")
+
+
+def test_conv_wgrad_config3_shape_closed_form_and_oracle(ctx):
+    # the weight gradient of benchmark config 3 (N32 C64 56x56, K128 3x3 pad 1).
+    # All-ones: DW = N * (rows a tap sees) * (columns it sees) = 32 * {56, 55}^2.
+    xd, wd = [32, 64, 56, 56], [128, 64, 3, 3]
+    yd = [32, 128, 56, 56]
+    cl = oracle.channels_last_strides
+    x = HT.from_logical(np.ones(xd), capi.BFLOAT16, cl(xd))
+    dy = HT.from_logical(np.ones(yd), capi.BFLOAT16, cl(yd))
+    dw = run_conv_wgrad(ctx, dy, x, wd, [1, 1], [1, 1], [1, 1], capi.BFLOAT16,
+                        tuned=True, w_dtype=capi.FLOAT).logical()
+    span = np.array([55.0, 56.0, 55.0])
+    assert np.array_equal(dw, np.broadcast_to(32.0 * np.outer(span, span), wd))
+    # random values on four images against the oracle
+    xd, yd = [4] + xd[1:], [4] + yd[1:]
+    x = HT.from_logical(rand(36, 0, xd), capi.BFLOAT16, cl(xd))
+    dy = HT.from_logical(rand(36, 1, yd), capi.BFLOAT16, cl(yd))
+    dw = run_conv_wgrad(ctx, dy, x, wd, [1, 1], [1, 1], [1, 1], capi.BFLOAT16,
+                        tuned=True).logical()
+    ref = oracle.conv_wgrad(dy.logical(), x.logical(), wd, [1, 1], [1, 1], [1, 1])
+    assert_close(dw, ref, capi.BFLOAT16, "config 3 wgrad")
 
 
 def test_conv_dgrad_needs_its_workspace(ctx):
