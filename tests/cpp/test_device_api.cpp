@@ -899,6 +899,57 @@ TEST("config 3 data gradient (reduced): bf16 NHWC on the MFMA kernel, scratch fr
   CHECK(worst <= 0.0);
 }
 
+TEST("config 3 weight gradient (reduced): bf16 NHWC on batched MFMA GEMMs, scratch from the plan's workspace") {
+  const int64_t n = 2, c = 64, h = 14, w = 14, k = 128;
+  Graph g = newGraph("cfg3_wgrad", DataType::BFloat16, DataType::Float);
+  auto DY = g.tensor(mk("dy", {n, k, h, w}, chlast({n, k, h, w}), DataType::BFloat16));
+  auto X = g.tensor(mk("x", {n, c, h, w}, chlast({n, c, h, w}), DataType::BFloat16));
+  ConvWGradAttr wa;
+  wa.setPadding({1, 1}).setStride({1, 1}).setDilation({1, 1});
+  auto DW = g.convWGrad(DY, X, wa);
+  DW->setDim({k, c, 3, 3}).setDataType(DataType::Float).setOutput(true);
+  REQUIRE_OK(g.validate());
+  REQUIRE_OK(g.compile(gpu(), true));
+  auto wsSize = g.getWorkspaceSize();
+  REQUIRE(!isError(wsSize) && wsSize->has_value());
+  CHECK(**wsSize > 0); // padded operand copies and partial sums
+  auto gf = randomVec(n * h * w * k, 41, -1.f, 1.f);
+  auto xf = randomVec(n * h * w * c, 42, -1.f, 1.f);
+  std::vector<bf16> gb(gf.size()), xb(xf.size());
+  for (size_t i = 0; i < gf.size(); ++i) gb[i] = (bf16)gf[i], gf[i] = (float)gb[i];
+  for (size_t i = 0; i < xf.size(); ++i) xb[i] = (bf16)xf[i], xf[i] = (float)xb[i];
+  Pack pack = {{DY, bufOf(DY, gb)}, {X, bufOf(X, xb)}, {DW, fill(DW, 0.f)}};
+  auto ws = workspaceFor(g);
+  for (int rep = 0; rep < 2; ++rep)
+    REQUIRE_OK(g.execute(gpu(), pack, ws));
+  auto out = readBack<float>(pack[DW]);
+  // physical layouts: dy [n][p][q][k], x [n][h][w][c], dw [k][r][s][c]
+  std::vector<double> ref(k * 9 * c, 0.0);
+  for (int64_t in = 0; in < n; ++in)
+    for (int64_t p = 0; p < h; ++p)
+      for (int64_t q = 0; q < w; ++q)
+        for (int64_t r = 0; r < 3; ++r)
+          for (int64_t s = 0; s < 3; ++s) {
+            const int64_t ih = p - 1 + r, iw = q - 1 + s;
+            if (ih < 0 || ih >= h || iw < 0 || iw >= w)
+              continue;
+            for (int64_t kk = 0; kk < k; ++kk) {
+              const double gy = gf[((in * h + p) * w + q) * k + kk];
+              for (int64_t cc = 0; cc < c; ++cc)
+                ref[((kk * 3 + r) * 3 + s) * c + cc] +=
+                    gy * xf[((in * h + ih) * w + iw) * c + cc];
+            }
+          }
+  REQUIRE(out.size() == ref.size());
+  double worst = 0, rms = 0;
+  for (double r : ref)
+    rms += r * r;
+  rms = std::sqrt(rms / ref.size());
+  for (size_t i = 0; i < ref.size(); ++i)
+    worst = std::max(worst, std::fabs(out[i] - ref[i]) - 1e-3 * (std::fabs(ref[i]) + rms));
+  CHECK(worst <= 0.0);
+}
+
 TEST("config 5a (reduced): int8 matmul is bit exact") {
   const int64_t m = 256, k = 512, n = 384;
   Graph g = newGraph("cfg5a", DataType::Int8);
