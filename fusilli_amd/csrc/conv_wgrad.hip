@@ -11,7 +11,7 @@
 // wherever the shifted pixel would leave the image.  For one filter row r the
 // S taps of a pixel are S * C consecutive elements, so
 //   partial[r][n][k][s * C + c] = sum_m DYp[n][m][k] * Xp[n][m + r * dil * pitch][s * C + c]
-// is one batched GEMM per filter row (A = DYp, M-contiguous; B = Xp with
+// is one batched GEMM per filter row, all rows in one launch (A = DYp, M-contiguous; B = Xp with
 // overlapping rows of S * C elements, row stride C; reduction over the 64-pixel
 // K slices of an image, or of an equal share of it; batch = image x share),
 // and DW is the sum of the partial results over the batch.
@@ -163,6 +163,7 @@ __global__ void conv_wgrad_sum_kernel(WgradSumArgs a, const float *part,
   const int64_t r = rem / a.K;
   const float *src = part + (r * a.N * a.K + k) * sc + j;
   float acc = 0.f;
+#pragma unroll 8 // independent loads: several in flight
   for (int64_t n = 0; n < a.N; ++n)
     acc += src[n * a.K * sc];
   const int64_t s = j / a.C, c = j - s * a.C;
@@ -204,12 +205,12 @@ int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                      dim3(256), 0, ctx->stream, ay, (const uint4 *)dy, (uint4 *)dyp);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   DevEpilogue epi{};
-  for (int64_t r = 0; r < p.R; ++r) {
-    const char *b = xp + r * p.dil_h * p.pitch * p.C * 2;
-    float *out = part + r * p.N * p.split * p.K * p.S * p.C;
-    if (fhip_fast_matmul(ctx, &p.mm, dyp, b, epi, out) != 0)
-      return 1;
-  }
+  // all filter rows in one launch: the outer batch dim steps B by one filter
+  // row of pixels and the output by one block of partial results
+  if (fhip_fast_matmul_outer(ctx, &p.mm, dyp, xp, epi, part, (int)p.R, 0,
+                             p.dil_h * p.pitch * p.C,
+                             p.N * p.split * p.K * p.S * p.C) != 0)
+    return 1;
   WgradSumArgs as;
   as.N = p.N * p.split, as.K = p.K, as.R = p.R, as.S = p.S, as.C = p.C;
   as.sk = d->w.dim[0] == 1 ? 0 : d->w.stride[0];

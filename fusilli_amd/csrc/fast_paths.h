@@ -10,6 +10,13 @@ bool fhip_fast_matmul_applicable(const fhip_matmul_desc *d);
 int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
                      const void *b, const DevEpilogue &epi, void *out);
 
+// The same with an outer batch dim of `outer` entries around the descriptor's
+// own (element strides per operand, 16-byte multiples; empty epilogue).
+int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
+                           const void *a, const void *b, const DevEpilogue &epi,
+                           void *out, int outer, int64_t a_outer,
+                           int64_t b_outer, int64_t o_outer);
+
 bool fhip_fast_conv_applicable(const fhip_conv_desc *d);
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                    const void *w, const DevEpilogue &epi, void *out);

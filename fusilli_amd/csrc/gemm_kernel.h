@@ -140,6 +140,10 @@ struct GemmArgs {
                               // non-contiguous one of the two matrix dims)
   int64_t a_batch, b_batch;   // batch strides in elements (0 = broadcast)
   int64_t o_sm, o_sn, o_batch; // output strides in elements
+  // optional outer batch dim (grid z) with strides of its own; fused operands
+  // do not see it
+  int64_t a_outer, b_outer, o_outer;
+  int32_t outer; // extent (0 or 1: none)
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
   // rows of an M tile that are computed and stored (0: all BM); a smaller
@@ -505,6 +509,7 @@ gemm_kernel(GemmArgs g) {
     tile_n = (pid % per_group) / group_rows;
   }
   const int64_t batch = blockIdx.y;
+  const int64_t outer = blockIdx.z;
 
   const int tile_rows = g.tile_rows ? g.tile_rows : BM;
   const int64_t m0 = (int64_t)tile_m * tile_rows, n0 = (int64_t)tile_n * BN;
@@ -564,21 +569,21 @@ gemm_kernel(GemmArgs g) {
       cv_chunk = ((l & 7) ^ kc_swz(row)) * 16; // same for every j
     }
   } else if constexpr (A_KC) {
-    a_base = g.a + batch * g.a_batch * ELEM + m0 * a_ldb;
+    a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * a_ldb;
     a_step = kTileKBytes;
     dma_setup<BM, ELEM, true, NW>(a_ldb, m0, m_end, off_a);
   } else {
-    a_base = g.a + batch * g.a_batch * ELEM + m0 * ELEM;
+    a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * ELEM;
     a_step = (int64_t)GA::kKRows * a_ldb;
     dma_setup<BM, ELEM, false, NW>(a_ldb, m0, m_end, off_a);
   }
   const char *b_base;
   int64_t b_step;
   if constexpr (B_KC) {
-    b_base = g.b + batch * g.b_batch * ELEM + n0 * b_ldb;
+    b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * b_ldb;
     b_step = kTileKBytes;
   } else {
-    b_base = g.b + batch * g.b_batch * ELEM + n0 * ELEM;
+    b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * ELEM;
     b_step = (int64_t)GB::kKRows * b_ldb;
   }
   dma_setup<BN, ELEM, B_KC, NW>(b_ldb, n0, g.N, off_b);
@@ -910,7 +915,7 @@ gemm_kernel(GemmArgs g) {
   const uint32_t band = lds0 + (uint32_t)wave * (BANDS * L::kBand);
   const uint32_t wr = band + (uint32_t)((l >> 5) * 4 * PITCH + (l & 31) * 4);
   const uint32_t rd = band + (uint32_t)((l / LPR) * PITCH + (l % LPR) * 32);
-  const int64_t ob = batch * g.o_batch;
+  const int64_t ob = batch * g.o_batch + outer * g.o_outer;
   const int64_t ncol = n0 + wn * WN + (l % LPR) * 8;
 
   // Lean path: the epilogue is linear with scalar / per-column operands (bias,
@@ -1284,7 +1289,8 @@ int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     configured = true;
   }
-  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch,
+                  (unsigned)(g.outer > 1 ? g.outer : 1));
   hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, ctx->stream, g);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;

@@ -163,7 +163,16 @@ bool fhip_fast_matmul_applicable(const fhip_matmul_desc *d) {
 
 int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
                      const void *b, const DevEpilogue &epi, void *out) {
+  return fhip_fast_matmul_outer(ctx, d, a, b, epi, out, 1, 0, 0, 0);
+}
+
+int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
+                           const void *a, const void *b, const DevEpilogue &epi,
+                           void *out, int outer, int64_t a_outer,
+                           int64_t b_outer, int64_t o_outer) {
   const GemmPlan p = make_plan(d);
+  FHIP_REQUIRE(ctx, outer >= 1 && outer <= 65535 && (outer == 1 || epi.count == 0),
+               "gemm: outer batch extent %d (no fused operands with it)", outer);
   FHIP_REQUIRE(ctx, p.ok, "gemm: descriptor not supported by the MFMA kernel");
   FHIP_REQUIRE(ctx, ((uintptr_t)a & 15) == 0 && ((uintptr_t)b & 15) == 0,
                "gemm: A and B must be 16-byte aligned");
@@ -181,6 +190,10 @@ int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
   g.o_sm = p.o_sm;
   g.o_sn = p.o_sn;
   g.o_batch = p.o_batch;
+  g.outer = outer;
+  g.a_outer = a_outer;
+  g.b_outer = b_outer;
+  g.o_outer = o_outer;
   g.c_dt = d->c.dtype;
   g.o_dt = d->out.dtype;
   g.tiles_m = (int)((p.M + p.bm - 1) / p.bm);
@@ -188,7 +201,8 @@ int fhip_fast_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
   {
     const int64_t oe = fhip_dtype_size(d->out.dtype);
     g.o_vec = p.o_sn == 1 && (p.o_sm * oe) % 16 == 0 &&
-              (p.o_batch * oe) % 16 == 0 && ((uintptr_t)out & 15) == 0;
+              (p.o_batch * oe) % 16 == 0 && (o_outer * oe) % 16 == 0 &&
+              ((uintptr_t)out & 15) == 0;
   }
   // epilogue strides on (batch, m, n)
   g.epi = epi;
