@@ -49,3 +49,39 @@ def test_supported_queries_need_no_gpu():
     assert lib.fhip_norm_fwd_supported(d) == 1  # generic strided kernel
     d.out = capi.TensorDesc.make([8192, 4095], [4095, 1], capi.BFLOAT16)
     assert lib.fhip_norm_fwd_supported(d) == 0  # dims disagree
+
+
+def test_gradient_and_batchnorm_queries_need_no_gpu():
+    lib = capi.load()
+    cl = lambda d: [d[1] * d[2] * d[3], 1, d[3] * d[1], d[1]]
+    xd, wd, yd = [32, 64, 56, 56], [128, 64, 3, 3], [32, 128, 56, 56]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
+    d.epilogue = capi.make_epilogue([])
+    assert lib.fhip_conv_dgrad_supported(d) == 2  # forward MFMA kernel, mirrored filter
+    assert lib.fhip_conv_wgrad_supported(d) == 2  # batched MFMA GEMMs
+    n = ctypes.c_size_t(0)
+    assert lib.fhip_conv_dgrad_workspace_size(d, ctypes.byref(n)) == 0
+    assert n.value == 128 * 64 * 9 * 2
+    assert lib.fhip_conv_wgrad_workspace_size(d, ctypes.byref(n)) == 0
+    assert n.value > 32 * 58 * 64 * (64 + 128) * 2  # padded X and DY grids
+    for i in range(2):
+        d.stride[i] = 2
+    d.y = capi.TensorDesc.make([32, 128, 28, 28], cl([32, 128, 28, 28]), capi.BFLOAT16)
+    assert lib.fhip_conv_dgrad_supported(d) == 1  # strided kernels
+    assert lib.fhip_conv_wgrad_supported(d) == 1
+    d.y = capi.TensorDesc.make([32, 128, 28, 27], cl([32, 128, 28, 27]), capi.BFLOAT16)
+    assert lib.fhip_conv_dgrad_supported(d) == 0  # DY extent disagrees
+
+    b = capi.BatchNormDesc()
+    b.x = b.y = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    b.running_dtype = b.stats_dtype = b.scale_dtype = b.bias_dtype = capi.FLOAT
+    b.epsilon = 1e-5
+    assert lib.fhip_batchnorm_fwd_supported(b) == 1
+    b.y = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    assert lib.fhip_batchnorm_fwd_supported(b) == 0
