@@ -2,7 +2,8 @@
 //
 //   DW[k, r, s, c] = sum over n, p, q of DY[n, p, q, k] * X[n, p + r*dil - pad_h, q + s - pad_w, c]
 //
-// (channels-last tensors, unit strides, one group, unit dilation along W).
+// (channels-last tensors, one group, unit dilation along W; written here for
+// unit strides, equal strides in both dims work the same way, see the plan).
 // Both operands are first copied into zero-padded grids of the same geometry,
 // [N][rows = H + 2 pad_h][pitch >= W + 2 pad_w] pixels with pitch a multiple of
 // 64: X shifted by the padding, DY in the top-left corner.  With m the flat
@@ -29,6 +30,8 @@ struct WgradPlan {
   int64_t pad_h = 0, pad_w = 0, dil_h = 1;
   int64_t rows = 0, pitch = 0, pix = 0; // padded grid
   int64_t split = 1; // GEMM batches per image (more workgroups, shorter K)
+  int64_t str = 1;   // convolution stride (same in both dims)
+  int64_t rows_y = 0, pix_y = 0; // DY's grid: rows / str rows of the same pitch
   size_t xp_bytes = 0, dyp_bytes = 0, part_bytes = 0;
   fhip_matmul_desc mm; // one filter row
 };
@@ -65,28 +68,34 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
     return p;
   if (d->w.dim[1] != d->x.dim[1]) // groups
     return p;
-  if (d->stride[0] != 1 || d->stride[1] != 1 || d->dilation[1] != 1)
+  if (d->stride[0] != d->stride[1] || d->dilation[1] != 1)
     return p;
+  p.str = d->stride[0];
   if (!wg_channels_last(d->x) || !wg_channels_last(d->y))
     return p;
   p.N = d->x.dim[0], p.C = d->x.dim[1], p.H = d->x.dim[2], p.W = d->x.dim[3];
   p.K = d->w.dim[0], p.R = d->w.dim[2], p.S = d->w.dim[3];
   p.P = d->y.dim[2], p.Q = d->y.dim[3];
   p.pad_h = d->padding[0], p.pad_w = d->padding[1], p.dil_h = d->dilation[0];
-  p.rows = p.H + 2 * p.pad_h;
+  // Strides: output pixel (p, q) reads input pixel (p * str + r * dil, q * str
+  // + s); with DY on a grid of the SAME pitch and rows / str rows, DY pixel m
+  // pairs with X pixel str * m + shift: B's row stride becomes str * C.
+  p.rows = (p.H + 2 * p.pad_h + p.str - 1) / p.str * p.str;
   p.pitch = (p.W + 2 * p.pad_w + 63) / 64 * 64;
   p.pix = p.rows * p.pitch;
-  if (p.P > p.rows || p.Q + p.S - 1 > p.pitch)
+  p.rows_y = p.rows / p.str;
+  p.pix_y = p.rows_y * p.pitch;
+  if (p.P > p.rows_y || (p.Q - 1) * p.str + p.S > p.pitch)
     return p;
   // guard behind the last image: the furthest tap of the last pixel
   const int64_t guard = (p.R - 1) * p.dil_h * p.pitch * p.C + p.S * p.C;
   p.xp_bytes = wg_align((size_t)(p.N * p.pix * p.C + guard) * 2);
-  p.dyp_bytes = wg_align((size_t)(p.N * p.pix * p.K) * 2);
+  p.dyp_bytes = wg_align((size_t)(p.N * p.pix_y * p.K) * 2);
   // An image's pixels are cut into `split` equal runs of whole 64-pixel
   // slices, each a batch entry of its own: the largest cut that keeps at
   // least 8 slices per run and at most ~1024 workgroups per launch.
   {
-    const int64_t slices = p.pix / 64;
+    const int64_t slices = p.pix_y / 64;
     const int64_t col_tiles = (p.S * p.C + 127) / 128, row_tiles = (p.K + 127) / 128;
     for (int64_t f = 1; f <= slices; ++f)
       if (slices % f == 0 && slices / f >= 8 &&
@@ -105,9 +114,9 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
     t.dim[0] = d0, t.dim[1] = d1, t.dim[2] = d2;
     t.stride[0] = s0, t.stride[1] = s1, t.stride[2] = s2;
   };
-  const int64_t nb = p.N * p.split, run = p.pix / p.split;
+  const int64_t nb = p.N * p.split, run = p.pix_y / p.split;
   set(m.a, dt, nb, p.K, run, run * p.K, 1, p.K);
-  set(m.b, dt, nb, run, p.S * p.C, run * p.C, p.C, 1);
+  set(m.b, dt, nb, run, p.S * p.C, p.str * run * p.C, p.str * p.C, 1);
   set(m.c, FHIP_FLOAT, nb, p.K, p.S * p.C, p.K * p.S * p.C, p.S * p.C, 1);
   m.out = m.c;
   m.out_dtype = FHIP_FLOAT;
@@ -199,8 +208,8 @@ int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
              (int64_t)(p.xp_bytes / 16)};
   hipLaunchKernelGGL(conv_pad_grid_kernel, dim3((unsigned)((ax.total + 255) / 256)),
                      dim3(256), 0, ctx->stream, ax, (const uint4 *)x, (uint4 *)xp);
-  PadArgs ay{p.N, p.rows, p.pitch, p.K, p.P, p.Q, 0, 0,
-             (int64_t)(p.N * p.pix * p.K * 2 / 16)};
+  PadArgs ay{p.N, p.rows_y, p.pitch, p.K, p.P, p.Q, 0, 0,
+             (int64_t)(p.N * p.pix_y * p.K * 2 / 16)};
   hipLaunchKernelGGL(conv_pad_grid_kernel, dim3((unsigned)((ay.total + 255) / 256)),
                      dim3(256), 0, ctx->stream, ay, (const uint4 *)dy, (uint4 *)dyp);
   FHIP_HIP_CHECK(ctx, hipGetLastError());

@@ -29,7 +29,7 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                          const void *w, void *dx, void *workspace);
 
 // Weight gradient as batched GEMMs over zero-padded copies of X and DY
-// (channels-last 16-bit tensors, unit strides, one group); needs
+// (channels-last 16-bit tensors, equal strides, one group); needs
 // `*workspace_bytes` of 256-byte aligned workspace.
 bool fhip_fast_conv_wgrad_applicable(const fhip_conv_desc *d,
                                      size_t *workspace_bytes);

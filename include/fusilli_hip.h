@@ -260,7 +260,7 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
  *      one group): it then needs fhip_conv_dgrad_workspace_size bytes of
  *      16-byte aligned workspace (a mirrored copy of the filter) and fails
  *      without them.  fhip_conv_wgrad_supported returns 2 for 16-bit
- *      channels-last X and DY with unit strides, one group, K >= 128 and
+ *      channels-last X and DY with equal strides, one group, K >= 128 and
  *      S * C >= 128 (batched MFMA GEMMs over zero-padded copies of both
  *      operands; 256-byte aligned workspace of
  *      fhip_conv_wgrad_workspace_size bytes). ----------------------------- */

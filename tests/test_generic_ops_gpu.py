@@ -345,20 +345,24 @@ def test_conv_dgrad_config3_shape_closed_form_and_oracle(ctx):
     dict(x=[3, 32, 9, 21], w=[136, 32, 2, 5], pad=[0, 2], d=[1, 1]),
     dict(x=[1, 128, 7, 70], w=[192, 128, 3, 1], pad=[2, 0], d=[2, 1]),
     dict(x=[5, 24, 16, 16], w=[128, 24, 1, 7], pad=[0, 3], d=[1, 1]),
+    dict(x=[2, 64, 15, 14], w=[128, 64, 3, 3], pad=[1, 1], d=[1, 1], s=2),
+    dict(x=[3, 48, 23, 31], w=[160, 48, 4, 3], pad=[2, 1], d=[2, 1], s=3),
+    dict(x=[2, 128, 16, 16], w=[256, 128, 1, 1], pad=[0, 0], d=[1, 1], s=2),
 ])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
 @pytest.mark.parametrize("w_nhwc", [True, False])
 def test_conv_wgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
-    # unit strides, one group, 16-bit channels-last X and DY, K >= 128 and
+    # equal strides, one group, 16-bit channels-last X and DY, K >= 128 and
     # S * C >= 128: batched MFMA GEMMs over zero-padded grids
-    yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], [1, 1], case["d"])
+    st = [case.get("s", 1)] * 2
+    yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], st, case["d"])
     cl = oracle.channels_last_strides
     x = HT.from_logical(rand(35, 0, case["x"]), dtype, cl(case["x"]))
     dy = HT.from_logical(rand(35, 2, yd), dtype, cl(yd))
-    dw = run_conv_wgrad(ctx, dy, x, case["w"], case["pad"], [1, 1], case["d"],
+    dw = run_conv_wgrad(ctx, dy, x, case["w"], case["pad"], st, case["d"],
                         dtype, nhwc=w_nhwc, tuned=True, w_dtype=capi.FLOAT)
     ref = oracle.conv_wgrad(dy.logical(), x.logical(), case["w"], case["pad"],
-                            [1, 1], case["d"])
+                            st, case["d"])
     assert_close(dw.logical(), ref, dtype, f"wgrad {case}")
 
 
