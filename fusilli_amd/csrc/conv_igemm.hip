@@ -295,13 +295,15 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
 }
 
 // ---------------------------------------------------------------------------
-// Data gradient on the same kernels.  With unit strides and one group
+// Data gradient on the same kernels.  With one group and (first) unit strides
 //   DX[n, c, i] = sum_{k, f} DY[n, k, i + pad - f * dil] * W[k, c, f]
 // is the forward convolution of DY (K channels) with the filter
 //   W'[c, k, f'] = W[k, c, F - 1 - f']   (taps mirrored, channel roles swapped)
 // under padding' = dil * (F - 1) - pad.  W' is small (the filter's size); it is
 // rebuilt in the caller's workspace on every call, channels-last, by a
-// transposing copy, and the forward kernel does the rest.
+// transposing copy, and the forward kernel does the rest.  Strides above one:
+// DY is spread over a zero grid first (DY(p, q) at (p * stride, q * stride)),
+// which is the unit-stride case again at stride^2 times the MFMA work.
 // (Reference node/conv_node.h:428-598; aten.convolution_backward, input
 // gradient.)
 // ---------------------------------------------------------------------------
@@ -311,6 +313,11 @@ struct DgradPlan {
   bool ok = false;
   fhip_conv_desc fwd; // the equivalent forward problem
   size_t filter_bytes = 0;
+  // strides above one: DY is first spread over a zero grid of the unit-stride
+  // output extent (element (p, q) at (p * stride, q * stride)), in workspace
+  // behind the mirrored filter
+  bool spread = false;
+  size_t spread_bytes = 0;
 };
 
 DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
@@ -327,7 +334,7 @@ DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
   f.spatial_rank = sp;
   for (int i = 0; i < sp; ++i) {
     if (d->stride[i] != 1)
-      return p;
+      p.spread = true;
     const int64_t pad = d->dilation[i] * (d->w.dim[2 + i] - 1) - d->padding[i];
     if (pad < 0)
       return p;
@@ -336,6 +343,23 @@ DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
     f.dilation[i] = d->dilation[i];
   }
   f.x = d->y; // DY plays the input
+  if (p.spread) {
+    // dense channels-last grid [N, K, unit-stride output extent]
+    int64_t st = f.x.dim[1];
+    f.x.stride[1] = 1;
+    for (int i = sp - 1; i >= 0; --i) {
+      f.x.dim[2 + i] = d->x.dim[2 + i] + 2 * d->padding[i] -
+                       d->dilation[i] * (d->w.dim[2 + i] - 1);
+      if (f.x.dim[2 + i] < (d->y.dim[2 + i] - 1) * d->stride[i] + 1)
+        return p;
+      f.x.stride[2 + i] = st;
+      st *= f.x.dim[2 + i];
+    }
+    f.x.stride[0] = st;
+    if (!is_channels_last(d->y) || (d->y.dim[1] * 2) % 16 != 0)
+      return p;
+    p.spread_bytes = (size_t)(st * f.x.dim[0]) * 2;
+  }
   f.y = d->x; // DX plays the output
   f.out = d->x;
   f.out_dtype = d->x.dtype;
@@ -354,9 +378,35 @@ DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
   f.w.stride[0] = st;
   if (!fhip_fast_conv_applicable(&f))
     return p;
-  p.filter_bytes = (size_t)(st * f.w.dim[0]) * fhip_dtype_size(f.w.dtype);
+  p.filter_bytes =
+      ((size_t)(st * f.w.dim[0]) * fhip_dtype_size(f.w.dtype) + 255) / 256 * 256;
   p.ok = true;
   return p;
+}
+
+struct SpreadArgs {
+  int64_t P, Q, Hd, Wd, cpp; // DY extent, grid extent, 16-byte chunks per pixel
+  int64_t sh, sw;            // convolution strides
+  int64_t total;             // chunks of the grid
+};
+
+// grid[n][h][w][:] = DY[n][h / sh][w / sw][:] where both divisions are exact
+// and inside DY, zeros elsewhere (both channels-last, 16-bit)
+__global__ void conv_spread_kernel(SpreadArgs a, const uint4 *src, uint4 *dst) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= a.total)
+    return;
+  const int64_t chunk = lin % a.cpp;
+  int64_t pixel = lin / a.cpp;
+  const int64_t w = pixel % a.Wd;
+  pixel /= a.Wd;
+  const int64_t h = pixel % a.Hd;
+  const int64_t n = pixel / a.Hd;
+  const int64_t p = h / a.sh, q = w / a.sw;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (p * a.sh == h && q * a.sw == w && p < a.P && q < a.Q)
+    v = src[((n * a.P + p) * a.Q + q) * a.cpp + chunk];
+  dst[lin] = v;
 }
 
 struct FlipArgs {
@@ -386,7 +436,7 @@ bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
                                      size_t *workspace_bytes) {
   const DgradPlan p = make_dgrad_plan(d);
   if (workspace_bytes)
-    *workspace_bytes = p.ok ? p.filter_bytes : 0;
+    *workspace_bytes = p.ok ? p.filter_bytes + p.spread_bytes : 0;
   return p.ok;
 }
 
@@ -413,5 +463,23 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                      total);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   DevEpilogue epi{};
+  if (p.spread) {
+    char *grid = (char *)workspace + p.filter_bytes;
+    SpreadArgs sa;
+    sa.P = sp == 2 ? d->y.dim[2] : 1;
+    sa.Q = d->y.dim[1 + sp];
+    sa.Hd = sp == 2 ? p.fwd.x.dim[2] : 1;
+    sa.Wd = p.fwd.x.dim[1 + sp];
+    sa.cpp = d->y.dim[1] * 2 / 16;
+    sa.sh = sp == 2 ? d->stride[0] : 1;
+    sa.sw = d->stride[sp - 1];
+    sa.total = (int64_t)(p.spread_bytes / 16);
+    FHIP_REQUIRE(ctx, ((uintptr_t)dy & 15) == 0, "conv dgrad: DY must be 16-byte aligned");
+    hipLaunchKernelGGL(conv_spread_kernel,
+                       dim3((unsigned)((sa.total + 255) / 256)), dim3(256), 0,
+                       ctx->stream, sa, (const uint4 *)dy, (uint4 *)grid);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    return fhip_fast_conv(ctx, &p.fwd, grid, workspace, epi, dx);
+  }
   return fhip_fast_conv(ctx, &p.fwd, dy, workspace, epi, dx);
 }

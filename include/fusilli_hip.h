@@ -256,10 +256,10 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
  *      (wgrad output), `y` describes DY.  `epilogue` must be empty; `out` and
  *      `out_dtype` are not read.  f32 accumulation, one rounding to the
  *      gradient's dtype.  fhip_conv_dgrad_supported returns 2 where the MFMA
- *      kernel takes the problem (16-bit channels-last tensors, unit strides,
- *      one group): it then needs fhip_conv_dgrad_workspace_size bytes of
- *      16-byte aligned workspace (a mirrored copy of the filter) and fails
- *      without them.  fhip_conv_wgrad_supported returns 2 for 16-bit
+ *      kernel takes the problem (16-bit channels-last tensors, one group):
+ *      it then needs fhip_conv_dgrad_workspace_size bytes of 256-byte aligned
+ *      workspace (a mirrored copy of the filter; with strides above one also
+ *      DY spread over a zero grid) and fails without them.  fhip_conv_wgrad_supported returns 2 for 16-bit
  *      channels-last X and DY with equal strides, one group, K >= 128 and
  *      S * C >= 128 (batched MFMA GEMMs over zero-padded copies of both
  *      operands; 256-byte aligned workspace of

@@ -297,6 +297,11 @@ def test_conv_backward_random_vs_oracle(ctx, case, dtype, nhwc):
     dict(x=[1, 16, 30, 9], w=[192, 16, 1, 1], pad=[0, 0], d=[1, 1]),
     dict(x=[2, 72, 11, 11], w=[64, 72, 5, 5], pad=[0, 3], d=[1, 1]),
     dict(x=[4, 32, 150], w=[64, 32, 4], pad=[2], d=[3]),
+    # strides above one: DY spread over a zero grid first
+    dict(x=[2, 64, 15, 14], w=[128, 64, 3, 3], pad=[1, 1], d=[1, 1], s=[2, 2]),
+    dict(x=[3, 24, 23, 31], w=[64, 24, 4, 3], pad=[2, 1], d=[2, 1], s=[3, 2]),
+    dict(x=[2, 128, 16, 16], w=[256, 128, 1, 1], pad=[0, 0], d=[1, 1], s=[2, 2]),
+    dict(x=[2, 16, 101], w=[64, 16, 5], pad=[2], d=[1], s=[4]),
 ])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
 @pytest.mark.parametrize("w_nhwc", [True, False])
@@ -304,7 +309,7 @@ def test_conv_dgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
     # unit strides, one group, 16-bit channels-last gradients: the forward
     # MFMA kernel on the mirrored filter (any filter layout)
     sp = len(case["pad"])
-    ones = [1] * sp
+    ones = case.get("s", [1] * sp)
     yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], ones, case["d"])
     w = HT.from_logical(rand(33, 1, case["w"], std=0.2), dtype,
                         oracle.channels_last_strides(case["w"]) if w_nhwc else None)
