@@ -761,6 +761,51 @@ TEST("samples: pointwise transposed add, scalar mul, AOT int32 add") {
   }
 }
 
+TEST("AOT: a graph with a data gradient (planner scratch) and a batch norm survives the artifact round trip") {
+  const int64_t n = 2, c = 64, h = 6, w = 6, k = 64;
+  std::shared_ptr<TensorAttr> dy[2], wt[2], dx[2], y[2];
+  auto build = [&](int i) {
+    auto g = std::make_unique<Graph>();
+    g->setName("aot_grad").setIODataType(DataType::BFloat16)
+        .setIntermediateDataType(DataType::Float).setComputeDataType(DataType::Float);
+    dy[i] = g->tensor(mk("dy", {n, k, h, w}, chlast({n, k, h, w}), DataType::BFloat16));
+    wt[i] = g->tensor(mk("w", {k, c, 1, 1}, chlast({k, c, 1, 1}), DataType::BFloat16));
+    ConvDGradAttr da;
+    da.setPadding({0, 0}).setStride({1, 1}).setDilation({1, 1});
+    dx[i] = g->convDGrad(dy[i], wt[i], da);
+    dx[i]->setDim({n, c, h, w}).setOutput(true);
+    BatchnormAttr ba;
+    ba.setForwardPhase(NormFwdPhase::INFERENCE)
+        .setEpsilon(g->tensor(TensorAttr(0.0f)))
+        .setMomentum(g->tensor(TensorAttr(0.1f)));
+    auto mean = g->tensor(mk("mean", {k}, {1}, DataType::Float));
+    auto var = g->tensor(mk("var", {k}, {1}, DataType::Float));
+    auto out = g->batchnorm(dy[i], nullptr, nullptr, mean, var, ba);
+    y[i] = out[0];
+    y[i]->setOutput(true);
+    return std::make_tuple(std::move(g), mean, var);
+  };
+  auto [producer, m0, v0] = build(0);
+  REQUIRE_OK(producer->validate());
+  REQUIRE_ASSIGN(auto bytes, producer->compileToArtifact(Backend::AMDGPU, true));
+  auto [consumer, m1, v1] = build(1);
+  REQUIRE_OK(consumer->validate());
+  REQUIRE_OK(consumer->loadFromArtifact(gpu(), bytes));
+  CHECK(consumer->getKernelCount() == std::optional<size_t>(2));
+  auto ws = consumer->getWorkspaceSize();
+  REQUIRE(!isError(ws) && ws->has_value());
+  CHECK(**ws >= static_cast<size_t>(k * c * 2)); // the mirrored filter
+  Pack pack = {{dy[1], fill(dy[1], bf16(1.f))}, {wt[1], fill(wt[1], bf16(0.5f))},
+               {dx[1], fill(dx[1], bf16(0.f))}, {y[1], fill(y[1], bf16(0.f))},
+               {m1, fill(m1, 0.5f)}, {v1, fill(v1, 4.f)}};
+  REQUIRE_OK(consumer->execute(gpu(), pack, workspaceFor(*consumer)));
+  CHECK(allEqual(readBack<bf16>(pack[dx[1]]), 32.f)); // K * 1 * 0.5
+  CHECK(allEqual(readBack<bf16>(pack[y[1]]), 0.25f)); // (1 - 0.5) / sqrt(4)
+  // a corrupted artifact is rejected
+  bytes[bytes.size() / 2] ^= 0x5a;
+  CHECK(isError(consumer->loadFromArtifact(gpu(), bytes)));
+}
+
 // ---- benchmark configs through the graph API ---------------------------------
 
 TEST("config 1: f32 matmul 1x256x512x256 vs host loop, rel 1e-4") {
