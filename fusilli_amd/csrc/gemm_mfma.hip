@@ -105,6 +105,8 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
     return p;
   if (!p.b_kc && (p.N * elem) % 16 != 0)
     return p;
+  if (p.batch > 65535) // grid y
+    return p;
   if (r == 3) {
     p.a_batch = d->a.dim[0] == 1 ? 0 : d->a.stride[0];
     p.b_batch = d->b.dim[0] == 1 ? 0 : d->b.stride[0];
