@@ -111,11 +111,28 @@ def bench_rmsnorm(ctx, steps, warmup, mul_kind="scalar", sets=5):
                      epilogue_operands=[gs[j]] if gs else ())
 
     wall_ms, ev_ms = timed_loop(ctx, launch, steps, warmup)
+    # spread of single launches (outside the timed region): batches of 10
+    # back-to-back launches between two events, so that the event overhead of
+    # an idle stream does not enter
+    batches = []
+    for b in range(100):
+        e0, e1 = ctx.event(), ctx.event()
+        e0.record()
+        for i in range(10):
+            launch(b * 10 + i)
+        e1.record()
+        ctx.sync()
+        batches.append(e1.elapsed_ms_since(e0) * 100.0)  # us per launch
+    mean = sum(batches) / len(batches)
+    std = (sum((t - mean) ** 2 for t in batches) / len(batches)) ** 0.5
     algo_bytes = 2 * n * 2 + cols * 2 + (n * 2 if mul_kind == "full" else 0)
     return {"wall_ms": wall_ms, "kernel_ms": ev_ms, "bytes": algo_bytes,
             "gbs_wall": algo_bytes / wall_ms / 1e6,
             "gbs_kernel": algo_bytes / ev_ms / 1e6,
-            "sets": sets}
+            "sets": sets,
+            "launch_us": {"min": round(min(batches), 2), "mean": round(mean, 2),
+                          "stddev": round(std, 2),
+                          "sample": "100 batches of 10 launches"}}
 
 
 # ---------------------------------------------------------------------------
@@ -482,7 +499,8 @@ def main():
                      "frac": round(r["gbs_kernel"] / HBM_PEAK_GBS, 4),
                      "traffic": RMSNORM_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": r["bytes"],
-                     "kernel_us": round(r["kernel_ms"] * 1e3, 2)},
+                     "kernel_us": round(r["kernel_ms"] * 1e3, 2),
+                     "launch_us": r["launch_us"]},
     }
     if not args.no_others:
         global MIN_WARM_MS
