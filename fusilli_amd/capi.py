@@ -170,6 +170,7 @@ SYMBOLS = {
     "fhip_abi_version": (c_int, []),
     "fhip_device_count": (c_int, [POINTER(c_int)]),
     "fhip_device_arch": (c_int, [c_int, c_char_p, c_size_t]),
+    "fhip_tuning_reload": (c_int, []),
     "fhip_ctx_create": (c_int, [c_int, _P, POINTER(_P)]),
     "fhip_ctx_destroy": (c_int, [_P]),
     "fhip_last_error": (c_char_p, [_P]),

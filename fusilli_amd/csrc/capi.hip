@@ -1,8 +1,58 @@
 // Context, memory, stream and event entry points of the C ABI, plus the
 // host-side descriptor helpers shared by the op entry points.
 #include "common.h"
+#include "fast_paths.h"
 
 #include <mutex>
+
+namespace {
+std::mutex g_knob_mu;
+FhipKnobs g_knobs;
+std::atomic<bool> g_knobs_ready{false};
+
+FhipKnobs parse_knobs() {
+  FhipKnobs k;
+  if (const char *e = getenv("FUSILLI_HIP_ROWNORM_WGS_PER_CU")) {
+    k.has_rownorm_wgs = true;
+    k.rownorm_wgs_per_cu = atoi(e);
+  }
+  if (const char *e = getenv("FUSILLI_HIP_ROWNORM_SHAPE"))
+    if (sscanf(e, "%d,%d", &k.rownorm_shape_w, &k.rownorm_shape_c) != 2)
+      k.rownorm_shape_w = k.rownorm_shape_c = 0;
+  k.rownorm_general = getenv("FUSILLI_HIP_ROWNORM_GENERAL") != nullptr;
+  if (const char *e = getenv("FUSILLI_HIP_CONV_TILE"))
+    if (sscanf(e, "%d,%d", &k.conv_tile_bm, &k.conv_tile_bn) != 2)
+      k.conv_tile_bm = k.conv_tile_bn = 0;
+  if (const char *e = getenv("FUSILLI_HIP_CONV_HALO"))
+    k.conv_halo = atoi(e);
+  if (const char *e = getenv("FUSILLI_HIP_CONV_BN"))
+    k.conv_bn = atoi(e);
+  if (const char *e = getenv("FUSILLI_HIP_CONV_ROWS"))
+    k.conv_rows = atoi(e);
+  if (const char *e = getenv("FUSILLI_HIP_GEMM_TILE"))
+    if (sscanf(e, "%d,%d", &k.gemm_tile_bm, &k.gemm_tile_bn) != 2)
+      k.gemm_tile_bm = k.gemm_tile_bn = 0;
+  return k;
+}
+} // namespace
+
+const FhipKnobs &fhip_knobs() {
+  if (!g_knobs_ready.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(g_knob_mu);
+    if (!g_knobs_ready.load(std::memory_order_relaxed)) {
+      g_knobs = parse_knobs();
+      g_knobs_ready.store(true, std::memory_order_release);
+    }
+  }
+  return g_knobs;
+}
+
+int fhip_tuning_reload(void) {
+  std::lock_guard<std::mutex> lock(g_knob_mu);
+  g_knobs = parse_knobs();
+  g_knobs_ready.store(true, std::memory_order_release);
+  return 0;
+}
 
 std::string &fhip_tls_error() {
   static thread_local std::string s;

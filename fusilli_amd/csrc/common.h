@@ -9,6 +9,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <string>
 
 #include "../../include/fusilli_hip.h"
@@ -22,6 +23,34 @@ struct fhip_ctx {
   bool owns_stream = false;
   int num_cus = 0;
   std::string err;
+};
+
+// Tuning / test knobs from the environment, parsed once per process (and again
+// on fhip_tuning_reload) instead of on every launch.
+struct FhipKnobs {
+  bool has_rownorm_wgs = false;
+  int rownorm_wgs_per_cu = 0;       // FUSILLI_HIP_ROWNORM_WGS_PER_CU
+  int rownorm_shape_w = 0, rownorm_shape_c = 0; // FUSILLI_HIP_ROWNORM_SHAPE "w,c"
+  bool rownorm_general = false;     // FUSILLI_HIP_ROWNORM_GENERAL
+  int conv_tile_bm = 0, conv_tile_bn = 0; // FUSILLI_HIP_CONV_TILE "bm,bn"
+  int conv_halo = -1;               // FUSILLI_HIP_CONV_HALO (-1: unset)
+  int conv_bn = 0;                  // FUSILLI_HIP_CONV_BN
+  int conv_rows = -1;               // FUSILLI_HIP_CONV_ROWS (-1: unset)
+  int gemm_tile_bm = 0, gemm_tile_bn = 0; // FUSILLI_HIP_GEMM_TILE "bm,bn"
+};
+const FhipKnobs &fhip_knobs();
+
+// "Done once per device" flag for per-kernel set-up such as
+// hipFuncSetAttribute: one bit per device ordinal, safe to test and set from
+// several threads (the set-up itself is idempotent).
+struct FhipOncePerDevice {
+  std::atomic<uint64_t> bits{0};
+  bool done(int device) const {
+    return (bits.load(std::memory_order_acquire) >> (device & 63)) & 1;
+  }
+  void mark(int device) {
+    bits.fetch_or(1ull << (device & 63), std::memory_order_release);
+  }
 };
 
 struct fhip_event {

@@ -152,10 +152,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
   // share a compute unit and cover each other's prologue and epilogue
   if (p.bn == 128 || p.bm == 128)
     p.bm = p.bn = 128;
-  if (const char *env = getenv("FUSILLI_HIP_CONV_TILE")) {
-    int bm = 0, bn = 0;
-    if (sscanf(env, "%d,%d", &bm, &bn) == 2 &&
-        (bm == 128 || bm == 256 || (bm == 512 && bn == 128)) &&
+  const FhipKnobs &knobs = fhip_knobs();
+  if (knobs.conv_tile_bm) {
+    const int bm = knobs.conv_tile_bm, bn = knobs.conv_tile_bn;
+    if ((bm == 128 || bm == 256 || (bm == 512 && bn == 128)) &&
         (bn == 128 || bn == 256) && bm >= bn)
       p.bm = bm, p.bn = bn;
   }
@@ -171,12 +171,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
       const int64_t rows = (bm + reach + 7) / 8 * 8;
       return rows * g.slices_per_tap * kTileKBytes + kTileKBytes;
     };
-    const char *env = getenv("FUSILLI_HIP_CONV_HALO");
-    const int want = env ? atoi(env) : -1; // 0 off, 128 / 256 tile, else auto
+    const int want = knobs.conv_halo; // 0 off, 128 / 256 tile, else auto
     // 64-wide column tiles: half the filter ring (FUSILLI_HIP_CONV_BN=64
     // forces them for wider outputs: tuning)
-    const char *bn_env = getenv("FUSILLI_HIP_CONV_BN");
-    const bool narrow = p.N <= 64 || (bn_env && atoi(bn_env) == 64);
+    const bool narrow = p.N <= 64 || knobs.conv_bn == 64;
     const int ring128 = narrow ? HaloShape<128, 64>::kRingBytes
                                : HaloShape<128>::kRingBytes;
     const int ring256 = narrow ? HaloShape<256, 64>::kRingBytes

@@ -75,6 +75,9 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
     return p;
   p.N = d->x.dim[0], p.C = d->x.dim[1], p.H = d->x.dim[2], p.W = d->x.dim[3];
   p.K = d->w.dim[0], p.R = d->w.dim[2], p.S = d->w.dim[3];
+  // the padding copies move whole 16-byte chunks of a pixel's channels
+  if (p.C % 8 != 0 || p.K % 8 != 0)
+    return p;
   p.P = d->y.dim[2], p.Q = d->y.dim[3];
   p.pad_h = d->padding[0], p.pad_w = d->padding[1], p.dil_h = d->dilation[0];
   // Strides: output pixel (p, q) reads input pixel (p * str + r * dil, q * str
@@ -196,8 +199,6 @@ int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   FHIP_REQUIRE(ctx, ((uintptr_t)workspace & 255) == 0 && ((uintptr_t)x & 15) == 0 &&
                         ((uintptr_t)dy & 15) == 0,
                "conv wgrad: workspace must be 256-byte and tensors 16-byte aligned");
-  FHIP_REQUIRE(ctx, p.C % 8 == 0 && p.K % 8 == 0,
-               "conv wgrad: channel counts must be multiples of 8");
   char *xp = (char *)workspace;
   char *dyp = xp + p.xp_bytes;
   float *part = (float *)(dyp + p.dyp_bytes);

@@ -1282,12 +1282,12 @@ int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
   constexpr int NW = GemmWaves<BM, BN>::value;
   constexpr int lds = GemmLds<BM, BN, NSTAGE, NW>::kBytes;
   auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC, NSTAGE, NW>;
-  static bool configured = false;
-  if (!configured) {
+  static FhipOncePerDevice configured;
+  if (!configured.done(ctx->device)) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
                             reinterpret_cast<const void *>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    configured = true;
+    configured.mark(ctx->device);
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), (unsigned)batch,
                   (unsigned)(g.outer > 1 ? g.outer : 1));
@@ -1347,13 +1347,13 @@ int conv_launch_halo(fhip_ctx *ctx, const GemmArgs &g) {
   // sharing a compute unit)
   const int lds = main_bytes > L::kEpiBytes ? main_bytes : L::kEpiBytes;
   auto kernel = gemm_kernel<KIND, BM, BN, A_HALO, true, STAGES, 4>;
-  static bool configured = false;
-  if (!configured) {
+  static FhipOncePerDevice configured;
+  if (!configured.done(ctx->device)) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
                             reinterpret_cast<const void *>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
                             160 * 1024));
-    configured = true;
+    configured.mark(ctx->device);
   }
   const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1);
   hipLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, g);

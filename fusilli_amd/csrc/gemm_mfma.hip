@@ -147,9 +147,9 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
     if (t2 < 200 && p.bm == 256)
       p.bm = 128;
   }
-  if (const char *env = getenv("FUSILLI_HIP_GEMM_TILE")) {
-    int bm = 0, bn = 0;
-    if (sscanf(env, "%d,%d", &bm, &bn) == 2 && (bm == 128 || bm == 256) &&
+  if (fhip_knobs().gemm_tile_bm) {
+    const int bm = fhip_knobs().gemm_tile_bm, bn = fhip_knobs().gemm_tile_bn;
+    if ((bm == 128 || bm == 256) &&
         (bn == 128 || bn == 256) && bm >= bn && bm <= p.M && bn <= p.N)
       p.bm = bm, p.bn = bn;
   }

@@ -69,9 +69,9 @@ bool fast_dtype(int dt) {
 bool pick_shape(int64_t inner, int vec, int *chunks, int *wpr) {
   const int64_t per_wave_chunk = 64 * (int64_t)vec;
   const int64_t need = (inner + per_wave_chunk - 1) / per_wave_chunk;
-  if (const char *env = getenv("FUSILLI_HIP_ROWNORM_SHAPE")) {
-    int w = 0, c = 0;
-    if (sscanf(env, "%d,%d", &w, &c) == 2 && (int64_t)w * c >= need) {
+  {
+    const int w = fhip_knobs().rownorm_shape_w, c = fhip_knobs().rownorm_shape_c;
+    if (w > 0 && (int64_t)w * c >= need) {
       for (const RowNormShape &sh : kRowNormShapes)
         if (sh.wpr == w && sh.chunks == c) {
           *wpr = w;
@@ -214,18 +214,18 @@ int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
   } else if (d->is_layernorm && scale_same && bias_same && epi.count == 0) {
     variant = RN_LN_SCALE_BIAS;
   }
-  if (getenv("FUSILLI_HIP_ROWNORM_GENERAL"))
+  if (fhip_knobs().rownorm_general)
     variant = RN_GENERAL; // tuning / test hook: force the general kernel
   bool launched;
   switch (d->x.dtype) {
   case FHIP_BFLOAT16:
-    launched = rownorm_launch_bf16(chunks, wpr, variant, g.rows, ctx->stream, g);
+    launched = rownorm_launch_bf16(chunks, wpr, variant, g.rows, ctx->num_cus, ctx->stream, g);
     break;
   case FHIP_HALF:
-    launched = rownorm_launch_f16(chunks, wpr, variant, g.rows, ctx->stream, g);
+    launched = rownorm_launch_f16(chunks, wpr, variant, g.rows, ctx->num_cus, ctx->stream, g);
     break;
   default:
-    launched = rownorm_launch_f32(chunks, wpr, variant, g.rows, ctx->stream, g);
+    launched = rownorm_launch_f32(chunks, wpr, variant, g.rows, ctx->num_cus, ctx->stream, g);
     break;
   }
   FHIP_REQUIRE(ctx, launched, "rownorm: no kernel for shape (%d, %d)", wpr,

@@ -2,6 +2,6 @@
 #include "rownorm_kernel.h"
 
 bool rownorm_launch_f16(int chunks, int wpr, int variant, int64_t rows,
-                         hipStream_t s, const RowNormArgs &g) {
-  return rownorm_launch_typed<_Float16>(chunks, wpr, variant, rows, s, g);
+                        int num_cus, hipStream_t s, const RowNormArgs &g) {
+  return rownorm_launch_typed<_Float16>(chunks, wpr, variant, rows, num_cus, s, g);
 }

@@ -432,7 +432,7 @@ constexpr RowNormShape kRowNormShapes[] = {
 };
 
 template <typename T, int WPR, int CHUNKS>
-void rownorm_launch_one(int variant, int64_t rows, hipStream_t s,
+void rownorm_launch_one(int variant, int64_t rows, int num_cus, hipStream_t s,
                         const RowNormArgs &g) {
   constexpr int rpw = RowNormGeom<WPR>::kRowsPerWg;
   // Workgroups walk the row-blocks with the per-column parameters in
@@ -444,10 +444,11 @@ void rownorm_launch_one(int variant, int64_t rows, hipStream_t s,
   // FUSILLI_HIP_ROWNORM_WGS_PER_CU overrides it (0: one row-block each).
   int64_t blocks = (rows + rpw - 1) / rpw;
   int per_cu = variant == RN_LN_SCALE_BIAS ? 20 : 24;
-  if (const char *env = getenv("FUSILLI_HIP_ROWNORM_WGS_PER_CU"))
-    per_cu = atoi(env);
-  if (per_cu > 0 && blocks > 256ll * per_cu)
-    blocks = 256ll * per_cu;
+  if (fhip_knobs().has_rownorm_wgs)
+    per_cu = fhip_knobs().rownorm_wgs_per_cu;
+  const int64_t cus = num_cus > 0 ? num_cus : 256;
+  if (per_cu > 0 && blocks > cus * per_cu)
+    blocks = cus * per_cu;
   const dim3 grid((unsigned)blocks);
   const dim3 block(RowNormGeom<WPR>::kThreads);
   switch (variant) {
@@ -477,10 +478,10 @@ void rownorm_launch_one(int variant, int64_t rows, hipStream_t s,
 // Returns false when (wpr, chunks) is not an instantiated pair.
 template <typename T>
 bool rownorm_launch_typed(int chunks, int wpr, int variant, int64_t rows,
-                          hipStream_t s, const RowNormArgs &g) {
+                          int num_cus, hipStream_t s, const RowNormArgs &g) {
 #define FHIP_ROWNORM_CASE(W, C)                                                \
   if (wpr == W && chunks == C) {                                               \
-    rownorm_launch_one<T, W, C>(variant, rows, s, g);                          \
+    rownorm_launch_one<T, W, C>(variant, rows, num_cus, s, g);                          \
     return true;                                                               \
   }
   FHIP_ROWNORM_CASE(1, 1)
@@ -497,10 +498,10 @@ bool rownorm_launch_typed(int chunks, int wpr, int variant, int64_t rows,
 }
 
 bool rownorm_launch_bf16(int chunks, int wpr, int variant, int64_t rows,
-                         hipStream_t s, const RowNormArgs &g);
+                        int num_cus, hipStream_t s, const RowNormArgs &g);
 bool rownorm_launch_f16(int chunks, int wpr, int variant, int64_t rows,
-                        hipStream_t s, const RowNormArgs &g);
+                        int num_cus, hipStream_t s, const RowNormArgs &g);
 bool rownorm_launch_f32(int chunks, int wpr, int variant, int64_t rows,
-                        hipStream_t s, const RowNormArgs &g);
+                        int num_cus, hipStream_t s, const RowNormArgs &g);
 
 #endif // FUSILLI_AMD_CSRC_ROWNORM_KERNEL_H

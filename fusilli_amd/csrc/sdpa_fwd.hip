@@ -646,13 +646,13 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
   const dim3 grid((unsigned)d->q.dim[1], (unsigned)d->q.dim[0],
                   (unsigned)(d->is_causal ? (n_qtiles + 1) / 2 : n_qtiles));
-  auto launch = [&](auto kernel, int lds_bytes, bool &configured) {
-    if (!configured) {
+  auto launch = [&](auto kernel, int lds_bytes, FhipOncePerDevice &configured) {
+    if (!configured.done(ctx->device)) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                               hipFuncAttributeMaxDynamicSharedMemorySize,
                               lds_bytes) != hipSuccess)
         return fhip_fail(ctx, "sdpa: cannot reserve LDS");
-      configured = true;
+      configured.mark(ctx->device);
     }
     hipLaunchKernelGGL(kernel, grid, dim3(kWaves * 64), lds_bytes, ctx->stream,
                        g);
@@ -660,10 +660,10 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
     return 0;
   };
   // one flag per kernel instance: [head dim][type][causal]
-  static bool configured[2][2][2] = {};
+  static FhipOncePerDevice configured[2][2][2];
   auto pick = [&](auto hd) {
     constexpr int HD = decltype(hd)::value;
-    bool(&cfg)[2][2] = configured[HD == 128];
+    FhipOncePerDevice(&cfg)[2][2] = configured[HD == 128];
     constexpr int lds = SdShape<HD>::kLdsB;
     if (p.bf16)
       return d->is_causal

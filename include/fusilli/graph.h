@@ -122,7 +122,18 @@ public:
                             ErrorCode::RuntimeFailure,
                             "Artifact does not match this graph (signature "
                             "mismatch)");
-    loadedPlan_ = std::move(*parsed);
+    // Only the plan this library derives from the graph is ever executed: the
+    // artifact has to be that plan byte for byte (steps, slots, workspace
+    // layout, argument table), so a stale or edited file with a valid
+    // checksum is rejected rather than run.
+    const std::vector<uint8_t> expect = plan::serialize(*own);
+    FUSILLI_RETURN_ERROR_IF(
+        expect.size() != bytes.size() ||
+            std::memcmp(expect.data(), bytes.data(), bytes.size()) != 0,
+        ErrorCode::RuntimeFailure,
+        "Artifact does not match the plan of this graph (stale or edited "
+        "artifact)");
+    loadedPlan_ = std::move(*own);
     loadedBackend_ = handle.getBackend();
     return ok();
   }

@@ -196,6 +196,12 @@ inline ErrorOr<Plan> deserialize(std::span<const uint8_t> bytes) {
   p.signature = getU64();
   p.workspaceBytes = getU64();
   const uint64_t nSteps = getU64(), nWs = getU64(), nArgs = getU64();
+  // counts are bounded by the byte count first, so the products cannot wrap
+  FUSILLI_RETURN_ERROR_IF(nSteps > bytes.size() / sizeof(Step) ||
+                              nWs > bytes.size() / sizeof(WorkspaceTensor) ||
+                              nArgs > bytes.size() / sizeof(ArgInfo),
+                          ErrorCode::RuntimeFailure,
+                          "Artifact length does not match its header");
   const uint64_t need = nSteps * sizeof(Step) + nWs * sizeof(WorkspaceTensor) +
                         nArgs * sizeof(ArgInfo);
   FUSILLI_RETURN_ERROR_IF(bytes.size() != header + need + 8,

@@ -184,6 +184,12 @@ int fhip_device_count(int *count);
 int fhip_device_arch(int device_id, char *buf, size_t buf_len);
 /* external_stream: a hipStream_t the caller owns, or NULL for a stream the
  * context creates (handle.h:89-112). */
+/* Tuning knobs (environment variables FUSILLI_HIP_*: tile shapes, grid caps)
+ * are parsed once per process, not per launch.  fhip_tuning_reload parses them
+ * again; call it only while no other thread is inside the library.  It has no
+ * counterpart in the reference, whose flags travel through
+ * FUSILLI_EXTRA_COMPILER_FLAGS at compile time (backend/backend.h:226-297). */
+int fhip_tuning_reload(void);
 int fhip_ctx_create(int device_id, void *external_stream, fhip_ctx **out);
 int fhip_ctx_destroy(fhip_ctx *ctx);
 const char *fhip_last_error(fhip_ctx *ctx);

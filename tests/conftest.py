@@ -19,3 +19,21 @@ def ctx():
     c = capi.Context(0)
     yield c
     c.close()
+
+
+@pytest.fixture
+def knobs(monkeypatch):
+    """Sets FUSILLI_HIP_* tuning variables for one test.  The library parses
+    them once per process, so every change is followed by fhip_tuning_reload,
+    also when the test ends and the variables are gone again."""
+    from fusilli_amd import capi
+    lib = capi.load()
+
+    def set_knobs(**kv):
+        for name, value in kv.items():
+            monkeypatch.setenv("FUSILLI_HIP_" + name, str(value))
+        assert lib.fhip_tuning_reload() == 0
+
+    yield set_knobs
+    monkeypatch.undo()
+    lib.fhip_tuning_reload()

@@ -985,6 +985,31 @@ TEST("graph: artifact contract") {
   auto corrupt = bytes;
   corrupt[corrupt.size() / 2] ^= 0x40;
   CHECK(isError(consumer.graph->loadFromArtifact(cpu, corrupt)));
+  // an edited artifact whose checksum was recomputed (same header, same
+  // signature field, one byte of a step changed) is not executed either
+  {
+    auto edited = bytes;
+    edited[16 + 8 * 8 + 40] ^= 0x01; // inside the first step
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i + 8 < edited.size(); ++i)
+      h = (h ^ edited[i]) * 1099511628211ull;
+    std::memcpy(edited.data() + edited.size() - 8, &h, 8);
+    CHECK_ERROR(consumer.graph->loadFromArtifact(cpu, edited),
+                ErrorCode::RuntimeFailure,
+                "Artifact does not match the plan of this graph (stale or "
+                "edited artifact)");
+    // counts that would wrap the length computation
+    auto huge = bytes;
+    const uint64_t big = ~0ull / 8;
+    std::memcpy(huge.data() + 16 + 5 * 8, &big, 8); // nSteps
+    h = 1469598103934665603ull;
+    for (size_t i = 0; i + 8 < huge.size(); ++i)
+      h = (h ^ huge[i]) * 1099511628211ull;
+    std::memcpy(huge.data() + huge.size() - 8, &h, 8);
+    CHECK_ERROR(consumer.graph->loadFromArtifact(cpu, huge),
+                ErrorCode::RuntimeFailure,
+                "Artifact length does not match its header");
+  }
   // an artifact of a different graph is rejected
   Graph g = newGraph("different");
   auto a = g.tensor(mk("a", {4, 4}, {4, 1}));

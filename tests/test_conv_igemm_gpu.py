@@ -75,9 +75,8 @@ def test_conv_igemm_random_vs_oracle(ctx, case, dtype):
 
 
 @pytest.mark.parametrize("tile", ["128,128", "256,128", "256,256", "512,128"])
-def test_conv_igemm_every_tile_shape(ctx, tile, monkeypatch):
-    monkeypatch.setenv("FUSILLI_HIP_CONV_TILE", tile)
-    monkeypatch.setenv("FUSILLI_HIP_CONV_HALO", "0")  # the gather kernel's tiles
+def test_conv_igemm_every_tile_shape(ctx, tile, knobs):
+    knobs(CONV_TILE=tile, CONV_HALO="0", CONV_ROWS="0")  # the gather kernel's tiles
     case = dict(x=[2, 64, 15, 17], w=[300, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1])
     x = cl(case["x"], 42, 0, capi.BFLOAT16)
     w = cl(case["w"], 42, 1, capi.BFLOAT16, std=0.1)
@@ -111,8 +110,8 @@ SAME_CASES = [
 @pytest.mark.parametrize("case", SAME_CASES)
 @pytest.mark.parametrize("halo", ["128", "256", "0"])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
-def test_conv_same_geometry_halo_and_gather(ctx, case, halo, dtype, monkeypatch):
-    monkeypatch.setenv("FUSILLI_HIP_CONV_HALO", halo)
+def test_conv_same_geometry_halo_and_gather(ctx, case, halo, dtype, knobs):
+    knobs(CONV_HALO=halo, CONV_ROWS="0")
     st = [1] * len(case["pad"])
     x = cl(case["x"], 46, 0, dtype)
     w = cl(case["w"], 46, 1, dtype, std=0.1)

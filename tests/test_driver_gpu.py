@@ -12,11 +12,15 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DRIVER = os.path.join(ROOT, "fusilli_amd", "bench", "bin", "driver")
 COMMANDS = os.path.join(ROOT, "fusilli_amd", "bench", "test_commands.txt")
+# every add_fusilli_benchmark command of the reference's
+# benchmarks/CMakeLists.txt:49-392, extracted as data
+REFERENCE_COMMANDS = os.path.join(ROOT, "fusilli_amd", "bench",
+                                  "reference_commands.txt")
 
 
-def commands():
+def commands(path=COMMANDS):
     out = []
-    for line in open(COMMANDS):
+    for line in open(path):
         line = line.strip()
         if line and not line.startswith("#") and not line.startswith("[SKIP]"):
             out.append(line)
@@ -39,6 +43,44 @@ def test_driver_command(cmd):
     assert rec["iter"] == want_iter
     assert rec["dispatch_count"] == "1"  # producer + pointwise chain fused
     assert float(rec["avg_us"]) > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cmd", commands(REFERENCE_COMMANDS))
+def test_driver_runs_the_reference_benchmark_commands(cmd):
+    # 2-D and 3-D convolutions in every direction and layout, layer norms of
+    # rank 2 to 4, (batched, transposed, mixed-type) matmuls, attention with
+    # mask / GQA / explicit scale: each must run unchanged and print its row.
+    proc = subprocess.run([DRIVER] + shlex.split(cmd), capture_output=True,
+                          text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().splitlines()
+    rec = dict(zip(lines[-2].split(","), lines[-1].split(",")))
+    assert rec["iter"] == "10"
+    # gradients with --bias add the bias-gradient reduction as a second step
+    steps = 2 if ("--bias" in cmd and (" -F 2 " in cmd or " -F 4 " in cmd)) else 1
+    assert int(rec["dispatch_count"]) == steps
+    assert float(rec["avg_us"]) > 0
+
+
+@pytest.mark.parametrize("bad", [
+    "conv -F 1 -n 1 -c 8 -H 8 -W 8 -k 8 -y 3 -x 3 -p 1 -q 1 -u 1 -v 1 -l 1 -j 1 "
+    "--in_layout NHWC --out_layout NHWC --fil_layout NHWC --spatial_dim 2 --nonsense 3",
+    "conv -F 1 -n 1 -c 8 -H 8 -W 8 -k 8 -y 3 -x 3 -p 1 -q 1 -u 1 -v 1 -l 1 -j 1 "
+    "--in_layout NDHWC --out_layout NDHWC --fil_layout NDHWC --spatial_dim 2",
+    "conv -F 1 -n 1 -c 8 -H 8 -W 8 -k 8 -y 3 -x 3 -p 1 -q 1 -u 1 -v 1 -l 1 -j 1 "
+    "--in_layout NDHWC --out_layout NDHWC --fil_layout NDHWC --spatial_dim 3",
+    "matmul -M 16 -N 32 -K 64 --a_type f32 --b_type f32 --out_type f32 --transC",
+    "sdpa -B 1 --heads_q 8 --heads_kv 8 --seq_q 64 --seq_kv 64 -d 64 -t f16 --causal --mask",
+    "layernorm -X 2x3x128 -F 1 -t f32 --layout NCHW",
+])
+def test_driver_rejects_what_it_does_not_implement(bad):
+    # unknown flags, layouts of the wrong rank, 3-D without its depth flags:
+    # an error before any device is touched, never a number for another problem
+    proc = subprocess.run([DRIVER] + shlex.split(bad), capture_output=True,
+                          text=True, timeout=60)
+    assert proc.returncode != 0
+    assert "driver:" in proc.stderr
 
 
 def test_driver_commands_file_has_every_subcommand():

@@ -166,3 +166,25 @@ def test_gemm_config5a_int8_full_size_bit_exact(ctx):
 
 def test_gemm_config5b_fp8_full_size(ctx):
     _full_size_rows_check(ctx, capi.FP8E4M3)
+
+
+def test_gemm_config5b_fp8_full_size_scaled_bf16_output(ctx):
+    # benchmark config 5b as stated: fp8 e4m3 operands quantised with
+    # per-tensor scales s = max|x| / 448, f32 accumulation, the product
+    # multiplied by s_a * s_b (a fused scalar MUL) and stored as bf16;
+    # rel 2e-2 against the oracle on sampled rows of the full-size result.
+    m, k, n = 4096, 8192, 4096
+    fa = rand(6, 0, [m, k], "uniform")
+    fb = rand(6, 1, [k, n], "uniform")
+    sa, sb = float(np.abs(fa).max()) / 448.0, float(np.abs(fb).max()) / 448.0
+    a = HT.from_logical(fa / sa, capi.FP8E4M3)
+    b = HT.from_logical(fb / sb, capi.FP8E4M3)
+    epi = [capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16, scalar=sa * sb)]
+    out = run(ctx, a, b, capi.FLOAT, out_dtype=capi.BFLOAT16, epilogue=epi).logical()
+    rows = np.array([0, 1, 33, 255, 256, 1023, 2048, 3071, 4064, 4095])
+    ref = oracle.matmul_rows(a.logical(), b.logical(), rows) * np.float32(sa * sb)
+    assert_close(out[rows], ref, capi.BFLOAT16, "config 5b scaled bf16")
+    # the dequantised product also tracks the unquantised one (fp8 has 3
+    # mantissa bits: about 3 % per element, averaged down over K = 8192)
+    exact = fa[rows].astype(np.float64) @ fb.astype(np.float64)
+    assert np.abs(out[rows] - exact).max() < 0.05 * np.abs(exact).max()

@@ -200,3 +200,85 @@ def test_norm_rejects_bad_descriptors(ctx):
     dx = x.upload(ctx)
     with pytest.raises(capi.FusilliHipError, match="dims differ"):
         ctx.norm_fwd(d, dx, None, None, dx)
+
+
+# ---- the benchmarked sizes: several row-blocks per workgroup ---------------
+def test_rmsnorm_config2_full_size_all_rows(ctx):
+    # benchmark config 2 exactly as bench.py launches it: bf16 X[8192, 4096],
+    # learned scale, eps 1e-6, f32 Y, fused scalar MUL, bf16 output.  At this
+    # size the grid is capped, so a workgroup walks more than one row-block
+    # with the scale held in registers; every row is checked.
+    rows, cols = 8192, 4096
+    x = HT.from_logical(rand(2, 0, [rows, cols]), capi.BFLOAT16)
+    s = HT.from_logical(rand(2, 1, [1, cols], mean=1.0, std=0.02), capi.BFLOAT16)
+    epi = [capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16, scalar=0.5)]
+    out = run_norm(ctx, x, s, None, eps=1e-6, y_dtype=capi.FLOAT, epilogue=epi,
+                   expect_path=2)
+    ref = oracle.rmsnorm(x.logical(), s.logical(), 1e-6) * 0.5
+    assert_close(out.logical(), ref, capi.BFLOAT16, "config 2 full size")
+
+
+def test_rmsnorm_config2_full_size_full_operand_mul(ctx):
+    # the same with a full-size second operand G[8192, 4096]
+    rows, cols = 8192, 4096
+    x = HT.from_logical(rand(2, 0, [rows, cols]), capi.BFLOAT16)
+    s = HT.from_logical(rand(2, 1, [1, cols], mean=1.0, std=0.02), capi.BFLOAT16)
+    g = HT.from_logical(rand(2, 3, [rows, cols]), capi.BFLOAT16)
+    epi = [capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16, operand=g.desc(),
+                            operand_index=0)]
+    out = run_norm(ctx, x, s, None, eps=1e-6, y_dtype=capi.FLOAT, epilogue=epi,
+                   epi_tensors=[g], expect_path=2)
+    ref = oracle.rmsnorm(x.logical(), s.logical(), 1e-6) * g.logical()
+    assert_close(out.logical(), ref, capi.BFLOAT16, "config 2 full operand")
+
+
+def test_layernorm_8192x4096_all_rows_with_stats(ctx):
+    # the LayerNorm line of the benchmark (bf16, scale and bias, training
+    # statistics), every row and both statistics against the oracle
+    rows, cols = 8192, 4096
+    x = HT.from_logical(rand(8, 0, [rows, cols], mean=0.3, std=1.5), capi.BFLOAT16)
+    s = HT.from_logical(rand(8, 1, [1, cols], mean=1.0, std=0.1), capi.BFLOAT16)
+    b = HT.from_logical(rand(8, 2, [1, cols], std=0.2), capi.BFLOAT16)
+    out, mean, rstd = run_norm(ctx, x, s, b, eps=1e-5, layernorm=True,
+                               stats=True, expect_path=2)
+    ref, rmean, rrstd = oracle.layernorm(x.logical(), s.logical(), b.logical(),
+                                         1e-5)
+    assert_close(out.logical(), ref, capi.BFLOAT16, "layernorm full size")
+    assert_close(mean.logical(), rmean.reshape(-1), capi.FLOAT, "mean", rtol=1e-4)
+    assert_close(rstd.logical(), rrstd.reshape(-1), capi.FLOAT, "rstd", rtol=1e-4)
+
+
+@pytest.mark.parametrize("rows,cols", [(4099, 512), (2051, 1024), (1029, 2048),
+                                       (700, 4096), (600, 16384)])
+@pytest.mark.parametrize("kind", ["rms_scalar", "rms_per_row", "rms_full", "ln"])
+def test_rownorm_several_row_blocks_per_workgroup(ctx, knobs, rows, cols, kind):
+    # One workgroup per compute unit (256 workgroups): every workgroup walks
+    # two to five row-blocks, reusing the column parameters it fetched once.
+    # At 512 / 1024 / 2048 columns a workgroup holds 4 / 4 / 2 rows at a time
+    # and the row count is no multiple of that (ragged last block).
+    knobs(ROWNORM_WGS_PER_CU=1)
+    x = HT.from_logical(rand(9, 0, [rows, cols], mean=0.1), capi.BFLOAT16)
+    s = HT.from_logical(rand(9, 1, [1, cols], mean=1.0, std=0.05), capi.BFLOAT16)
+    if kind == "ln":
+        b = HT.from_logical(rand(9, 2, [1, cols], std=0.2), capi.BFLOAT16)
+        out, mean, rstd = run_norm(ctx, x, s, b, eps=1e-5, layernorm=True,
+                                   stats=True, expect_path=2)
+        ref, rmean, rrstd = oracle.layernorm(x.logical(), s.logical(),
+                                             b.logical(), 1e-5)
+        assert_close(mean.logical(), rmean.reshape(-1), capi.FLOAT, "mean", rtol=1e-4)
+        assert_close(rstd.logical(), rrstd.reshape(-1), capi.FLOAT, "rstd", rtol=1e-4)
+    else:
+        ref = oracle.rmsnorm(x.logical(), s.logical(), 1e-6)
+        if kind == "rms_scalar":
+            epi, ops = [capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16, scalar=0.5)], []
+            ref = ref * 0.5
+        else:
+            gd = [rows, 1] if kind == "rms_per_row" else [rows, cols]
+            g = HT.from_logical(rand(9, 3, gd), capi.BFLOAT16)
+            epi = [capi.epilogue_op(capi.PW["MUL"], capi.BFLOAT16,
+                                    operand=g.desc(), operand_index=0)]
+            ops = [g]
+            ref = ref * g.logical()
+        out = run_norm(ctx, x, s, None, eps=1e-6, y_dtype=capi.FLOAT,
+                       epilogue=epi, epi_tensors=ops, expect_path=2)
+    assert_close(out.logical(), ref, capi.BFLOAT16, f"{kind} {rows}x{cols}")
