@@ -196,6 +196,7 @@ SYMBOLS = {
     "fhip_conv_dgrad_workspace_size": (c_int, [POINTER(ConvDesc), POINTER(c_size_t)]),
     "fhip_conv_dgrad_supported": (c_int, [POINTER(ConvDesc)]),
     "fhip_conv_dgrad": (c_int, [_P, POINTER(ConvDesc), _P, _P, _P, _P, c_size_t]),
+    "fhip_conv_dgrad_static": (c_int, [_P, POINTER(ConvDesc), _P, _P, _P]),
     "fhip_conv_wgrad_workspace_size": (c_int, [POINTER(ConvDesc), POINTER(c_size_t)]),
     "fhip_conv_wgrad_supported": (c_int, [POINTER(ConvDesc)]),
     "fhip_conv_wgrad": (c_int, [_P, POINTER(ConvDesc), _P, _P, _P, _P, c_size_t]),
@@ -389,6 +390,12 @@ class Context:
         self._check(self.lib.fhip_conv_dgrad(self.handle, byref(d), _p(dy),
                                              _p(w), _p(dx), _p(workspace),
                                              need))
+
+    def conv_dgrad_static(self, d: ConvDesc, dy, w, dx):
+        """The data gradient on the library's static scratch: no workspace
+        argument and no allocation inside the call."""
+        self._check(self.lib.fhip_conv_dgrad_static(self.handle, byref(d),
+                                                    _p(dy), _p(w), _p(dx)))
 
     def conv_dgrad_workspace(self, d: ConvDesc) -> int:
         n = c_size_t(0)

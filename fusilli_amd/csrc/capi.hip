@@ -214,6 +214,13 @@ int fhip_ctx_create(int device_id, void *external_stream, fhip_ctx **out) {
     }
     c->owns_stream = true;
   }
+  if (fhip_conv_dgrad_static_setup(c) != 0) {
+    fhip_tls_error() = c->err;
+    if (c->owns_stream)
+      (void)hipStreamDestroy(c->stream);
+    delete c;
+    return 1;
+  }
   *out = c;
   return 0;
 }

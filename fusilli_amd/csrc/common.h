@@ -22,6 +22,8 @@ struct fhip_ctx {
   hipStream_t stream = nullptr;
   bool owns_stream = false;
   int num_cus = 0;
+  // this device's copy of the data gradient's static scratch array
+  void *dgrad_static_scratch = nullptr;
   std::string err;
 };
 

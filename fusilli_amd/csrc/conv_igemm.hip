@@ -430,6 +430,33 @@ __global__ void conv_flip_filter_kernel(FlipArgs a, const uint16_t *src,
 
 } // namespace
 
+// Scratch of the entry point that allocates nothing (fhip_conv_dgrad_static):
+// the mirrored filter and, with strides above one, DY spread over its zero
+// grid live here instead of in caller workspace.  Every device that loads the
+// library holds its own copy at its own address until the process ends; the
+// address is resolved once per device by fhip_conv_dgrad_static_setup and kept
+// in the context.  In host code the array's name is only a handle for that
+// query, never a pointer to pass on.
+static __device__ __align__(256) unsigned char
+    dgrad_static_scratch[FHIP_CONV_DGRAD_STATIC_MAX_BYTES];
+
+int fhip_conv_dgrad_static_setup(fhip_ctx *ctx) {
+  // one slot per device ordinal; written under the context-creation lock
+  constexpr int kMaxDevices = 64;
+  static void *per_device[kMaxDevices] = {};
+  FHIP_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices,
+               "device ordinal %d beyond the static scratch table", ctx->device);
+  if (!per_device[ctx->device]) {
+    void *ptr = nullptr;
+    FHIP_HIP_CHECK(ctx, hipGetSymbolAddress(&ptr, HIP_SYMBOL(dgrad_static_scratch)));
+    FHIP_REQUIRE(ctx, ptr != nullptr && ((uintptr_t)ptr & 255) == 0,
+                 "static scratch address not resolved");
+    per_device[ctx->device] = ptr;
+  }
+  ctx->dgrad_static_scratch = per_device[ctx->device];
+  return 0;
+}
+
 bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
                                      size_t *workspace_bytes) {
   const DgradPlan p = make_dgrad_plan(d);

@@ -28,6 +28,10 @@ bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
 int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                          const void *w, void *dx, void *workspace);
 
+// Resolves this device's address of the static scratch array behind
+// fhip_conv_dgrad_static into the context (device current, creation lock held).
+int fhip_conv_dgrad_static_setup(fhip_ctx *ctx);
+
 // Weight gradient as batched GEMMs over zero-padded copies of X and DY
 // (channels-last 16-bit tensors, equal strides, one group); needs
 // `*workspace_bytes` of 256-byte aligned workspace.

@@ -1200,6 +1200,33 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   return 0;
 }
 
+int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
+                           const void *dy, const void *w, void *dx) {
+  FHIP_REQUIRE(ctx, ctx != nullptr, "fhip_conv_dgrad_static: null context");
+  if (conv_bwd_validate(ctx, d, "fhip_conv_dgrad_static") != 0)
+    return 1;
+  FHIP_REQUIRE(ctx, dy && w && dx, "fhip_conv_dgrad_static: null tensor pointer");
+  FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  size_t need = 0;
+  if (fhip_fast_conv_dgrad_applicable(d, &need)) {
+    FHIP_REQUIRE(ctx, need <= (size_t)FHIP_CONV_DGRAD_STATIC_MAX_BYTES,
+                 "fhip_conv_dgrad_static: this descriptor needs %zu bytes of "
+                 "scratch, the static array holds %zu; use fhip_conv_dgrad "
+                 "with caller workspace",
+                 need, (size_t)FHIP_CONV_DGRAD_STATIC_MAX_BYTES);
+    FHIP_REQUIRE(ctx, ctx->dgrad_static_scratch != nullptr,
+                 "fhip_conv_dgrad_static: scratch address not resolved");
+    return fhip_fast_conv_dgrad(ctx, d, dy, w, dx, ctx->dgrad_static_scratch);
+  }
+  // the strided kernel uses no scratch at all
+  const ConvBwdArgs g = conv_bwd_args(d, true);
+  const int64_t total = fhip_desc_volume(d->x);
+  hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),
+                     dim3(256), 0, ctx->stream, g, dy, w, dx, total);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
 int fhip_conv_wgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
   FHIP_REQUIRE(nullptr, d && bytes, "fhip_conv_wgrad_workspace_size: null");
   *bytes = 0;

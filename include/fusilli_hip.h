@@ -275,6 +275,18 @@ int fhip_conv_dgrad_supported(const fhip_conv_desc *d);
 int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                     const void *w, void *dx, void *workspace,
                     size_t workspace_bytes);
+/* fhip_conv_dgrad without any allocation and without caller workspace.  It has
+ * no counterpart in the reference; it exists for callers that cannot allocate
+ * device memory around the call (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  The mirrored filter (and DY's zero
+ * grid for strides above one) live in a per-device static array of
+ * FHIP_CONV_DGRAD_STATIC_MAX_BYTES inside the library; descriptors whose
+ * fhip_conv_dgrad_workspace_size exceeds that fail with a message.  Same
+ * kernels and results as fhip_conv_dgrad.  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two contexts) race. */
+#define FHIP_CONV_DGRAD_STATIC_MAX_BYTES (8u << 20)
+int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
+                           const void *dy, const void *w, void *dx);
 int fhip_conv_wgrad_workspace_size(const fhip_conv_desc *d, size_t *bytes);
 int fhip_conv_wgrad_supported(const fhip_conv_desc *d);
 int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
