@@ -461,6 +461,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-others", action="store_true")
+    ap.add_argument("--only", default="",
+                    help="comma-separated substrings: run only the matching "
+                         "lines of `others` (tuning runs; skips the CPU baseline)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain copy kernel of known size (counter "
                          "calibration) and print its figures")
@@ -511,40 +514,49 @@ def main():
             result["warmup_launches"] = LAST_WARMUP
             others[name] = result
 
-        r2 = bench_rmsnorm(ctx, args.steps, args.warmup, "full")
-        other("rmsnorm_bf16_8192x4096_mul_full_operand", {
-            "value": round(r2["gbs_kernel"], 1), "unit": "GB/s",
-            "frac_of_hbm_peak": round(r2["gbs_kernel"] / HBM_PEAK_GBS, 4),
-            "kernel_us": round(r2["kernel_ms"] * 1e3, 2), "bytes": r2["bytes"]})
-        other("layernorm_bf16_8192x4096_scale_bias",
-              bench_layernorm(ctx, args.steps, args.warmup))
-        other("pointwise_add_bf16_8192x4096_bias_row",
-              bench_pointwise(ctx, max(5, args.steps // 4), 2, "ADD"))
-        other("pointwise_gelu_bf16_8192x4096",
-              bench_pointwise(ctx, max(5, args.steps // 4), 2, "GELU_FWD"))
-        other("reduce_sum_bf16_8192x4096_rows",
-              bench_reduce(ctx, args.steps, args.warmup, "SUM"))
-        other("reduce_amax_bf16_8192x4096_rows",
-              bench_reduce(ctx, args.steps, args.warmup, "AMAX"))
-        other("matmul_f32_1x256x512x256",
-              bench_matmul_f32_c1(ctx, max(10, args.steps // 4), 3))
+        def rms_full():
+            r2 = bench_rmsnorm(ctx, args.steps, args.warmup, "full")
+            return {"value": round(r2["gbs_kernel"], 1), "unit": "GB/s",
+                    "frac_of_hbm_peak": round(r2["gbs_kernel"] / HBM_PEAK_GBS, 4),
+                    "kernel_us": round(r2["kernel_ms"] * 1e3, 2), "bytes": r2["bytes"]}
+
         ksteps, kwarm = max(10, args.steps // 10), max(3, args.warmup // 5)
-        other("matmul_int8_4096x8192x4096_i32",
-              bench_matmul(ctx, ksteps, kwarm, "int8"))
-        other("matmul_fp8e4m3_4096x8192x4096_scaled_bf16_out",
-              bench_matmul(ctx, ksteps, kwarm, "fp8"))
-        other("matmul_bf16_4096x4096x4096",
-              bench_matmul(ctx, ksteps, kwarm, "bf16", 4096, 4096, 4096))
-        other("conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu",
-              bench_conv(ctx, max(20, args.steps // 4), kwarm))
-        other("conv_dgrad_bf16_n32c64h56w56_k128r3s3",
-              bench_conv_dgrad(ctx, max(20, args.steps // 4), kwarm))
-        other("conv_wgrad_bf16_n32c64h56w56_k128r3s3",
-              bench_conv_wgrad(ctx, max(20, args.steps // 10), kwarm))
-        other("sdpa_fwd_bf16_causal_b4h32s2048d128",
-              bench_sdpa(ctx, max(20, args.steps // 4), kwarm))
+        lines = [
+            ("rmsnorm_bf16_8192x4096_mul_full_operand", rms_full),
+            ("layernorm_bf16_8192x4096_scale_bias",
+             lambda: bench_layernorm(ctx, args.steps, args.warmup)),
+            ("pointwise_add_bf16_8192x4096_bias_row",
+             lambda: bench_pointwise(ctx, max(5, args.steps // 4), 2, "ADD")),
+            ("pointwise_gelu_bf16_8192x4096",
+             lambda: bench_pointwise(ctx, max(5, args.steps // 4), 2, "GELU_FWD")),
+            ("reduce_sum_bf16_8192x4096_rows",
+             lambda: bench_reduce(ctx, args.steps, args.warmup, "SUM")),
+            ("reduce_amax_bf16_8192x4096_rows",
+             lambda: bench_reduce(ctx, args.steps, args.warmup, "AMAX")),
+            ("matmul_f32_1x256x512x256",
+             lambda: bench_matmul_f32_c1(ctx, max(10, args.steps // 4), 3)),
+            ("matmul_int8_4096x8192x4096_i32",
+             lambda: bench_matmul(ctx, ksteps, kwarm, "int8")),
+            ("matmul_fp8e4m3_4096x8192x4096_scaled_bf16_out",
+             lambda: bench_matmul(ctx, ksteps, kwarm, "fp8")),
+            ("matmul_bf16_4096x4096x4096",
+             lambda: bench_matmul(ctx, ksteps, kwarm, "bf16", 4096, 4096, 4096)),
+            ("conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu",
+             lambda: bench_conv(ctx, max(20, args.steps // 4), kwarm)),
+            ("conv_dgrad_bf16_n32c64h56w56_k128r3s3",
+             lambda: bench_conv_dgrad(ctx, max(20, args.steps // 4), kwarm)),
+            ("conv_wgrad_bf16_n32c64h56w56_k128r3s3",
+             lambda: bench_conv_wgrad(ctx, max(20, args.steps // 10), kwarm)),
+            ("sdpa_fwd_bf16_causal_b4h32s2048d128",
+             lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm)),
+        ]
+        wanted = [w for w in args.only.split(",") if w]
+        for name, fn in lines:
+            if wanted and not any(w in name for w in wanted):
+                continue
+            other(name, fn())
         line["others"] = others
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not args.only:
         line["cpu_baseline"] = cpu_baseline_rmsnorm()
     ctx.close()
     print(json.dumps(line))

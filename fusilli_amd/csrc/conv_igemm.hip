@@ -238,11 +238,14 @@ int conv_launch_f16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
 }
 
 bool fhip_fast_conv_applicable(const fhip_conv_desc *d) {
-  return make_plan(d).ok;
+  return make_plan(d).ok || fhip_fast_conv_rf_applicable(d);
 }
 
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                    const void *w, const DevEpilogue &epi, void *out) {
+  if (((uintptr_t)out & 15) == 0 &&
+      fhip_fast_conv_rf_applicable_on(d, ctx->num_cus))
+    return fhip_fast_conv_rf(ctx, d, x, w, epi, out);
   const ConvPlan p = make_plan(d);
   FHIP_REQUIRE(ctx, p.ok, "conv: descriptor not supported by the MFMA kernel");
   FHIP_REQUIRE(ctx, ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0,

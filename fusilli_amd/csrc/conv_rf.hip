@@ -1,0 +1,682 @@
+// Convolution forward with the filter held in registers.
+//
+// For channels-last tensors with unit stride and unit dilation and a filter
+// small enough that a 32-channel slice of it fits a wavefront's registers
+// (R * S * C <= 640: the 3 x 3 x 64 family), the whole problem is one pass:
+//
+//   * a workgroup (4 wavefronts, one per SIMD, the full 512-register file
+//     each) owns TR output rows of one image and 128 output channels; each
+//     wavefront owns 32 of those channels and keeps its 32 x (R*S*C) filter
+//     slice in registers as ready-made MFMA A operands for the kernel's whole
+//     life (loaded once, straight from global memory);
+//   * the tile's input rows plus halo go into LDS once, by LDS-DMA, into a
+//     zero-padded image (W + S - 1 pixels per row, rows above / below the image
+//     as zeros) with a pixel pitch of C * 2 + 16 bytes: every filter tap is then
+//     a constant byte offset from an output pixel's slab address, no border
+//     masks exist, and the pitch keeps the 16-byte fragment reads of 16
+//     consecutive pixels on distinct banks;
+//   * the product is computed transposed, OUT^T[channel, pixel] = W . X^T, with
+//     v_mfma_f32_16x16x32: the pixels' B fragments are one ds_read_b128 per 16
+//     pixels and K-step, feeding two MFMAs (the wavefront's two 16-channel
+//     tiles).  A lane then holds 8 consecutive output channels of one pixel:
+//     bias / scale / ReLU run on the accumulators and the result leaves with
+//     one 16-byte store per lane, no trip through LDS;
+//   * pixels are processed in groups of 5 blocks of 16; the epilogue and the
+//     stores of group g - 1 are issued between the MFMAs of group g (two
+//     accumulator sets alternate), and the fragments of a group's first K-step
+//     are fetched during the previous group's last one, so the matrix pipe
+//     sees one continuous stream and the output leaves while it works.
+//
+// Reference semantics: aten.convolution, groups = 1 (reference
+// support/asm_emitter.h:690-701, node/conv_node.h:38-56) followed by the fused
+// pointwise chain (support/asm_emitter.h:1806-2122).
+#include "common.h"
+#include "fast_paths.h"
+#include "gemm_kernel.h"
+
+#ifdef RF_PROFILE // experiment builds: cycle stamps of workgroup 0
+__device__ uint64_t rf_prof[64];
+#define RF_STAMP(i)                                                            \
+  do {                                                                         \
+    if (blockIdx.x == 0 && threadIdx.x == 0)                                   \
+      rf_prof[i] = __builtin_amdgcn_s_memtime();                               \
+  } while (0)
+#else
+#define RF_STAMP(i)                                                            \
+  do {                                                                         \
+  } while (0)
+#endif
+#ifndef RF_VARIANT_NAME
+#define RF_VARIANT_NAME "default"
+#endif
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kRfWaves = 8;      // two per SIMD
+constexpr int kRfThreads = kRfWaves * 64;
+constexpr int kRfChannels = 128; // output channels per workgroup
+constexpr int kRfMaxNI = 16;     // KB of LDS per slab row, at most
+
+// Compile-time geometry shared by the kernel and the host's LDS budget.
+template <int C, int R, int S> struct RfGeom {
+  static constexpr int kCPP = C * 2 / 16 + 1;   // chunks per slab pixel (one is padding)
+  static constexpr int kNK = R * S * (C / 32);  // K-steps of 32 channels
+  static constexpr int kNKA = (kNK + 1) / 2;    // K-steps staged first
+  // filter stage: per wavefront one KB per (K-step, tile) of the larger part
+  static constexpr int kStageBytes = 4 * kNKA * 2 * 1024;
+};
+
+struct ConvRfArgs {
+  const char *x, *w;
+  char *out;
+  int32_t N, H, W, P, Q;
+  int32_t K;               // output channels, a multiple of 128
+  int32_t pad_h, pad_w;
+  int32_t TR;              // output rows per tile
+  int32_t tiles_per_image; // ceil(P / TR)
+  int32_t ntiles;          // N * tiles_per_image
+  int32_t kgroups;         // K / 128
+  int32_t NI;              // 1 KB LDS-DMA instructions per slab row
+  uint32_t magic_q, magic_ni;
+  uint32_t x_bytes, w_bytes;
+  int32_t o_dt;
+  int32_t lds_spare;  // byte offset of a spare KB behind the slab
+  int32_t unit_scale; // every op of the chain is additive with factor 1
+  // linear epilogue before the optional ReLU: per op y = mul ? y * o : a * y + b * o
+  int32_t nops;
+  float lin_a[FHIP_MAX_EPILOGUE], lin_b[FHIP_MAX_EPILOGUE];
+  int32_t lin_mul[FHIP_MAX_EPILOGUE];
+  DevEpilogue epi; // operand pointers; stride[2] = per-channel step
+};
+
+template <int KIND>
+__device__ __forceinline__ f32x4 rf_mfma(const u32x4 &a, const u32x4 &b,
+                                         const f32x4 &c) {
+  if constexpr (KIND == GK_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+        __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+        __builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rf_rsrc(const void *base,
+                                                          uint32_t bytes) {
+  const uint64_t b64 = (uint64_t)base;
+  const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64);
+  const uint32_t bhi = __builtin_amdgcn_readfirstlane((uint32_t)(b64 >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc(
+      (void *)(((uint64_t)bhi << 32) | blo), 0,
+      (int)__builtin_amdgcn_readfirstlane(bytes), 0x00020000);
+}
+
+template <int KIND, int C, int R, int S, bool RELU, bool UNIT>
+__global__ __launch_bounds__(kRfThreads)
+__attribute__((amdgpu_waves_per_eu(2, 2))) void
+conv_rf_kernel(ConvRfArgs g) {
+  // scalar arguments as locals (only the loop over the epilogue table indexes
+  // the argument block at run time)
+  const int a_Q = g.Q;
+  const int a_kgroups = g.kgroups;
+  const int a_TR = g.TR;
+  const int a_P = g.P;
+  const int a_NI = g.NI;
+  const int a_K = g.K;
+  const int a_tiles_per_image = g.tiles_per_image;
+  const int a_ntiles = g.ntiles;
+  const int a_W = g.W;
+  const int a_H = g.H;
+  const int a_pad_w = g.pad_w;
+  const int a_pad_h = g.pad_h;
+  const uint32_t a_magic_q = g.magic_q;
+  const uint32_t a_magic_ni = g.magic_ni;
+  const uint32_t a_x_bytes = g.x_bytes;
+  const uint32_t a_w_bytes = g.w_bytes;
+  const int a_nops = g.nops;
+  constexpr int CPP = RfGeom<C, R, S>::kCPP; // 16-byte chunks per slab pixel
+  constexpr int PITCH = CPP * 16;
+  constexpr int KPT = C / 32;                // K-steps per filter tap
+  constexpr int NK = RfGeom<C, R, S>::kNK;   // K-steps
+  constexpr int NKA = RfGeom<C, R, S>::kNKA; // K-steps of the filter's first part
+  // fragment buffers (K-steps in flight); a divisor of NK, so that a block's
+  // K-step j always sits in buffer j % RING
+  constexpr int RING = NK % 6 == 0 ? 6 : (NK % 4 == 0 ? 4 : 3);
+  constexpr int FROW = R * S * C * 2;        // bytes of a filter row
+  static_assert(C % 32 == 0 && NK % RING == 0 && NKA >= RING, "filter too small for this kernel");
+  static_assert((S - 1) * PITCH + (KPT - 1) * 64 + 48 < 65536, "ds offset range");
+
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int slice = wave & 3; // 32 output channels; wavefronts w and w + 4 share a SIMD
+  const int half = wave >> 2; // which of the pair: its pixel blocks, its filter tile
+  const int l = threadIdx.x & 63;
+  const int px = l & 15, q = l >> 4;
+  const uint32_t rowpitch = (uint32_t)a_NI * 1024u;
+  // LDS: [filter stage, one part per channel slice | slab]
+  const uint32_t lds_f = lds0 + (uint32_t)slice * (NKA * 2 * 1024);
+  const uint32_t lds_s = lds0 + RfGeom<C, R, S>::kStageBytes;
+
+  // this workgroup's channel group stays fixed; tiles are strided over
+  const int kg = (int)(blockIdx.x % (unsigned)a_kgroups);
+  const int tile0 = (int)(blockIdx.x / (unsigned)a_kgroups);
+  const int tile_step = (int)(gridDim.x / (unsigned)a_kgroups);
+  const int ch_wave = kg * kRfChannels + slice * 32;
+  RF_STAMP(0);
+
+  // ---- filter slice -> registers, through LDS --------------------------------
+  // MFMA row rho of tile t is output channel ch_wave + 8 * (rho / 4) + 4 * t +
+  // rho % 4, so that a lane's 8 results (rows 4 q .. 4 q + 3 of both tiles) are
+  // 8 consecutive channels.  K-step j covers the 64 bytes at j * 64 of a
+  // channel's R * S * C run; MFMA lane (rho, kq) takes the 16 bytes of K
+  // quarter kq.  Loading those straight into registers would touch four cache
+  // lines per lane quad (adjacent lanes are adjacent rho: rows FROW bytes
+  // apart), so each (K-step, tile) fragment is first written to one KB of LDS
+  // by one LDS-DMA instruction whose lane quads each fetch the 64 contiguous
+  // bytes of one row: DMA lane d carries row d / 4, quarter (d % 4) ^ (row / 4
+  // % 4) -- the XOR spreads the 16 rows that a fragment read of one quarter
+  // touches over all banks -- and the MFMA lane reads its 16 bytes back from
+  // position rho * 4 + (kq ^ (rho / 4 % 4)).  The two wavefronts of a slice
+  // stage one tile each and both read all fragments.  The K-step is the
+  // instructions' scalar offset (the immediate offset would also move the LDS
+  // destination), so there is no address arithmetic per instruction.
+  u32x4 filt[NK][2];
+  const __amdgpu_buffer_rsrc_t rw = rf_rsrc(g.w, a_w_bytes);
+  uint32_t fvoff;
+  {
+    const int rho = l >> 2, kq = (l & 3) ^ ((rho >> 2) & 3);
+    const int ch = ch_wave + 8 * (rho >> 2) + 4 * half + (rho & 3);
+    fvoff = (uint32_t)ch * (uint32_t)FROW + (uint32_t)kq * 16u;
+  }
+  const uint32_t fread = lds_f + (uint32_t)(px * 4 + (q ^ ((px >> 2) & 3))) * 16u;
+  auto filter_dma = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
+    constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
+    gemm_static_for<J1 - J0>([&](auto dc) {
+      constexpr int j = J0 + decltype(dc)::value;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rw,
+          (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(
+              lds_f + (uint32_t)(((j - J0) * 2 + half) * 1024)),
+          16, (int)fvoff, j * 64, 0, 0);
+    });
+  };
+  auto filter_read = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
+    constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
+    gemm_static_for<J1 - J0>([&](auto dc) {
+      constexpr int j = J0 + decltype(dc)::value;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        filt[j][t] = *(const GEMM_AS3 u32x4 *)(uintptr_t)(
+            fread + (uint32_t)(((j - J0) * 2 + t) * 1024));
+    });
+  };
+  using JA0 = std::integral_constant<int, 0>;
+  using JA1 = std::integral_constant<int, NKA>;
+  using JB1 = std::integral_constant<int, NK>;
+  filter_dma(JA0{}, JA1{});
+  RF_STAMP(14);
+
+  const __amdgpu_buffer_rsrc_t rx = rf_rsrc(g.x, a_x_bytes);
+  // lane part of the slab addressing: lane = CPP * la + lb
+  const int lane_a = (l * (65536 / CPP + 1)) >> 16;
+  const int lane_b = l - lane_a * CPP;
+  float sc[8], sh[8];
+  f32x4 acc0[2];
+
+  bool first = true; // the filter's second part is still on its way
+  for (int tile = tile0; tile < a_ntiles; tile += tile_step) {
+    const int n = tile / a_tiles_per_image;
+    const int p0 = (tile - n * a_tiles_per_image) * a_TR;
+    const int tr = a_P - p0 < a_TR ? a_P - p0 : a_TR;
+    const int npix = tr * a_Q;
+    const int rows_in = tr + R - 1;
+    const int ih0 = p0 - a_pad_h;
+
+    // ---- slab: rows_in rows of NI KB by LDS-DMA; wavefront w loads KB w, w + 8, ...
+    // LDS chunk x = i * 64 + lane of a slab row is chunk x % CPP of slab pixel
+    // x / CPP, i.e. input pixel (ih0 + row, x / CPP - pad_w); the padding chunk,
+    // pixels outside the image and the tail of a row's last KB read as zeros.
+    for (int idx = wave; idx < rows_in * a_NI; idx += kRfWaves) {
+      const int sr = (int)conv_div(idx, a_NI, a_magic_ni);
+      const int i = idx - sr * a_NI;
+      const int ih = ih0 + sr;
+      const bool row_ok = (unsigned)ih < (unsigned)a_H;
+      const int soff = row_ok ? ((n * a_H + ih) * a_W) * (C * 2) : 0;
+      // x = i * 64 + lane = CPP * (ua + la) + (ub + lb): scalar and lane parts
+      const int ua = ((i * 64) * (65536 / CPP + 1)) >> 16;
+      const int ub = i * 64 - ua * CPP;
+      const int t = lane_b + ub;
+      const int wrap = t >= CPP ? 1 : 0;
+      const int c = t - wrap * CPP;
+      const int iw = lane_a + ua + wrap - a_pad_w;
+      const bool ok = row_ok && c < CPP - 1 && (unsigned)iw < (unsigned)a_W;
+      const uint32_t off = ok ? (uint32_t)(iw * (C * 2) + c * 16) : 0x80000000u;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rx,
+          (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(lds_s + (uint32_t)idx * 1024u),
+          16, (int)off, soff, 0, 0);
+    }
+    if (first) {
+      // ---- epilogue constants: y = acc * sc[c] + sh[c] for the lane's 8 channels
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        sc[c] = 1.f;
+        sh[c] = 0.f;
+      }
+      for (int e = 0; e < a_nops; ++e) {
+        const DevEpiOp &o = g.epi.op[e];
+        // the 8 operand values of an op are fetched by loads issued back to back
+        float ovs[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          ovs[c] = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
+        if (o.kind == FHIP_OPERAND_TENSOR) {
+          int64_t off[8];
+#pragma unroll
+          for (int c = 0; c < 8; ++c)
+            off[c] = (int64_t)(ch_wave + 8 * q + c) * o.stride[2];
+          load_operand_vec<8>(o.ptr, o.operand_dtype, off, ovs);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const float ov = ovs[c];
+          if (g.lin_mul[e]) {
+            sc[c] *= ov;
+            sh[c] *= ov;
+          } else {
+            sc[c] *= g.lin_a[e];
+            sh[c] = sh[c] * g.lin_a[e] + g.lin_b[e] * ov;
+          }
+        }
+      }
+      // with unit scales (UNIT: the host found every op additive with factor
+      // 1) the shift is the accumulators' start value and the multiply-add
+      // drops out of the epilogue
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc0[t][i] = UNIT ? sh[4 * t + i] : 0.f;
+    }
+    RF_STAMP(1);
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+    RF_STAMP(2);
+    gemm_barrier();
+    RF_STAMP(3);
+    if (first) {
+      // first part of the filter into registers; the stage is refilled with
+      // the second part once every wavefront has read the first
+      filter_read(JA0{}, JA1{});
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
+      gemm_barrier();
+      filter_dma(JA1{}, JB1{});
+    }
+
+    // outputs of this tile: dense rows of K channels, pixel index tile-relative
+    const __amdgpu_buffer_rsrc_t ro =
+        rf_rsrc(g.out + ((int64_t)(n * a_P + p0) * a_Q) * a_K * 2,
+                (uint32_t)npix * (uint32_t)a_K * 2u);
+    const uint32_t lane_out = (uint32_t)(ch_wave + 8 * q) * 2u;
+    const int nblocks = (npix + 15) >> 4;
+
+    // Slab address (filter row 0, this lane's K quarter) and output offset of
+    // this lane's pixel of block b.
+    auto block_setup = [&](int b, uint32_t &base, uint32_t &ooff) __attribute__((always_inline)) {
+      const int pl = b * 16 + px;
+      const int plc = pl < npix ? pl : npix - 1;
+      const int prow = (int)conv_div(plc, a_Q, a_magic_q);
+      const int pcol = plc - prow * a_Q;
+      base = lds_s + (uint32_t)prow * rowpitch + (uint32_t)pcol * PITCH + (uint32_t)q * 16u;
+      ooff = pl < npix ? (uint32_t)pl * (uint32_t)a_K * 2u + lane_out : 0x80000000u;
+    };
+    u32x4 frag[RING];
+    auto fetch = [&](auto jc, uint32_t base) __attribute__((always_inline)) {
+      constexpr int j = decltype(jc)::value;
+      constexpr int tap = j / KPT, part = j % KPT;
+      constexpr int r = tap / S, s = tap % S;
+      frag[j % RING] = *(const GEMM_AS3 u32x4 *)(uintptr_t)(
+          base + (uint32_t)r * rowpitch + (uint32_t)(s * PITCH + part * 64));
+    };
+    f32x4 acc[2];
+    uint32_t base, ooff, nbase, nooff;
+    // K-steps [J0, J1) of the block at `base`; the first fragments of the next
+    // block (at `nbase`) are fetched during the last steps.
+    auto ksteps = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
+      constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
+      gemm_static_for<J1 - J0>([&](auto dc) {
+        constexpr int j = J0 + decltype(dc)::value;
+        constexpr int ahead = j + RING - 1;
+        if constexpr (ahead < NK)
+          fetch(std::integral_constant<int, ahead>{}, base);
+        else
+          fetch(std::integral_constant<int, ahead - NK>{}, nbase);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+          acc[t] = rf_mfma<KIND>(filt[j][t], frag[j % RING], j == 0 ? acc0[t] : acc[t]);
+      });
+    };
+    // scale / ReLU, rounding and the 16-byte store of a finished block
+    auto finish = [&](const float (&yin)[8], uint32_t off) __attribute__((always_inline)) {
+      float y[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        y[c] = UNIT ? yin[c] : __builtin_fmaf(yin[c], sc[c], sh[c]);
+      // (scalar words: bit-casting an element of a vector in place reads
+      // element 0)
+      uint32_t w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        // one packed round-to-nearest-even conversion per pair (a vector
+        // conversion: inline asm here would hide the MFMA -> VALU hazard of
+        // its operands from the compiler's hazard handling)
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        const f2 pair = {y[2 * i], y[2 * i + 1]};
+        if constexpr (KIND == GK_BF16) {
+          typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+          const b2 r = __builtin_convertvector(pair, b2);
+          w[i] = __builtin_bit_cast(uint32_t, r);
+        } else {
+          typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+          const h2 r = __builtin_convertvector(pair, h2);
+          w[i] = __builtin_bit_cast(uint32_t, r);
+        }
+        if constexpr (RELU) {
+          // max(x, 0) on the rounded pair: as 16-bit integers the negative
+          // values (and -0) are exactly the patterns below zero
+          typedef short s2 __attribute__((ext_vector_type(2)));
+          const s2 v = __builtin_bit_cast(s2, w[i]);
+          w[i] = __builtin_bit_cast(uint32_t,
+                                    __builtin_elementwise_max(v, s2{0, 0}));
+        }
+      }
+      const u32x4 pk = {w[0], w[1], w[2], w[3]};
+      __builtin_amdgcn_raw_buffer_store_b128(pk, ro, (int)off, 0, 0);
+    };
+
+    // This wavefront's blocks: half, half + 2, ...  (block indices past the
+    // last one address the last pixel and store nothing).
+    int b = half;
+    block_setup(b, base, ooff);
+    gemm_static_for<RING - 1>([&](auto jc) { fetch(jc, base); });
+    RF_STAMP(4);
+    if (first) {
+      // The first block (of every wavefront: the barrier in its middle is the
+      // workgroup's) runs its first K-steps on the first part of the filter.
+      block_setup(b + 2, nbase, nooff);
+      ksteps(JA0{}, JA1{});
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+      gemm_barrier();
+      filter_read(JA1{}, JB1{});
+      ksteps(JA1{}, JB1{});
+      float y[8];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          y[4 * t + i] = acc[t][i];
+      const uint32_t done_off = ooff;
+      b += 2;
+      base = nbase;
+      ooff = nooff;
+      first = false;
+      finish(y, done_off);
+    }
+    RF_STAMP(5);
+    for (; b < nblocks; b += 2) {
+      block_setup(b + 2, nbase, nooff);
+      ksteps(JA0{}, JB1{});
+      float y[8];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          y[4 * t + i] = acc[t][i];
+      const uint32_t done_off = ooff;
+      base = nbase;
+      ooff = nooff;
+      finish(y, done_off);
+    }
+    RF_STAMP(12);
+    // every wavefront is done with the slab before the next tile overwrites it
+    if (tile + tile_step < a_ntiles) {
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+      gemm_barrier();
+    }
+  }
+  RF_STAMP(13);
+}
+
+struct RfPlan {
+  bool ok = false;
+  int kind = 0;
+  int C = 0, R = 0, S = 0;
+  bool relu = false;
+  ConvRfArgs a{};
+  int lds = 0;
+  int grid = 0;
+};
+
+bool rf_channels_last(const fhip_tensor_desc &t) {
+  int64_t expect = 1;
+  int order[FHIP_MAX_RANK];
+  int n = 0;
+  order[n++] = 1;
+  for (int i = t.rank - 1; i >= 2; --i)
+    order[n++] = i;
+  order[n++] = 0;
+  for (int i = 0; i < n; ++i) {
+    const int d = order[i];
+    if (t.dim[d] != 1 && t.stride[d] != expect)
+      return false;
+    expect *= t.dim[d];
+  }
+  return true;
+}
+
+// The (C, R, S) instances that are compiled.
+bool rf_instance(int C, int R, int S) {
+  return C == 64 && R == 3 && S == 3;
+}
+
+RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
+  RfPlan p;
+  const FhipKnobs &knobs = fhip_knobs();
+  if (knobs.conv_rows == 0)
+    return p;
+  if (d->spatial_rank != 2 || d->x.dtype != d->w.dtype)
+    return p;
+  if (d->x.dtype == FHIP_BFLOAT16)
+    p.kind = GK_BF16;
+  else if (d->x.dtype == FHIP_HALF)
+    p.kind = GK_F16;
+  else
+    return p;
+  if (d->out.dtype != d->x.dtype) // the element kind also fixes the rounding
+    return p;
+  if (d->y.dtype != FHIP_FLOAT && !(d->epilogue.count == 0 && d->y.dtype == d->out.dtype))
+    return p;
+  const int64_t C = d->x.dim[1], K = d->w.dim[0];
+  if (d->w.dim[1] != C || K % kRfChannels != 0)
+    return p;
+  const int64_t R = d->w.dim[2], S = d->w.dim[3];
+  if (!rf_instance((int)C, (int)R, (int)S))
+    return p;
+  for (int i = 0; i < 2; ++i)
+    if (d->stride[i] != 1 || d->dilation[i] != 1)
+      return p;
+  if (!rf_channels_last(d->x) || !rf_channels_last(d->w) || !rf_channels_last(d->out))
+    return p;
+  ConvRfArgs &a = p.a;
+  a.N = (int32_t)d->x.dim[0], a.H = (int32_t)d->x.dim[2], a.W = (int32_t)d->x.dim[3];
+  a.P = (int32_t)d->y.dim[2], a.Q = (int32_t)d->y.dim[3];
+  a.K = (int32_t)K;
+  a.pad_h = (int32_t)d->padding[0], a.pad_w = (int32_t)d->padding[1];
+  if (a.P != a.H + 2 * a.pad_h - (int)R + 1 || a.Q != a.W + 2 * a.pad_w - (int)S + 1)
+    return p;
+  const int64_t x_bytes = (int64_t)a.N * a.H * a.W * C * 2;
+  const int64_t o_tile_max = (int64_t)a.P * a.Q * K * 2;
+  if (x_bytes >= (1ll << 31) || o_tile_max >= (1ll << 31) || K * R * S * C * 2 >= (1ll << 31))
+    return p;
+  a.x_bytes = (uint32_t)x_bytes;
+  a.w_bytes = (uint32_t)(K * R * S * C * 2);
+  // epilogue: linear ops with scalar / per-channel operands and f32
+  // intermediates, optionally closed by one ReLU
+  int nops = d->epilogue.count;
+  if (nops > 0 && d->epilogue.op[nops - 1].mode == FHIP_PW_RELU_FWD) {
+    p.relu = true;
+    --nops;
+  }
+  {
+    GemmArgs tmp{};
+    tmp.c_dt = d->y.dtype;
+    tmp.o_dt = d->out.dtype;
+    for (int i = 0; i < d->epilogue.count; ++i) {
+      const fhip_epilogue_op &o = d->epilogue.op[i];
+      if (o.operand_kind == FHIP_OPERAND_TENSOR) {
+        int64_t st[FHIP_MAX_RANK];
+        if (!fhip_broadcast_strides(o.operand, d->y.rank, d->y.dim, st))
+          return p;
+        // per-channel vectors only
+        if ((d->y.dim[0] != 1 && st[0] != 0) || (d->y.dim[2] != 1 && st[2] != 0) ||
+            (d->y.dim[3] != 1 && st[3] != 0))
+          return p;
+        const int dt = o.operand.dtype;
+        if (dt != FHIP_FLOAT && dt != FHIP_BFLOAT16 && dt != FHIP_HALF)
+          return p;
+        tmp.epi.op[i].stride[2] = st[1];
+      }
+    }
+    gemm_fill_linear(d->epilogue, tmp);
+    if (!tmp.epi_reg)
+      return p;
+    a.unit_scale = 1;
+    for (int i = 0; i < nops; ++i) {
+      if (tmp.lin_relu[i])
+        return p; // a ReLU in the middle of the chain
+      a.lin_a[i] = tmp.lin_a[i];
+      a.lin_b[i] = tmp.lin_b[i];
+      a.lin_mul[i] = tmp.lin_mul[i];
+      if (tmp.lin_mul[i] || tmp.lin_a[i] != 1.f)
+        a.unit_scale = 0;
+    }
+  }
+  a.nops = nops;
+  a.o_dt = d->out.dtype;
+  // slab geometry
+  const int cpp = (int)C * 2 / 16 + 1;
+  const int wp = a.W + (int)S - 1 + 0; // = W + 2 * pad_w
+  if (a.W + 2 * a.pad_w != a.Q + (int)S - 1)
+    return p;
+  a.NI = ((a.W + 2 * a.pad_w) * cpp + 63) / 64;
+  (void)wp;
+  if (a.NI > kRfMaxNI)
+    return p;
+  // LDS: the filter stage (one KB per K-step and tile of the larger filter
+  // part, per wavefront) in front of the slab
+  const int stage = 4 * (int)((R * S * (C / 32) + 1) / 2) * 2 * 1024;
+  const int64_t lds_cap = 160 * 1024 - stage - 1024;
+  // rows per tile: the choice that fills whole rounds of the machine best
+  const int cus = num_cus > 0 ? num_cus : 256;
+  const int kgroups = (int)(K / kRfChannels);
+  double best = 0;
+  int best_tr = 0;
+  for (int tr = 1; tr <= a.P; ++tr) {
+    const int64_t lds = (int64_t)(tr + R - 1) * a.NI * 1024;
+    if (lds > lds_cap)
+      break;
+    const int64_t tiles = (int64_t)a.N * ((a.P + tr - 1) / tr) * kgroups;
+    const int64_t rounds = (tiles + cus - 1) / cus;
+    const int64_t blocks = ((int64_t)tr * a.Q + 15) / 16;
+    // time of a round ~ the blocks of the busier wavefront of a pair plus a
+    // fixed set-up share
+    const double cost = (double)rounds * ((blocks + 1) / 2 * 2 * 16 + 96);
+    const double eff = (double)a.N * a.P * a.Q * kgroups / (cost * cus);
+    if (eff > best + 1e-9) {
+      best = eff;
+      best_tr = tr;
+    }
+  }
+  if (knobs.conv_rows > 0 && knobs.conv_rows <= a.P &&
+      (int64_t)(knobs.conv_rows + R - 1) * a.NI * 1024 <= lds_cap)
+    best_tr = knobs.conv_rows;
+  if (best_tr == 0)
+    return p;
+  // small problems that leave most of the machine idle stay with the tiled kernels
+  if (best < 0.5 && knobs.conv_rows < 0)
+    return p;
+  a.TR = best_tr;
+  a.tiles_per_image = (a.P + a.TR - 1) / a.TR;
+  a.ntiles = a.N * a.tiles_per_image;
+  a.kgroups = kgroups;
+  a.magic_q = conv_magic(a.Q);
+  a.magic_ni = conv_magic(a.NI);
+  p.C = (int)C, p.R = (int)R, p.S = (int)S;
+  a.lds_spare = stage + (a.TR + (int)R - 1) * a.NI * 1024;
+  p.lds = a.lds_spare + 1024;
+  const int64_t items = (int64_t)a.ntiles * kgroups;
+  const int64_t slots = (int64_t)cus / kgroups * kgroups > 0 ? (int64_t)cus / kgroups * kgroups : kgroups;
+  p.grid = (int)(items < slots ? items : slots);
+  p.ok = true;
+  return p;
+}
+
+template <int KIND, int C, int R, int S, bool RELU, bool UNIT>
+int rf_launch(fhip_ctx *ctx, const RfPlan &p) {
+  auto kernel = conv_rf_kernel<KIND, C, R, S, RELU, UNIT>;
+  static FhipOncePerDevice configured;
+  if (!configured.done(ctx->device)) {
+    FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
+                            reinterpret_cast<const void *>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024));
+    configured.mark(ctx->device);
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)p.grid), dim3(kRfThreads), p.lds,
+                     ctx->stream, p.a);
+  FHIP_HIP_CHECK(ctx, hipGetLastError());
+  return 0;
+}
+
+template <int KIND, int C, int R, int S>
+int rf_launch_relu(fhip_ctx *ctx, const RfPlan &p) {
+  if (p.a.unit_scale)
+    return p.relu ? rf_launch<KIND, C, R, S, true, true>(ctx, p)
+                  : rf_launch<KIND, C, R, S, false, true>(ctx, p);
+  return p.relu ? rf_launch<KIND, C, R, S, true, false>(ctx, p)
+                : rf_launch<KIND, C, R, S, false, false>(ctx, p);
+}
+
+template <int KIND> int rf_launch_shape(fhip_ctx *ctx, const RfPlan &p) {
+  if (p.C == 64 && p.R == 3 && p.S == 3)
+    return rf_launch_relu<KIND, 64, 3, 3>(ctx, p);
+  return fhip_fail(ctx, "conv: no register-filter kernel for this filter");
+}
+
+} // namespace
+
+bool fhip_fast_conv_rf_applicable(const fhip_conv_desc *d) {
+  return make_rf_plan(d, 256).ok;
+}
+bool fhip_fast_conv_rf_applicable_on(const fhip_conv_desc *d, int num_cus) {
+  return make_rf_plan(d, num_cus).ok;
+}
+
+int fhip_fast_conv_rf(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
+                      const void *w, const DevEpilogue &epi, void *out) {
+  RfPlan p = make_rf_plan(d, ctx->num_cus);
+  FHIP_REQUIRE(ctx, p.ok, "conv: descriptor not supported by the register-filter kernel");
+  FHIP_REQUIRE(ctx, ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+                        ((uintptr_t)out & 15) == 0,
+               "conv: X, W and OUT must be 16-byte aligned");
+  p.a.x = (const char *)x;
+  p.a.w = (const char *)w;
+  p.a.out = (char *)out;
+  p.a.epi = epi;
+  for (int i = 0; i < epi.count; ++i)
+    p.a.epi.op[i].stride[2] = epi.op[i].stride[1]; // per-channel step
+  return p.kind == GK_BF16 ? rf_launch_shape<GK_BF16>(ctx, p)
+                           : rf_launch_shape<GK_F16>(ctx, p);
+}

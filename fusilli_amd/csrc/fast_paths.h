@@ -21,6 +21,14 @@ bool fhip_fast_conv_applicable(const fhip_conv_desc *d);
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                    const void *w, const DevEpilogue &epi, void *out);
 
+// The same problem on the register-filter kernel (unit stride and dilation,
+// 3 x 3 x 64 filters, K a multiple of 128, 16-bit output, linear epilogue that
+// may end in a ReLU); fhip_fast_conv tries it first.
+bool fhip_fast_conv_rf_applicable(const fhip_conv_desc *d);
+bool fhip_fast_conv_rf_applicable_on(const fhip_conv_desc *d, int num_cus);
+int fhip_fast_conv_rf(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
+                      const void *w, const DevEpilogue &epi, void *out);
+
 // Data gradient through the forward kernel (unit strides, one group); needs
 // `*workspace_bytes` of 16-byte aligned workspace for the mirrored filter.
 bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,

@@ -186,3 +186,71 @@ def test_conv_igemm_headline_shape(ctx):
         ref = oracle.conv_fprop(xl[img:img + 1], w.logical(), pad, st, dil)
         ref = np.maximum(ref + bias.logical(), 0.0)
         assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"image {img}")
+
+
+# ---- register-filter kernel (3 x 3 x 64 filters, unit stride, K % 128 == 0) -----
+RF_CASES = [
+    # rows per tile forced (CONV_ROWS): image geometry, channels
+    # width not a multiple of 16, rows not a multiple of the tile height
+    dict(x=[2, 64, 13, 21], k=128, pad=[1, 1], rows=4),
+    # one row per tile (halo rows dominate), two channel groups
+    dict(x=[1, 64, 9, 17], k=256, pad=[1, 1], rows=1),
+    # no padding: output smaller than input
+    dict(x=[3, 64, 12, 19], k=128, pad=[0, 0], rows=5),
+    # padding 2: output larger than input, rows of zeros above and below
+    dict(x=[2, 64, 7, 30], k=128, pad=[2, 2], rows=3),
+    # asymmetric padding
+    dict(x=[2, 64, 10, 16], k=128, pad=[0, 2], rows=8),
+    # more tiles than compute units: workgroups walk several tiles
+    dict(x=[40, 64, 16, 8], k=128, pad=[1, 1], rows=2),
+    # whole image per tile, a single group of blocks and a ragged one
+    dict(x=[2, 64, 6, 11], k=128, pad=[1, 1], rows=6),
+    # wide image (several KB of slab per row)
+    dict(x=[1, 64, 5, 100], k=128, pad=[1, 1], rows=2),
+]
+
+
+@pytest.mark.parametrize("case", RF_CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("epi_kind", ["bias_relu", "none", "scale_bias"])
+def test_conv_register_filter_kernel_vs_oracle(ctx, knobs, case, dtype, epi_kind):
+    xd, wd = case["x"], [case["k"], 64, 3, 3]
+    pad, st, dil = case["pad"], [1, 1], [1, 1]
+    x = cl(xd, 47, 0, dtype)
+    w = cl(wd, 47, 1, dtype, std=0.05)
+    bias = HT.from_logical(rand(47, 2, [1, case["k"], 1, 1]), dtype,
+                           oracle.channels_last_strides([1, case["k"], 1, 1]))
+    ref = oracle.conv_fprop(x.logical(), w.logical(), pad, st, dil)
+    if epi_kind == "bias_relu":
+        epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0,
+                                operand=bias.desc()),
+               capi.epilogue_op(capi.PW["RELU_FWD"], dtype)]
+        ops = [bias]
+        ref = np.maximum(ref + bias.logical(), 0.0)
+    elif epi_kind == "scale_bias":
+        epi = [capi.epilogue_op(capi.PW["MUL"], capi.FLOAT, scalar=0.25),
+               capi.epilogue_op(capi.PW["SUB"], dtype, operand_index=0,
+                                operand=bias.desc())]
+        ops = [bias]
+        ref = ref * 0.25 - bias.logical()
+    else:
+        epi, ops = [], []
+    got = {}
+    for rows in (case["rows"], 0):  # the register-filter kernel, then the tiled one
+        knobs(CONV_ROWS=rows)
+        got[rows] = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=dtype,
+                        epilogue=epi, epi_tensors=ops).logical()
+        assert_close(got[rows], ref, dtype, f"rows={rows} {case} {epi_kind}")
+
+
+def test_conv_register_filter_kernel_chosen_rows(ctx, knobs):
+    # the planner's own tile height on a mid-sized problem (no knob), and the
+    # all-ones closed form there: 64 channels x taps inside the image
+    xd, wd = [16, 64, 28, 28], [256, 64, 3, 3]
+    ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
+    ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
+    out = run(ctx, ones_x, ones_w, [1, 1], [1, 1], [1, 1], capi.FLOAT,
+              out_dtype=capi.BFLOAT16).logical()
+    taps = np.full(28, 3.0); taps[[0, -1]] = 2.0
+    assert np.array_equal(out, np.broadcast_to(64.0 * taps[:, None] * taps[None, :],
+                                               out.shape))
