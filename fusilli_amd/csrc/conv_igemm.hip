@@ -242,11 +242,21 @@ bool fhip_fast_conv_applicable(const fhip_conv_desc *d) {
 }
 
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
-                   const void *w, const DevEpilogue &epi, void *out) {
-  if (((uintptr_t)out & 15) == 0 &&
-      fhip_fast_conv_rf_applicable_on(d, ctx->num_cus))
-    return fhip_fast_conv_rf(ctx, d, x, w, epi, out);
+                   const void *w, const DevEpilogue &epi, void *out,
+                   bool *handled) {
+  if (handled)
+    *handled = true;
+  bool taken = false;
+  if (fhip_fast_conv_rf(ctx, d, x, w, epi, out, &taken) != 0)
+    return 1;
+  if (taken)
+    return 0;
   const ConvPlan p = make_plan(d);
+  if (handled) {
+    *handled = p.ok;
+    if (!p.ok)
+      return 0;
+  }
   FHIP_REQUIRE(ctx, p.ok, "conv: descriptor not supported by the MFMA kernel");
   FHIP_REQUIRE(ctx, ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0,
                "conv: X and W must be 16-byte aligned");

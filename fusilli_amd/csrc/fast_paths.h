@@ -18,16 +18,21 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
                            int64_t b_outer, int64_t o_outer);
 
 bool fhip_fast_conv_applicable(const fhip_conv_desc *d);
+// With `handled` the call plans once and reports whether a tuned kernel was
+// launched; a descriptor that none takes is then no error.
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
-                   const void *w, const DevEpilogue &epi, void *out);
+                   const void *w, const DevEpilogue &epi, void *out,
+                   bool *handled = nullptr);
 
 // The same problem on the register-filter kernel (unit stride and dilation,
 // 3 x 3 x 64 filters, K a multiple of 128, 16-bit output, linear epilogue that
 // may end in a ReLU); fhip_fast_conv tries it first.
 bool fhip_fast_conv_rf_applicable(const fhip_conv_desc *d);
-bool fhip_fast_conv_rf_applicable_on(const fhip_conv_desc *d, int num_cus);
+// With `handled` the call plans once and reports whether it launched; a
+// descriptor it does not take is then no error.
 int fhip_fast_conv_rf(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
-                      const void *w, const DevEpilogue &epi, void *out);
+                      const void *w, const DevEpilogue &epi, void *out,
+                      bool *handled = nullptr);
 
 // Data gradient through the forward kernel (unit strides, one group); needs
 // `*workspace_bytes` of 16-byte aligned workspace for the mirrored filter.

@@ -1064,8 +1064,11 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   if (fhip_build_epilogue(ctx, d->epilogue, d->y.rank, d->y.dim,
                           epilogue_operands, &epi) != 0)
     return 1;
-  if (fhip_fast_conv_applicable(d))
-    return fhip_fast_conv(ctx, d, x, w, epi, out);
+  bool tuned = false;
+  if (fhip_fast_conv(ctx, d, x, w, epi, out, &tuned) != 0)
+    return 1;
+  if (tuned)
+    return 0;
 
   ConvArgs g{};
   g.y = make_dims(d->y);
