@@ -161,8 +161,10 @@ def make_epilogue(ops: Sequence[EpilogueOp]) -> Epilogue:
     return e
 
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
-                         "libfusilli_hip.so")
+# FUSILLI_HIP_LIBRARY names another build of the library (tuning runs that
+# compare builds side by side); the default is the in-tree one.
+_LIB_PATH = os.environ.get("FUSILLI_HIP_LIBRARY") or os.path.join(
+    os.path.dirname(os.path.abspath(__file__)), "lib", "libfusilli_hip.so")
 
 # name -> (restype, argtypes); every symbol include/fusilli_hip.h declares.
 _P = c_void_p
