@@ -431,6 +431,76 @@ def calibrate_copy(ctx, steps):
             "gbs": round(2 * n * 4 / ev_ms / 1e6, 1)}
 
 
+def roofline_of(result):
+    """The `roofline` object of one `others` line, from the figures its bench
+    function measured: algorithmic bytes (or flops) of one call over the
+    HIP-event time of one call, against the HBM (or dense MFMA) peak."""
+    us = result.get("kernel_us", result.get("call_us"))
+    if "bytes" in result:
+        achieved = result["bytes"] / us / 1e3
+        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "kernel_us": us, "traffic": None}
+    achieved = result["work"] / us / 1e6
+    peak = achieved / result["frac_of_mfma_peak"] if result["frac_of_mfma_peak"] else None
+    return {"bound": "mfma", "achieved": round(achieved, 1),
+            "peak": round(peak, 1) if peak else None,
+            "unit": result["unit"], "frac": result["frac_of_mfma_peak"],
+            "kernel_us": us, "traffic": None}
+
+
+def _timed_cpu(fn, seconds_budget):
+    fn()  # warm (page-in, thread pool)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds_budget:
+            return reps, dt
+
+
+def cpu_baseline_others(seconds_budget=4.0):
+    """The CPU oracle (float64 accumulation, OpenMP) on bounded samples of the
+    matmul, convolution and attention workloads of `others`."""
+    from oracle import oracle
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    out = {}
+    # int8 matmul: 32 rows of the 4096 x 8192 x 4096 product
+    m, n, k, rows = 4096, 4096, 8192, 32
+    a = synth.integers(5, 0, rows * k, -127, 127).astype(np.int8).reshape(rows, k)
+    b = synth.integers(5, 1, k * n, -127, 127).astype(np.int8).reshape(k, n)
+    idx = np.arange(rows)
+    reps, dt = _timed_cpu(lambda: oracle.matmul_rows(a, b, idx), seconds_budget)
+    out["matmul_int8_4096x8192x4096_i32"] = {
+        "value": round(2.0 * rows * n * k * reps / dt / 1e12, 5), "unit": "TOP/s",
+        "cores": threads, "kind": "port",
+        "sample": f"{reps} passes over {rows} of {m} output rows, {dt:.1f} s"}
+    # convolution: one image of the 32
+    c, h, w, kk, r = 64, 56, 56, 128, 3
+    x = synth.f32_to_bf16_bits(synth.normal(8, 0, c * h * w))
+    x = oracle.dequantize(x, capi.BFLOAT16).reshape(1, h, w, c).transpose(0, 3, 1, 2)
+    wt = synth.f32_to_bf16_bits(synth.normal(8, 1, kk * c * r * r, 0.0, 0.05))
+    wt = oracle.dequantize(wt, capi.BFLOAT16).reshape(kk, r, r, c).transpose(0, 3, 1, 2)
+    reps, dt = _timed_cpu(lambda: oracle.conv_fprop(x, wt, [1, 1], [1, 1], [1, 1]),
+                          seconds_budget)
+    out["conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu"] = {
+        "value": round(2.0 * h * w * kk * c * r * r * reps / dt / 1e12, 5),
+        "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"{reps} passes over 1 of 32 images (convolution only), {dt:.1f} s"}
+    # attention: two of the 128 (batch, head) pairs
+    sq, dd, heads = 2048, 128, 2
+    q, kx, v = (oracle.dequantize(
+        synth.f32_to_bf16_bits(synth.normal(9, i, heads * sq * dd)), capi.BFLOAT16
+    ).reshape(1, heads, sq, dd) for i in range(3))
+    reps, dt = _timed_cpu(lambda: oracle.sdpa(q, kx, v, is_causal=True), seconds_budget)
+    out["sdpa_fwd_bf16_causal_b4h32s2048d128"] = {
+        "value": round(4.0 * heads * sq * sq * dd / 2 * reps / dt / 1e12, 5),
+        "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"{reps} passes over {heads} of 128 (batch, head) pairs, {dt:.1f} s"}
+    return out
+
+
 def cpu_baseline_rmsnorm(seconds_budget=12.0):
     """The oracle's bf16 RMSNorm * scalar on the host cores over a row sample."""
     from oracle import oracle
@@ -501,6 +571,9 @@ def main():
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(r["gbs_kernel"] / HBM_PEAK_GBS, 4),
                      "traffic": RMSNORM_TRAFFIC_BYTES,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                       "of an earlier run, scaled by a plain "
+                                       "copy (profiles/); not measured by this run",
                      "algorithmic_bytes_per_launch": r["bytes"],
                      "kernel_us": round(r["kernel_ms"] * 1e3, 2),
                      "launch_us": r["launch_us"]},
@@ -512,6 +585,7 @@ def main():
 
         def other(name, result):
             result["warmup_launches"] = LAST_WARMUP
+            result["roofline"] = roofline_of(result)
             others[name] = result
 
         def rms_full():
@@ -558,6 +632,8 @@ def main():
         line["others"] = others
     if not args.no_cpu_baseline and not args.only:
         line["cpu_baseline"] = cpu_baseline_rmsnorm()
+        if not args.no_others:
+            line["cpu_baseline"]["others"] = cpu_baseline_others()
     ctx.close()
     print(json.dumps(line))
 
