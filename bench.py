@@ -286,8 +286,9 @@ def bench_conv_dgrad(ctx, steps, warmup):
 
 def bench_conv_wgrad(ctx, steps, warmup):
     """Weight gradient of C3: DY bf16 NHWC [32,128,56,56], X [32,64,56,56] ->
-    DW KRSC [128,64,3,3]; zero-padded copies of both operands, one batched
-    MFMA GEMM per filter row, a sum over the batch (6 kernels per call)."""
+    DW KRSC [128,64,3,3]; one MFMA kernel that reads X and DY in place and
+    leaves one block of partial sums per workgroup, then their sum (2 kernels
+    per call)."""
     n, c, h, w, k, r = 32, 64, 56, 56, 128, 3
     cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
     xd, wd, yd = [n, c, h, w], [k, c, r, r], [n, k, h, w]
@@ -310,7 +311,7 @@ def bench_conv_wgrad(ctx, steps, warmup):
     return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
             "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
             "call_us": round(ev_ms * 1e3, 2), "work": flop,
-            "kernels_per_call": 6}
+            "kernels_per_call": 2}
 
 
 def bench_reduce(ctx, steps, warmup, mode="SUM", sets=5):

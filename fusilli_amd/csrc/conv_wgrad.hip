@@ -186,6 +186,8 @@ __global__ void conv_wgrad_sum_kernel(WgradSumArgs a, const float *part,
 
 bool fhip_fast_conv_wgrad_applicable(const fhip_conv_desc *d,
                                      size_t *workspace_bytes) {
+  if (fhip_fast_conv_wgrad_direct_applicable(d, workspace_bytes))
+    return true;
   const WgradPlan p = make_wgrad_plan(d);
   if (workspace_bytes)
     *workspace_bytes = p.ok ? p.xp_bytes + p.dyp_bytes + p.part_bytes : 0;
@@ -194,6 +196,8 @@ bool fhip_fast_conv_wgrad_applicable(const fhip_conv_desc *d,
 
 int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                          const void *x, void *dw, void *workspace) {
+  if (fhip_fast_conv_wgrad_direct_applicable(d, nullptr))
+    return fhip_fast_conv_wgrad_direct(ctx, d, dy, x, dw, workspace);
   const WgradPlan p = make_wgrad_plan(d);
   FHIP_REQUIRE(ctx, p.ok, "conv wgrad: descriptor not supported by the MFMA path");
   FHIP_REQUIRE(ctx, ((uintptr_t)workspace & 255) == 0 && ((uintptr_t)x & 15) == 0 &&

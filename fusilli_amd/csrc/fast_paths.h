@@ -53,6 +53,15 @@ bool fhip_fast_conv_wgrad_applicable(const fhip_conv_desc *d,
 int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                          const void *x, void *dw, void *workspace);
 
+// Weight gradient of 3 x 3, padding-1, unit-stride convolutions straight from
+// X and DY (no operand copies): one MFMA kernel plus the sum of its partial
+// results; `*workspace_bytes` of 256-byte aligned workspace hold those.
+bool fhip_fast_conv_wgrad_direct_applicable(const fhip_conv_desc *d,
+                                            size_t *workspace_bytes);
+int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
+                                const void *dy, const void *x, void *dw,
+                                void *workspace);
+
 bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d);
 int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
                    const void *k, const void *v, void *o);

@@ -64,17 +64,19 @@ def test_gradient_and_batchnorm_queries_need_no_gpu():
         d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
     d.epilogue = capi.make_epilogue([])
     assert lib.fhip_conv_dgrad_supported(d) == 2  # forward MFMA kernel, mirrored filter
-    assert lib.fhip_conv_wgrad_supported(d) == 2  # batched MFMA GEMMs
+    assert lib.fhip_conv_wgrad_supported(d) == 2  # the kernel that reads X and DY in place
     n = ctypes.c_size_t(0)
     assert lib.fhip_conv_dgrad_workspace_size(d, ctypes.byref(n)) == 0
     assert n.value == 128 * 64 * 9 * 2
     assert lib.fhip_conv_wgrad_workspace_size(d, ctypes.byref(n)) == 0
-    assert n.value > 32 * 58 * 64 * (64 + 128) * 2  # padded X and DY grids
+    assert n.value == 256 * 9 * 1024 * 4  # 256 workgroups' partial sums, 36 KB each
     for i in range(2):
         d.stride[i] = 2
     d.y = capi.TensorDesc.make([32, 128, 28, 28], cl([32, 128, 28, 28]), capi.BFLOAT16)
     assert lib.fhip_conv_dgrad_supported(d) == 2  # DY spread over a zero grid
-    assert lib.fhip_conv_wgrad_supported(d) == 2  # B rows two pixels apart
+    assert lib.fhip_conv_wgrad_supported(d) == 2  # batched GEMMs, B rows two pixels apart
+    assert lib.fhip_conv_wgrad_workspace_size(d, ctypes.byref(n)) == 0
+    assert n.value > 32 * 58 * 64 * 64 * 2  # zero-padded copies of X and DY
     d.y = capi.TensorDesc.make([32, 128, 28, 27], cl([32, 128, 28, 27]), capi.BFLOAT16)
     assert lib.fhip_conv_dgrad_supported(d) == 0  # DY extent disagrees
 

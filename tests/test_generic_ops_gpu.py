@@ -371,6 +371,46 @@ def test_conv_wgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
     assert_close(dw.logical(), ref, dtype, f"wgrad {case}")
 
 
+@pytest.mark.parametrize("case", [
+    # [N, C, H, W], K: 3 x 3 filters, padding 1, unit strides, images of up to
+    # 56 columns, C and K multiples of 32 -- the kernel that reads X and DY in place
+    dict(x=[2, 64, 12, 12], k=128),     # small batch: image rows cut into chunks
+    dict(x=[1, 32, 5, 7], k=32),        # fewer rows than wavefronts
+    dict(x=[3, 32, 17, 56], k=64),      # widest row, rows not a multiple of 8
+    dict(x=[2, 96, 9, 33], k=32),       # three K-steps and a bit
+    dict(x=[5, 32, 1, 1], k=32),        # one pixel per image
+    dict(x=[70, 64, 10, 16], k=128),    # several images per workgroup, last group short
+    dict(x=[40, 32, 23, 48], k=32),     # whole K-steps only
+])
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_conv_wgrad_direct_kernel_vs_oracle(ctx, case, dtype, knobs):
+    xd, wd = case["x"], [case["k"], case["x"][1], 3, 3]
+    yd = [xd[0], case["k"], xd[2], xd[3]]
+    cl = oracle.channels_last_strides
+    x = HT.from_logical(rand(37, 0, xd), dtype, cl(xd))
+    dy = HT.from_logical(rand(37, 1, yd), dtype, cl(yd))
+    ref = oracle.conv_wgrad(dy.logical(), x.logical(), wd, [1, 1], [1, 1], [1, 1])
+    dw = run_conv_wgrad(ctx, dy, x, wd, [1, 1], [1, 1], [1, 1], dtype, tuned=True,
+                        w_dtype=capi.FLOAT)
+    assert_close(dw.logical(), ref, dtype, f"direct wgrad {case}")
+    # DW in the tensors' own dtype, filter laid out KCRS
+    dw = run_conv_wgrad(ctx, dy, x, wd, [1, 1], [1, 1], [1, 1], dtype, nhwc=False,
+                        tuned=True)
+    assert_close(dw.logical(), ref, dtype, f"direct wgrad {case}, KCRS")
+    # the workspace is only the partial sums: one 36 KB block per workgroup
+    d = conv_bwd_desc(x, HT.empty(wd, dtype, cl(wd)), dy, [1, 1], [1, 1], [1, 1])
+    assert ctx.conv_wgrad_workspace(d) % (9 * 16 * 64 * 4) == 0
+    # switched off, the same descriptor runs on the batched-GEMM path or the
+    # generic kernel and agrees
+    knobs(WGRAD_DIRECT="0")
+    assert ctx.conv_wgrad_workspace(d) % (9 * 16 * 64 * 4) != 0 or \
+        ctx.conv_wgrad_workspace(d) == 0
+    tuned = ctx.lib.fhip_conv_wgrad_supported(d) == 2
+    dw = run_conv_wgrad(ctx, dy, x, wd, [1, 1], [1, 1], [1, 1], dtype, tuned=tuned,
+                        w_dtype=capi.FLOAT)
+    assert_close(dw.logical(), ref, dtype, f"wgrad without the direct kernel {case}")
+
+
 def test_conv_wgrad_config3_shape_closed_form_and_oracle(ctx):
     # the weight gradient of benchmark config 3 (N32 C64 56x56, K128 3x3 pad 1).
     # All-ones: DW = N * (rows a tap sees) * (columns it sees) = 32 * {56, 55}^2.
