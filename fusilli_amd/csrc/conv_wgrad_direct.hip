@@ -31,6 +31,18 @@
 #include "fast_paths.h"
 #include "gemm_kernel.h"
 
+#ifndef WD_EXP
+#define WD_EXP 0 // timing experiments: 1 no MFMA, 2 no loads in the loop, 4 no LDS sum, 8 no fragment reads
+#endif
+
+#ifdef WD_PROFILE // experiment builds: cycle stamps of workgroup 0 replace its results
+#define WD_STAMP(i) st[i] = __builtin_amdgcn_s_memtime()
+#else
+#define WD_STAMP(i)                                                            \
+  do {                                                                         \
+  } while (0)
+#endif
+
 namespace {
 
 constexpr int kWdWaves = 8;
@@ -44,16 +56,19 @@ constexpr int kWdMaxW = 56;
 constexpr int kWdBlock = 9 * 16 * 64; // partial sums of one workgroup (floats)
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 struct WgDirectArgs {
   const char *x, *dy;
   float *part;
   int32_t N, H, W, C, K;
-  int32_t rpw;    // image rows per wavefront
-  int32_t chunks; // row chunks (8 * rpw rows) per image
+  int32_t rpw;    // image rows per pair of wavefronts (w, w + 4) that share a SIMD
+  int32_t rfirst; // of which wavefront w takes the first rfirst, w + 4 the rest
+  int32_t chunks; // row chunks (4 * rpw rows) per image
   int32_t ipw;    // images per workgroup
   int32_t nparts; // workgroups per (k, c) block
   int32_t ctypes; // C / 32
+  uint32_t magic_ctypes;
   uint32_t x_bytes, dy_bytes;
 };
 
@@ -63,6 +78,11 @@ __device__ __forceinline__ f32x16 wd_mfma(const u32x2 &a0, const u32x2 &a1,
                                           const f32x16 &c) {
   const u32x4 a = {a0.x, a0.y, a1.x, a1.y};
   const u32x4 b = {b0.x, b0.y, b1.x, b1.y};
+  if (WD_EXP & 1) {
+    f32x16 r = c;
+    asm volatile("" : "+v"(r) : "v"(a), "v"(b));
+    return r;
+  }
   if constexpr (KIND == GK_BF16)
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
         __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -79,6 +99,10 @@ __device__ __forceinline__ f32x16 wd_mfma(const u32x2 &a0, const u32x2 &a1,
 template <int OFFSET>
 __device__ __forceinline__ void wd_read_tr(u32x2 &dst, uint32_t addr) {
   static_assert(OFFSET >= 0 && OFFSET < 65536, "16-bit offset field");
+  if (WD_EXP & 8) {
+    asm volatile("" : "=v"(dst) : "v"(addr));
+    return;
+  }
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
                : "=v"(dst)
                : "v"(addr), "n"(OFFSET));
@@ -106,24 +130,33 @@ __global__ __launch_bounds__(kWdThreads)
 __attribute__((amdgpu_waves_per_eu(2, 2))) void
 conv_wgrad_direct_kernel(WgDirectArgs g) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+#ifdef WD_PROFILE
+  uint64_t st[8] = {};
+#endif
+  WD_STAMP(0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int l = threadIdx.x & 63;
   const int a_H = g.H, a_W = g.W, a_C = g.C, a_K = g.K, a_N = g.N;
-  const int a_rpw = g.rpw, a_chunks = g.chunks, a_ipw = g.ipw;
+  const int a_rpw = g.rpw, a_ipw = g.ipw;
 
-  // workgroup -> (k block, c block), images, row chunk
-  const int type = (int)(blockIdx.x / (unsigned)g.nparts);
-  const int part = (int)(blockIdx.x - (unsigned)type * (unsigned)g.nparts);
-  const int kb = type / g.ctypes, cb = type - kb * g.ctypes;
-  const int igroup = part / a_chunks, chunk = part - igroup * a_chunks;
+  // workgroup (x, y, z) -> row chunk, image group, (k block, c block)
+  const int chunk = (int)blockIdx.x, igroup = (int)blockIdx.y, type = (int)blockIdx.z;
+  const int kb = conv_div(type, g.ctypes, g.magic_ctypes), cb = type - kb * g.ctypes;
   const int n0 = igroup * a_ipw;
   const int n1 = n0 + a_ipw < a_N ? n0 + a_ipw : a_N;
-  const int p0 = (chunk * kWdWaves + wave) * a_rpw;
+  // rows: the pair (w, w + 4) of a SIMD shares a_rpw rows; the first of the
+  // pair, which the SIMD serves first, takes the larger part
+  const int second = wave >> 2;
+  const int p0 = (chunk * 4 + (wave & 3)) * a_rpw + (second ? g.rfirst : 0);
+  const int share = second ? a_rpw - g.rfirst : g.rfirst;
   int nrows = a_H - p0;
-  nrows = nrows < a_rpw ? nrows : a_rpw;
+  nrows = nrows < share ? nrows : share;
   nrows = nrows > 0 ? nrows : 0;
-  const int n_it = nrows > 0 ? nrows + 2 : 0;
+  // Step t of a wavefront's walk brings DY row p0 - 1 + t into registers and,
+  // from t = 2 on, multiplies X row p0 + t - 2 with the three DY rows held:
+  // the newest is filter row 0, the oldest filter row 2.
+  const int n_st = nrows > 0 ? nrows + 2 : 0;
 
   // ---- LDS-DMA lane offsets (relative to a row's first byte) --------------------
   // instruction j fills pixel slots 16 j .. 16 j + 15 of a row slice: lane d
@@ -161,59 +194,78 @@ conv_wgrad_direct_kernel(WgDirectArgs g) {
     for (int i = 0; i < 16; ++i)
       acc[t][i] = 0.f;
 
-  for (int n = n0; n < n1; ++n) {
-    // group gi of loads: X row p0 - 1 + gi into X slot xs, DY row p0 + gi into
-    // DY slot gi % 2; rows outside the image (or this wavefront's share of DY)
-    // arrive as zeros.  Always eight instructions, so the waits can count.
-    auto issue = [&](int gi, int xs) __attribute__((always_inline)) {
-      const int rho = p0 - 1 + gi;
-      const bool xok = (unsigned)rho < (unsigned)a_H && gi < n_it;
-      const __amdgpu_buffer_rsrc_t rsx = xok ? rx : rnone;
-      const int xoff = xok ? ((n * a_H + rho) * a_W) * a_C * 2 : 0;
-      const uint32_t xdst = wbase + (uint32_t)xs * kWdRow;
+  for (int n = n0; n < n1 && n_st > 0; ++n) {
+    // Loads of step t: four instructions each, so that the waits can count.
+    // Rows outside the image arrive as zeros (DY rows of the neighbouring
+    // wavefronts' shares are real: they are this share's halo).
+    auto issue_y = [&](int t) __attribute__((always_inline)) {
+      const int row = p0 - 1 + t;
+      const bool ok = t < n_st && (unsigned)row < (unsigned)a_H;
+      const __amdgpu_buffer_rsrc_t rs = ok ? ry : rnone;
+      const int off = ok ? ((n * a_H + row) * a_W) * a_K * 2 : 0;
+      const uint32_t dst = wbase + (uint32_t)(kWdXSlots + (t & 1)) * kWdRow;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsx, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(xdst + j * 1024u),
-            16, (int)xrel[j], xoff, 0, 0);
-      const bool yok = gi < nrows;
-      const __amdgpu_buffer_rsrc_t rsy = yok ? ry : rnone;
-      const int yoff = yok ? ((n * a_H + p0 + gi) * a_W) * a_K * 2 : 0;
-      const uint32_t ydst = wbase + (uint32_t)(kWdXSlots + (gi & 1)) * kWdRow;
+            rs, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst + j * 1024u),
+            16, (int)yrel[j], off, 0, 0);
+    };
+    auto issue_x = [&](int t, int xs) __attribute__((always_inline)) {
+      const int row = p0 + t - 2;
+      const bool ok = t < n_st;
+      const __amdgpu_buffer_rsrc_t rs = ok ? rx : rnone;
+      const int off = ok ? ((n * a_H + row) * a_W) * a_C * 2 : 0;
+      const uint32_t dst = wbase + (uint32_t)xs * kWdRow;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsy, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(ydst + j * 1024u),
-            16, (int)yrel[j], yoff, 0, 0);
+            rs, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst + j * 1024u),
+            16, (int)xrel[j], off, 0, 0);
     };
 
-    // DY fragments of three rows: dyf[j] holds row it with it % 3 == j
+    // DY fragments of three rows: dyf[j] holds the row of step t, t % 3 == j
     u32x2 dyf[3][4][2];
-#pragma unroll
-    for (int j = 0; j < 3; ++j)
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-        dyf[j][ks][0] = dyf[j][ks][1] = u32x2{0u, 0u};
 
-    if (n_it > 0) {
-      issue(0, 0);
-      issue(1, 1);
-    }
+    WD_STAMP(1);
+    issue_y(0);
+    issue_y(1);
+    issue_x(2, 0);
+    WD_STAMP(2);
 
-    // iteration it (it % 3 == J): X row p0 - 1 + it against DY rows it, it - 1,
-    // it - 2 of this wavefront's share
-    auto body = [&](auto jc, int it) __attribute__((always_inline)) {
+    auto read_y = [&](auto jc, int t) __attribute__((always_inline)) {
       constexpr int J = decltype(jc)::value;
-      constexpr int J1 = (J + 2) % 3, J2 = (J + 1) % 3;
-      // group `it` has landed when only the eight loads of group it + 1 are out
-      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(8));
-      const uint32_t ya = ybase + (uint32_t)(it & 1) * kWdRow;
+      const uint32_t ya = ybase + (uint32_t)(t & 1) * kWdRow;
       gemm_static_for<4>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
         wd_read_tr<ks * 1024>(dyf[J][ks][0], ya);
         wd_read_tr<ks * 1024 + 256>(dyf[J][ks][1], ya);
       });
-      const uint32_t xa = xbase + (uint32_t)J * kWdRow;
+    };
+    // steps 0 and 1: a DY row into registers, its slot refilled.  The order of
+    // all loads is Y0 Y1 X2 | Y2 X3 | Y3 | X4 Y4 | X5 Y5 ...: from step 2 on a
+    // step finds exactly eight loads issued after the ones it needs.
+    auto light = [&](auto jc, auto vmc, int t) __attribute__((always_inline)) {
+      if (!(WD_EXP & 2))
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(decltype(vmc)::value));
+      read_y(jc, t);
+      wd_wait_lgkm<0>();
+      if (!(WD_EXP & 2)) {
+        issue_y(t + 2);
+        if (t == 0)
+          issue_x(3, 1);
+      }
+    };
+    // step t >= 2 (t % 3 == J): X row p0 + t - 2 against the three DY rows
+    auto full = [&](auto jc, auto vmc, int t) __attribute__((always_inline)) {
+      constexpr int J = decltype(jc)::value;
+      constexpr int J1 = (J + 2) % 3, J2 = (J + 1) % 3;
+      constexpr int XS = (J + 1) % 3; // (t - 2) % 3
+      // the loads of this step have landed when only the eight issued after
+      // them are out
+      if (!(WD_EXP & 2))
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(decltype(vmc)::value));
+      read_y(jc, t);
+      const uint32_t xa = xbase + (uint32_t)XS * kWdRow;
       u32x2 xf[2][3][2];
       auto read_x = [&](auto kc) __attribute__((always_inline)) {
         constexpr int ks = decltype(kc)::value;
@@ -224,13 +276,13 @@ conv_wgrad_direct_kernel(WgDirectArgs g) {
         });
       };
       read_x(std::integral_constant<int, 0>{});
-      // the DY row is in registers: its slot (and the X slot read last
-      // iteration) can be refilled
+      // the DY row is in registers: its slot, and the X slot read in the
+      // step before, can be refilled
       wd_wait_lgkm<6>();
-      issue(it + 2, (J + 2) % 3);
-      // Every MFMA runs: rows that do not exist (outside the image, or DY
-      // rows of another wavefront's share) were loaded as zeros, so the
-      // accumulators are updated in place by straight-line code.
+      if (!(WD_EXP & 2)) {
+        issue_x(t + 2, J);
+        issue_y(t + 2);
+      }
       gemm_static_for<4>([&](auto kc) {
         constexpr int ks = decltype(kc)::value;
         if constexpr (ks + 1 < 4) {
@@ -272,49 +324,81 @@ conv_wgrad_direct_kernel(WgDirectArgs g) {
       });
     };
 
-    int it = 0;
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using V8 = std::integral_constant<int, 8>;
+    using V12 = std::integral_constant<int, 12>;
+    light(I0{}, V8{}, 0);
+    light(I1{}, V12{}, 1);
+    int t = 2;
     while (true) {
-      if (it >= n_it)
+      if (t >= n_st)
         break;
-      body(std::integral_constant<int, 0>{}, it);
-      ++it;
-      if (it >= n_it)
+      full(I2{}, V8{}, t);
+      ++t;
+      if (t >= n_st)
         break;
-      body(std::integral_constant<int, 1>{}, it);
-      ++it;
-      if (it >= n_it)
+      full(I0{}, V8{}, t);
+      ++t;
+      if (t >= n_st)
         break;
-      body(std::integral_constant<int, 2>{}, it);
-      ++it;
+      full(I1{}, V8{}, t);
+      ++t;
     }
-    // the two groups still in flight land before the next image reuses the slots
+    // the loads still in flight land before the next image reuses the slots
     __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
   }
 
-  // ---- sum of the eight wavefronts through LDS, one filter row at a time ------
+  // ---- sum of the eight wavefronts through LDS, half of the block at a time ---
+  WD_STAMP(4);
   __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
   __syncthreads();
-  float *scr = (float *)smem; // [wavefront][48 = 3 taps x 16 registers][64 lanes]
-  float *dst = g.part + (size_t)blockIdx.x * kWdBlock;
-  gemm_static_for<3>([&](auto rc) {
-    constexpr int r = decltype(rc)::value;
+  WD_STAMP(5);
+  const unsigned wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  f32x4 *dst4 = (f32x4 *)(g.part + (size_t)wg * kWdBlock);
+  if (WD_EXP & 4) {
+    float v = 0.f;
 #pragma unroll
-    for (int s = 0; s < 3; ++s)
+    for (int t = 0; t < 9; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i)
-        scr[(wave * 48 + s * 16 + i) * 64 + l] = acc[r * 3 + s][i];
+        v += acc[t][i];
+    ((float *)dst4)[wave * 64 + l] = v;
+    return;
+  }
+  // entry e = 4 * tap + j is registers 4 j .. 4 j + 3 of a tap's accumulator:
+  // one 16-byte LDS access per lane
+  f32x4 *scr4 = (f32x4 *)smem; // [wavefront][18 entries][64 lanes]
+  constexpr int kHalf = 18 * 64;
+  gemm_static_for<2>([&](auto hc) {
+    constexpr int h = decltype(hc)::value;
+    gemm_static_for<18>([&](auto kc) {
+      constexpr int k = decltype(kc)::value;
+      constexpr int e = 18 * h + k, tap = e / 4, j = e % 4;
+      const f32x4 v = {acc[tap][4 * j], acc[tap][4 * j + 1], acc[tap][4 * j + 2],
+                       acc[tap][4 * j + 3]};
+      scr4[(wave * 18 + k) * 64 + l] = v;
+    });
     __syncthreads();
+    for (int f = (int)threadIdx.x; f < kHalf; f += kWdThreads) {
+      f32x4 sum = scr4[f];
 #pragma unroll
-    for (int e6 = 0; e6 < 6; ++e6) {
-      const int e = wave * 6 + e6;
-      float sum = 0.f;
-#pragma unroll
-      for (int v = 0; v < kWdWaves; ++v)
-        sum += scr[(v * 48 + e) * 64 + l];
-      dst[(r * 48 + e) * 64 + l] = sum;
+      for (int v = 1; v < kWdWaves; ++v) {
+        const f32x4 o = scr4[v * kHalf + f];
+        sum[0] += o[0], sum[1] += o[1], sum[2] += o[2], sum[3] += o[3];
+      }
+      dst4[h * kHalf + f] = sum;
     }
     __syncthreads();
   });
+#ifdef WD_PROFILE
+  __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+  WD_STAMP(6);
+  if (wg == 0 && l == 0)
+    for (int i = 0; i < 8; ++i)
+      ((uint64_t *)dst4)[wave * 8 + i] = st[i];
+#endif
 }
 
 struct WgDirectSumArgs {
@@ -323,33 +407,41 @@ struct WgDirectSumArgs {
   int32_t dt;
 };
 
-// DW[k][c][r][s] = sum over the workgroups of a (k, c) block of their partial
-// sums, in workgroup order; one thread per output element.
-__global__ void conv_wgrad_direct_sum_kernel(WgDirectSumArgs a, const float *part,
-                                             void *dw, int64_t total) {
-  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (lin >= total)
-    return;
-  const int lane = (int)(lin & 63), i = (int)((lin >> 6) & 15);
-  const int tap = (int)((lin >> 10) % 9);
+// DW[k][c][r][s] = sum of the partial results of a (k, c) block's workgroups.
+// 64 outputs per workgroup of 256 threads: thread (o, j) adds the partials
+// j, j + 4, ... (all loads independent), the four sums are added in order.
+// A partial block is [entry e = 4 * tap + i / 4][lane][i % 4].
+__global__ __launch_bounds__(256) void
+conv_wgrad_direct_sum_kernel(WgDirectSumArgs a, const float *part, void *dw) {
+  __shared__ float red[4][64];
+  const int o = threadIdx.x & 63, j = threadIdx.x >> 6;
+  const int64_t lin = (int64_t)blockIdx.x * 64 + o;
   const int type = (int)(lin / kWdBlock);
-  const float *src = part + (int64_t)type * a.nparts * kWdBlock + lin % kWdBlock;
+  const int within = (int)(lin - (int64_t)type * kWdBlock);
+  const float *src = part + (int64_t)type * a.nparts * kWdBlock + within;
   float acc = 0.f;
-#pragma unroll 8 // independent loads: several in flight
-  for (int p = 0; p < a.nparts; ++p)
+#pragma unroll 8
+  for (int p = j; p < a.nparts; p += 4)
     acc += src[(int64_t)p * kWdBlock];
+  red[j][o] = acc;
+  __syncthreads();
+  if (j != 0)
+    return;
+  acc = ((red[0][o] + red[1][o]) + red[2][o]) + red[3][o];
+  const int comp = within & 3, lane = (within >> 2) & 63, e = within >> 8;
+  const int tap = e >> 2, i = 4 * (e & 3) + comp;
   const int kb = type / a.ctypes, cb = type - kb * a.ctypes;
   const int64_t k = kb * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
   const int64_t c = cb * 32 + (lane & 31);
-  const int r = tap / 3, s = tap - r * 3;
-  fhip_store<float>(dw, a.dt, k * a.sk + c * a.sc + r * a.sr + s * a.ss, acc);
+  const int r = tap / 3, sx = tap - r * 3;
+  fhip_store<float>(dw, a.dt, k * a.sk + c * a.sc + r * a.sr + sx * a.ss, acc);
 }
 
 struct WgDirectPlan {
   bool ok = false;
   int kind = GK_BF16;
   WgDirectArgs a{};
-  int grid = 0;
+  dim3 grid;
   size_t part_bytes = 0;
 };
 
@@ -371,7 +463,8 @@ bool wd_channels_last(const fhip_tensor_desc &t) {
 
 WgDirectPlan make_wd_plan(const fhip_conv_desc *d, int num_cus) {
   WgDirectPlan p;
-  if (fhip_knobs().wgrad_direct == 0)
+  const FhipKnobs &knobs = fhip_knobs();
+  if (knobs.wgrad_direct == 0)
     return p;
   if (d->spatial_rank != 2)
     return p;
@@ -419,19 +512,27 @@ WgDirectPlan make_wd_plan(const fhip_conv_desc *d, int num_cus) {
     ipw = types * N / cus;
     ipw = ipw < 1 ? 1 : ipw;
   }
-  const int64_t rpw = (H + kWdWaves * chunks - 1) / (kWdWaves * chunks);
-  chunks = (H + kWdWaves * rpw - 1) / (kWdWaves * rpw);
+  // rows per pair of wavefronts
+  const int64_t rpw = (H + 4 * chunks - 1) / (4 * chunks);
+  chunks = (H + 4 * rpw - 1) / (4 * rpw);
+  int64_t rfirst = (rpw + 1) / 2;
+  if (knobs.wgrad_first_rows > 0 && knobs.wgrad_first_rows <= rpw)
+    rfirst = knobs.wgrad_first_rows;
   const int64_t igroups = (N + ipw - 1) / ipw;
   const int64_t nparts = igroups * chunks;
   if (types * nparts >= (1ll << 31) / kWdBlock)
     return p;
   WgDirectArgs &a = p.a;
   a.N = (int32_t)N, a.H = (int32_t)H, a.W = (int32_t)W, a.C = (int32_t)C, a.K = (int32_t)K;
-  a.rpw = (int32_t)rpw, a.chunks = (int32_t)chunks, a.ipw = (int32_t)ipw;
+  a.rpw = (int32_t)rpw, a.rfirst = (int32_t)rfirst;
+  a.chunks = (int32_t)chunks, a.ipw = (int32_t)ipw;
   a.nparts = (int32_t)nparts, a.ctypes = (int32_t)(C / 32);
+  a.magic_ctypes = conv_magic(a.ctypes);
   a.x_bytes = (uint32_t)x_bytes, a.dy_bytes = (uint32_t)dy_bytes;
-  p.grid = (int)(types * nparts);
-  p.part_bytes = (size_t)p.grid * kWdBlock * sizeof(float);
+  if (chunks > 65535 || igroups > 65535 || types > 65535)
+    return p;
+  p.grid = dim3((unsigned)chunks, (unsigned)igroups, (unsigned)types);
+  p.part_bytes = (size_t)(types * nparts) * kWdBlock * sizeof(float);
   p.ok = true;
   return p;
 }
@@ -445,8 +546,7 @@ template <int KIND> int wd_launch(fhip_ctx *ctx, const WgDirectPlan &p) {
                             hipFuncAttributeMaxDynamicSharedMemorySize, kWdLds));
     configured.mark(ctx->device);
   }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)p.grid), dim3(kWdThreads), kWdLds,
-                     ctx->stream, p.a);
+  hipLaunchKernelGGL(kernel, p.grid, dim3(kWdThreads), kWdLds, ctx->stream, p.a);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }
@@ -484,9 +584,8 @@ int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
   s.ss = d->w.dim[3] == 1 ? 0 : d->w.stride[3];
   s.dt = d->w.dtype;
   const int64_t total = (int64_t)(p.a.C / 32) * (p.a.K / 32) * kWdBlock;
-  hipLaunchKernelGGL(conv_wgrad_direct_sum_kernel,
-                     dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                     ctx->stream, s, (const float *)p.a.part, dw, total);
+  hipLaunchKernelGGL(conv_wgrad_direct_sum_kernel, dim3((unsigned)(total / 64)),
+                     dim3(256), 0, ctx->stream, s, (const float *)p.a.part, dw);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }
