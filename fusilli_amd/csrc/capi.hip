@@ -31,8 +31,6 @@ FhipKnobs parse_knobs() {
     k.conv_rows = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_WGRAD_DIRECT"))
     k.wgrad_direct = atoi(e);
-  if (const char *e = getenv("FUSILLI_HIP_WGRAD_FIRST_ROWS"))
-    k.wgrad_first_rows = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_GEMM_TILE"))
     if (sscanf(e, "%d,%d", &k.gemm_tile_bm, &k.gemm_tile_bn) != 2)
       k.gemm_tile_bm = k.gemm_tile_bn = 0;

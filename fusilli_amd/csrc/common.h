@@ -40,7 +40,6 @@ struct FhipKnobs {
   int conv_rows = -1;               // FUSILLI_HIP_CONV_ROWS (-1: unset)
   int gemm_tile_bm = 0, gemm_tile_bn = 0; // FUSILLI_HIP_GEMM_TILE "bm,bn"
   int wgrad_direct = -1;            // FUSILLI_HIP_WGRAD_DIRECT (-1: unset, 0: off)
-  int wgrad_first_rows = 0;         // FUSILLI_HIP_WGRAD_FIRST_ROWS
 };
 const FhipKnobs &fhip_knobs();
 

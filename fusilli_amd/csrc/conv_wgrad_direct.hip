@@ -515,9 +515,7 @@ WgDirectPlan make_wd_plan(const fhip_conv_desc *d, int num_cus) {
   // rows per pair of wavefronts
   const int64_t rpw = (H + 4 * chunks - 1) / (4 * chunks);
   chunks = (H + 4 * rpw - 1) / (4 * rpw);
-  int64_t rfirst = (rpw + 1) / 2;
-  if (knobs.wgrad_first_rows > 0 && knobs.wgrad_first_rows <= rpw)
-    rfirst = knobs.wgrad_first_rows;
+  const int64_t rfirst = (rpw + 1) / 2;
   const int64_t igroups = (N + ipw - 1) / ipw;
   const int64_t nparts = igroups * chunks;
   if (types * nparts >= (1ll << 31) / kWdBlock)
