@@ -73,6 +73,23 @@ int fhip_fail(fhip_ctx *ctx, const char *fmt, ...) {
   return 1;
 }
 
+int fhip_ctx_scratch(fhip_ctx *ctx, size_t bytes, void **out) {
+  if (bytes > ctx->scratch_bytes) {
+    FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+    if (ctx->scratch) {
+      FHIP_HIP_CHECK(ctx, hipStreamSynchronize(ctx->stream));
+      FHIP_HIP_CHECK(ctx, hipFree(ctx->scratch));
+      ctx->scratch = nullptr;
+      ctx->scratch_bytes = 0;
+    }
+    const size_t want = bytes < (64u << 10) ? (64u << 10) : bytes;
+    FHIP_HIP_CHECK(ctx, hipMalloc(&ctx->scratch, want));
+    ctx->scratch_bytes = want;
+  }
+  *out = ctx->scratch;
+  return 0;
+}
+
 bool fhip_check_desc(fhip_ctx *ctx, const fhip_tensor_desc &t,
                      const char *what) {
   if (t.rank < 1 || t.rank > FHIP_MAX_RANK) {
@@ -235,6 +252,8 @@ int fhip_ctx_destroy(fhip_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
   }
+  if (ctx->scratch)
+    (void)hipFree(ctx->scratch);
   delete ctx;
   return 0;
 }

@@ -24,8 +24,15 @@ struct fhip_ctx {
   int num_cus = 0;
   // this device's copy of the data gradient's static scratch array
   void *dgrad_static_scratch = nullptr;
+  // device memory for kernels' partial results, owned by the context (one
+  // stream: its users are ordered); grown on demand, freed with the context
+  void *scratch = nullptr;
+  size_t scratch_bytes = 0;
   std::string err;
 };
+// At least `bytes` of 256-byte aligned scratch in *out.  Growing it allocates
+// (after the stream has drained): not for callers under graph capture.
+int fhip_ctx_scratch(fhip_ctx *ctx, size_t bytes, void **out);
 
 // Tuning / test knobs from the environment, parsed once per process (and again
 // on fhip_tuning_reload) instead of on every launch.

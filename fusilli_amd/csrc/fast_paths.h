@@ -71,6 +71,13 @@ int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
                    const void *scale, const void *bias, const DevEpilogue &epi,
                    void *out, void *mean, void *inv_variance);
 
+// Rows too long for the register-resident kernels (rownorm_long.hip); the
+// layout conditions are the caller's (rownorm.hip).
+bool fhip_norm_long_applicable(const fhip_norm_desc *d);
+int fhip_norm_long(fhip_ctx *ctx, const fhip_norm_desc *d, int64_t inner,
+                   const void *x, const void *scale, const void *bias, void *out,
+                   void *mean, void *inv_variance);
+
 bool fhip_fast_reduce_applicable(const fhip_reduce_desc *d);
 int fhip_fast_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
                      void *y);

@@ -107,8 +107,10 @@ bool fhip_fast_norm_applicable(const fhip_norm_desc *d) {
   const int vec = 16 / fhip_dtype_size(x.dtype);
   if (lay.inner % vec != 0)
     return false;
+  // rows that do not fit the register-resident kernels go to the long-row
+  // kernels (no fused pointwise chain there)
   int chunks, wpr;
-  if (!pick_shape(lay.inner, vec, &chunks, &wpr))
+  if (!pick_shape(lay.inner, vec, &chunks, &wpr) && !fhip_norm_long_applicable(d))
     return false;
   const int64_t xrs = x.dim[0] > 1 ? x.stride[0] : lay.inner;
   const int64_t ors = d->out.dim[0] > 1 ? d->out.stride[0] : lay.inner;
@@ -149,10 +151,9 @@ int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
   const InnerLayout lay = inner_layout(d->x);
   const int vec = 16 / fhip_dtype_size(d->x.dtype);
   int chunks = 1, wpr = 1;
-  FHIP_REQUIRE(ctx, pick_shape(lay.inner, vec, &chunks, &wpr),
-               "rownorm: row of %lld elements exceeds the register-resident "
-               "kernel",
-               (long long)lay.inner);
+  if (!pick_shape(lay.inner, vec, &chunks, &wpr))
+    return fhip_norm_long(ctx, d, lay.inner, x, scale, bias, out, mean,
+                          inv_variance);
   RowNormArgs g{};
   g.x = x;
   g.scale = scale;

@@ -169,6 +169,56 @@ def test_layernorm_vs_oracle(ctx, dtype, train):
         assert_close(res[2].logical(), rstd.reshape(-1), capi.FLOAT, "rstd")
 
 
+@pytest.mark.parametrize("case", [
+    # rows too long for the register-resident kernels (more than 16384 16-byte
+    # chunks): segments of a row on many workgroups, two passes
+    dict(dims=[3, 8, 64, 130], dtype=capi.FLOAT, nhwc=False, affine=False),
+    dict(dims=[3, 8, 64, 130], dtype=capi.FLOAT, nhwc=True, affine=True),
+    dict(dims=[2, 16, 96, 100], dtype=capi.BFLOAT16, nhwc=True, affine=True),
+    dict(dims=[5, 16, 96, 100], dtype=capi.HALF, nhwc=False, affine=True),
+    dict(dims=[1, 140000], dtype=capi.HALF, nhwc=False, affine=False),
+    # the reference's benchmark shapes (benchmarks/CMakeLists.txt, layernorm)
+    dict(dims=[16, 128, 64, 32], dtype=capi.FLOAT, nhwc=False, affine=False),
+    dict(dims=[16, 128, 64, 32], dtype=capi.BFLOAT16, nhwc=True, affine=True),
+])
+@pytest.mark.parametrize("train", [False, True])
+def test_layernorm_long_rows_vs_oracle(ctx, case, train):
+    dims, dtype = case["dims"], case["dtype"]
+    lay = oracle.channels_last_strides if case["nhwc"] else (lambda d: None)
+    x = HT.from_logical(rand(23, 0, dims, mean=3.0, std=2.0), dtype, lay(dims))
+    s = b = None
+    if case["affine"]:
+        sd = [1] + dims[1:]
+        s = HT.from_logical(rand(23, 1, sd, mean=1.0, std=0.1), dtype, lay(sd))
+        b = HT.from_logical(rand(23, 2, sd), dtype, lay(sd))
+    res = run_norm(ctx, x, s, b, eps=1e-5, layernorm=True, stats=train,
+                   expect_path=2)
+    y, mean, rstd = oracle.layernorm(
+        x.logical(), None if s is None else s.logical(),
+        None if b is None else b.logical(), 1e-5)
+    out = res[0] if train else res
+    assert_close(out.logical(), y, dtype, f"long-row layernorm {case}")
+    if train:
+        assert_close(res[1].logical(), mean.reshape(-1), capi.FLOAT, "mean")
+        assert_close(res[2].logical(), rstd.reshape(-1), capi.FLOAT, "rstd")
+
+
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.FLOAT])
+def test_rmsnorm_long_rows_vs_oracle(ctx, dtype):
+    rows, cols = 3, 150016
+    x = HT.from_logical(rand(24, 0, [rows, cols]), dtype)
+    s = HT.from_logical(rand(24, 1, [1, cols], mean=1.0, std=0.02), dtype)
+    out = run_norm(ctx, x, s, None, eps=1e-6, expect_path=2)
+    assert_close(out.logical(), oracle.rmsnorm(x.logical(), s.logical(), 1e-6),
+                 dtype, "long-row rmsnorm")
+    # a fused pointwise chain on such rows stays on the generic kernel
+    out = run_norm(ctx, x, s, None, eps=1e-6, expect_path=1,
+                   epilogue=[capi.epilogue_op(capi.PW["MUL"], dtype, scalar=0.5)])
+    assert_close(out.logical(),
+                 oracle.rmsnorm(x.logical(), s.logical(), 1e-6) * 0.5, dtype,
+                 "long-row rmsnorm with a fused MUL", rtol=2e-2 if dtype == capi.BFLOAT16 else None)
+
+
 def test_layernorm_reference_two_value_pattern(ctx):
     # samples/layernorm/layernorm_utils.h:25-82: x0 = 2b, x1 = 2b+2 =>
     # y = scale*(-/+ 1/sqrt(1+eps)) + bias, mean = 2b+1, rstd = 1/sqrt(1+eps).
