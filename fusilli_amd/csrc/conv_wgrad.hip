@@ -27,6 +27,7 @@ namespace {
 struct WgradPlan {
   bool ok = false;
   int64_t N = 0, H = 0, W = 0, C = 0, K = 0, P = 0, Q = 0, R = 0, S = 0;
+  int64_t Kp = 0; // channels of the padded DY grid: K, or 128 for narrower outputs
   int64_t pad_h = 0, pad_w = 0, dil_h = 1;
   int64_t rows = 0, pitch = 0, pix = 0; // padded grid
   int64_t split = 1; // GEMM batches per image (more workgroups, shorter K)
@@ -78,6 +79,8 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
   // the padding copies move whole 16-byte chunks of a pixel's channels
   if (p.C % 8 != 0 || p.K % 8 != 0)
     return p;
+  // the GEMM's tiles want at least 128 rows: narrower gradients are zero-padded
+  p.Kp = p.K < 128 ? 128 : p.K;
   p.P = d->y.dim[2], p.Q = d->y.dim[3];
   p.pad_h = d->padding[0], p.pad_w = d->padding[1], p.dil_h = d->dilation[0];
   // Strides: output pixel (p, q) reads input pixel (p * str + r * dil, q * str
@@ -93,7 +96,7 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
   // guard behind the last image: the furthest tap of the last pixel
   const int64_t guard = (p.R - 1) * p.dil_h * p.pitch * p.C + p.S * p.C;
   p.xp_bytes = wg_align((size_t)(p.N * p.pix * p.C + guard) * 2);
-  p.dyp_bytes = wg_align((size_t)(p.N * p.pix_y * p.K) * 2);
+  p.dyp_bytes = wg_align((size_t)(p.N * p.pix_y * p.Kp) * 2);
   // An image's pixels are cut into `split` equal runs of whole 64-pixel
   // slices, each a batch entry of its own: the largest cut that keeps at
   // least 8 slices per run and at most ~1024 workgroups per launch.
@@ -105,7 +108,7 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
           p.N * f * col_tiles * row_tiles <= 1024)
         p.split = f;
   }
-  p.part_bytes = wg_align((size_t)(p.R * p.N * p.split * p.K * p.S * p.C) * 4);
+  p.part_bytes = wg_align((size_t)(p.R * p.N * p.split * p.Kp * p.S * p.C) * 4);
   if (p.xp_bytes >= (1ull << 32) || p.dyp_bytes >= (1ull << 32))
     return p;
   fhip_matmul_desc &m = p.mm;
@@ -118,9 +121,9 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
     t.stride[0] = s0, t.stride[1] = s1, t.stride[2] = s2;
   };
   const int64_t nb = p.N * p.split, run = p.pix_y / p.split;
-  set(m.a, dt, nb, p.K, run, run * p.K, 1, p.K);
+  set(m.a, dt, nb, p.Kp, run, run * p.Kp, 1, p.Kp);
   set(m.b, dt, nb, run, p.S * p.C, p.str * run * p.C, p.str * p.C, 1);
-  set(m.c, FHIP_FLOAT, nb, p.K, p.S * p.C, p.K * p.S * p.C, p.S * p.C, 1);
+  set(m.c, FHIP_FLOAT, nb, p.Kp, p.S * p.C, p.Kp * p.S * p.C, p.S * p.C, 1);
   m.out = m.c;
   m.out_dtype = FHIP_FLOAT;
   if (!fhip_fast_matmul_applicable(&m))
@@ -131,6 +134,7 @@ WgradPlan make_wgrad_plan(const fhip_conv_desc *d) {
 
 struct PadArgs {
   int64_t N, rows, pitch, ch;  // destination grid, channels per pixel
+  int64_t src_ch;              // channels per source pixel (<= ch: the rest is zero)
   int64_t h, w;                // source extent
   int64_t off_h, off_w;        // destination position of source pixel (0, 0)
   int64_t total;               // 16-byte chunks of the destination
@@ -151,13 +155,15 @@ __global__ void conv_pad_grid_kernel(PadArgs a, const uint4 *src, uint4 *dst) {
   const int64_t n = pixel / a.rows;
   const int64_t sr = row - a.off_h, sc = col - a.off_w;
   uint4 v = make_uint4(0, 0, 0, 0);
-  if (n < a.N && sr >= 0 && sr < a.h && sc >= 0 && sc < a.w)
-    v = src[((n * a.h + sr) * a.w + sc) * cpp + chunk];
+  const int64_t scpp = a.src_ch / 8;
+  if (n < a.N && sr >= 0 && sr < a.h && sc >= 0 && sc < a.w && chunk < scpp)
+    v = src[((n * a.h + sr) * a.w + sc) * scpp + chunk];
   dst[lin] = v;
 }
 
 struct WgradSumArgs {
   int64_t N, K, R, S, C;
+  int64_t Kp; // rows of a partial result (K, or 128 for narrower gradients)
   int64_t sk, sc, sr, ss; // element strides of DW [K, C, R, S]
   int32_t dt;
 };
@@ -173,11 +179,11 @@ __global__ void conv_wgrad_sum_kernel(WgradSumArgs a, const float *part,
   int64_t rem = lin / sc;
   const int64_t k = rem % a.K;
   const int64_t r = rem / a.K;
-  const float *src = part + (r * a.N * a.K + k) * sc + j;
+  const float *src = part + (r * a.N * a.Kp + k) * sc + j;
   float acc = 0.f;
 #pragma unroll 8 // independent loads: several in flight
   for (int64_t n = 0; n < a.N; ++n)
-    acc += src[n * a.K * sc];
+    acc += src[n * a.Kp * sc];
   const int64_t s = j / a.C, c = j - s * a.C;
   fhip_store<float>(dw, a.dt, k * a.sk + c * a.sc + r * a.sr + s * a.ss, acc);
 }
@@ -209,12 +215,12 @@ int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   // X into its padded grid (the guard behind the last image included: the
   // grid is extended by whole zero images' worth of chunks up to the buffer's
   // end), DY into the top-left corner of the same grid
-  PadArgs ax{p.N, p.rows, p.pitch, p.C, p.H, p.W, p.pad_h, p.pad_w,
+  PadArgs ax{p.N, p.rows, p.pitch, p.C, p.C, p.H, p.W, p.pad_h, p.pad_w,
              (int64_t)(p.xp_bytes / 16)};
   hipLaunchKernelGGL(conv_pad_grid_kernel, dim3((unsigned)((ax.total + 255) / 256)),
                      dim3(256), 0, ctx->stream, ax, (const uint4 *)x, (uint4 *)xp);
-  PadArgs ay{p.N, p.rows_y, p.pitch, p.K, p.P, p.Q, 0, 0,
-             (int64_t)(p.N * p.pix_y * p.K * 2 / 16)};
+  PadArgs ay{p.N, p.rows_y, p.pitch, p.Kp, p.K, p.P, p.Q, 0, 0,
+             (int64_t)(p.N * p.pix_y * p.Kp * 2 / 16)};
   hipLaunchKernelGGL(conv_pad_grid_kernel, dim3((unsigned)((ay.total + 255) / 256)),
                      dim3(256), 0, ctx->stream, ay, (const uint4 *)dy, (uint4 *)dyp);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
@@ -223,10 +229,11 @@ int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   // row of pixels and the output by one block of partial results
   if (fhip_fast_matmul_outer(ctx, &p.mm, dyp, xp, epi, part, (int)p.R, 0,
                              p.dil_h * p.pitch * p.C,
-                             p.N * p.split * p.K * p.S * p.C) != 0)
+                             p.N * p.split * p.Kp * p.S * p.C) != 0)
     return 1;
   WgradSumArgs as;
   as.N = p.N * p.split, as.K = p.K, as.R = p.R, as.S = p.S, as.C = p.C;
+  as.Kp = p.Kp;
   as.sk = d->w.dim[0] == 1 ? 0 : d->w.stride[0];
   as.sc = d->w.dim[1] == 1 ? 0 : d->w.stride[1];
   as.sr = d->w.dim[2] == 1 ? 0 : d->w.stride[2];

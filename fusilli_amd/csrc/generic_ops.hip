@@ -429,9 +429,13 @@ __global__ void generic_conv_dgrad_kernel(ConvBwdArgs g, const void *dy,
 // and 64 filter channels: lane = channel (channels-last X is read in
 // contiguous runs, the DY value is the same for the whole wavefront), the four
 // wavefronts split the pixels and their sums meet in LDS.  The pixel
-// decomposition is wavefront-uniform.
+// decomposition is wavefront-uniform.  Filters are small and batches large:
+// with gridDim.z > 1 the pixels are cut into that many runs, one workgroup
+// each, whose sums go to `partial` [run][k][tap][fc] for
+// generic_conv_wgrad_sum_kernel.
 __global__ __launch_bounds__(256) void generic_conv_wgrad_kernel(
-    ConvBwdArgs g, const void *dy, const void *x, void *dw) {
+    ConvBwdArgs g, const void *dy, const void *x, void *dw, float *partial,
+    int64_t per_run) {
   __shared__ float part[4][64];
   const int sp = g.spatial;
   int64_t fvol = 1;
@@ -453,14 +457,16 @@ __global__ __launch_bounds__(256) void generic_conv_wgrad_kernel(
   int64_t ovol = 1;
   for (int i = 0; i < sp; ++i)
     ovol *= g.y_dim[2 + i];
-  const int64_t total = g.y_dim[0] * ovol;
+  const int64_t all = g.y_dim[0] * ovol;
+  const int64_t first = (int64_t)blockIdx.z * per_run;
+  const int64_t total = first + per_run < all ? first + per_run : all;
   const int64_t y_k = k * g.y.s[1], x_c = c * g.x.s[1];
   // This wavefront's pixels are wave, wave + 4, ...: coordinates advance by
   // carries (no division in the loop), and eight pixels' loads are in flight
   // together.
   int64_t o[3] = {0, 0, 0}, n = 0;
   {
-    int64_t rem = wave;
+    int64_t rem = first + wave;
     for (int i = sp - 1; i >= 0; --i) {
       o[i] = rem % g.y_dim[2 + i];
       rem /= g.y_dim[2 + i];
@@ -469,7 +475,7 @@ __global__ __launch_bounds__(256) void generic_conv_wgrad_kernel(
   }
   constexpr int U = 8;
   float acc = 0.f;
-  for (int64_t it = wave; it < total; it += 4 * U) {
+  for (int64_t it = first + wave; it < total; it += 4 * U) {
     int64_t yo[U], xo[U];
     bool ok[U];
 #pragma unroll
@@ -512,11 +518,94 @@ __global__ __launch_bounds__(256) void generic_conv_wgrad_kernel(
   __syncthreads();
   if (wave == 0 && fc < fC) {
     const float sum = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+    if (gridDim.z > 1) {
+      partial[((int64_t)blockIdx.z * gridDim.x + blockIdx.x) * fC + fc] = sum;
+      return;
+    }
     int64_t off = k * g.w.s[0] + fc * g.w.s[1];
     for (int i = 0; i < sp; ++i)
       off += f[i] * g.w.s[2 + i];
     fhip_store<float>(dw, g.w_dt, off, sum);
   }
+}
+
+// The same sum for filters with few channels per group (lane = channel would
+// leave most of a wavefront idle): one workgroup per filter element
+// (k, fc, tap), its 256 threads stride over the output pixels -- consecutive
+// threads read consecutive pixels of DY and X -- and their sums meet in LDS.
+__global__ __launch_bounds__(256) void generic_conv_wgrad_pixel_kernel(
+    ConvBwdArgs g, const void *dy, const void *x, void *dw) {
+  __shared__ float part[4];
+  const int sp = g.spatial;
+  // blockIdx.x = ((k * fC + fc) * f0 + ..) in DW's logical order
+  int64_t rem = blockIdx.x;
+  int64_t f[3] = {0, 0, 0};
+  int64_t w_off = 0;
+  for (int i = sp - 1; i >= 0; --i) {
+    f[i] = rem % g.w_dim[2 + i];
+    rem /= g.w_dim[2 + i];
+    w_off += f[i] * g.w.s[2 + i];
+  }
+  const int64_t fC = g.w_dim[1];
+  const int64_t fc = rem % fC, k = rem / fC;
+  w_off += k * g.w.s[0] + fc * g.w.s[1];
+  const int64_t kPerGroup = g.w_dim[0] / g.groups;
+  const int64_t c = (k / kPerGroup) * fC + fc;
+  uint32_t od[3] = {1, 1, 1};
+  uint32_t ovol = 1;
+  for (int i = 0; i < sp; ++i) {
+    od[i] = (uint32_t)g.y_dim[2 + i];
+    ovol *= od[i];
+  }
+  const uint32_t total = (uint32_t)g.y_dim[0] * ovol; // the host checked the range
+  const int64_t y_k = k * g.y.s[1], x_c = c * g.x.s[1];
+  float acc = 0.f;
+  for (uint32_t pix = threadIdx.x; pix < total; pix += 256) {
+    uint32_t r = pix;
+    int64_t yy = y_k, xx = x_c;
+    bool inside = true;
+    for (int i = sp - 1; i >= 0; --i) {
+      const uint32_t o = r % od[i];
+      r /= od[i];
+      const int64_t xi = (int64_t)o * g.str[i] - g.pad[i] + f[i] * g.dil[i];
+      inside = inside && xi >= 0 && xi < g.x_dim[2 + i];
+      yy += (int64_t)o * g.y.s[2 + i];
+      xx += xi * g.x.s[2 + i];
+    }
+    yy += (int64_t)r * g.y.s[0];
+    xx += (int64_t)r * g.x.s[0];
+    if (inside)
+      acc += fhip_load<float>(dy, g.y_dt, yy) * fhip_load<float>(x, g.x_dt, xx);
+  }
+  acc = wave_sum(acc);
+  if ((threadIdx.x & 63) == 0)
+    part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    fhip_store<float>(dw, g.w_dt, w_off, (part[0] + part[1]) + (part[2] + part[3]));
+}
+
+// DW = sum of the runs' partial sums, in run order; one thread per element.
+__global__ __launch_bounds__(256) void generic_conv_wgrad_sum_kernel(
+    ConvBwdArgs g, const float *partial, void *dw, int64_t elems, int runs) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= elems)
+    return;
+  float sum = 0.f;
+#pragma unroll 8
+  for (int r = 0; r < runs; ++r)
+    sum += partial[(int64_t)r * elems + lin];
+  const int sp = g.spatial;
+  const int64_t fC = g.w_dim[1];
+  const int64_t fc = lin % fC;
+  int64_t tap = lin / fC;
+  int64_t off = fc * g.w.s[1];
+  for (int i = sp - 1; i >= 0; --i) {
+    off += (tap % g.w_dim[2 + i]) * g.w.s[2 + i];
+    tap /= g.w_dim[2 + i];
+  }
+  off += tap * g.w.s[0]; // what is left is k
+  fhip_store<float>(dw, g.w_dt, off, sum);
 }
 
 constexpr int kSdpaMaxDvPerLane = 8; // Dv <= 512
@@ -1286,8 +1375,45 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   const ConvBwdArgs g = conv_bwd_args(d, false);
   if (fhip_desc_volume(d->w) == 0)
     return 0;
+  int64_t pixels = d->y.dim[0];
+  for (int i = 0; i < d->spatial_rank; ++i)
+    pixels *= d->y.dim[2 + i];
+  // few channels per group: one workgroup per filter element, threads over pixels
+  if (d->w.dim[1] < 32 && pixels < (1ll << 31) && fhip_desc_volume(d->w) < (1ll << 31)) {
+    hipLaunchKernelGGL(generic_conv_wgrad_pixel_kernel,
+                       dim3((unsigned)fhip_desc_volume(d->w)), dim3(256), 0,
+                       ctx->stream, g, dy, x, dw);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    return 0;
+  }
+  // Few workgroups (one per filter tap and output channel) and many pixels:
+  // cut the pixels into runs of at least 256 until the launch has about 16
+  // workgroups per compute unit; the runs' sums meet in the context's scratch.
+  const int64_t wgs = (int64_t)grid.x * grid.y;
+  const int64_t cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  int64_t runs = (16 * cus + wgs - 1) / wgs;
+  runs = runs < pixels / 256 ? runs : pixels / 256;
+  runs = runs < 1024 ? runs : 1024;
+  if (runs < 2 || grid.y != 1) {
+    hipLaunchKernelGGL(generic_conv_wgrad_kernel, grid, dim3(256), 0, ctx->stream,
+                       g, dy, x, dw, (float *)nullptr, pixels);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    return 0;
+  }
+  // whole groups of 32 pixels (4 wavefronts x 8 in flight) per run
+  int64_t per_run = (pixels + runs - 1) / runs;
+  per_run = (per_run + 31) / 32 * 32;
+  runs = (pixels + per_run - 1) / per_run;
+  const int64_t elems = (int64_t)grid.x * d->w.dim[1];
+  void *scratch = nullptr;
+  if (fhip_ctx_scratch(ctx, (size_t)(runs * elems) * sizeof(float), &scratch) != 0)
+    return 1;
+  grid.z = (unsigned)runs;
   hipLaunchKernelGGL(generic_conv_wgrad_kernel, grid, dim3(256), 0, ctx->stream,
-                     g, dy, x, dw);
+                     g, dy, x, dw, (float *)scratch, per_run);
+  hipLaunchKernelGGL(generic_conv_wgrad_sum_kernel,
+                     dim3((unsigned)((elems + 255) / 256)), dim3(256), 0,
+                     ctx->stream, g, (const float *)scratch, dw, elems, (int)runs);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }

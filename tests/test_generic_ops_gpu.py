@@ -353,6 +353,10 @@ def test_conv_dgrad_config3_shape_closed_form_and_oracle(ctx):
     dict(x=[2, 64, 15, 14], w=[128, 64, 3, 3], pad=[1, 1], d=[1, 1], s=2),
     dict(x=[3, 48, 23, 31], w=[160, 48, 4, 3], pad=[2, 1], d=[2, 1], s=3),
     dict(x=[2, 128, 16, 16], w=[256, 128, 1, 1], pad=[0, 0], d=[1, 1], s=2),
+    # fewer than 128 output channels: DY is zero-padded to 128 (the shape class
+    # of the reference's wgrad benchmark: C = K = 48, 3 x 3, padding 2)
+    dict(x=[4, 48, 20, 16], w=[48, 48, 3, 3], pad=[2, 2], d=[1, 1]),
+    dict(x=[3, 64, 9, 13], w=[8, 64, 3, 3], pad=[1, 1], d=[1, 1]),
 ])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
 @pytest.mark.parametrize("w_nhwc", [True, False])
