@@ -50,14 +50,16 @@ bool is_channels_last(const fhip_tensor_desc &t) {
 // Strides `st` of an operand over the output dims [n, k, spatial...]: do the
 // pixel dims (n, p, q) collapse to one stride `sm` per flattened pixel index?
 bool pixel_stride(const int64_t *st, const int64_t *dim, int sp, int64_t *sm) {
-  const int pix_dims[3] = {1 + sp, sp == 2 ? 2 : -1, 0}; // q, p, n
+  int pix_dims[FHIP_MAX_RANK]; // fastest first: last spatial dim .. first, then n
+  int np = 0;
+  for (int i = 1 + sp; i >= 2; --i)
+    pix_dims[np++] = i;
+  pix_dims[np++] = 0;
   int64_t mult = 1;
   bool have = false;
   *sm = 0;
-  for (int i = 0; i < 3; ++i) {
+  for (int i = 0; i < np; ++i) {
     const int dd = pix_dims[i];
-    if (dd < 0)
-      continue;
     if (dim[dd] != 1) {
       if (!have) {
         if (st[dd] % mult != 0)
@@ -73,8 +75,49 @@ bool pixel_stride(const int64_t *st, const int64_t *dim, int sp, int64_t *sm) {
   return true;
 }
 
-ConvPlan make_plan(const fhip_conv_desc *d) {
+void set_channels_last(fhip_tensor_desc &t, int dtype, int64_t d0, int64_t d1,
+                       int64_t d2, int64_t d3) {
+  t.rank = 4;
+  t.dtype = dtype;
+  t.dim[0] = d0, t.dim[1] = d1, t.dim[2] = d2, t.dim[3] = d3;
+  t.stride[1] = 1;
+  t.stride[3] = d1;
+  t.stride[2] = d1 * d3;
+  t.stride[0] = d1 * d3 * d2;
+}
+
+// A 3-D convolution whose filter is 1 x 1 in H and W (unit strides, no padding
+// there) over dense channels-last tensors is the 2-D convolution of
+// [N, C, D, H * W] images with an [fd, 1] filter: `f` receives that problem
+// (geometry only -- the fused operands keep the original descriptor's shape).
+bool fold_3d(const fhip_conv_desc *d, fhip_conv_desc *f) {
+  if (d->spatial_rank != 3 || d->x.rank != 5)
+    return false;
+  if (d->w.dim[3] != 1 || d->w.dim[4] != 1 || d->stride[1] != 1 ||
+      d->stride[2] != 1 || d->padding[1] != 0 || d->padding[2] != 0)
+    return false;
+  if (!is_channels_last(d->x) || !is_channels_last(d->w) ||
+      !is_channels_last(d->out) || !is_channels_last(d->y))
+    return false;
+  *f = *d;
+  const int64_t hw = d->x.dim[3] * d->x.dim[4];
+  set_channels_last(f->x, d->x.dtype, d->x.dim[0], d->x.dim[1], d->x.dim[2], hw);
+  set_channels_last(f->w, d->w.dtype, d->w.dim[0], d->w.dim[1], d->w.dim[2], 1);
+  set_channels_last(f->y, d->y.dtype, d->y.dim[0], d->y.dim[1], d->y.dim[2], hw);
+  set_channels_last(f->out, d->out.dtype, d->out.dim[0], d->out.dim[1],
+                    d->out.dim[2], hw);
+  f->spatial_rank = 2;
+  f->padding[1] = 0, f->stride[1] = 1, f->dilation[1] = 1;
+  f->padding[2] = 0, f->stride[2] = 1, f->dilation[2] = 1;
+  return true;
+}
+
+// `d` is the geometry that runs (possibly folded and channel-padded); the
+// fused operands are described over `orig`'s output dims.
+ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr) {
   ConvPlan p;
+  if (!orig)
+    orig = d;
   if (d->spatial_rank != 2 && d->spatial_rank != 1)
     return p;
   if (d->x.dtype != d->w.dtype)
@@ -140,10 +183,10 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
     if (!f(o.operand.dtype))
       return p;
     int64_t st[FHIP_MAX_RANK];
-    if (!fhip_broadcast_strides(o.operand, d->y.rank, d->y.dim, st))
+    if (!fhip_broadcast_strides(o.operand, orig->y.rank, orig->y.dim, st))
       return p;
     int64_t sm;
-    if (!pixel_stride(st, d->y.dim, sp, &sm))
+    if (!pixel_stride(st, orig->y.dim, orig->spatial_rank, &sm))
       return p;
   }
   p.bn = p.N > 128 ? 256 : 128;
@@ -220,6 +263,75 @@ ConvPlan make_plan(const fhip_conv_desc *d) {
   return p;
 }
 
+// The problem that the MFMA kernel runs for descriptor `d`: `d` itself, its
+// 2-D fold, and / or a copy with the channels zero-padded to a multiple of 64
+// (the kernel's K slices are 128 bytes of one filter tap).
+struct ConvResolved {
+  ConvPlan plan;
+  fhip_conv_desc run;  // geometry of the launch
+  bool padded = false; // X and W are first copied into the context's scratch
+  int64_t C = 0, Cp = 0, x_pixels = 0, w_pixels = 0;
+  size_t x_bytes = 0, w_bytes = 0;
+};
+
+ConvResolved resolve(const fhip_conv_desc *d) {
+  ConvResolved r;
+  fhip_conv_desc folded;
+  const fhip_conv_desc *g = fold_3d(d, &folded) ? &folded : d;
+  r.run = *g;
+  r.plan = make_plan(g, d);
+  if (r.plan.ok)
+    return r;
+  // channel padding: 16-bit channels-last tensors, whole 16-byte chunks
+  const int64_t C = g->x.dim[1];
+  if ((g->spatial_rank != 2 && g->spatial_rank != 1) || g->x.rank != 2 + g->spatial_rank)
+    return r;
+  if (g->x.dtype != g->w.dtype ||
+      (g->x.dtype != FHIP_BFLOAT16 && g->x.dtype != FHIP_HALF))
+    return r;
+  if (g->w.dim[1] != C || C % 8 != 0 || C % 64 == 0)
+    return r;
+  if (!is_channels_last(g->x) || !is_channels_last(g->w))
+    return r;
+  const int64_t Cp = (C + 63) / 64 * 64;
+  fhip_conv_desc pd = *g;
+  auto widen = [&](fhip_tensor_desc &t) {
+    // channels-last strides of the same dims with Cp channels
+    t.dim[1] = Cp;
+    int64_t expect = Cp;
+    for (int i = t.rank - 1; i >= 2; --i) {
+      t.stride[i] = expect;
+      expect *= t.dim[i];
+    }
+    t.stride[0] = expect;
+    t.stride[1] = 1;
+  };
+  widen(pd.x);
+  widen(pd.w);
+  r.plan = make_plan(&pd, d);
+  if (!r.plan.ok)
+    return r;
+  r.run = pd;
+  r.padded = true;
+  r.C = C, r.Cp = Cp;
+  r.x_pixels = fhip_desc_volume(g->x) / C;
+  r.w_pixels = fhip_desc_volume(g->w) / C;
+  r.x_bytes = ((size_t)(r.x_pixels * Cp * 2) + 255) / 256 * 256;
+  r.w_bytes = ((size_t)(r.w_pixels * Cp * 2) + 255) / 256 * 256;
+  return r;
+}
+
+// dst[pixel][0 .. Cp) = src[pixel][0 .. C), zeros behind; one 16-byte chunk per thread
+__global__ void conv_pad_channels_kernel(const uint4 *src, uint4 *dst, int64_t pixels,
+                                         int32_t c8, int32_t cp8) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= pixels * cp8)
+    return;
+  const int64_t pixel = lin / cp8;
+  const int32_t chunk = (int32_t)(lin - pixel * cp8);
+  dst[lin] = chunk < c8 ? src[pixel * c8 + chunk] : make_uint4(0, 0, 0, 0);
+}
+
 } // namespace
 
 int conv_launch_bf16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
@@ -238,7 +350,7 @@ int conv_launch_f16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
 }
 
 bool fhip_fast_conv_applicable(const fhip_conv_desc *d) {
-  return make_plan(d).ok || fhip_fast_conv_rf_applicable(d);
+  return fhip_fast_conv_rf_applicable(d) || resolve(d).plan.ok;
 }
 
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
@@ -251,7 +363,8 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     return 1;
   if (taken)
     return 0;
-  const ConvPlan p = make_plan(d);
+  const ConvResolved res = resolve(d);
+  const ConvPlan &p = res.plan;
   if (handled) {
     *handled = p.ok;
     if (!p.ok)
@@ -260,7 +373,25 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   FHIP_REQUIRE(ctx, p.ok, "conv: descriptor not supported by the MFMA kernel");
   FHIP_REQUIRE(ctx, ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0,
                "conv: X and W must be 16-byte aligned");
-  const int sp = d->spatial_rank;
+  if (res.padded) {
+    // channel counts that are no multiple of 64: zero-padded copies of X and W
+    void *scratch = nullptr;
+    if (fhip_ctx_scratch(ctx, res.x_bytes + res.w_bytes, &scratch) != 0)
+      return 1;
+    char *xp = (char *)scratch, *wp = xp + res.x_bytes;
+    const int32_t c8 = (int32_t)(res.C / 8), cp8 = (int32_t)(res.Cp / 8);
+    const int64_t xt = res.x_pixels * cp8, wt = res.w_pixels * cp8;
+    hipLaunchKernelGGL(conv_pad_channels_kernel, dim3((unsigned)((xt + 255) / 256)),
+                       dim3(256), 0, ctx->stream, (const uint4 *)x, (uint4 *)xp,
+                       res.x_pixels, c8, cp8);
+    hipLaunchKernelGGL(conv_pad_channels_kernel, dim3((unsigned)((wt + 255) / 256)),
+                       dim3(256), 0, ctx->stream, (const uint4 *)w, (uint4 *)wp,
+                       res.w_pixels, c8, cp8);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    x = xp;
+    w = wp;
+  }
+  const int sp = d->spatial_rank; // of the descriptor the fused operands follow
   GemmArgs g{};
   g.conv = p.geom;
   g.a = (const char *)x;

@@ -1,8 +1,9 @@
 """Implicit-GEMM convolution (MFMA kernel) through the C ABI vs the oracle.
 
 Shapes here satisfy the tuned kernel's contract (channels-last bf16/f16,
-C * 2 bytes a multiple of 128, groups = 1); each test asserts that the tuned
-kernel is the one chosen, so a silent fall back to the generic kernel fails.
+C a multiple of 8 -- channel counts that are no multiple of 64 run on
+zero-padded copies --, groups = 1); each test asserts that the tuned kernel is
+the one chosen, so a silent fall back to the generic kernel fails.
 """
 import numpy as np
 import pytest
@@ -61,6 +62,46 @@ CASES = [
     # 1-D convolution
     dict(x=[2, 64, 50], w=[48, 64, 5], pad=[2], s=[2], d=[1]),
 ]
+
+
+RESHAPED_CASES = [
+    # channel counts that are no multiple of 64 run on zero-padded copies: the
+    # reference's NHWC benchmark shape (C = K = 48, 3 x 3, padding 2, dilation 2
+    # or 1), a wider one with a ragged channel tail, 1-D
+    dict(x=[3, 48, 20, 16], w=[48, 48, 3, 3], pad=[2, 2], s=[1, 1], d=[2, 2]),
+    dict(x=[2, 48, 20, 16], w=[48, 48, 3, 3], pad=[2, 2], s=[1, 1], d=[1, 1]),
+    dict(x=[2, 200, 9, 7], w=[72, 200, 2, 3], pad=[1, 0], s=[2, 1], d=[1, 1]),
+    dict(x=[2, 24, 70], w=[40, 24, 5], pad=[2], s=[1], d=[1]),
+    # 3-D convolutions with a 1 x 1 filter in H and W fold into 2-D ones: the
+    # reference's NDHWC benchmark shape class (depth filter 2, depth stride 2),
+    # with and without a channel tail, with depth padding and dilation
+    dict(x=[2, 288, 2, 12, 8], w=[96, 288, 2, 1, 1], pad=[0, 0, 0], s=[2, 1, 1], d=[1, 1, 1]),
+    dict(x=[2, 64, 5, 6, 10], w=[136, 64, 3, 1, 1], pad=[1, 0, 0], s=[1, 1, 1], d=[1, 1, 1]),
+    dict(x=[1, 40, 7, 5, 9], w=[24, 40, 2, 1, 1], pad=[2, 0, 0], s=[2, 1, 1], d=[2, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("case", RESHAPED_CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("bias", [False, True])
+def test_conv_padded_channels_and_folded_3d_vs_oracle(ctx, case, dtype, bias):
+    x = cl(case["x"], 43, 0, dtype)
+    w = cl(case["w"], 43, 1, dtype, std=0.1)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"],
+                            case["d"])
+    if not bias:
+        out = run(ctx, x, w, case["pad"], case["s"], case["d"], dtype)
+        assert_close(out.logical(), ref, dtype, str(case))
+        return
+    k = case["w"][0]
+    bd = [1, k] + [1] * (len(case["x"]) - 2)
+    b = HT.from_logical(rand(43, 2, bd), dtype)
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT,
+              out_dtype=dtype,
+              epilogue=[capi.epilogue_op(capi.PW["ADD"], dtype, operand_index=0,
+                                         operand=b.desc())],
+              epi_tensors=[b])
+    assert_close(out.logical(), ref + b.logical(), dtype, f"{case} + bias")
 
 
 @pytest.mark.parametrize("case", CASES)
@@ -142,9 +183,10 @@ def test_conv_igemm_bias_relu_residual(ctx):
 
 
 def test_conv_igemm_not_chosen_outside_contract(ctx):
-    # C = 48 (96 bytes per pixel) and grouped filters keep the generic kernel
-    x = cl([1, 48, 8, 8], 44, 0, capi.BFLOAT16)
-    w = cl([16, 48, 3, 3], 44, 1, capi.BFLOAT16, std=0.1)
+    # C = 44 (not whole 16-byte chunks per pixel) and grouped filters keep the
+    # generic kernel
+    x = cl([1, 44, 8, 8], 44, 0, capi.BFLOAT16)
+    w = cl([16, 44, 3, 3], 44, 1, capi.BFLOAT16, std=0.1)
     out = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.BFLOAT16, expect_tuned=False)
     ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
     assert_close(out.logical(), ref, capi.BFLOAT16)

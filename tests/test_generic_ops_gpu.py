@@ -239,7 +239,10 @@ def test_conv_dgrad_all_ones_known_answer(ctx, grouped):
     dyd, wd = [n, k, 8, 8], [k, fc, 1, 1]
     dy = HT.from_logical(np.ones(dyd), capi.HALF, oracle.channels_last_strides(dyd))
     w = HT.from_logical(np.ones(wd), capi.HALF)
-    dx = run_conv_dgrad(ctx, dy, w, [n, c, 8, 8], [0, 0], [1, 1], [1, 1], capi.HALF)
+    # one group: the forward MFMA kernel on the mirrored filter (K = 16 channels
+    # of DY, zero-padded to 64); grouped: the generic kernel
+    dx = run_conv_dgrad(ctx, dy, w, [n, c, 8, 8], [0, 0], [1, 1], [1, 1], capi.HALF,
+                        tuned=not grouped)
     assert np.all(dx.logical() == float(k // (c // fc)))
 
 
@@ -264,7 +267,10 @@ def test_conv_wgrad_all_ones_known_answer(ctx, variant):
     dict(x=[2, 6, 10, 11], w=[6, 2, 3, 3], pad=[1, 2], s=[3, 2], d=[1, 1]),
     dict(x=[1, 8, 13], w=[8, 2, 4], pad=[2], s=[3], d=[2]),
     dict(x=[1, 4, 5, 6, 7], w=[2, 4, 2, 3, 3], pad=[1, 0, 1], s=[1, 2, 1], d=[1, 1, 1]),
-    dict(x=[3, 16, 20, 20], w=[24, 16, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    # channels-last 16-bit, one group, unit strides, K a multiple of 8: the data
+    # gradient runs on the forward MFMA kernel (DY's 24 channels padded to 64)
+    dict(x=[3, 16, 20, 20], w=[24, 16, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1],
+         dgrad_mfma=True),
 ])
 @pytest.mark.parametrize("dtype", [capi.FLOAT, capi.BFLOAT16])
 @pytest.mark.parametrize("nhwc", [False, True])
@@ -276,7 +282,9 @@ def test_conv_backward_random_vs_oracle(ctx, case, dtype, nhwc):
     w = HT.from_logical(rand(32, 1, case["w"], std=0.2), dtype, lay(case["w"]))
     dy = HT.from_logical(rand(32, 2, yd), dtype, lay(yd))
     dx = run_conv_dgrad(ctx, dy, w, case["x"], case["pad"], case["s"],
-                        case["d"], dtype, nhwc)
+                        case["d"], dtype, nhwc,
+                        tuned=case.get("dgrad_mfma", False) and nhwc
+                        and dtype == capi.BFLOAT16)
     assert_close(dx.logical(),
                  oracle.conv_dgrad(dy.logical(), w.logical(), case["x"],
                                    case["pad"], case["s"], case["d"]),
