@@ -17,6 +17,7 @@
 #include <unordered_map>
 #include <unordered_set>
 
+#include "cache.h"
 #include "plan.h"
 
 namespace fusilli {
@@ -73,25 +74,117 @@ public:
   }
 
   // ---- compilation ------------------------------------------------------------
-  // JIT: plan for the handle's backend and load the plan.
+  // JIT: plan for the handle's backend, through the on-disk cache, and load
+  // the plan.  `remove` = true deletes the cache files when this Graph goes
+  // out of scope (reference graph.h:127-146).
   ErrorObject compile(const Handle &handle, bool remove = false) {
     FUSILLI_ASSIGN_OR_RETURN(auto bytes,
                              compileToArtifact(handle.getBackend(), remove));
     return loadFromArtifact(handle, bytes);
   }
 
-  // AOT: the serialised plan.  Needs no handle; does not disturb a loaded
-  // plan.  `remove` is accepted for source compatibility (there is no
-  // on-disk cache to clean).
+  // AOT: the serialised plan, read back from the cache file that holds it.
+  // Needs no handle; does not disturb a loaded plan.
   ErrorOr<std::vector<uint8_t>> compileToArtifact(Backend backend,
                                                   bool remove = false) {
-    (void)remove;
+    FUSILLI_ASSIGN_OR_RETURN(std::string text, emitAsm());
+    FUSILLI_ASSIGN_OR_RETURN(std::filesystem::path artifact,
+                             getCompiledArtifact(backend, text, remove));
+    (void)artifact;
+    return cache_->output.readBytes();
+  }
+
+  // A textual description of the validated graph (tensors, nodes, planned
+  // steps): what the cache compares to decide whether its artifact is still
+  // this graph's.  Takes the place of the reference's MLIR text
+  // (graph.h:407-419); backend-independent.
+  ErrorOr<std::string> emitAsm() {
+    FUSILLI_RETURN_ERROR_IF(!isValidated_, ErrorCode::NotValidated,
+                            "Graph must be validated before being compiled");
+    plan::Planner planner(subNodes_, fullGraphInputsSorted_,
+                          fullGraphOutputsSorted_, Backend::CPU);
+    FUSILLI_ASSIGN_OR_RETURN(plan::Plan p, planner.run());
+    std::ostringstream os;
+    os << "fusilli.graph @" << getName() << " {\n";
+    auto tensorLine = [&](const char *what, const TensorAttr &t) {
+      os << "  " << what << " %" << t.getName() << " : dims[";
+      for (size_t i = 0; i < t.getDim().size(); ++i)
+        os << (i ? "," : "") << t.getDim()[i];
+      os << "] strides[";
+      for (size_t i = 0; i < t.getStride().size(); ++i)
+        os << (i ? "," : "") << t.getStride()[i];
+      os << "] dtype " << static_cast<int>(t.getDataType()) << "\n";
+    };
+    for (const auto &t : fullGraphInputsSorted_)
+      tensorLine("input", *t);
+    for (const auto &t : fullGraphOutputsSorted_)
+      tensorLine("output", *t);
+    for (const auto &n : subNodes_)
+      os << "  node " << static_cast<int>(n->getType()) << " '" << n->getName()
+         << "'\n";
+    os << "  steps " << p.steps.size() << " workspace " << p.workspaceBytes
+       << " plan 0x" << std::hex << p.signature << std::dec << "\n";
+    for (const plan::Step &st : p.steps) {
+      os << "    step kind " << st.kind << " slots";
+      for (int sl : st.slot)
+        os << ' ' << sl;
+      os << "\n";
+    }
+    os << "}\n";
+    return ok(os.str());
+  }
+
+  // The path of the artifact in the cache, (re)generating the cache files
+  // unless they are still valid for this instance: same paths (graph name),
+  // same description, same planner key (backend).  `reCompiled` reports
+  // whether they were regenerated (reference graph.h:428-447, 557-644; the
+  // cache is per Graph instance: a new instance always regenerates).
+  ErrorOr<std::filesystem::path>
+  getCompiledArtifact(Backend backend, const std::string &generatedAsm,
+                      bool remove, std::optional<bool> *reCompiled = nullptr) {
+    FUSILLI_ASSIGN_OR_RETURN(bool valid, validateCache(backend, generatedAsm));
+    if (valid) {
+      if (reCompiled)
+        *reCompiled = false;
+      return ok(cache_->output.path);
+    }
     FUSILLI_RETURN_ERROR_IF(!isValidated_, ErrorCode::NotValidated,
                             "Graph must be validated before being compiled");
     plan::Planner planner(subNodes_, fullGraphInputsSorted_,
                           fullGraphOutputsSorted_, backend);
     FUSILLI_ASSIGN_OR_RETURN(plan::Plan p, planner.run());
-    return ok(plan::serialize(p));
+    const std::vector<uint8_t> bytes = plan::serialize(p);
+    cache_.reset(); // the old files (if owned) go first: same names
+    FUSILLI_ASSIGN_OR_RETURN(
+        CacheFile input, CacheFile::create(getName(), kCacheInputFileName, remove));
+    FUSILLI_ASSIGN_OR_RETURN(
+        CacheFile output,
+        CacheFile::create(getName(), kCacheOutputFileName, remove));
+    FUSILLI_ASSIGN_OR_RETURN(
+        CacheFile command,
+        CacheFile::create(getName(), kCacheCommandFileName, remove));
+    FUSILLI_CHECK_ERROR(input.write(generatedAsm));
+    FUSILLI_CHECK_ERROR(output.write(bytes));
+    FUSILLI_CHECK_ERROR(command.write(plannerKey(backend)));
+    cache_.emplace(CachedAssets{std::move(input), std::move(output),
+                                std::move(command)});
+    if (reCompiled)
+      *reCompiled = true;
+    return ok(cache_->output.path);
+  }
+
+  // Contents of one of this instance's cache files.
+  ErrorOr<std::string> readCompilationCacheFile(CachedAssetsType type) {
+    FUSILLI_RETURN_ERROR_IF(!cache_.has_value(), ErrorCode::FileSystemFailure,
+                            "Cache not populated yet");
+    switch (type) {
+    case CachedAssetsType::Input:
+      return cache_->input.read();
+    case CachedAssetsType::Output:
+      return cache_->output.read();
+    default:
+      return cache_->command.read();
+    }
   }
 
   // Loads a plan produced by this or an identically built graph.  Replaces
@@ -136,6 +229,36 @@ public:
     loadedPlan_ = std::move(*own);
     loadedBackend_ = handle.getBackend();
     return ok();
+  }
+
+  // What produced an artifact: changes with the backend and the plan format.
+  static std::string plannerKey(Backend backend) {
+    return std::string("fusilli_hip plan --backend=") + backendName(backend) +
+           " --format=" + std::string(plan::kMagic, sizeof(plan::kMagic)) + "\n";
+  }
+
+  // The cache is valid when this instance generated it, the graph's name (the
+  // paths) has not changed since, the files still exist, and the description
+  // and the planner key they hold are the ones asked for.
+  ErrorOr<bool> validateCache(Backend backend, const std::string &generatedAsm) {
+    if (!cache_.has_value())
+      return ok(false);
+    if (cache_->input.path != CacheFile::getPath(getName(), kCacheInputFileName) ||
+        cache_->output.path != CacheFile::getPath(getName(), kCacheOutputFileName) ||
+        cache_->command.path != CacheFile::getPath(getName(), kCacheCommandFileName))
+      return ok(false);
+    FUSILLI_ASSIGN_OR_RETURN(CacheFile input,
+                             CacheFile::open(getName(), kCacheInputFileName));
+    FUSILLI_ASSIGN_OR_RETURN(CacheFile output,
+                             CacheFile::open(getName(), kCacheOutputFileName));
+    FUSILLI_ASSIGN_OR_RETURN(CacheFile command,
+                             CacheFile::open(getName(), kCacheCommandFileName));
+    (void)output;
+    FUSILLI_ASSIGN_OR_RETURN(std::string inputContents, input.read());
+    if (inputContents != generatedAsm)
+      return ok(false);
+    FUSILLI_ASSIGN_OR_RETURN(std::string commandContents, command.read());
+    return ok(commandContents == plannerKey(backend));
   }
 
   // nullopt until a plan is loaded; must be called before execute().
@@ -644,6 +767,8 @@ private:
 
   bool isValidated_ = false;
   std::optional<plan::Plan> loadedPlan_;
+  // this instance's cache files; never shared between instances
+  std::optional<CachedAssets> cache_;
   std::optional<Backend> loadedBackend_;
   std::optional<size_t> workspaceSize_;
   // plans for buffer extents that differ from the declared ones

@@ -878,7 +878,7 @@ TEST("graph: compile/execute preconditions") {
   auto st = c.graph->execute(cpu, pack, nullptr);
   CHECK(st.getCode() == ErrorCode::NotCompiled);
 
-  REQUIRE_OK(c.graph->compile(cpu));
+  REQUIRE_OK(c.graph->compile(cpu, /*remove=*/true));
   CHECK(c.graph->getKernelCount() == std::optional<size_t>(1));
   CHECK_ERROR(c.graph->execute(cpu, pack, nullptr), ErrorCode::InvalidArgument,
               "Graph::execute requires getWorkspaceSize() to be called before "
@@ -921,7 +921,7 @@ TEST("graph: virtual and scalar tensors must stay out of the variant pack") {
   out->setOutput(true);
   REQUIRE_OK(g.validate());
   REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
-  REQUIRE_OK(g.compile(cpu));
+  REQUIRE_OK(g.compile(cpu, /*remove=*/true));
   REQUIRE_ASSIGN(auto ws, g.getWorkspaceSize());
   REQUIRE(ws.has_value());
   CHECK(*ws >= 2 * 5 * 4); // the virtual tensor between the two kernels
@@ -957,7 +957,7 @@ TEST("graph: artifact contract") {
   {
     auto producer = makeConvGraph("aot_producer");
     REQUIRE_OK(producer.graph->validate());
-    REQUIRE_ASSIGN(bytes, producer.graph->compileToArtifact(Backend::CPU));
+    REQUIRE_ASSIGN(bytes, producer.graph->compileToArtifact(Backend::CPU, /*remove=*/true));
   }
   CHECK(!bytes.empty());
   // another instance's artifact loads into an identically built graph
@@ -965,7 +965,7 @@ TEST("graph: artifact contract") {
   REQUIRE_ASSIGN(auto ws, consumer.graph->getWorkspaceSize());
   CHECK(ws.has_value());
   // compileToArtifact for another backend leaves the loaded state alone
-  REQUIRE_ASSIGN(auto other, consumer.graph->compileToArtifact(Backend::AMDGPU));
+  REQUIRE_ASSIGN(auto other, consumer.graph->compileToArtifact(Backend::AMDGPU, /*remove=*/true));
   CHECK(!other.empty());
   REQUIRE_ASSIGN(auto ws2, consumer.graph->getWorkspaceSize());
   CHECK(ws2.has_value());
@@ -1022,6 +1022,106 @@ TEST("graph: artifact contract") {
               "Artifact does not match this graph (signature mismatch)");
 }
 
+TEST("cache: files, RAII removal, hit and miss") {
+  namespace fs = std::filesystem;
+  // files live under ${FUSILLI_CACHE_DIR}/.cache/fusilli/<graph>/<file>
+  const fs::path dir = CacheFile::getCacheDir();
+  CHECK(dir.filename() == "fusilli");
+  CHECK(CacheFile::getPath("g", "f") == dir / "g" / "f");
+  // a name cannot leave the cache directory
+  CHECK(CacheFile::getPath("../x/y", "f") == dir / ".._x_y" / "f");
+  {
+    REQUIRE_ASSIGN(CacheFile kept, CacheFile::create("cache_case", "kept", false));
+    {
+      REQUIRE_ASSIGN(CacheFile temp, CacheFile::create("cache_case", "temp", true));
+      REQUIRE_OK(temp.write(std::string("abc")));
+      REQUIRE_ASSIGN(std::string back, temp.read());
+      CHECK(back == "abc");
+      REQUIRE_ASSIGN(CacheFile again, CacheFile::open("cache_case", "temp"));
+      CHECK(again.path == temp.path);
+      // moving hands the removal over
+      CacheFile moved = std::move(temp);
+      CHECK(fs::exists(moved.path));
+    }
+    CHECK(!fs::exists(CacheFile::getPath("cache_case", "temp")));
+    CHECK(isError(CacheFile::open("cache_case", "temp")));
+    CHECK(fs::exists(kept.path)); // remove = false survives its object
+    fs::remove(kept.path);
+    fs::remove(kept.path.parent_path());
+  }
+
+  // the reference's cache test (tests/test_graph.cpp:242-299)
+  auto cg = makeConvGraph("cache_graph");
+  Graph &g = *cg.graph;
+  CHECK_ERROR(g.emitAsm(), ErrorCode::NotValidated,
+              "Graph must be validated before being compiled");
+  REQUIRE_OK(g.validate());
+  REQUIRE_ASSIGN(std::string text, g.emitAsm());
+  CHECK(text.find("fusilli.graph @cache_graph") == 0);
+  std::optional<bool> re;
+  REQUIRE_ASSIGN(fs::path artifact, g.getCompiledArtifact(Backend::CPU, text, true, &re));
+  CHECK(re.has_value() && *re); // empty cache: generated
+  CHECK(fs::exists(artifact));
+  re.reset();
+  REQUIRE_OK(g.getCompiledArtifact(Backend::CPU, text, true, &re));
+  CHECK(re.has_value() && !*re); // hit
+  re.reset();
+  REQUIRE_OK(g.getCompiledArtifact(Backend::AMDGPU, text, true, &re));
+  CHECK(re.has_value() && *re); // another backend: another planner key
+  re.reset();
+  REQUIRE_OK(g.getCompiledArtifact(Backend::AMDGPU, text, true, &re));
+  CHECK(re.has_value() && !*re);
+  re.reset();
+  REQUIRE_OK(g.getCompiledArtifact(Backend::CPU, text + " ", true, &re));
+  CHECK(re.has_value() && *re); // another description
+  re.reset();
+  REQUIRE_OK(g.getCompiledArtifact(Backend::CPU, text + " ", true, &re));
+  CHECK(re.has_value() && !*re);
+  REQUIRE_ASSIGN(std::string cmd, g.readCompilationCacheFile(CachedAssetsType::Command));
+  CHECK(cmd.find("--backend=CPU") != std::string::npos);
+  REQUIRE_ASSIGN(std::string in, g.readCompilationCacheFile(CachedAssetsType::Input));
+  CHECK(in == text + " ");
+  // a deleted file is a miss, not an error of the second kind
+  fs::remove(artifact);
+  CHECK(isError(g.getCompiledArtifact(Backend::CPU, text + " ", true, &re)));
+  const fs::path old_dir = artifact.parent_path();
+  g.setName("cache_graph_renamed");
+  re.reset();
+  REQUIRE_ASSIGN(fs::path artifact2, g.getCompiledArtifact(Backend::CPU, text + " ", true, &re));
+  CHECK(re.has_value() && *re); // new name, new paths
+  CHECK(artifact2.parent_path() != old_dir);
+  CHECK(!fs::exists(old_dir)); // the old files went with their objects
+
+  // compile() goes through the cache; remove = true cleans up with the Graph
+  fs::path compiled_dir;
+  {
+    REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+    auto tmp = makeConvGraph("cache_compile");
+    REQUIRE_OK(tmp.graph->validate());
+    REQUIRE_OK(tmp.graph->compile(cpu, /*remove=*/true));
+    compiled_dir = CacheFile::getPath("cache_compile", kCacheOutputFileName).parent_path();
+    CHECK(fs::exists(compiled_dir / kCacheOutputFileName));
+    CHECK(fs::exists(compiled_dir / kCacheInputFileName));
+    CHECK(fs::exists(compiled_dir / kCacheCommandFileName));
+    // the artifact in the cache is what compileToArtifact returns
+    REQUIRE_ASSIGN(auto bytes, tmp.graph->compileToArtifact(Backend::CPU, true));
+    REQUIRE_ASSIGN(CacheFile f, CacheFile::open("cache_compile", kCacheOutputFileName));
+    REQUIRE_ASSIGN(auto disk, f.readBytes());
+    CHECK(bytes == disk);
+  }
+  CHECK(!fs::exists(compiled_dir));
+  // remove = false keeps the files
+  {
+    REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
+    auto tmp = makeConvGraph("cache_keep");
+    REQUIRE_OK(tmp.graph->validate());
+    REQUIRE_OK(tmp.graph->compile(cpu));
+  }
+  const fs::path keep_dir = CacheFile::getPath("cache_keep", "x").parent_path();
+  CHECK(fs::exists(keep_dir / kCacheOutputFileName));
+  fs::remove_all(keep_dir);
+}
+
 TEST("planner: fusion decisions") {
   REQUIRE_ASSIGN(Handle cpu, Handle::create(Backend::CPU));
   // conv -> add(bias) -> relu fuses into one kernel, no workspace
@@ -1041,7 +1141,7 @@ TEST("planner: fusion decisions") {
     auto o = g.pointwise(t, relu);
     o->setOutput(true);
     REQUIRE_OK(g.validate());
-    REQUIRE_OK(g.compile(cpu));
+    REQUIRE_OK(g.compile(cpu, /*remove=*/true));
     CHECK(g.getKernelCount() == std::optional<size_t>(1));
     REQUIRE_ASSIGN(auto ws, g.getWorkspaceSize());
     CHECK(*ws == 0);
@@ -1059,7 +1159,7 @@ TEST("planner: fusion decisions") {
     auto o = g.pointwise(y, g.tensor(TensorAttr(0.5f)), mul);
     o->setOutput(true);
     REQUIRE_OK(g.validate());
-    REQUIRE_OK(g.compile(cpu));
+    REQUIRE_OK(g.compile(cpu, /*remove=*/true));
     CHECK(g.getKernelCount() == std::optional<size_t>(1));
   }
   // a virtual tensor with two consumers is not fused away
@@ -1076,7 +1176,7 @@ TEST("planner: fusion decisions") {
     auto o = g.pointwise(r, c, p2); // c is read twice
     o->setOutput(true);
     REQUIRE_OK(g.validate());
-    REQUIRE_OK(g.compile(cpu));
+    REQUIRE_OK(g.compile(cpu, /*remove=*/true));
     CHECK(g.getKernelCount() == std::optional<size_t>(3));
   }
 }

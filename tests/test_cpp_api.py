@@ -3,6 +3,7 @@ GPU; the device binary runs the reference samples' known answers end to end on
 Backend::AMDGPU."""
 import os
 import subprocess
+import tempfile
 
 import pytest
 
@@ -13,7 +14,15 @@ def _run(name, timeout):
     path = os.path.join(BIN, name)
     assert os.path.exists(path), \
         f"{path} missing: run `python -c 'import __graft_entry__ as g; g.build()'`"
-    proc = subprocess.run([path], capture_output=True, text=True, timeout=timeout)
+    # the graphs' cache files go to a directory of this run
+    with tempfile.TemporaryDirectory(prefix="fusilli_cache_") as cache:
+        env = dict(os.environ, FUSILLI_CACHE_DIR=cache)
+        proc = subprocess.run([path], capture_output=True, text=True,
+                              timeout=timeout, env=env)
+        left = [os.path.join(d, f) for d, _, fs in os.walk(cache) for f in fs]
+    # every test compiles with remove = true or cleans up after itself
+    # (reference tests/test_cache_empty.sh)
+    assert not left, f"{name} left cache files behind: {left[:5]}"
     tail = "\n".join(proc.stdout.splitlines()[-60:])
     assert proc.returncode == 0, f"{name} failed:\n{tail}\n{proc.stderr[-2000:]}"
     assert "0 failed checks" in proc.stdout, tail
