@@ -4,11 +4,12 @@
 // small enough that a 32-channel slice of it fits a wavefront's registers
 // (R * S * C <= 640: the 3 x 3 x 64 family), the whole problem is one pass:
 //
-//   * a workgroup (4 wavefronts, one per SIMD, the full 512-register file
-//     each) owns TR output rows of one image and 128 output channels; each
-//     wavefront owns 32 of those channels and keeps its 32 x (R*S*C) filter
-//     slice in registers as ready-made MFMA A operands for the kernel's whole
-//     life (loaded once, straight from global memory);
+//   * a workgroup (8 wavefronts, two per SIMD) owns TR output rows of one
+//     image and 128 output channels; the wavefronts w and w + 4 share 32 of
+//     those channels, both keep that 32 x (R*S*C) filter slice in registers as
+//     ready-made MFMA A operands for the kernel's whole life (staged once
+//     through LDS, so that the global reads are whole 64-byte runs of a filter
+//     row), and they take alternate blocks of 16 pixels;
 //   * the tile's input rows plus halo go into LDS once, by LDS-DMA, into a
 //     zero-padded image (W + S - 1 pixels per row, rows above / below the image
 //     as zeros) with a pixel pitch of C * 2 + 16 bytes: every filter tap is then
@@ -21,11 +22,9 @@
 //     tiles).  A lane then holds 8 consecutive output channels of one pixel:
 //     bias / scale / ReLU run on the accumulators and the result leaves with
 //     one 16-byte store per lane, no trip through LDS;
-//   * pixels are processed in groups of 5 blocks of 16; the epilogue and the
-//     stores of group g - 1 are issued between the MFMAs of group g (two
-//     accumulator sets alternate), and the fragments of a group's first K-step
-//     are fetched during the previous group's last one, so the matrix pipe
-//     sees one continuous stream and the output leaves while it works.
+//   * the fragments run through a ring of registers a few K-steps ahead of the
+//     MFMAs, across block boundaries, and a block's epilogue and store are
+//     issued while the SIMD's other wavefront keeps the matrix pipe busy.
 //
 // Reference semantics: aten.convolution, groups = 1 (reference
 // support/asm_emitter.h:690-701, node/conv_node.h:38-56) followed by the fused
