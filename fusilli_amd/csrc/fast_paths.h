@@ -64,7 +64,7 @@ int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
 
 bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d);
 int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
-                   const void *k, const void *v, void *o);
+                   const void *k, const void *v, const void *mask, void *o);
 
 bool fhip_fast_norm_applicable(const fhip_norm_desc *d);
 int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,

@@ -1487,7 +1487,7 @@ int fhip_sdpa_fwd(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
   if (fhip_fast_sdpa_applicable(d))
-    return fhip_fast_sdpa(ctx, d, q, k, v, o);
+    return fhip_fast_sdpa(ctx, d, q, k, v, mask, o);
 
   SdpaArgs g{};
   g.B = d->q.dim[0];

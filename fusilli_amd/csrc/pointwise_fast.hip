@@ -30,6 +30,8 @@ struct PwFastArgs {
   int32_t o_dt;
   int32_t mode;
   int32_t num_inputs;
+  int32_t hoist_rows; // IN_ROW operands are the same for every chunk of a
+                      // thread: load them once
   fhip_pointwise_params params;
 };
 
@@ -226,11 +228,27 @@ __device__ __forceinline__ void evaluate(const PwFastArgs &g,
 }
 
 // A workgroup walks chunks of UNROLL * 256 consecutive vectors; all loads of
-// a chunk are issued before the first value is used.
+// a chunk are issued before the first value is used.  When the distance
+// between a workgroup's chunks is a multiple of a broadcast row's length
+// (hoist_rows), a thread meets the same row elements in every chunk and keeps
+// them in registers.
 template <int NIN, int MODE, int DT, int UNROLL>
 __global__ __launch_bounds__(256) void pointwise_fast_kernel(PwFastArgs g) {
   const int32_t nvec = (int32_t)g.nvec;
   const int32_t chunks = (nvec + 256 * UNROLL - 1) / (256 * UNROLL);
+  const bool hoist = g.hoist_rows != 0;
+  Raw rows[UNROLL][NIN];
+  if (hoist) {
+    const int32_t v0 = (int32_t)blockIdx.x * (256 * UNROLL) + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int32_t v = v0 + u * 256 < nvec ? v0 + u * 256 : nvec - 1;
+#pragma unroll
+      for (int i = 0; i < NIN; ++i)
+        if (g.kind[i] == IN_ROW)
+          fetch_raw<DT>(g, i, v, rows[u][i]);
+    }
+  }
   for (int32_t ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
     const int32_t v0 = ch * (256 * UNROLL) + threadIdx.x;
     Raw raw[UNROLL][NIN];
@@ -239,8 +257,12 @@ __global__ __launch_bounds__(256) void pointwise_fast_kernel(PwFastArgs g) {
       // lanes past the end re-read the last vector and store nothing
       const int32_t v = v0 + u * 256 < nvec ? v0 + u * 256 : nvec - 1;
 #pragma unroll
-      for (int i = 0; i < NIN; ++i)
-        fetch_raw<DT>(g, i, v, raw[u][i]);
+      for (int i = 0; i < NIN; ++i) {
+        if (hoist && g.kind[i] == IN_ROW)
+          raw[u][i] = rows[u][i];
+        else
+          fetch_raw<DT>(g, i, v, raw[u][i]);
+      }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -258,16 +280,45 @@ __global__ __launch_bounds__(256) void pointwise_fast_kernel(PwFastArgs g) {
   }
 }
 
-constexpr int kUnroll = 4;
+// Two vectors per lane and chunk and up to 32 workgroups per compute unit
+// measured best on 8192 x 4096 bf16 (ADD of a bias row 24.7 -> 23.7-24.1 us,
+// GELU 25.9 -> 24.6 us against four vectors and 8 workgroups).
+constexpr int kUnroll = 2;
+constexpr int kWgsPerCu = 32;
+
+int64_t pw_gcd(int64_t a, int64_t b) {
+  while (b) {
+    const int64_t t = a % b;
+    a = b;
+    b = t;
+  }
+  return a;
+}
 
 template <int NIN, int MODE, int DT>
-void launch_dt(fhip_ctx *ctx, const PwFastArgs &g) {
-  // up to eight workgroups per compute unit, each walking several chunks of
-  // a large tensor
-  int64_t blocks = (g.nvec + 256 * kUnroll - 1) / (256 * kUnroll);
-  const int64_t cap = 256 * 8;
+void launch_dt(fhip_ctx *ctx, const PwFastArgs &g0) {
+  PwFastArgs g = g0;
+  // a bounded number of workgroups per compute unit, each walking several
+  // chunks of a large tensor
+  const int64_t chunk = 256 * kUnroll;
+  int64_t blocks = (g.nvec + chunk - 1) / chunk;
+  const int64_t cap = 256 * kWgsPerCu;
   if (blocks > cap)
     blocks = cap;
+  // broadcast rows: a grid that is a multiple of `need` workgroups puts every
+  // thread on the same row elements in all of its chunks
+  int64_t need = 1;
+  bool has_row = false;
+  for (int i = 0; i < g.num_inputs; ++i)
+    if (g.kind[i] == IN_ROW) {
+      has_row = true;
+      const int64_t n = g.span[i] / pw_gcd(g.span[i], chunk);
+      need = need / pw_gcd(need, n) * n;
+    }
+  if (has_row && need <= blocks) {
+    blocks = blocks / need * need;
+    g.hoist_rows = 1;
+  }
   hipLaunchKernelGGL((pointwise_fast_kernel<NIN, MODE, DT, kUnroll>),
                      dim3((unsigned)blocks), dim3(256), 0, ctx->stream, g);
 }

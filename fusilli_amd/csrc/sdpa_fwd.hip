@@ -15,6 +15,10 @@
 //     accumulator O^T is rescaled only when some row maximum moved;
 //   * causal workgroups stop at the diagonal, and a wavefront skips tiles that
 //     lie wholly above its own rows;
+//   * a mask tensor (boolean, or additive in f32 / bf16 / f16, broadcast over
+//     batch and heads as its dims say) is read straight into registers, four
+//     consecutive keys per load, at the top of a round -- one MFMA phase ahead
+//     of the softmax that folds it into the scores;
 //   * the two wavefronts of a SIMD (w and w + 4) alternate: a tile is an MFMA
 //     phase (S^T of tile t and the O^T update of tile t - 1, 32 MFMAs) and a
 //     vector-ALU phase (online softmax of tile t) of about equal length,
@@ -26,7 +30,8 @@
 //
 // Reference semantics: aten.scaled_dot_product_attention (reference
 // support/asm_emitter.h:2409-2468, node/sdpa_node.h:36-236), GQA by head
-// repetition, causal mask aligned top-left.
+// repetition, causal mask aligned top-left; mask tensors as in
+// node/sdpa_node.h:138-176 (rank 4, every dim 1 or the full extent).
 #include "common.h"
 #include "fast_paths.h"
 
@@ -75,6 +80,12 @@ struct SdpaArgs {
   int32_t Sq, Skv, group; // group = Hq / Hkv
   int32_t causal;
   float scale_log2e; // softmax scale * log2(e)
+  // mask tensor (kernels with MASK): strides in elements, 0 where broadcast;
+  // the key stride is 1
+  const char *mask;
+  int64_t m_sb, m_sh, m_sq;
+  uint32_t m_bytes; // bytes of one (batch, head) slab
+  int32_t m_dt;     // FHIP_BOOLEAN / FHIP_FLOAT / FHIP_BFLOAT16 / FHIP_HALF
 };
 
 template <int N, typename F> __device__ __forceinline__ void sd_static_for(F &&f) {
@@ -211,8 +222,9 @@ __device__ __forceinline__ void sd_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <bool BF16, bool CAUSAL, int HD>
+template <bool BF16, bool CAUSAL, int HD, bool MASK>
 __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
+  static_assert(!(CAUSAL && MASK), "a mask tensor excludes the causal flag");
   using C = SdShape<HD>;
   constexpr int kD = HD;
   constexpr int kRowB = C::kRowB, kTileB = C::kTileB;
@@ -293,6 +305,35 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   };
   const __amdgpu_buffer_rsrc_t k_rsrc = slab_rsrc(kp, k_bytes);
   const __amdgpu_buffer_rsrc_t v_rsrc = slab_rsrc(vp, v_bytes);
+  // Mask: a lane's 32 scores of a tile are 8 runs of 4 consecutive keys (run i
+  // starts at key 32 * (i / 4) + 8 * (i % 4) + 4 * half), one load each; the
+  // element size picks the load width.  Runs past the slab's end read as
+  // zeros; their keys are dead anyway.
+  const int m_esh = !MASK ? 0 : g.m_dt == FHIP_BOOLEAN ? 0 : g.m_dt == FHIP_FLOAT ? 2 : 1;
+  __amdgpu_buffer_rsrc_t m_rsrc = k_rsrc;
+  uint32_t m_off = 0;
+  if constexpr (MASK) {
+    m_rsrc = slab_rsrc(g.mask + ((b * g.m_sb + h * g.m_sh) << m_esh), g.m_bytes);
+    const int qr = qrow < g.Sq ? qrow : g.Sq - 1;
+    m_off = (uint32_t)(((int64_t)qr * g.m_sq + half * 4) << m_esh);
+  }
+  u32x4 mraw[MASK ? 8 : 1];
+  auto load_mask = [&](int t) {
+    const int so = (t * kBKV) << m_esh;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int run = 32 * (i / 4) + 8 * (i % 4);
+      if (m_esh == 0) {
+        mraw[i].x = __builtin_amdgcn_raw_buffer_load_b32(m_rsrc, (int)m_off + run, so, 0);
+      } else if (m_esh == 1) {
+        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(m_rsrc, (int)m_off + run * 2, so, 0);
+        mraw[i].x = v.x;
+        mraw[i].y = v.y;
+      } else {
+        mraw[i] = __builtin_amdgcn_raw_buffer_load_b128(m_rsrc, (int)m_off + run * 4, so, 0);
+      }
+    }
+  };
   auto issue_kv = [&](const __amdgpu_buffer_rsrc_t &r, uint32_t tile_bytes,
                       const uint32_t (&off)[kLoadsPerTile], int t,
                       uint32_t stage) {
@@ -378,6 +419,10 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   int sl_prev = kStages - 1, sl_cur = 0, sl_next = 1;
 #pragma clang loop unroll(disable)
   for (int t = 0; t <= tiles; ++t) {
+    // (the mask first: the waits below count the K / V loads issued after it)
+    if constexpr (MASK)
+      if (t < tiles)
+        load_mask(t);
     issue_k(t + 2, sl_prev);
     issue_v(t + 1, sl_next);
     // ---- MFMA phase -----------------------------------------------------------
@@ -470,15 +515,46 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     // ---- vector-ALU phase -------------------------------------------------------
     if (active(t)) {
       const int kv0 = t * kBKV;
+      // with a mask the scores are scaled here, with the mask folded in, and
+      // the softmax below runs on them with unit scale
+      const float sl2 = MASK ? 1.0f : g.scale_log2e;
+      if constexpr (MASK) {
+        constexpr float kLog2e = 1.4426950408889634f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const u32x4 w = mraw[kb * 4 + (r >> 2)];
+            const int e = r & 3;
+            const float sc = s[kb][r] * g.scale_log2e;
+            if (m_esh == 0) {
+              s[kb][r] = ((w.x >> (8 * e)) & 0xffu) != 0 ? sc : -INFINITY;
+            } else if (m_esh == 1) {
+              const uint32_t hw = ((e < 2 ? w.x : w.y) >> (16 * (e & 1))) & 0xffffu;
+              const float mv = g.m_dt == FHIP_BFLOAT16
+                                   ? __builtin_bit_cast(float, hw << 16)
+                                   : (float)__builtin_bit_cast(_Float16, (uint16_t)hw);
+              s[kb][r] = __builtin_fmaf(mv, kLog2e, sc);
+            } else {
+              // (through a scalar: bit-casting a vector's element in place
+              // reads element 0)
+              const uint32_t word = e == 0 ? w.x : e == 1 ? w.y : e == 2 ? w.z : w.w;
+              s[kb][r] = __builtin_fmaf(__builtin_bit_cast(float, word), kLog2e, sc);
+            }
+          }
+      }
       const bool edge = (CAUSAL && kv0 + kBKV - 1 > qw0) || kv0 + kBKV > g.Skv;
       if (edge) {
+        // (masked kernels use -inf: a row may see dead keys before its first
+        // live one, and exp2(-inf - reference) is 0 whatever the reference)
+        const float gone = MASK ? -INFINITY : kNegBig;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int key = kv0 + kb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
             const bool dead = key >= g.Skv || (CAUSAL && key > qrow);
-            s[kb][r] = dead ? kNegBig : s[kb][r];
+            s[kb][r] = dead ? gone : s[kb][r];
           }
       }
       float mx = s[0][0];
@@ -494,19 +570,18 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
       // then at most 2^kMaxSlack, sums and outputs stay far inside float
       // range, and O = sum(p v) / sum(p) does not depend on the reference
       // point; the rescaling of O^T becomes rare.
-      const bool moved = (mx - m_run) * g.scale_log2e > kMaxSlack;
+      const bool moved = (mx - m_run) * sl2 > kMaxSlack;
       const float m_new = moved ? mx : m_run;
-      const float mc = m_new * g.scale_log2e;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * g.scale_log2e);
+      const float mc = m_new * sl2;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
       m_run = m_new;
       float psum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * g.scale_log2e - mc);
-          const float p1 =
-              __builtin_amdgcn_exp2f(s[kb][r + 1] * g.scale_log2e - mc);
+          const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * sl2 - mc);
+          const float p1 = __builtin_amdgcn_exp2f(s[kb][r + 1] * sl2 - mc);
           psum += p0 + p1;
           pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = sd_pack<BF16>(p0, p1);
         }
@@ -569,11 +644,42 @@ struct SdpaPlan {
   bool ok = false;
   bool bf16 = true;
   int hd = 128;
+  bool mask = false;
+  int64_t m_st[4] = {0, 0, 0, 0}; // mask strides over [B, Hq, Sq, Skv]
+  uint32_t m_bytes = 0;
 };
+
+// A mask the kernel can read: rank 4, boolean / f32 / bf16 / f16, unit key
+// stride, and every run of 4 keys a load fetches whole and aligned (extents
+// and the other strides multiples of 4), one (batch, head) slab below 2 GiB.
+bool plan_mask(const fhip_sdpa_desc *d, SdpaPlan &p) {
+  const fhip_tensor_desc &m = d->mask;
+  if (d->is_causal || m.rank != 4)
+    return false;
+  if (m.dtype != FHIP_BOOLEAN && m.dtype != FHIP_FLOAT &&
+      m.dtype != FHIP_BFLOAT16 && m.dtype != FHIP_HALF)
+    return false;
+  const int64_t dims[4] = {d->q.dim[0], d->q.dim[1], d->q.dim[2], d->k.dim[2]};
+  if (!fhip_broadcast_strides(m, 4, dims, p.m_st))
+    return false;
+  const int64_t Sq = dims[2], Skv = dims[3];
+  if (p.m_st[3] != 1 || Skv % 4 != 0)
+    return false;
+  for (int i = 0; i < 3; ++i)
+    if (p.m_st[i] < 0 || p.m_st[i] % 4 != 0)
+      return false;
+  const int64_t bytes =
+      ((Sq - 1) * p.m_st[2] + Skv) * (int64_t)fhip_dtype_size(m.dtype);
+  if (bytes >= (1ll << 31))
+    return false;
+  p.m_bytes = (uint32_t)bytes;
+  p.mask = true;
+  return true;
+}
 
 SdpaPlan make_plan(const fhip_sdpa_desc *d) {
   SdpaPlan p;
-  if (d->mask.rank != 0)
+  if (d->mask.rank != 0 && !plan_mask(d, p))
     return p;
   const int dt = d->q.dtype;
   if (dt != FHIP_BFLOAT16 && dt != FHIP_HALF)
@@ -617,7 +723,7 @@ bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d) {
 }
 
 int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
-                   const void *k, const void *v, void *o) {
+                   const void *k, const void *v, const void *mask, void *o) {
   const SdpaPlan p = make_plan(d);
   FHIP_REQUIRE(ctx, p.ok, "sdpa: descriptor not supported by the MFMA kernel");
   FHIP_REQUIRE(ctx,
@@ -640,6 +746,16 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   g.Skv = (int32_t)d->k.dim[2];
   g.group = (int32_t)(d->q.dim[1] / d->k.dim[1]);
   g.causal = d->is_causal;
+  if (p.mask) {
+    FHIP_REQUIRE(ctx, mask != nullptr, "sdpa: mask descriptor without a mask");
+    FHIP_REQUIRE(ctx,
+                 ((uintptr_t)mask & (4 * fhip_dtype_size(d->mask.dtype) - 1)) == 0,
+                 "sdpa: the mask must be aligned to four of its elements");
+    g.mask = (const char *)mask;
+    g.m_sb = p.m_st[0], g.m_sh = p.m_st[1], g.m_sq = p.m_st[2];
+    g.m_bytes = p.m_bytes;
+    g.m_dt = d->mask.dtype;
+  }
   const float scale =
       d->has_scale ? d->scale : 1.0f / sqrtf((float)d->q.dim[3]);
   g.scale_log2e = scale * 1.4426950408889634f;
@@ -659,19 +775,23 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
     FHIP_HIP_CHECK(ctx, hipGetLastError());
     return 0;
   };
-  // one flag per kernel instance: [head dim][type][causal]
-  static FhipOncePerDevice configured[2][2][2];
+  // one flag per kernel instance: [head dim][type][plain / causal / mask]
+  static FhipOncePerDevice configured[2][2][3];
   auto pick = [&](auto hd) {
     constexpr int HD = decltype(hd)::value;
-    FhipOncePerDevice(&cfg)[2][2] = configured[HD == 128];
+    FhipOncePerDevice(&cfg)[2][3] = configured[HD == 128];
     constexpr int lds = SdShape<HD>::kLdsB;
+    if (p.mask)
+      return p.bf16
+                 ? launch(sdpa_fwd_kernel<true, false, HD, true>, lds, cfg[1][2])
+                 : launch(sdpa_fwd_kernel<false, false, HD, true>, lds, cfg[0][2]);
     if (p.bf16)
       return d->is_causal
-                 ? launch(sdpa_fwd_kernel<true, true, HD>, lds, cfg[1][1])
-                 : launch(sdpa_fwd_kernel<true, false, HD>, lds, cfg[1][0]);
+                 ? launch(sdpa_fwd_kernel<true, true, HD, false>, lds, cfg[1][1])
+                 : launch(sdpa_fwd_kernel<true, false, HD, false>, lds, cfg[1][0]);
     return d->is_causal
-               ? launch(sdpa_fwd_kernel<false, true, HD>, lds, cfg[0][1])
-               : launch(sdpa_fwd_kernel<false, false, HD>, lds, cfg[0][0]);
+               ? launch(sdpa_fwd_kernel<false, true, HD, false>, lds, cfg[0][1])
+               : launch(sdpa_fwd_kernel<false, false, HD, false>, lds, cfg[0][0]);
   };
   return p.hd == 128 ? pick(std::integral_constant<int, 128>{})
                      : pick(std::integral_constant<int, 64>{});

@@ -1,8 +1,9 @@
 """Flash-attention forward (MFMA kernel) through the C ABI vs the oracle.
 
-Every case satisfies the tuned kernel's contract (bf16/f16, head dim 64 or 128,
-no mask tensor) and asserts that the tuned kernel is chosen, so a silent fall
-back to the generic kernel fails the test.
+Every case satisfies the tuned kernel's contract (bf16/f16, head dim 64 or 128;
+mask tensors with unit key stride and extents that are multiples of 4) and
+asserts that the tuned kernel is chosen, so a silent fall back to the generic
+kernel fails the test.
 """
 import numpy as np
 import pytest
@@ -14,17 +15,21 @@ from helpers import HT, assert_close, rand
 pytestmark = pytest.mark.gpu
 
 
-def run(ctx, q, k, v, causal=False, scale=None, o_strides=None, expect_tuned=True):
+def run(ctx, q, k, v, causal=False, scale=None, o_strides=None, expect_tuned=True,
+        mask=None):
     out = HT.empty([q.dims[0], q.dims[1], q.dims[2], v.dims[3]], q.dtype, o_strides)
     d = capi.SdpaDesc()
     d.q, d.k, d.v, d.o = q.desc(), k.desc(), v.desc(), out.desc()
+    if mask is not None:
+        d.mask = mask.desc()
     d.is_causal = int(causal)
     if scale is not None:
         d.has_scale, d.scale = 1, scale
     assert ctx.lib.fhip_sdpa_fwd_supported(d) == (2 if expect_tuned else 1)
     bufs = [t.upload(ctx) for t in (q, k, v)]
     dout = out.upload(ctx)
-    ctx.sdpa_fwd(d, bufs[0], bufs[1], bufs[2], dout)
+    dm = mask.upload(ctx) if mask is not None else None
+    ctx.sdpa_fwd(d, bufs[0], bufs[1], bufs[2], dout, mask=dm)
     return out.fetch(ctx, dout)
 
 
@@ -106,6 +111,78 @@ def test_flash_uniform_scores_causal_gives_prefix_means(ctx, hd):
     vl = v.logical()[0, 0]
     ref = np.cumsum(vl, axis=0) / np.arange(1, S + 1)[:, None]
     assert_close(out.logical()[0, 0], ref, capi.BFLOAT16)
+
+
+MASK_CASES = [
+    # the reference benchmark's shape: mask [B, 1, Sq, Skv] of the I/O type
+    dict(B=1, Hq=8, Hkv=8, Sq=64, Skv=64, mdims="b1qk"),
+    # ragged query tile, several key tiles with a partial last one
+    dict(B=2, Hq=3, Hkv=3, Sq=300, Skv=200, mdims="b1qk"),
+    # per-head masks, GQA, more than one query tile
+    dict(B=1, Hq=4, Hkv=2, Sq=513, Skv=260, mdims="bhqk"),
+    # one mask for every batch entry and head
+    dict(B=2, Hq=2, Hkv=2, Sq=130, Skv=132, mdims="11qk"),
+    # one mask row for every query (padding mask)
+    dict(B=2, Hq=2, Hkv=1, Sq=70, Skv=324, mdims="b11k"),
+]
+
+
+def mask_dims(c):
+    full = dict(b=c["B"], h=c["Hq"], q=c["Sq"], k=c["Skv"])
+    return [1 if ch == "1" else full[ch] for ch in c["mdims"]]
+
+
+@pytest.mark.parametrize("case", MASK_CASES)
+@pytest.mark.parametrize("kind", ["same", "f32", "bool"])
+@pytest.mark.parametrize("dtype,hd", [(capi.BFLOAT16, 128), (capi.HALF, 64),
+                                      (capi.HALF, 128), (capi.BFLOAT16, 64)])
+def test_flash_mask_vs_oracle(ctx, case, kind, dtype, hd):
+    c = case
+    q = HT.from_logical(rand(56, 0, [c["B"], c["Hq"], c["Sq"], hd]), dtype)
+    k = HT.from_logical(rand(56, 1, [c["B"], c["Hkv"], c["Skv"], hd]), dtype)
+    v = HT.from_logical(rand(56, 2, [c["B"], c["Hkv"], c["Skv"], hd]), dtype)
+    md = mask_dims(c)
+    if kind == "bool":
+        keep = rand(56, 3, md, "uniform") > 0.2
+        # whole key tiles masked at the front of some rows, no row without a key
+        keep[..., ::3, :128] = False
+        keep[..., -1] = True
+        mask, mref = HT.from_logical(keep, capi.BOOLEAN), keep
+    else:
+        mask = HT.from_logical(rand(56, 3, md) * 3.0,
+                               dtype if kind == "same" else capi.FLOAT)
+        mref = mask.logical()
+    out = run(ctx, q, k, v, mask=mask)
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), mask=mref)
+    assert_close(out.logical(), ref, dtype, f"{case} {kind}")
+
+
+def test_flash_mask_minus_infinity_and_dead_rows(ctx):
+    # additive -inf entries; a query with every key masked yields NaN, as
+    # softmax over an empty set does in aten, and leaves its neighbours alone
+    B, H, Sq, Skv, hd = 1, 2, 96, 128, 64
+    q = HT.from_logical(rand(57, 0, [B, H, Sq, hd]), capi.HALF)
+    k = HT.from_logical(rand(57, 1, [B, H, Skv, hd]), capi.HALF)
+    v = HT.from_logical(rand(57, 2, [B, H, Skv, hd]), capi.HALF)
+    m = rand(57, 3, [B, 1, Sq, Skv]).astype(np.float32)
+    m[..., 5:40] = -np.inf
+    m[0, 0, 17, :] = -np.inf
+    mask = HT.from_logical(m, capi.FLOAT)
+    out = run(ctx, q, k, v, mask=mask).logical()
+    assert np.all(np.isnan(out[:, :, 17, :]))
+    rows = np.arange(Sq) != 17
+    ref = oracle.sdpa(q.logical(), k.logical(), v.logical(), mask=m)
+    assert_close(out[:, :, rows, :], ref[:, :, rows, :], capi.HALF)
+
+
+def test_flash_mask_outside_contract_runs_generic(ctx):
+    # a key count that is no multiple of 4: mask rows are not 4-element aligned
+    q = HT.from_logical(rand(58, 0, [1, 2, 40, 64]), capi.HALF)
+    k = HT.from_logical(rand(58, 1, [1, 2, 66, 64]), capi.HALF)
+    mask = HT.from_logical(rand(58, 3, [1, 1, 40, 66]), capi.HALF)
+    out = run(ctx, q, k, k, mask=mask, expect_tuned=False)
+    ref = oracle.sdpa(q.logical(), k.logical(), k.logical(), mask=mask.logical())
+    assert_close(out.logical(), ref, capi.HALF)
 
 
 def test_flash_not_chosen_outside_contract(ctx):
