@@ -62,6 +62,19 @@ int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
                                 const void *dy, const void *x, void *dw,
                                 void *workspace);
 
+// Register-blocked direct kernels for any layout, dtype, group count and 1 - 3
+// spatial dims (conv_direct.hip): the path of the convolutions the MFMA
+// kernels do not take.  The weight gradient keeps its partial sums in the
+// context's scratch buffer.
+bool fhip_direct_conv_applicable(const fhip_conv_desc *d);
+int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
+                           const void *x, const void *w, const DevEpilogue &epi,
+                           void *out);
+int fhip_direct_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d,
+                           const void *dy, const void *w, void *dx);
+int fhip_direct_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d,
+                           const void *dy, const void *x, void *dw);
+
 bool fhip_fast_sdpa_applicable(const fhip_sdpa_desc *d);
 int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
                    const void *k, const void *v, const void *mask, void *o);

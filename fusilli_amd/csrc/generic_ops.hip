@@ -93,15 +93,17 @@ __global__ void generic_matmul_kernel(MatmulArgs g, const void *a,
   fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
 }
 
-// f32 x f32 matmul on the f32 matrix instruction (v_mfma_f32_32x32x2_f32), any
-// strides, batch broadcasting and epilogue of the strided kernel above.  A
+// Floating-point matmul on the f32 matrix instruction (v_mfma_f32_32x32x2_f32):
+// any strides, batch broadcasting and epilogue of the strided kernel above;
+// f32, bf16 and f16 operands (also mixed) are widened to f32 as they are
+// staged, which is exact.  A
 // workgroup of 4 wavefronts owns a 64 x 64 output tile of one batch entry and
 // walks K in steps of 16 through LDS (As[k][m], Bs[k][n]); the next step's
 // global loads are in flight while the current one is multiplied.
 constexpr int kF32Tile = 64, kF32K = 16, kF32Pitch = kF32Tile + 4;
 
 __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
-    MatmulArgs g, const float *a, const float *b, void *out, int tiles_n) {
+    MatmulArgs g, const void *a, const void *b, void *out, int tiles_n) {
   typedef float f32x16 __attribute__((ext_vector_type(16)));
   __shared__ float As[kF32K][kF32Pitch], Bs[kF32K][kF32Pitch];
   const int rank = g.out.rank;
@@ -142,8 +144,12 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
     for (int i = 0; i < 4; ++i) {
       const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
       const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
-      ra[i] = m < M && ka < g.K ? a[ab + m * a_sm + ka * g.a_k] : 0.f;
-      rb[i] = n < N && kb < g.K ? b[bb + n * b_sn + kb * g.b_k] : 0.f;
+      ra[i] = m < M && ka < g.K
+                  ? fhip_load<float>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
+                  : 0.f;
+      rb[i] = n < N && kb < g.K
+                  ? fhip_load<float>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
+                  : 0.f;
     }
   };
   f32x16 acc;
@@ -192,7 +198,7 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
 // the partial sums meet in LDS and every wavefront finishes a quarter of the
 // accumulator registers.
 __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
-    MatmulArgs g, const float *a, const float *b, void *out, int tiles_n) {
+    MatmulArgs g, const void *a, const void *b, void *out, int tiles_n) {
   typedef float f32x16 __attribute__((ext_vector_type(16)));
   constexpr int T = 32, PITCH = T + 4;
   __shared__ float As[4][kF32K][PITCH], Bs[4][kF32K][PITCH];
@@ -232,8 +238,12 @@ __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
     for (int i = 0; i < 8; ++i) {
       const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
       const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
-      ra[i] = m < M && ka < g.K ? a[ab + m * a_sm + ka * g.a_k] : 0.f;
-      rb[i] = n < N && kb < g.K ? b[bb + n * b_sn + kb * g.b_k] : 0.f;
+      ra[i] = m < M && ka < g.K
+                  ? fhip_load<float>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
+                  : 0.f;
+      rb[i] = n < N && kb < g.K
+                  ? fhip_load<float>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
+                  : 0.f;
     }
   };
   f32x16 acc;
@@ -798,19 +808,38 @@ __device__ __forceinline__ CT red_combine(int kind, CT a, CT b) {
   return a + b;
 }
 
-template <typename CT>
-__global__ __launch_bounds__(256) void generic_reduce_kernel(ReduceArgs g,
-                                                             const void *x,
-                                                             void *y) {
+// One workgroup per output element and slice of the reduced index range
+// (gridDim.y slices of `per_slice` indices; with several slices the
+// workgroup's result goes to partial[slice][output] for
+// generic_reduce_finish_kernel).  SMALL: the reduced index fits 32 bits, and
+// the index arithmetic runs in them.
+template <typename CT, bool SMALL>
+__global__ __launch_bounds__(256) void generic_reduce_kernel(
+    ReduceArgs g, const void *x, void *y, CT *partial, int64_t per_slice) {
   __shared__ CT lds[256];
   int64_t ocoord[FHIP_MAX_RANK], rcoord[FHIP_MAX_RANK];
   unravel((int64_t)blockIdx.x, g.y, ocoord);
   const int rank = g.y.rank;
   const int64_t base = dot(ocoord, g.xs, rank);
   CT acc = (CT)g.identity;
-  for (int64_t i = threadIdx.x; i < g.red_count; i += blockDim.x) {
-    unravel(i, g.red, rcoord);
-    const CT v = fhip_load<CT>(x, g.x_dt, base + dot(rcoord, g.xs, rank));
+  const int64_t first = (int64_t)blockIdx.y * per_slice;
+  const int64_t last =
+      first + per_slice < g.red_count ? first + per_slice : g.red_count;
+  for (int64_t i = first + threadIdx.x; i < last; i += blockDim.x) {
+    int64_t off = base;
+    if (SMALL) {
+      uint32_t rem = (uint32_t)i;
+      for (int r = rank - 1; r >= 0; --r) {
+        const uint32_t dim = (uint32_t)g.red.dim[r];
+        const uint32_t q = rem / dim;
+        off += (int64_t)(rem - q * dim) * g.xs.s[r];
+        rem = q;
+      }
+    } else {
+      unravel(i, g.red, rcoord);
+      off += dot(rcoord, g.xs, rank);
+    }
+    const CT v = fhip_load<CT>(x, g.x_dt, off);
     acc = red_combine<CT>(g.comb_kind, acc, red_map<CT>(g.map_kind, v));
   }
   lds[threadIdx.x] = acc;
@@ -823,12 +852,35 @@ __global__ __launch_bounds__(256) void generic_reduce_kernel(ReduceArgs g,
   }
   if (threadIdx.x == 0) {
     CT r = lds[0];
+    if (gridDim.y > 1) {
+      partial[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = r;
+      return;
+    }
     if (g.post_kind == RPOST_MEAN)
       r = r / (CT)g.red_count;
     else if (g.post_kind == RPOST_SQRT)
       r = sqrt(r);
     fhip_store<CT>(y, g.y_dt, dot(ocoord, g.ys, rank), r);
   }
+}
+
+// Combines the slices' results of one output element in slice order.
+template <typename CT>
+__global__ __launch_bounds__(256) void generic_reduce_finish_kernel(
+    ReduceArgs g, const CT *partial, void *y, int64_t outs, int slices) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= outs)
+    return;
+  CT r = partial[o];
+  for (int s = 1; s < slices; ++s)
+    r = red_combine<CT>(g.comb_kind, r, partial[(int64_t)s * outs + o]);
+  if (g.post_kind == RPOST_MEAN)
+    r = r / (CT)g.red_count;
+  else if (g.post_kind == RPOST_SQRT)
+    r = sqrt(r);
+  int64_t ocoord[FHIP_MAX_RANK];
+  unravel(o, g.y, ocoord);
+  fhip_store<CT>(y, g.y_dt, dot(ocoord, g.ys, g.y.rank), r);
 }
 
 // --------------------------------------------------------------------------
@@ -1047,7 +1099,10 @@ int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
   g.o_dt = d->out.dtype;
   g.epi = epi;
   const int64_t total = fhip_desc_volume(d->c);
-  if (d->a.dtype == FHIP_FLOAT && d->b.dtype == FHIP_FLOAT) {
+  auto widens = [](int dt) {
+    return dt == FHIP_FLOAT || dt == FHIP_BFLOAT16 || dt == FHIP_HALF;
+  };
+  if (widens(d->a.dtype) && widens(d->b.dtype)) {
     const int64_t M = d->c.dim[r - 2], N = d->c.dim[r - 1];
     const int64_t tm = (M + kF32Tile - 1) / kF32Tile, tn = (N + kF32Tile - 1) / kF32Tile;
     const int64_t batch = total / (M * N);
@@ -1057,15 +1112,13 @@ int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
       // few tiles: 32 x 32 tiles with K split over the wavefronts
       hipLaunchKernelGGL(splitk_matmul_f32_kernel,
                          dim3((unsigned)(sm * sn), (unsigned)batch), dim3(256),
-                         0, ctx->stream, g, (const float *)a, (const float *)b,
-                         out, (int)sn);
+                         0, ctx->stream, g, a, b, out, (int)sn);
       FHIP_HIP_CHECK(ctx, hipGetLastError());
       return 0;
     }
     if (tm * tn < (1ll << 31) && batch <= 65535 && tn < (1ll << 31)) {
       hipLaunchKernelGGL(tiled_matmul_f32_kernel, dim3((unsigned)(tm * tn), (unsigned)batch),
-                         dim3(256), 0, ctx->stream, g, (const float *)a,
-                         (const float *)b, out, (int)tn);
+                         dim3(256), 0, ctx->stream, g, a, b, out, (int)tn);
       FHIP_HIP_CHECK(ctx, hipGetLastError());
       return 0;
     }
@@ -1158,6 +1211,8 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     return 1;
   if (tuned)
     return 0;
+  if (fhip_direct_conv_applicable(d))
+    return fhip_direct_conv_fprop(ctx, d, x, w, epi, out);
 
   ConvArgs g{};
   g.y = make_dims(d->y);
@@ -1284,6 +1339,8 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                  need, workspace ? workspace_bytes : (size_t)0);
     return fhip_fast_conv_dgrad(ctx, d, dy, w, dx, workspace);
   }
+  if (fhip_direct_conv_applicable(d))
+    return fhip_direct_conv_dgrad(ctx, d, dy, w, dx);
   const ConvBwdArgs g = conv_bwd_args(d, true);
   const int64_t total = fhip_desc_volume(d->x);
   hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),
@@ -1310,7 +1367,9 @@ int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
                  "fhip_conv_dgrad_static: scratch address not resolved");
     return fhip_fast_conv_dgrad(ctx, d, dy, w, dx, ctx->dgrad_static_scratch);
   }
-  // the strided kernel uses no scratch at all
+  // the direct and the strided kernel use no scratch at all
+  if (fhip_direct_conv_applicable(d))
+    return fhip_direct_conv_dgrad(ctx, d, dy, w, dx);
   const ConvBwdArgs g = conv_bwd_args(d, true);
   const int64_t total = fhip_desc_volume(d->x);
   hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),
@@ -1372,6 +1431,8 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   (void)workspace;
   (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  if (fhip_direct_conv_applicable(d))
+    return fhip_direct_conv_wgrad(ctx, d, dy, x, dw);
   const ConvBwdArgs g = conv_bwd_args(d, false);
   if (fhip_desc_volume(d->w) == 0)
     return 0;
@@ -1811,12 +1872,43 @@ int fhip_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
     break;
   }
   const int64_t outs = fhip_desc_volume(d->y);
-  if (needs_double(d->x.dtype))
-    hipLaunchKernelGGL(generic_reduce_kernel<double>, dim3((unsigned)outs),
-                       dim3(256), 0, ctx->stream, g, x, y);
-  else
-    hipLaunchKernelGGL(generic_reduce_kernel<float>, dim3((unsigned)outs),
-                       dim3(256), 0, ctx->stream, g, x, y);
+  if (outs == 0)
+    return 0;
+  // few outputs over long ranges: slices of the range on workgroups of their
+  // own (about two workgroups per compute unit, at least 2048 indices each),
+  // combined in slice order by a second kernel
+  const int64_t cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+  int64_t slices = 2 * cus / outs;
+  const int64_t most = g.red_count / 2048;
+  slices = slices < most ? slices : most;
+  slices = slices < 1024 ? slices : 1024;
+  slices = slices < 1 ? 1 : slices;
+  int64_t per_slice = (g.red_count + slices - 1) / slices;
+  per_slice = per_slice < 1 ? 1 : per_slice;
+  slices = g.red_count > 0 ? (g.red_count + per_slice - 1) / per_slice : 1;
+  const bool small = g.red_count < (1ll << 31);
+  const dim3 grid((unsigned)outs, (unsigned)slices);
+  auto run = [&](auto zero) {
+    using CT = decltype(zero);
+    void *scratch = nullptr;
+    if (slices > 1 &&
+        fhip_ctx_scratch(ctx, (size_t)(slices * outs) * sizeof(CT), &scratch) != 0)
+      return 1;
+    if (small)
+      hipLaunchKernelGGL((generic_reduce_kernel<CT, true>), grid, dim3(256), 0,
+                         ctx->stream, g, x, y, (CT *)scratch, per_slice);
+    else
+      hipLaunchKernelGGL((generic_reduce_kernel<CT, false>), grid, dim3(256), 0,
+                         ctx->stream, g, x, y, (CT *)scratch, per_slice);
+    if (slices > 1)
+      hipLaunchKernelGGL(generic_reduce_finish_kernel<CT>,
+                         dim3((unsigned)((outs + 255) / 256)), dim3(256), 0,
+                         ctx->stream, g, (const CT *)scratch, y, outs,
+                         (int)slices);
+    return 0;
+  };
+  if ((needs_double(d->x.dtype) ? run(0.0) : run(0.f)) != 0)
+    return 1;
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;
 }
