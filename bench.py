@@ -389,26 +389,94 @@ def bench_layernorm(ctx, steps, warmup, sets=5):
             "kernel_us": round(ev_ms * 1e3, 2), "bytes": nbytes}
 
 
-def bench_sdpa(ctx, steps, warmup, b=4, h=32, sq=2048, d=128):
-    """C4: SDPA forward bf16 causal B4 H32 S2048 D128 ([B,H,S,D] contiguous)."""
+def bench_sdpa(ctx, steps, warmup, b=4, h=32, sq=2048, d=128, masked=False):
+    """C4: SDPA forward bf16 causal B4 H32 S2048 D128 ([B,H,S,D] contiguous);
+    `masked`: the same tensors under an additive bf16 mask [B,1,S,S] (shared
+    by the heads, as the reference's benchmark driver builds it) instead of
+    the causal flag."""
     dims = [b, h, sq, d]
     strides = [h * sq * d, sq * d, d, 1]
     desc = capi.SdpaDesc()
     desc.q = desc.k = desc.v = desc.o = capi.TensorDesc.make(dims, strides, capi.BFLOAT16)
-    desc.is_causal = 1
+    desc.is_causal = 0 if masked else 1
+    mask = None
+    if masked:
+        desc.mask = capi.TensorDesc.make([b, 1, sq, sq], [sq * sq, sq * sq, sq, 1],
+                                         capi.BFLOAT16)
+        mask = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(9, 7, b * sq * sq)))
     assert ctx.lib.fhip_sdpa_fwd_supported(desc) == 2, "MFMA SDPA not chosen"
     n = b * h * sq * d
     q, k, v = (ctx.to_device(synth.f32_to_bf16_bits(synth.normal(9, i, n)))
                for i in range(3))
     out = ctx.alloc(n * 2)
-    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.sdpa_fwd(desc, q, k, v, out),
-                                steps, warmup)
+    wall_ms, ev_ms = timed_loop(
+        ctx, lambda i: ctx.sdpa_fwd(desc, q, k, v, out, mask=mask), steps, warmup)
     # causal: only the lower triangle of the S x S score matrix is computed
-    flop = 4.0 * b * h * sq * sq * d / 2
+    flop = 4.0 * b * h * sq * sq * d / (1 if masked else 2)
     return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
             "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
             "kernel_us": round(ev_ms * 1e3, 2), "work": flop,
-            "flop_convention": "4*B*H*S*S*D/2 (causal half)"}
+            "flop_convention": "4*B*H*S*S*D" + ("" if masked else "/2 (causal half)")}
+
+
+def bench_layernorm_long(ctx, steps, warmup, rows=16, cols=128 * 64 * 32):
+    """The reference benchmark's LayerNorm shape, 16 x (128 * 64 * 32) bf16
+    with scale and bias: rows of 262144 elements, normalised by two kernels
+    per call (segment statistics, then the normalisation)."""
+    d = capi.NormDesc()
+    d.x = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.scale = capi.TensorDesc.make([1, cols], [cols, 1], capi.BFLOAT16)
+    d.bias = capi.TensorDesc.make([1, cols], [cols, 1], capi.BFLOAT16)
+    d.y = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.out = capi.TensorDesc.make([rows, cols], [cols, 1], capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.epsilon = 1e-5
+    d.is_layernorm = 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_norm_fwd_supported(d) == 2, "long-row norm not chosen"
+    n = rows * cols
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(12, 0, n)))
+    scale = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(12, 1, cols, 1.0, 0.02)))
+    bias = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(12, 2, cols, 0.0, 0.02)))
+    y = ctx.alloc(n * 2)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.norm_fwd(d, x, scale, bias, y),
+                                steps, warmup)
+    nbytes = 2 * n * 2 + 2 * cols * 2
+    return {"value": round(nbytes / ev_ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "call_us": round(ev_ms * 1e3, 2), "bytes": nbytes, "kernels_per_call": 2,
+            "note": "8 MB of X: the whole call is a few launch latencies long"}
+
+
+def bench_conv_padded(ctx, steps, warmup):
+    """The reference benchmark's conv2d_nhwc_fp16 shape: N16 C48 48x32, K48
+    3x3, padding 2 -- a channel count that is no multiple of 64, so X and W
+    are first copied into zero-padded 64-channel tensors (3 kernels per call)."""
+    n, c, h, w, k, r, pad = 16, 48, 48, 32, 48, 3, 2
+    p, q = h + 2 * pad - (r - 1), w + 2 * pad - (r - 1)
+    cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
+    xd, wd, yd = [n, c, h, w], [k, c, r, r], [n, k, p, q]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.HALF)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.HALF)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.HALF)
+    d.out = capi.TensorDesc.make(yd, cl(yd), capi.HALF)
+    d.out_dtype = capi.HALF
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = pad, 1, 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_conv_fprop_supported(d) == 2, "MFMA conv not chosen"
+    x = ctx.to_device(synth.normal(8, 3, n * c * h * w).astype(np.float16))
+    wt = ctx.to_device(synth.normal(8, 4, k * c * r * r, 0.0, 0.05).astype(np.float16))
+    out = ctx.alloc(n * k * p * q * 2)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.conv_fprop(d, x, wt, out),
+                                steps, warmup)
+    flop = 2.0 * n * p * q * k * c * r * r
+    return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
+            "call_us": round(ev_ms * 1e3, 2), "work": flop, "kernels_per_call": 3,
+            "note": "1.4 GFLOP: launch-latency bound"}
 
 
 def calibrate_copy(ctx, steps):
@@ -624,6 +692,12 @@ def main():
              lambda: bench_conv_wgrad(ctx, max(20, args.steps // 10), kwarm)),
             ("sdpa_fwd_bf16_causal_b4h32s2048d128",
              lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm)),
+            ("sdpa_fwd_bf16_mask_b4h32s2048d128",
+             lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm, masked=True)),
+            ("layernorm_bf16_16x262144_long_rows",
+             lambda: bench_layernorm_long(ctx, max(20, args.steps // 4), kwarm)),
+            ("conv_fprop_f16_n16c48h48w32_k48r3s3_padded_channels",
+             lambda: bench_conv_padded(ctx, max(20, args.steps // 4), kwarm)),
         ]
         wanted = [w for w in args.only.split(",") if w]
         for name, fn in lines:

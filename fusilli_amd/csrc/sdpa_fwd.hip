@@ -16,9 +16,12 @@
 //   * causal workgroups stop at the diagonal, and a wavefront skips tiles that
 //     lie wholly above its own rows;
 //   * a mask tensor (boolean, or additive in f32 / bf16 / f16, broadcast over
-//     batch and heads as its dims say) is read straight into registers, four
-//     consecutive keys per load, at the top of a round -- one MFMA phase ahead
-//     of the softmax that folds it into the scores;
+//     batch and heads as its dims say): every wavefront brings the 32 x 64
+//     mask elements of its next tile into an LDS region of its own by LDS-DMA
+//     (whole rows, coalesced) and reads them back in the score layout, four
+//     consecutive keys per lane and read, one MFMA phase after the load was
+//     issued; masks whose rows are not 16-byte aligned are read straight into
+//     registers instead (MASK == 1), four keys per load;
 //   * the two wavefronts of a SIMD (w and w + 4) alternate: a tile is an MFMA
 //     phase (S^T of tile t and the O^T update of tile t - 1, 32 MFMAs) and a
 //     vector-ALU phase (online softmax of tile t) of about equal length,
@@ -68,6 +71,9 @@ template <int HD> struct SdShape {
   static constexpr int kLdsB = kRingB > kWaves * 32 * kOutPitch
                                    ? kRingB
                                    : kWaves * 32 * kOutPitch;
+  // kernels that stage the mask: 8 KB per wavefront behind the rings
+  static constexpr int kMaskB = 8192;
+  static constexpr int kLdsMaskB = kLdsB + kWaves * kMaskB;
 };
 
 struct SdpaArgs {
@@ -80,6 +86,7 @@ struct SdpaArgs {
   int32_t Sq, Skv, group; // group = Hq / Hkv
   int32_t causal;
   float scale_log2e; // softmax scale * log2(e)
+  float scale;       // softmax scale
   // mask tensor (kernels with MASK): strides in elements, 0 where broadcast;
   // the key stride is 1
   const char *mask;
@@ -182,6 +189,14 @@ __device__ __forceinline__ void sd_read_tr16(u32x2 &dst, uint32_t addr) {
                : "v"(addr), "n"(OFFSET));
 }
 template <int OFFSET>
+__device__ __forceinline__ void sd_read_b32(uint32_t &dst, uint32_t addr) {
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET));
+}
+template <int OFFSET>
+__device__ __forceinline__ void sd_read_b64(u32x2 &dst, uint32_t addr) {
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFFSET));
+}
+template <int OFFSET>
 __device__ __forceinline__ void sd_read_b128(u32x4 &dst, uint32_t addr) {
   static_assert(OFFSET >= 0 && OFFSET < 65536, "16-bit offset field");
   asm volatile("ds_read_b128 %0, %1 offset:%2"
@@ -222,7 +237,8 @@ __device__ __forceinline__ void sd_barrier() {
   asm volatile("" ::: "memory");
 }
 
-template <bool BF16, bool CAUSAL, int HD, bool MASK>
+// MASK: 0 no mask tensor, 1 mask read into registers, 2 mask staged in LDS
+template <bool BF16, bool CAUSAL, int HD, int MASK>
 __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   static_assert(!(CAUSAL && MASK), "a mask tensor excludes the causal flag");
   using C = SdShape<HD>;
@@ -306,33 +322,81 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   const __amdgpu_buffer_rsrc_t k_rsrc = slab_rsrc(kp, k_bytes);
   const __amdgpu_buffer_rsrc_t v_rsrc = slab_rsrc(vp, v_bytes);
   // Mask: a lane's 32 scores of a tile are 8 runs of 4 consecutive keys (run i
-  // starts at key 32 * (i / 4) + 8 * (i % 4) + 4 * half), one load each; the
-  // element size picks the load width.  Runs past the slab's end read as
-  // zeros; their keys are dead anyway.
+  // starts at key 32 * (i / 4) + 8 * (i % 4) + 4 * half); the element size
+  // picks the access width.  Runs past the slab's end read as zeros; their
+  // keys are dead anyway.
   const int m_esh = !MASK ? 0 : g.m_dt == FHIP_BOOLEAN ? 0 : g.m_dt == FHIP_FLOAT ? 2 : 1;
   __amdgpu_buffer_rsrc_t m_rsrc = k_rsrc;
-  uint32_t m_off = 0;
-  if constexpr (MASK) {
+  if constexpr (MASK != 0)
     m_rsrc = slab_rsrc(g.mask + ((b * g.m_sb + h * g.m_sh) << m_esh), g.m_bytes);
+  // MASK == 1: one register load per run, issued at the top of a round
+  uint32_t m_off = 0;
+  if constexpr (MASK == 1) {
     const int qr = qrow < g.Sq ? qrow : g.Sq - 1;
     m_off = (uint32_t)(((int64_t)qr * g.m_sq + half * 4) << m_esh);
   }
-  u32x4 mraw[MASK ? 8 : 1];
+  u32x4 mreg[MASK == 1 ? 8 : 1];
   auto load_mask = [&](int t) {
     const int so = (t * kBKV) << m_esh;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int run = 32 * (i / 4) + 8 * (i % 4);
       if (m_esh == 0) {
-        mraw[i].x = __builtin_amdgcn_raw_buffer_load_b32(m_rsrc, (int)m_off + run, so, 0);
+        mreg[i].x = __builtin_amdgcn_raw_buffer_load_b32(m_rsrc, (int)m_off + run, so, 0);
       } else if (m_esh == 1) {
         const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(m_rsrc, (int)m_off + run * 2, so, 0);
-        mraw[i].x = v.x;
-        mraw[i].y = v.y;
+        mreg[i].x = v.x;
+        mreg[i].y = v.y;
       } else {
-        mraw[i] = __builtin_amdgcn_raw_buffer_load_b128(m_rsrc, (int)m_off + run * 4, so, 0);
+        mreg[i] = __builtin_amdgcn_raw_buffer_load_b128(m_rsrc, (int)m_off + run * 4, so, 0);
       }
     }
+  };
+  // MASK == 2: the tile's 32 rows of 64 elements go to this wavefront's LDS
+  // region by LDS-DMA, 1 KB (16 / 8 / 4 whole rows) per instruction; chunk c of
+  // row r sits at position c ^ ((r / 2) % chunks-per-row), which spreads the
+  // runs that the lanes of a read touch over the banks.
+  const uint32_t m_lds = lds0 + (uint32_t)C::kLdsB + (uint32_t)wave * C::kMaskB;
+  uint32_t m_dma[MASK == 2 ? 8 : 1]; // lane offsets of the DMA instructions
+  uint32_t m_rd[MASK == 2 ? 8 : 1];  // LDS address of this lane's run i
+  if constexpr (MASK == 2) {
+    const int cpr = 4 << m_esh;        // 16-byte chunks per row
+    const int rows_per = 64 / cpr;     // rows per instruction
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = j * rows_per + l / cpr;
+      const int c = (l % cpr) ^ ((row >> 1) & (cpr - 1));
+      const int qr = qw0 + row < g.Sq ? qw0 + row : g.Sq - 1;
+      m_dma[j] = (uint32_t)((((int64_t)qr * g.m_sq) << m_esh) + c * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int bo = (32 * (i / 4) + 8 * (i % 4) + 4 * half) << m_esh;
+      const int c = (bo >> 4) ^ ((lq >> 1) & (cpr - 1));
+      m_rd[i] = m_lds + (uint32_t)(lq * (64 << m_esh) + (c << 4) + (bo & 15));
+    }
+  }
+  auto issue_mask = [&](int t) {
+    const int so = t < tiles ? (t * kBKV) << m_esh : 0;
+    const int n = 2 << m_esh; // instructions per tile
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < n)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            m_rsrc,
+            (SD_AS3 char *)(uintptr_t)__builtin_amdgcn_readfirstlane(m_lds + j * 1024u),
+            16, (int)m_dma[j], so, 0, 0);
+  };
+  // the staged loads still in flight next to the K / V loads of a round
+  auto wait_all_but_round = [&]() {
+    if (MASK != 2)
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+    else if (m_esh == 0)
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile + 2));
+    else if (m_esh == 1)
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile + 4));
+    else
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile + 8));
   };
   auto issue_kv = [&](const __amdgpu_buffer_rsrc_t &r, uint32_t tile_bytes,
                       const uint32_t (&off)[kLoadsPerTile], int t,
@@ -402,6 +466,8 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   // the top of round t (K tile t + 2, V tile t + 1) reuse the stages of K tile
   // t - 1 and V tile t - 2 and have to land by barrier t + 1.
   const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
+  if constexpr (MASK == 2)
+    issue_mask(0); // older than every K / V load: landed by the first wait
   issue_k(0, 0);
   issue_v(0, 0);
   issue_k(1, 1);
@@ -420,7 +486,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
 #pragma clang loop unroll(disable)
   for (int t = 0; t <= tiles; ++t) {
     // (the mask first: the waits below count the K / V loads issued after it)
-    if constexpr (MASK)
+    if constexpr (MASK == 1)
       if (t < tiles)
         load_mask(t);
     issue_k(t + 2, sl_prev);
@@ -516,32 +582,80 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     if (active(t)) {
       const int kv0 = t * kBKV;
       // with a mask the scores are scaled here, with the mask folded in, and
-      // the softmax below runs on them with unit scale
-      const float sl2 = MASK ? 1.0f : g.scale_log2e;
-      if constexpr (MASK) {
-        constexpr float kLog2e = 1.4426950408889634f;
+      // the softmax below converts them to log2 units
+      const float sl2 = MASK ? 1.4426950408889634f : g.scale_log2e;
+      if constexpr (MASK != 0) {
+        // s <- s * scale + mask, or -inf where a boolean mask is false (one
+        // multiply-add per score; the softmax below then runs in natural-log
+        // units, its scale being log2(e))
+        auto fold = [&](const u32x4 (&mraw)[8]) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+          for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const u32x4 w = mraw[kb * 4 + (r >> 2)];
-            const int e = r & 3;
-            const float sc = s[kb][r] * g.scale_log2e;
-            if (m_esh == 0) {
-              s[kb][r] = ((w.x >> (8 * e)) & 0xffu) != 0 ? sc : -INFINITY;
-            } else if (m_esh == 1) {
-              const uint32_t hw = ((e < 2 ? w.x : w.y) >> (16 * (e & 1))) & 0xffffu;
-              const float mv = g.m_dt == FHIP_BFLOAT16
-                                   ? __builtin_bit_cast(float, hw << 16)
-                                   : (float)__builtin_bit_cast(_Float16, (uint16_t)hw);
-              s[kb][r] = __builtin_fmaf(mv, kLog2e, sc);
-            } else {
-              // (through a scalar: bit-casting a vector's element in place
-              // reads element 0)
-              const uint32_t word = e == 0 ? w.x : e == 1 ? w.y : e == 2 ? w.z : w.w;
-              s[kb][r] = __builtin_fmaf(__builtin_bit_cast(float, word), kLog2e, sc);
+            for (int r = 0; r < 16; ++r) {
+              const u32x4 w = mraw[kb * 4 + (r >> 2)];
+              const int e = r & 3;
+              if (m_esh == 0) {
+                s[kb][r] = ((w.x >> (8 * e)) & 0xffu) != 0 ? s[kb][r] * g.scale
+                                                           : -INFINITY;
+              } else if (m_esh == 1) {
+                const uint32_t word = e < 2 ? w.x : w.y;
+                float mv;
+                if (g.m_dt == FHIP_BFLOAT16)
+                  mv = __builtin_bit_cast(float, (e & 1) ? (word & 0xffff0000u)
+                                                         : (word << 16));
+                else
+                  mv = (float)__builtin_bit_cast(
+                      _Float16, (uint16_t)((e & 1) ? word >> 16 : word));
+                s[kb][r] = __builtin_fmaf(s[kb][r], g.scale, mv);
+              } else {
+                // (through a scalar: bit-casting a vector's element in place
+                // reads element 0)
+                const uint32_t word = e == 0 ? w.x : e == 1 ? w.y : e == 2 ? w.z : w.w;
+                s[kb][r] = __builtin_fmaf(s[kb][r], g.scale,
+                                          __builtin_bit_cast(float, word));
+              }
             }
+        };
+        if constexpr (MASK == 1) {
+          fold(mreg);
+        } else {
+          u32x4 mraw[8];
+          // the tile's mask was issued a round ago, before this round's K / V
+          __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+          asm volatile("" ::: "memory");
+          if (m_esh == 2) {
+            sd_static_for<8>([&](auto ic) {
+              sd_read_b128<0>(mraw[decltype(ic)::value], m_rd[decltype(ic)::value]);
+            });
+            sd_wait_pin<0>(mraw[0], mraw[1], mraw[2], mraw[3], mraw[4], mraw[5],
+                           mraw[6], mraw[7]);
+          } else if (m_esh == 1) {
+            u32x2 t2[8];
+            sd_static_for<8>([&](auto ic) {
+              sd_read_b64<0>(t2[decltype(ic)::value], m_rd[decltype(ic)::value]);
+            });
+            sd_wait_pin<0>(t2[0], t2[1], t2[2], t2[3], t2[4], t2[5], t2[6], t2[7]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              mraw[i].x = t2[i].x;
+              mraw[i].y = t2[i].y;
+            }
+          } else {
+            uint32_t t1[8];
+            sd_static_for<8>([&](auto ic) {
+              sd_read_b32<0>(t1[decltype(ic)::value], m_rd[decltype(ic)::value]);
+            });
+            sd_wait_pin<0>(t1[0], t1[1], t1[2], t1[3], t1[4], t1[5], t1[6], t1[7]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              mraw[i].x = t1[i];
           }
+          // the region is free again: next tile's mask (younger than this
+          // round's K / V loads, so the waits at the barriers leave it alone)
+          issue_mask(t + 1);
+          fold(mraw);
+        }
       }
       const bool edge = (CAUSAL && kv0 + kBKV - 1 > qw0) || kv0 + kBKV > g.Skv;
       if (edge) {
@@ -597,7 +711,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     }
     // wavefronts 0..3 end their round here
     if (!team) {
-      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+      wait_all_but_round();
       sd_barrier();
     }
     sl_prev = sl_cur;
@@ -645,6 +759,7 @@ struct SdpaPlan {
   bool bf16 = true;
   int hd = 128;
   bool mask = false;
+  bool mask_rows16 = false;       // every mask row starts and ends on 16 bytes
   int64_t m_st[4] = {0, 0, 0, 0}; // mask strides over [B, Hq, Sq, Skv]
   uint32_t m_bytes = 0;
 };
@@ -674,6 +789,10 @@ bool plan_mask(const fhip_sdpa_desc *d, SdpaPlan &p) {
     return false;
   p.m_bytes = (uint32_t)bytes;
   p.mask = true;
+  const int64_t es = (int64_t)fhip_dtype_size(m.dtype);
+  p.mask_rows16 = Skv * es % 16 == 0;
+  for (int i = 0; i < 3; ++i)
+    p.mask_rows16 = p.mask_rows16 && p.m_st[i] * es % 16 == 0;
   return true;
 }
 
@@ -730,6 +849,7 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
                (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) &
                 15) == 0,
                "sdpa: Q, K, V, O must be 16-byte aligned");
+  bool staged_mask = false;
   SdpaArgs g{};
   g.q = (const char *)q;
   g.k = (const char *)k;
@@ -751,6 +871,7 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
     FHIP_REQUIRE(ctx,
                  ((uintptr_t)mask & (4 * fhip_dtype_size(d->mask.dtype) - 1)) == 0,
                  "sdpa: the mask must be aligned to four of its elements");
+    staged_mask = p.mask_rows16 && ((uintptr_t)mask & 15) == 0;
     g.mask = (const char *)mask;
     g.m_sb = p.m_st[0], g.m_sh = p.m_st[1], g.m_sq = p.m_st[2];
     g.m_bytes = p.m_bytes;
@@ -759,6 +880,7 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   const float scale =
       d->has_scale ? d->scale : 1.0f / sqrtf((float)d->q.dim[3]);
   g.scale_log2e = scale * 1.4426950408889634f;
+  g.scale = scale;
   const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
   const dim3 grid((unsigned)d->q.dim[1], (unsigned)d->q.dim[0],
                   (unsigned)(d->is_causal ? (n_qtiles + 1) / 2 : n_qtiles));
@@ -775,23 +897,28 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
     FHIP_HIP_CHECK(ctx, hipGetLastError());
     return 0;
   };
-  // one flag per kernel instance: [head dim][type][plain / causal / mask]
-  static FhipOncePerDevice configured[2][2][3];
+  // one flag per kernel instance: [head dim][type][plain / causal / mask in
+  // registers / mask staged in LDS]
+  static FhipOncePerDevice configured[2][2][4];
   auto pick = [&](auto hd) {
     constexpr int HD = decltype(hd)::value;
-    FhipOncePerDevice(&cfg)[2][3] = configured[HD == 128];
+    FhipOncePerDevice(&cfg)[2][4] = configured[HD == 128];
     constexpr int lds = SdShape<HD>::kLdsB;
-    if (p.mask)
+    constexpr int lds_mask = SdShape<HD>::kLdsMaskB;
+    if (p.mask && staged_mask)
       return p.bf16
-                 ? launch(sdpa_fwd_kernel<true, false, HD, true>, lds, cfg[1][2])
-                 : launch(sdpa_fwd_kernel<false, false, HD, true>, lds, cfg[0][2]);
+                 ? launch(sdpa_fwd_kernel<true, false, HD, 2>, lds_mask, cfg[1][3])
+                 : launch(sdpa_fwd_kernel<false, false, HD, 2>, lds_mask, cfg[0][3]);
+    if (p.mask)
+      return p.bf16 ? launch(sdpa_fwd_kernel<true, false, HD, 1>, lds, cfg[1][2])
+                    : launch(sdpa_fwd_kernel<false, false, HD, 1>, lds, cfg[0][2]);
     if (p.bf16)
       return d->is_causal
-                 ? launch(sdpa_fwd_kernel<true, true, HD, false>, lds, cfg[1][1])
-                 : launch(sdpa_fwd_kernel<true, false, HD, false>, lds, cfg[1][0]);
+                 ? launch(sdpa_fwd_kernel<true, true, HD, 0>, lds, cfg[1][1])
+                 : launch(sdpa_fwd_kernel<true, false, HD, 0>, lds, cfg[1][0]);
     return d->is_causal
-               ? launch(sdpa_fwd_kernel<false, true, HD, false>, lds, cfg[0][1])
-               : launch(sdpa_fwd_kernel<false, false, HD, false>, lds, cfg[0][0]);
+               ? launch(sdpa_fwd_kernel<false, true, HD, 0>, lds, cfg[0][1])
+               : launch(sdpa_fwd_kernel<false, false, HD, 0>, lds, cfg[0][0]);
   };
   return p.hd == 128 ? pick(std::integral_constant<int, 128>{})
                      : pick(std::integral_constant<int, 64>{});
