@@ -31,6 +31,8 @@ FhipKnobs parse_knobs() {
     k.conv_rows = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_WGRAD_DIRECT"))
     k.wgrad_direct = atoi(e);
+  if (const char *e = getenv("FUSILLI_HIP_DGRAD_ROWS"))
+    k.dgrad_rf = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_GEMM_TILE"))
     if (sscanf(e, "%d,%d", &k.gemm_tile_bm, &k.gemm_tile_bn) != 2)
       k.gemm_tile_bm = k.gemm_tile_bn = 0;

@@ -613,6 +613,10 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                          const void *w, void *dx, void *workspace) {
   const DgradPlan p = make_dgrad_plan(d);
   FHIP_REQUIRE(ctx, p.ok, "conv dgrad: descriptor not supported by the MFMA kernel");
+  // the register-filter kernel needs neither the mirrored filter nor workspace
+  if (fhip_fast_conv_dgrad_rf_applicable(d) &&
+      (((uintptr_t)dy | (uintptr_t)w | (uintptr_t)dx) & 15) == 0)
+    return fhip_fast_conv_dgrad_rf(ctx, d, dy, w, dx);
   FHIP_REQUIRE(ctx, ((uintptr_t)workspace & 15) == 0,
                "conv dgrad: workspace must be 16-byte aligned");
   const int sp = d->spatial_rank;

@@ -41,6 +41,13 @@ bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
 int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                          const void *w, void *dx, void *workspace);
 
+// Data gradient of 3 x 3 convolutions over 128 output channels with the filter
+// in registers (conv_rf_dgrad.hip): one kernel, W read as it lies, no
+// workspace.  fhip_fast_conv_dgrad takes it where it applies.
+bool fhip_fast_conv_dgrad_rf_applicable(const fhip_conv_desc *d);
+int fhip_fast_conv_dgrad_rf(fhip_ctx *ctx, const fhip_conv_desc *d,
+                            const void *dy, const void *w, void *dx);
+
 // Resolves this device's address of the static scratch array behind
 // fhip_conv_dgrad_static into the context (device current, creation lock held).
 int fhip_conv_dgrad_static_setup(fhip_ctx *ctx);

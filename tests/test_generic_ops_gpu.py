@@ -401,6 +401,35 @@ def test_conv_dgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
                  dtype, f"dgrad {case}")
 
 
+@pytest.mark.parametrize("case", [
+    # [N, C, H, W] of DX, padding: 3 x 3 filters over K = 128 gradient channels,
+    # C a multiple of 64 -- the kernel that keeps the filter in registers and
+    # reads W as it lies
+    dict(x=[2, 64, 12, 12], pad=1),     # small: the efficiency rule is overridden
+    dict(x=[1, 64, 5, 7], pad=1),       # fewer pixel blocks than wavefronts
+    dict(x=[3, 128, 17, 40], pad=1),    # two channel groups, ragged last tile
+    dict(x=[2, 64, 9, 56], pad=0),      # widest slab row; DY smaller than DX
+    dict(x=[2, 64, 11, 30], pad=2),     # DY larger than DX
+    dict(x=[40, 64, 20, 20], pad=1),    # several tiles per workgroup
+])
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("rows", [2, 5])
+def test_conv_dgrad_register_filter_vs_oracle(ctx, case, dtype, rows, knobs):
+    xd, wd, pad = case["x"], [128, case["x"][1], 3, 3], [case["pad"]] * 2
+    yd = oracle.conv_output_dims(xd, wd, pad, [1, 1], [1, 1])
+    cl = oracle.channels_last_strides
+    dy = HT.from_logical(rand(36, 0, yd), dtype, cl(yd))
+    w = HT.from_logical(rand(36, 1, wd, std=0.1), dtype, cl(wd))
+    ref = oracle.conv_dgrad(dy.logical(), w.logical(), xd, pad, [1, 1], [1, 1])
+    knobs(DGRAD_ROWS=rows)  # rows per tile (forces the kernel)
+    dx = run_conv_dgrad(ctx, dy, w, xd, pad, [1, 1], [1, 1], dtype, tuned=True)
+    assert_close(dx.logical(), ref, dtype, f"dgrad rf {case} rows {rows}")
+    # the same call on the tiled kernel (mirrored filter in workspace)
+    knobs(DGRAD_ROWS=0)
+    dx2 = run_conv_dgrad(ctx, dy, w, xd, pad, [1, 1], [1, 1], dtype, tuned=True)
+    assert_close(dx2.logical(), ref, dtype, f"dgrad tiled {case}")
+
+
 def test_conv_dgrad_config3_shape_closed_form_and_oracle(ctx):
     # the data gradient of benchmark config 3 (N32 C64 56x56, K128 3x3 pad 1).
     # All-ones: DX = K * (taps whose output pixel exists) = 128 * {9, 6, 4}.
