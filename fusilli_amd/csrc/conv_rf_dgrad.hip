@@ -7,26 +7,29 @@
 // DY as the image, the mirrored and transposed filter and padding R - 1 - pad,
 // with two differences that shape the kernel:
 //
-//   * the reduction is twice as long (9 taps x 128 channels of DY) and the
-//     output half as wide, so a wavefront keeps the filter of 16 output
-//     channels -- 36 K-steps x 4 registers = 144 -- and a workgroup of 8
-//     wavefronts (4 channel slices x 2 that alternate pixel blocks) owns 64
-//     output channels: one v_mfma_f32_16x16x32 per 16 pixels and K-step, a lane
-//     ends up with 4 consecutive channels of one pixel (8-byte stores);
+//   * the reduction is twice as long (9 taps x 128 channels of DY): the filter
+//     of 32 output channels is 36 K-steps x 2 tiles x 4 = 288 registers, more
+//     than a wavefront has at two per SIMD (and 16 channels per wavefront
+//     would read one LDS fragment per MFMA: the LDS, not the matrix pipe, then
+//     sets the pace -- measured: 24.6 us).  So a workgroup is 4 wavefronts, one
+//     per SIMD with the whole register file (2 channel slices of 32 x 2 that
+//     alternate pixel blocks = 64 output channels), every fragment read feeds
+//     two v_mfma_f32_16x16x32, and a lane ends up with 8 consecutive channels
+//     of one pixel (16-byte stores);
 //   * no mirrored copy of the filter is made: W's rows [k][r][s][c] are staged
 //     as they lie, 32 k x 64 c per K-step by LDS-DMA (tap R - 1 - r', S - 1 -
 //     s' for the kernel's tap r', s'), and the transposing LDS read hands a
-//     lane the 8 consecutive k of its channel, the MFMA's A operand.  The
-//     filter passes through a stage of NK / NP K-steps in NP rounds during the
-//     first pixel block, so that the input slab has most of the LDS.
+//     lane the 8 consecutive k of its channel, the MFMA's A operand.  The whole
+//     filter (144 KB) is staged at once, before the first slab.
 //
 // The slab (tile rows plus halo, zero-padded, pixel pitch 128 * 2 + 16 bytes)
-// and the fragment ring are those of conv_rf.hip.  DY is twice the size of the
-// output, so the slab loads are what the kernel has to hide: two slab buffers
-// alternate, the next tile's rows arrive by LDS-DMA while the current tile is
-// multiplied (the second buffer lies over the filter stage, which is dead once
-// the filter is in registers).  Fragment reads are written as asm with their
-// own wait counts, so that they do not wait for the loads in flight.
+// and the fragment ring are those of conv_rf.hip; tiles may also split the
+// image's width, so that they come out as whole rounds of the machine.  DY is
+// twice the size of the output, so the slab loads are what the kernel has to
+// hide: two slab buffers alternate (under the filter stage until the filter is
+// in registers), the next tile's rows arrive by LDS-DMA while the current tile
+// is multiplied.  Fragment reads are written as asm with their own wait
+// counts, so that they do not wait for the loads in flight.
 //
 // Reference semantics: node/conv_node.h:427-598 (ConvDGradNode),
 // aten.convolution_backward, input gradient.
@@ -47,7 +50,7 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kRdWaves = 8; // two per SIMD
+constexpr int kRdWaves = 4; // one per SIMD: the whole register file each
 constexpr int kRdThreads = kRdWaves * 64;
 constexpr int kRdChannels = 64; // output channels per workgroup
 constexpr int kRdMaxNI = 16;    // KB of LDS per slab row, at most
@@ -60,7 +63,8 @@ struct RfDgradArgs {
   int32_t CO;       // DX's channels, a multiple of 64
   int32_t pad_h, pad_w; // of the forward-shaped problem: R - 1 - padding
   int32_t TR, tiles_per_image, ntiles, kgroups, NI;
-  uint32_t magic_q;
+  int32_t TQ, ctiles; // output columns per tile (Q = TQ * ctiles), column tiles per row tile
+  uint32_t magic_q;   // of TQ
   uint32_t dy_bytes, w_bytes;
 };
 
@@ -98,24 +102,22 @@ template <int N> __device__ __forceinline__ void rd_wait_lgkm(u32x4 &reg) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(N));
 }
 
-// CK: channels of DY (the reduction); NP: rounds the filter is staged in
-template <int CK, int R, int S, int NP> struct RdGeom {
+// CK: channels of DY (the reduction)
+template <int CK, int R, int S> struct RdGeom {
   static constexpr int kCPP = CK * 2 / 16 + 1;  // chunks per slab pixel (one is padding)
   static constexpr int kKPT = CK / 32;          // K-steps per tap
   static constexpr int kNK = R * S * kKPT;      // K-steps of 32 channels
-  static constexpr int kNKP = kNK / NP;         // K-steps per staging round
-  static constexpr int kStageBytes = kNKP * 4096; // 32 k x 64 c x 2 bytes per K-step
+  static constexpr int kStageBytes = kNK * 4096; // 32 k x 64 c x 2 bytes per K-step
 };
 
-template <int KIND, int CK, int R, int S, int NP>
+template <int KIND, int CK, int R, int S>
 __global__ __launch_bounds__(kRdThreads)
-__attribute__((amdgpu_waves_per_eu(2, 2))) void
+__attribute__((amdgpu_waves_per_eu(1, 1))) void
 conv_rf_dgrad_kernel(RfDgradArgs g) {
-  using G = RdGeom<CK, R, S, NP>;
-  constexpr int CPP = G::kCPP, PITCH = CPP * 16, KPT = G::kKPT, NK = G::kNK,
-                NKP = G::kNKP;
-  constexpr int RING = 6; // fragment buffers (K-steps in flight)
-  static_assert(CK % 32 == 0 && NK % NP == 0 && NK % RING == 0 && NKP >= RING,
+  using G = RdGeom<CK, R, S>;
+  constexpr int CPP = G::kCPP, PITCH = CPP * 16, KPT = G::kKPT, NK = G::kNK;
+  constexpr int RING = 6;  // fragment buffers (K-steps in flight)
+  static_assert(RING == 6 && CK % 32 == 0 && NK % RING == 0 && NK >= 3 * RING,
                 "filter shape not covered");
   static_assert((S - 1) * PITCH + (KPT - 1) * 64 + 48 < 65536, "ds offset range");
   const int a_Q = g.Q, a_P = g.P, a_TR = g.TR, a_NI = g.NI, a_CO = g.CO;
@@ -123,6 +125,7 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
   const int a_tiles_per_image = g.tiles_per_image, a_ntiles = g.ntiles;
   const int a_kgroups = g.kgroups;
   const uint32_t a_magic_q = g.magic_q;
+  const int a_TQ = g.TQ, a_ctiles = g.ctiles;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
 #ifdef RD_PROFILE
@@ -132,19 +135,18 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
   RD_STAMP(0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const int slice = wave & 3; // 16 output channels; wavefronts w and w + 4 share a SIMD
-  const int half = wave >> 2; // which of the pair: its pixel blocks
+  const int slice = wave & 1; // 32 output channels
+  const int half = wave >> 1; // which of the two that alternate pixel blocks
   const int l = threadIdx.x & 63;
   const int px = l & 15, q = l >> 4;
   const uint32_t rowpitch = (uint32_t)a_NI * 1024u;
-  // slab buffers: the first tile's behind the filter stage, the other over it
+  // two slab buffers; the filter stage lies over them until the filter is in
+  // registers
   const uint32_t slab_bytes = (uint32_t)(a_TR + R - 1) * rowpitch;
-  const uint32_t buf1 = lds0;
-  const uint32_t buf0 =
-      lds0 + (slab_bytes > (uint32_t)G::kStageBytes ? slab_bytes : (uint32_t)G::kStageBytes);
+  const uint32_t buf0 = lds0, buf1 = lds0 + slab_bytes;
 
   const int kg = (int)(blockIdx.x % (unsigned)a_kgroups);
-  const int ch_wave = kg * kRdChannels + slice * 16;
+  const int ch_wave = kg * kRdChannels + slice * 32;
   // Tiles of a workgroup.  Workgroups go to the 8 XCDs round-robin; with one
   // channel group and a multiple of 8 workgroups, XCD x takes a contiguous
   // eighth of the tiles, so that the halo rows neighbouring tiles share are
@@ -164,66 +166,93 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
   // tap' = (r', s'), which is filter tap (R - 1 - r', S - 1 - s').  Its stage
   // slot holds 32 rows (k) of this workgroup's 64 channels (128 bytes), written
   // by four LDS-DMA instructions (8 rows each: lane d carries chunk d % 8 of
-  // row d / 8); wavefront (slice, half) issues instruction `slice` of the
-  // K-steps whose parity is `half`.
+  // row d / 8); wavefront w issues the K-steps j = w, w + 4, ...
   const int64_t wrow = (int64_t)R * S * a_CO * 2; // bytes between W's k rows
   const __amdgpu_buffer_rsrc_t rw = rd_rsrc(g.w, g.w_bytes);
-  const uint32_t fvoff = (uint32_t)((slice * 8 + (l >> 3)) * wrow + kg * 128 + (l & 7) * 16);
-  auto filter_dma = [&](auto pc) __attribute__((always_inline)) {
-    constexpr int p = decltype(pc)::value;
-    gemm_static_for<NKP>([&](auto jc) {
-      constexpr int jj = decltype(jc)::value, j = p * NKP + jj;
-      constexpr int tap = j / KPT, part = j % KPT;
-      constexpr int src = (R - 1 - tap / S) * S + (S - 1 - tap % S);
-      if ((jj & 1) == half)
+  {
+    uint32_t fvoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fvoff[i] = (uint32_t)((i * 8 + (l >> 3)) * wrow + kg * 128 + (l & 7) * 16);
+    gemm_static_for<NK / 4>([&](auto jc) {
+      const int j = decltype(jc)::value * 4 + wave;
+      const int tap = j / KPT, part = j - tap * KPT;
+      const int src = (R - 1 - tap / S) * S + (S - 1 - tap % S);
+      const int soff = (int)(part * 32 * wrow + src * a_CO * 2);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             rw,
             (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(
-                lds0 + (uint32_t)(jj * 4096 + slice * 1024)),
-            16, (int)fvoff, (int)(part * 32 * wrow + src * a_CO * 2), 0, 0);
+                lds0 + (uint32_t)(j * 4096 + i * 1024)),
+            16, (int)fvoff[i], soff, 0, 0);
     });
-  };
-  // MFMA lane (rho = l % 16, kq = l / 16) takes channel ch_wave + rho, k = 8 kq
-  // .. 8 kq + 7: two transposing reads of 4 k each; the 16 lanes of a group
-  // address rows 8 kq + rho / 4 (+ 4), channels 4 (rho % 4) ..+3 of the slice.
-  u32x4 filt[NK];
-  const uint32_t fread = lds0 + (uint32_t)((8 * q + (px >> 2)) * 128 + slice * 32 + (px & 3) * 8);
-  auto filter_read = [&](auto pc) __attribute__((always_inline)) {
-    constexpr int p = decltype(pc)::value;
-    gemm_static_for<NKP>([&](auto jc) {
-      constexpr int jj = decltype(jc)::value, j = p * NKP + jj;
-      const u32x2 lo = __builtin_bit_cast(
-          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                     (GEMM_AS3 s16x4 *)(uintptr_t)(fread + jj * 4096)));
-      const u32x2 hi = __builtin_bit_cast(
-          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                     (GEMM_AS3 s16x4 *)(uintptr_t)(fread + jj * 4096 + 512)));
-      filt[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+  }
+  // MFMA row rho of tile t is output channel ch_wave + 8 * (rho / 4) + 4 * t +
+  // rho % 4, so that a lane's 8 results (rows 4 q .. 4 q + 3 of both tiles) are
+  // 8 consecutive channels.  MFMA lane (rho = l % 16, kq = l / 16) takes k = 8
+  // kq .. 8 kq + 7 of its channel: two transposing reads of 4 k each, for which
+  // the 16 lanes of a group address rows 8 kq + rho / 4 (+ 4) and the four
+  // channels 8 (rho % 4) + 4 t ..+3 of the slice.
+  // (with one wavefront per SIMD the compiler has the accumulation registers
+  // as well: it keeps most of these 288 registers there, where the MFMA takes
+  // its A operand from directly)
+  u32x4 filt[NK][2];
+  __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+  gemm_barrier();
+  RD_STAMP(1);
+  {
+    const uint32_t fread =
+        lds0 + (uint32_t)((8 * q + (px >> 2)) * 128 + slice * 64 + (px & 3) * 16);
+    gemm_static_for<NK>([&](auto jc) {
+      constexpr int j = decltype(jc)::value;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const u32x2 lo = __builtin_bit_cast(
+            u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                       (GEMM_AS3 s16x4 *)(uintptr_t)(fread + j * 4096 + t * 8)));
+        const u32x2 hi = __builtin_bit_cast(
+            u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                       (GEMM_AS3 s16x4 *)(uintptr_t)(fread + j * 4096 + t * 8 + 512)));
+        const u32x4 f = {lo.x, lo.y, hi.x, hi.y};
+        filt[j][t] = f;
+      }
     });
-  };
-  filter_dma(std::integral_constant<int, 0>{});
+  }
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // the reads returned
+  gemm_barrier(); // the stage is dead: slabs may cover it
 
   const __amdgpu_buffer_rsrc_t rx = rd_rsrc(g.dy, g.dy_bytes);
   const __amdgpu_buffer_rsrc_t rnone = rd_rsrc(g.dy, 0); // every lane out of range
 
   // ---- slab of a tile: its rows plus halo by LDS-DMA; wavefront w loads rows
-  // w, w + 8, ...  LDS chunk x = i * 64 + lane of a slab row is chunk x % CPP
-  // of slab pixel x / CPP, i.e. input column x / CPP - pad_w; the padding
-  // chunk, columns outside the image and the tail of the row's last KB read as
-  // zeros.  The lane offsets are the same for every row and tile.
-  uint32_t rel[kRdMaxNI];
-#pragma unroll
-  for (int i = 0; i < kRdMaxNI; ++i) {
-    const int xk = i * 64 + l;
-    const int sp = (xk * (65536 / CPP + 1)) >> 16; // xk / CPP for xk < 2^12
-    const int c = xk - sp * CPP;
-    const int iw = sp - a_pad_w;
-    const bool ok = c < CPP - 1 && (unsigned)iw < (unsigned)a_W;
-    rel[i] = ok ? (uint32_t)(iw * (CK * 2) + c * 16) : 0x80000000u;
-  }
+  // w, w + 4, ...  LDS chunk x = i * 64 + lane of a slab row is chunk x % CPP
+  // of slab pixel x / CPP, i.e. input column q0 - pad_w + x / CPP; the padding
+  // chunk, columns outside the image or the tile's reach and the tail of the
+  // row's last KB read as zeros.
+  // tile -> (image, first output row, first output column)
+  auto tile_origin = [&](int tile, int &n, int &p0, int &q0) __attribute__((always_inline)) {
+    const int rt = tile / a_ctiles; // row tile of the batch
+    q0 = (tile - rt * a_ctiles) * a_TQ;
+    n = rt / a_tiles_per_image;
+    p0 = (rt - n * a_tiles_per_image) * a_TR;
+  };
   auto issue_slab = [&](int tile, uint32_t dst0) __attribute__((always_inline)) {
-    const int n = tile / a_tiles_per_image;
-    const int p0 = (tile - n * a_tiles_per_image) * a_TR;
+    int n, p0, q0;
+    tile_origin(tile, n, p0, q0);
+    // slab pixel sp is input column q0 - pad_w + sp; only the TQ + S - 1
+    // columns the tile needs are fetched
+    uint32_t rel[kRdMaxNI];
+#pragma unroll
+    for (int i = 0; i < kRdMaxNI; ++i) {
+      const int xk = i * 64 + l;
+      const int sp = (xk * (65536 / CPP + 1)) >> 16; // xk / CPP for xk < 2^12
+      const int c = xk - sp * CPP;
+      const int iw = q0 - a_pad_w + sp;
+      const bool ok = c < CPP - 1 && sp < a_TQ + S - 1 && (unsigned)iw < (unsigned)a_W;
+      rel[i] = ok ? (uint32_t)(iw * (CK * 2) + c * 16) : 0x80000000u;
+    }
     const int tr = a_P - p0 < a_TR ? a_P - p0 : a_TR;
     const int rows_in = tr + R - 1;
     const int ih0 = p0 - a_pad_h;
@@ -243,34 +272,34 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
   };
   if (tile0 < tile_end)
     issue_slab(tile0, buf0);
+  RD_STAMP(2);
 
-  bool first = true; // the filter is not in registers yet
-  int cur = 0;       // buffer of the current tile
+  int cur = 0; // buffer of the current tile
   for (int tile = tile0; tile < tile_end; tile += tile_step) {
-    const int n = tile / a_tiles_per_image;
-    const int p0 = (tile - n * a_tiles_per_image) * a_TR;
+    int n, p0, q0;
+    tile_origin(tile, n, p0, q0);
     const int tr = a_P - p0 < a_TR ? a_P - p0 : a_TR;
-    const int npix = tr * a_Q;
+    const int npix = tr * a_TQ;
     const uint32_t lds_s = cur ? buf1 : buf0;
     const int next = tile + tile_step;
-    // this tile's slab (and the filter's first round) has landed, and every
-    // wavefront has left the previous tile: its buffer is free
+    // this tile's slab has landed, and every wavefront has left the previous
+    // tile: its buffer is free for the next tile's rows
     __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
     gemm_barrier();
 #ifdef RD_PROFILE
     if (iter == 0)
-      RD_STAMP(1);
+      RD_STAMP(3);
     if (iter == 1)
-      RD_STAMP(4);
+      RD_STAMP(5);
 #endif
-    if (!first && next < tile_end)
+    if (next < tile_end)
       issue_slab(next, cur ? buf0 : buf1);
 
-    // outputs of this tile: dense rows of CO channels, pixel index tile-relative
+    // outputs of this tile: TQ pixels of CO channels out of every image row
     const __amdgpu_buffer_rsrc_t ro =
-        rd_rsrc(g.dx + ((int64_t)(n * a_P + p0) * a_Q) * a_CO * 2,
-                (uint32_t)npix * (uint32_t)a_CO * 2u);
-    const uint32_t lane_out = (uint32_t)(ch_wave + 4 * q) * 2u;
+        rd_rsrc(g.dx + ((int64_t)(n * a_P + p0) * a_Q + q0) * a_CO * 2,
+                (uint32_t)((tr - 1) * a_Q + a_TQ) * (uint32_t)a_CO * 2u);
+    const uint32_t lane_out = (uint32_t)(ch_wave + 8 * q) * 2u;
     const int nblocks = (npix + 15) >> 4;
 
     // Slab addresses (one per filter row, this lane's K quarter) and output
@@ -278,46 +307,68 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
     auto block_setup = [&](int b, uint32_t (&base)[R], uint32_t &ooff) __attribute__((always_inline)) {
       const int pl = b * 16 + px;
       const int plc = pl < npix ? pl : npix - 1;
-      const int prow = (int)conv_div(plc, a_Q, a_magic_q);
-      const int pcol = plc - prow * a_Q;
+      const int prow = (int)conv_div(plc, a_TQ, a_magic_q);
+      const int pcol = plc - prow * a_TQ;
       base[0] = lds_s + (uint32_t)prow * rowpitch + (uint32_t)pcol * PITCH + (uint32_t)q * 16u;
 #pragma unroll
       for (int r = 1; r < R; ++r)
         base[r] = base[r - 1] + rowpitch;
-      ooff = pl < npix ? (uint32_t)pl * (uint32_t)a_CO * 2u + lane_out : 0x80000000u;
+      ooff = pl < npix ? (uint32_t)(prow * a_Q + pcol) * (uint32_t)a_CO * 2u + lane_out
+                       : 0x80000000u;
     };
     u32x4 frag[RING];
-    auto fetch = [&](auto jc, const uint32_t (&base)[R]) __attribute__((always_inline)) {
+    auto fetch = [&](auto jc, const uint32_t (&base)[R], u32x4 &dst) __attribute__((always_inline)) {
       constexpr int j = decltype(jc)::value;
       constexpr int tap = j / KPT, part = j % KPT;
       constexpr int r = tap / S, s = tap % S;
-      rd_read_b128<s * PITCH + part * 64>(frag[j % RING], base[r]);
+      rd_read_b128<s * PITCH + part * 64>(dst, base[r]);
     };
-    f32x4 acc;
+    f32x4 acc[2];
     uint32_t base[R], nbase[R], ooff, nooff;
-    // K-steps [J0, J1) of the block at `base`; the first fragments of the next
-    // block (at `nbase`) are fetched during the last steps.  RING reads are in
-    // flight when a step waits for its own, the oldest.
-    auto ksteps = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
-      constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
-      gemm_static_for<J1 - J0>([&](auto dc) {
-        constexpr int j = J0 + decltype(dc)::value;
+    // The K-steps of the block at `base`.  Step j fetches the fragment of step
+    // j + RING - 1; the first RING - 1 fragments of the NEXT block (at `nbase`)
+    // are fetched into registers of their own a dozen steps before the end, so
+    // that they have landed when the block ends: values that cross the loop's
+    // back edge may be copied there, which must not happen to a register a
+    // load is still to write.  LDS returns in order, so a step waits until at
+    // most `younger` reads issued after its own fragment's are outstanding.
+    u32x4 nfrag[RING - 1];
+    constexpr int NF0 = NK - 2 * RING; // step of the first early fetch
+    auto ksteps = [&]() __attribute__((always_inline)) {
+      gemm_static_for<NK>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
         constexpr int ahead = j + RING - 1;
         if constexpr (ahead < NK)
-          fetch(std::integral_constant<int, ahead>{}, base);
-        else
-          fetch(std::integral_constant<int, ahead - NK>{}, nbase);
-        rd_wait_lgkm<RING - 1>(frag[j % RING]);
-        acc = rd_mfma<KIND>(filt[j], frag[j % RING], j == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc);
-      });
-    };
-    // rounding and the 8-byte store of a finished block
-    auto finish = [&](const f32x4 &y, uint32_t off) __attribute__((always_inline)) {
-      typedef float f2 __attribute__((ext_vector_type(2)));
-      uint32_t w[2];
+          fetch(std::integral_constant<int, ahead>{}, base, frag[ahead % RING]);
+        if constexpr (j >= NF0 && j < NF0 + RING - 1)
+          fetch(std::integral_constant<int, j - NF0>{}, nbase, nfrag[j - NF0]);
+        constexpr int regular = NK - 1 - j < RING - 1 ? NK - 1 - j : RING - 1;
+        // early fetches issued at steps j - (RING - 1) .. j
+        constexpr int lo = j - (RING - 1) > NF0 ? j - (RING - 1) : NF0;
+        constexpr int hi = j < NF0 + RING - 2 ? j : NF0 + RING - 2;
+        constexpr int early = hi >= lo ? hi - lo + 1 : 0;
+        rd_wait_lgkm<regular + early>(frag[j % RING]);
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const f2 pair = {y[2 * i], y[2 * i + 1]};
+        for (int t = 0; t < 2; ++t) {
+          acc[t] = rd_mfma<KIND>(filt[j][t], frag[j % RING],
+                                 j == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[t]);
+        }
+      });
+      // every read has returned (the early ones long ago)
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(nfrag[0]), "+v"(nfrag[1]), "+v"(nfrag[2]), "+v"(nfrag[3]),
+                     "+v"(nfrag[4]));
+#pragma unroll
+      for (int k = 0; k < RING - 1; ++k)
+        frag[k] = nfrag[k];
+    };
+    // rounding and the 16-byte store of a finished block
+    auto finish = [&](uint32_t off) __attribute__((always_inline)) {
+      typedef float f2 __attribute__((ext_vector_type(2)));
+      uint32_t w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const f2 pair = {acc[i >> 1][2 * (i & 1)], acc[i >> 1][2 * (i & 1) + 1]};
         if constexpr (KIND == GK_BF16) {
           typedef __bf16 b2 __attribute__((ext_vector_type(2)));
           w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, b2));
@@ -326,70 +377,31 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
           w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, h2));
         }
       }
-      __builtin_amdgcn_raw_buffer_store_b64(u32x2{w[0], w[1]}, ro, (int)off, 0, 19);
+      __builtin_amdgcn_raw_buffer_store_b128(u32x4{w[0], w[1], w[2], w[3]}, ro, (int)off, 0, 19);
     };
-    auto next_block = [&]() __attribute__((always_inline)) {
+
+    // This wavefront's blocks: half, half + 2, ...  (a block index past the
+    // last one addresses the last pixel and stores nothing).
+    int b = half;
+    block_setup(b, base, ooff);
+    gemm_static_for<RING - 1>(
+        [&](auto jc) { fetch(jc, base, frag[decltype(jc)::value]); });
+    for (; b < nblocks; b += 2) {
+      block_setup(b + 2, nbase, nooff);
+      ksteps();
+      const uint32_t done_off = ooff;
 #pragma unroll
       for (int r = 0; r < R; ++r)
         base[r] = nbase[r];
       ooff = nooff;
-    };
-
-    // This wavefront's blocks: half, half + 2, ...  (block indices past the
-    // last one address the last pixel and store nothing).
-    int b = half;
-    block_setup(b, base, ooff);
-    if (first) {
-      // The first block (of every wavefront: the barriers in its middle are
-      // the workgroup's) takes the filter in as it goes: round p of the stage
-      // is read, refilled with round p + 1 once every wavefront has read it,
-      // and its K-steps run while that lands.
-      block_setup(b + 2, nbase, nooff);
-      gemm_static_for<NP>([&](auto pc) {
-        constexpr int p = decltype(pc)::value;
-        filter_read(pc);
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // the reads returned
-        gemm_barrier();
-        if constexpr (p + 1 < NP)
-          filter_dma(std::integral_constant<int, p + 1>{});
-        else if (next < tile_end) // the stage is dead: the next slab may cover it
-          issue_slab(next, buf1);
-        if constexpr (p == 0)
-          gemm_static_for<RING - 1>([&](auto jc) { fetch(jc, base); });
-        ksteps(std::integral_constant<int, p * NKP>{},
-               std::integral_constant<int, (p + 1) * NKP>{});
-        if constexpr (p + 1 < NP) {
-          __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
-          gemm_barrier();
-        }
-      });
-      const f32x4 y = acc;
-      const uint32_t done_off = ooff;
-      b += 2;
-      next_block();
-      first = false;
-      finish(y, done_off);
-      RD_STAMP(2);
-    } else {
-      gemm_static_for<RING - 1>([&](auto jc) { fetch(jc, base); });
-    }
-    for (; b < nblocks; b += 2) {
-      block_setup(b + 2, nbase, nooff);
-      ksteps(std::integral_constant<int, 0>{}, std::integral_constant<int, NK>{});
-      const f32x4 y = acc;
-      const uint32_t done_off = ooff;
-      next_block();
-      finish(y, done_off);
+      finish(done_off);
     }
     // the fragments fetched ahead for a block that does not exist
     __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
     cur ^= 1;
 #ifdef RD_PROFILE
     if (iter == 0)
-      RD_STAMP(3);
-    if (iter == 1)
-      RD_STAMP(5);
+      RD_STAMP(4);
     ++iter;
 #endif
   }
@@ -426,7 +438,7 @@ bool rd_channels_last(const fhip_tensor_desc &t) {
   return true;
 }
 
-constexpr int kRdCK = 128, kRdR = 3, kRdS = 3, kRdNP = 2;
+constexpr int kRdCK = 128, kRdR = 3, kRdS = 3;
 
 RdPlan make_rd_plan(const fhip_conv_desc *d, int num_cus) {
   RdPlan p;
@@ -468,39 +480,53 @@ RdPlan make_rd_plan(const fhip_conv_desc *d, int num_cus) {
     return p;
   a.dy_bytes = (uint32_t)dy_bytes;
   a.w_bytes = (uint32_t)w_bytes;
-  using G = RdGeom<kRdCK, kRdR, kRdS, kRdNP>;
-  a.NI = ((a.W + 2 * a.pad_w) * G::kCPP + 63) / 64;
-  if (a.NI > kRdMaxNI)
-    return p;
-  // two slab buffers, the second over the filter stage
+  using G = RdGeom<kRdCK, kRdR, kRdS>;
+  // two slab buffers, under the filter stage until the filter is in registers
   const int64_t lds_total = 160 * 1024;
-  // rows per tile: the choice that fills whole rounds of the machine best
+  auto lds_of = [&](int tr, int ni) {
+    const int64_t slab = (int64_t)(tr + kRdR - 1) * ni * 1024;
+    return 2 * slab > G::kStageBytes ? 2 * slab : (int64_t)G::kStageBytes;
+  };
+  // Tile = TR output rows x TQ output columns (Q = TQ * ctiles): the split
+  // that fills whole rounds of the machine best.  Time of a round ~ the blocks
+  // of the busier wavefront of a pair plus a share that grows with the slab
+  // bytes a tile loads (measured on N32 56 x 56 with full-width tiles: 2 rows
+  // per tile 24.8 us, 3 rows 25.9 us, 1 row 28.7 us).
   const int cus = num_cus > 0 ? num_cus : 256;
   const int kgroups = (int)(CO / kRdChannels);
   double best = 0;
-  int best_tr = 0;
-  for (int tr = 1; tr <= a.P; ++tr) {
-    const int64_t slab = (int64_t)(tr + kRdR - 1) * a.NI * 1024;
-    if (slab + (slab > G::kStageBytes ? slab : G::kStageBytes) > lds_total)
-      break;
-    const int64_t tiles = (int64_t)a.N * ((a.P + tr - 1) / tr) * kgroups;
-    const int64_t rounds = (tiles + cus - 1) / cus;
-    const int64_t blocks = ((int64_t)tr * a.Q + 15) / 16;
-    // time of a round ~ the blocks of the busier wavefront of a pair plus a
-    // share that grows with the slab rows a tile loads (measured on N32 56 x
-    // 56: 2 rows per tile 24.8 us, 3 rows 25.9 us, 1 row 28.7 us)
-    const double cost =
-        (double)rounds * ((blocks + 1) / 2 * 2 * 16 + 32 * (tr + kRdR - 1));
-    const double eff = (double)a.N * a.P * a.Q * kgroups / (cost * cus);
-    if (eff > best + 1e-9) {
-      best = eff;
-      best_tr = tr;
+  int best_tr = 0, best_ct = 1;
+  for (int ct = 1; ct <= 4; ct *= 2) {
+    if (a.Q % ct != 0)
+      continue;
+    const int tq = a.Q / ct;
+    const int ni = ((tq + kRdS - 1) * G::kCPP + 63) / 64;
+    if (ni > kRdMaxNI || (ct > 1 && tq < 16))
+      continue;
+    for (int tr = 1; tr <= a.P; ++tr) {
+      if (lds_of(tr, ni) > lds_total)
+        break;
+      const int64_t tiles = (int64_t)a.N * ((a.P + tr - 1) / tr) * ct * kgroups;
+      const int64_t rounds = (tiles + cus - 1) / cus;
+      const int64_t blocks = ((int64_t)tr * tq + 15) / 16;
+      const double cost =
+          (double)rounds * ((blocks + 1) / 2 * 2 * 16 + 2 * (tr + kRdR - 1) * ni);
+      const double eff = (double)a.N * a.P * a.Q * kgroups / (cost * cus);
+      if (eff > best + 1e-9) {
+        best = eff;
+        best_tr = tr;
+        best_ct = ct;
+      }
     }
   }
-  if (knobs.dgrad_rf > 0 && knobs.dgrad_rf <= a.P) {
-    const int64_t slab = (int64_t)(knobs.dgrad_rf + kRdR - 1) * a.NI * 1024;
-    if (slab + (slab > G::kStageBytes ? slab : G::kStageBytes) <= lds_total)
-      best_tr = knobs.dgrad_rf;
+  if (knobs.dgrad_rf > 0) {
+    // rows per tile, and column tiles in the hundreds: 207 = 7 rows, 2 column tiles
+    const int tr = knobs.dgrad_rf % 100, ct = knobs.dgrad_rf >= 100 ? knobs.dgrad_rf / 100 : 1;
+    if (tr >= 1 && tr <= a.P && ct >= 1 && a.Q % ct == 0) {
+      const int ni = ((a.Q / ct + kRdS - 1) * G::kCPP + 63) / 64;
+      if (ni <= kRdMaxNI && lds_of(tr, ni) <= lds_total)
+        best_tr = tr, best_ct = ct;
+    }
   }
   if (best_tr == 0)
     return p;
@@ -508,14 +534,14 @@ RdPlan make_rd_plan(const fhip_conv_desc *d, int num_cus) {
   if (best < 0.3 && knobs.dgrad_rf < 0)
     return p;
   a.TR = best_tr;
+  a.ctiles = best_ct;
+  a.TQ = a.Q / best_ct;
+  a.NI = ((a.TQ + kRdS - 1) * G::kCPP + 63) / 64;
   a.tiles_per_image = (a.P + a.TR - 1) / a.TR;
-  a.ntiles = a.N * a.tiles_per_image;
+  a.ntiles = a.N * a.tiles_per_image * a.ctiles;
   a.kgroups = kgroups;
-  a.magic_q = conv_magic(a.Q);
-  {
-    const int slab = (a.TR + kRdR - 1) * a.NI * 1024;
-    p.lds = slab + (slab > G::kStageBytes ? slab : G::kStageBytes);
-  }
+  a.magic_q = conv_magic(a.TQ);
+  p.lds = (int)lds_of(a.TR, a.NI);
   const int64_t items = (int64_t)a.ntiles * kgroups;
   const int64_t slots =
       (int64_t)cus / kgroups * kgroups > 0 ? (int64_t)cus / kgroups * kgroups : kgroups;
@@ -525,7 +551,7 @@ RdPlan make_rd_plan(const fhip_conv_desc *d, int num_cus) {
 }
 
 template <int KIND> int rd_launch(fhip_ctx *ctx, const RdPlan &p) {
-  auto kernel = conv_rf_dgrad_kernel<KIND, kRdCK, kRdR, kRdS, kRdNP>;
+  auto kernel = conv_rf_dgrad_kernel<KIND, kRdCK, kRdR, kRdS>;
   static FhipOncePerDevice configured;
   if (!configured.done(ctx->device)) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(

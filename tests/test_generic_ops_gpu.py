@@ -413,7 +413,7 @@ def test_conv_dgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
     dict(x=[40, 64, 20, 20], pad=1),    # several tiles per workgroup
 ])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
-@pytest.mark.parametrize("rows", [2, 5])
+@pytest.mark.parametrize("rows", [2, 5, 203, 407])
 def test_conv_dgrad_register_filter_vs_oracle(ctx, case, dtype, rows, knobs):
     xd, wd, pad = case["x"], [128, case["x"][1], 3, 3], [case["pad"]] * 2
     yd = oracle.conv_output_dims(xd, wd, pad, [1, 1], [1, 1])
@@ -421,7 +421,9 @@ def test_conv_dgrad_register_filter_vs_oracle(ctx, case, dtype, rows, knobs):
     dy = HT.from_logical(rand(36, 0, yd), dtype, cl(yd))
     w = HT.from_logical(rand(36, 1, wd, std=0.1), dtype, cl(wd))
     ref = oracle.conv_dgrad(dy.logical(), w.logical(), xd, pad, [1, 1], [1, 1])
-    knobs(DGRAD_ROWS=rows)  # rows per tile (forces the kernel)
+    # rows per tile, + 100 x column tiles: forces the kernel and its tiling
+    # (splits the width does not allow fall back to the kernel's own choice)
+    knobs(DGRAD_ROWS=rows)
     dx = run_conv_dgrad(ctx, dy, w, xd, pad, [1, 1], [1, 1], dtype, tuned=True)
     assert_close(dx.logical(), ref, dtype, f"dgrad rf {case} rows {rows}")
     # the same call on the tiled kernel (mirrored filter in workspace)
