@@ -116,8 +116,13 @@ __attribute__((amdgpu_waves_per_eu(1, 1))) void
 conv_rf_dgrad_kernel(RfDgradArgs g) {
   using G = RdGeom<CK, R, S>;
   constexpr int CPP = G::kCPP, PITCH = CPP * 16, KPT = G::kKPT, NK = G::kNK;
-  constexpr int RING = 6;  // fragment buffers (K-steps in flight)
-  static_assert(RING == 6 && CK % 32 == 0 && NK % RING == 0 && NK >= 3 * RING,
+#ifndef RD_RING
+#define RD_RING 9
+#endif
+  constexpr int RING = RD_RING; // fragment buffers (K-steps in flight)
+  constexpr int NFE = RING - 1; // fragments of the next block fetched early
+  constexpr int NF0 = NK - 2 * NFE - RING - 1; // step of the first early fetch, then every other step
+  static_assert(RING <= 9 && CK % 32 == 0 && NK % RING == 0 && NF0 >= 0,
                 "filter shape not covered");
   static_assert((S - 1) * PITCH + (KPT - 1) * 64 + 48 < 65536, "ds offset range");
   const int a_Q = g.Q, a_P = g.P, a_TR = g.TR, a_NI = g.NI, a_CO = g.CO;
@@ -172,8 +177,13 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
   {
     uint32_t fvoff[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      fvoff[i] = (uint32_t)((i * 8 + (l >> 3)) * wrow + kg * 128 + (l & 7) * 16);
+    for (int i = 0; i < 4; ++i) {
+      // chunk c of stage row r sits at position c ^ 4 * (r / 2 % 2): the 64 lanes
+      // of a fragment read then meet 4 to a bank pair instead of 8
+      const int row = i * 8 + (l >> 3);
+      const int c = (l & 7) ^ (((row >> 1) & 1) << 2);
+      fvoff[i] = (uint32_t)(row * wrow + kg * 128 + c * 16);
+    }
     gemm_static_for<NK / 4>([&](auto jc) {
       const int j = decltype(jc)::value * 4 + wave;
       const int tap = j / KPT, part = j - tap * KPT;
@@ -202,8 +212,9 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
   gemm_barrier();
   RD_STAMP(1);
   {
+    const int frow = 8 * q + (px >> 2);
     const uint32_t fread =
-        lds0 + (uint32_t)((8 * q + (px >> 2)) * 128 + slice * 64 + (px & 3) * 16);
+        lds0 + (uint32_t)(frow * 128 + (((slice * 4 + (px & 3)) ^ (((frow >> 1) & 1) << 2)) << 4));
     gemm_static_for<NK>([&](auto jc) {
       constexpr int j = decltype(jc)::value;
 #pragma unroll
@@ -332,35 +343,46 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
     // back edge may be copied there, which must not happen to a register a
     // load is still to write.  LDS returns in order, so a step waits until at
     // most `younger` reads issued after its own fragment's are outstanding.
-    u32x4 nfrag[RING - 1];
-    constexpr int NF0 = NK - 2 * RING; // step of the first early fetch
+    u32x4 nfrag[NFE];
     auto ksteps = [&]() __attribute__((always_inline)) {
       gemm_static_for<NK>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         constexpr int ahead = j + RING - 1;
         if constexpr (ahead < NK)
           fetch(std::integral_constant<int, ahead>{}, base, frag[ahead % RING]);
-        if constexpr (j >= NF0 && j < NF0 + RING - 1)
-          fetch(std::integral_constant<int, j - NF0>{}, nbase, nfrag[j - NF0]);
+        if constexpr (j >= NF0 && j < NF0 + 2 * NFE && (j - NF0) % 2 == 0)
+          fetch(std::integral_constant<int, (j - NF0) / 2>{}, nbase, nfrag[(j - NF0) / 2]);
+        // reads issued after this step's fragment's: the regular ones of the
+        // steps since, and the early ones issued at steps j - (RING - 1) .. j
         constexpr int regular = NK - 1 - j < RING - 1 ? NK - 1 - j : RING - 1;
-        // early fetches issued at steps j - (RING - 1) .. j
-        constexpr int lo = j - (RING - 1) > NF0 ? j - (RING - 1) : NF0;
-        constexpr int hi = j < NF0 + RING - 2 ? j : NF0 + RING - 2;
-        constexpr int early = hi >= lo ? hi - lo + 1 : 0;
+        constexpr int early = [] {
+          int n = 0;
+          for (int k = 0; k < NFE; ++k) {
+            const int st = NF0 + 2 * k;
+            n += (st >= j - (RING - 1) && st <= j) ? 1 : 0;
+          }
+          return n;
+        }();
+        static_assert(regular + early <= 15, "lgkmcnt is a 4-bit field");
         rd_wait_lgkm<regular + early>(frag[j % RING]);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
           acc[t] = rd_mfma<KIND>(filt[j][t], frag[j % RING],
                                  j == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[t]);
         }
+        // (keeps the step's MFMAs at its reads: with registers to spare the
+        // compiler would otherwise gather all reads of a block in front of all
+        // its MFMAs, or put off the second tile's MFMAs to the block's end, and
+        // nothing would overlap.  The empty statement orders both accumulators
+        // among the reads, which are volatile as well.)
+        asm volatile("" : "+a"(acc[0]), "+a"(acc[1]));
+        __builtin_amdgcn_sched_barrier(0);
       });
       // every read has returned (the early ones long ago)
-      asm volatile("s_waitcnt lgkmcnt(0)"
-                   : "+v"(nfrag[0]), "+v"(nfrag[1]), "+v"(nfrag[2]), "+v"(nfrag[3]),
-                     "+v"(nfrag[4]));
-#pragma unroll
-      for (int k = 0; k < RING - 1; ++k)
-        frag[k] = nfrag[k];
+      gemm_static_for<NFE>([&](auto kc) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(nfrag[decltype(kc)::value]));
+        frag[decltype(kc)::value] = nfrag[decltype(kc)::value];
+      });
     };
     // rounding and the 16-byte store of a finished block
     auto finish = [&](uint32_t off) __attribute__((always_inline)) {
