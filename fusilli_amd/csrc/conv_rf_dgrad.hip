@@ -249,21 +249,34 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
     n = rt / a_tiles_per_image;
     p0 = (rt - n * a_tiles_per_image) * a_TR;
   };
+  // s_sp / s_off: slab pixel and byte offset (pixel and chunk) of this lane's
+  // chunk of instruction i, the same for every tile; a chunk that no tile
+  // fetches has a pixel far below zero, which fails the column test.
+  int s_sp[kRdMaxNI];
+  uint32_t s_off[kRdMaxNI];
+#pragma unroll
+  for (int i = 0; i < kRdMaxNI; ++i)
+    if (i < a_NI) {
+      const int xk = i * 64 + l;
+      const int sp = (xk * (65536 / CPP + 1)) >> 16; // xk / CPP for xk < 2^12
+      const int c = xk - sp * CPP;
+      const bool ok = c < CPP - 1 && sp < a_TQ + S - 1;
+      s_sp[i] = ok ? sp : -0x40000000;
+      s_off[i] = (uint32_t)(sp * (CK * 2) + c * 16);
+    }
   auto issue_slab = [&](int tile, uint32_t dst0) __attribute__((always_inline)) {
     int n, p0, q0;
     tile_origin(tile, n, p0, q0);
     // slab pixel sp is input column q0 - pad_w + sp; only the TQ + S - 1
     // columns the tile needs are fetched
+    const int iw0 = q0 - a_pad_w;
     uint32_t rel[kRdMaxNI];
 #pragma unroll
-    for (int i = 0; i < kRdMaxNI; ++i) {
-      const int xk = i * 64 + l;
-      const int sp = (xk * (65536 / CPP + 1)) >> 16; // xk / CPP for xk < 2^12
-      const int c = xk - sp * CPP;
-      const int iw = q0 - a_pad_w + sp;
-      const bool ok = c < CPP - 1 && sp < a_TQ + S - 1 && (unsigned)iw < (unsigned)a_W;
-      rel[i] = ok ? (uint32_t)(iw * (CK * 2) + c * 16) : 0x80000000u;
-    }
+    for (int i = 0; i < kRdMaxNI; ++i)
+      if (i < a_NI)
+        rel[i] = (unsigned)(iw0 + s_sp[i]) < (unsigned)a_W
+                     ? s_off[i] + (uint32_t)(iw0 * (CK * 2))
+                     : 0x80000000u;
     const int tr = a_P - p0 < a_TR ? a_P - p0 : a_TR;
     const int rows_in = tr + R - 1;
     const int ih0 = p0 - a_pad_h;
@@ -402,9 +415,11 @@ conv_rf_dgrad_kernel(RfDgradArgs g) {
       __builtin_amdgcn_raw_buffer_store_b128(u32x4{w[0], w[1], w[2], w[3]}, ro, (int)off, 0, 19);
     };
 
-    // This wavefront's blocks: half, half + 2, ...  (a block index past the
-    // last one addresses the last pixel and stores nothing).
-    int b = half;
+    // This wavefront's blocks: b0, b0 + 2, ... with b0 = half on even tiles of
+    // the workgroup and 1 - half on odd ones, so that the odd block of a tile
+    // falls to either pair of wavefronts in turn.  (A block index past the last
+    // one addresses the last pixel and stores nothing.)
+    int b = half ^ cur;
     block_setup(b, base, ooff);
     gemm_static_for<RING - 1>(
         [&](auto jc) { fetch(jc, base, frag[decltype(jc)::value]); });
