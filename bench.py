@@ -692,6 +692,8 @@ def main():
              lambda: bench_conv_wgrad(ctx, max(20, args.steps // 10), kwarm)),
             ("sdpa_fwd_bf16_causal_b4h32s2048d128",
              lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm)),
+            ("sdpa_fwd_bf16_causal_b4h32s2048d64",
+             lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm, d=64)),
             ("sdpa_fwd_bf16_mask_b4h32s2048d128",
              lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm, masked=True)),
             ("layernorm_bf16_16x262144_long_rows",
