@@ -479,6 +479,36 @@ def bench_conv_padded(ctx, steps, warmup):
             "note": "1.4 GFLOP: launch-latency bound"}
 
 
+def bench_conv_grouped(ctx, steps, warmup):
+    """Grouped convolution on the MFMA kernels: N32 C256 56x56 -> K256, 3x3,
+    padding 1, 4 groups of 64 -> 64 channels (bf16 channels-last), one launch
+    whose outer grid dimension is the group."""
+    n, c, h, w, k, r, groups = 32, 256, 56, 56, 256, 3, 4
+    cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
+    xd, wd, yd = [n, c, h, w], [k, c // groups, r, r], [n, k, h, w]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.FLOAT)
+    d.out = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_conv_fprop_supported(d) == 2, "MFMA conv not chosen"
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 5, n * c * h * w)))
+    wt = ctx.to_device(synth.f32_to_bf16_bits(
+        synth.normal(8, 6, k * (c // groups) * r * r, 0.0, 0.05)))
+    out = ctx.alloc(n * k * h * w * 2)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.conv_fprop(d, x, wt, out),
+                                steps, warmup)
+    flop = 2.0 * n * h * w * k * (c // groups) * r * r
+    return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
+            "call_us": round(ev_ms * 1e3, 2), "work": flop, "kernels_per_call": 1}
+
+
 def calibrate_copy(ctx, steps):
     """Plain copy of known size (pointwise IDENTITY over 64 Mi int32 = 256 MiB
     read + 256 MiB written, on the strided kernel: one ordinary 4-byte load
@@ -698,6 +728,8 @@ def main():
              lambda: bench_sdpa(ctx, max(20, args.steps // 4), kwarm, masked=True)),
             ("layernorm_bf16_16x262144_long_rows",
              lambda: bench_layernorm_long(ctx, max(20, args.steps // 4), kwarm)),
+            ("conv_fprop_bf16_n32c256h56w56_k256r3s3_groups4",
+             lambda: bench_conv_grouped(ctx, max(20, args.steps // 10), kwarm)),
             ("conv_fprop_f16_n16c48h48w32_k48r3s3_padded_channels",
              lambda: bench_conv_padded(ctx, max(20, args.steps // 4), kwarm)),
         ]

@@ -26,6 +26,11 @@ struct ConvPlan {
   int bm = 256, bn = 128;
   bool halo = false;
   int tile_rows = 0; // halo mode: rows per M tile (<= bm)
+  // grouped convolution: one GEMM per group (the kernel's outer batch dim)
+  // over the group's channel runs of X, its rows of W and its columns of OUT;
+  // N and K are a group's
+  int groups = 1;
+  int64_t channels_out = 0; // of all groups
 };
 
 // strides equal the dense channels-last strides of dims (unit dims are free)
@@ -130,9 +135,11 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
     return p;
   const int elem = 2;
   const int sp = d->spatial_rank;
-  const int64_t C = d->x.dim[1];
-  if (d->w.dim[1] != C) // grouped convolutions take the generic kernel
+  const int64_t Call = d->x.dim[1];
+  const int64_t C = d->w.dim[1]; // channels of one group
+  if (C <= 0 || Call % C != 0 || d->w.dim[0] % (Call / C) != 0)
     return p;
+  p.groups = (int)(Call / C);
   if ((C * elem) % kTileKBytes != 0)
     return p;
   if (!is_channels_last(d->x) || !is_channels_last(d->w) ||
@@ -158,15 +165,17 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
   g.pad_w = (int32_t)d->padding[sp - 1];
   g.str_w = (int32_t)d->stride[sp - 1];
   g.dil_w = (int32_t)d->dilation[sp - 1];
+  g.x_pitch = (int32_t)(Call * elem);
   g.slices_per_tap = (int32_t)(C * elem / kTileKBytes);
   p.M = d->x.dim[0] * g.P * g.Q;
-  p.N = d->w.dim[0];
+  p.channels_out = d->w.dim[0];
+  p.N = d->w.dim[0] / p.groups;
   p.K = R * g.S * C;
   // 32-bit byte offsets in the gather; one validity bit per filter row and
   // one per filter column
-  const int64_t x_bytes = d->x.dim[0] * (int64_t)g.H * g.W * C * elem;
+  const int64_t x_bytes = d->x.dim[0] * (int64_t)g.H * g.W * Call * elem;
   if (x_bytes >= (1ll << 31) || p.M >= (1ll << 31) || R > 16 || g.S > 16 ||
-      p.K * elem >= (1ll << 23))
+      p.K * elem >= (1ll << 23) || p.groups > 65535)
     return p;
   g.x_bytes = (uint32_t)x_bytes;
   g.R = (int32_t)R;
@@ -402,15 +411,23 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   g.K = p.K;
   g.a_ld = 0;
   g.b_ld = p.K; // filter rows are R*S*C contiguous elements
-  g.o_sm = p.N; // OUT is dense channels-last: consecutive pixels are N apart
+  g.o_sm = p.channels_out; // OUT is dense channels-last: pixels are all groups' channels apart
   g.o_sn = 1;
   g.o_batch = 0;
+  if (p.groups > 1) {
+    g.outer = p.groups;
+    g.a_outer = p.geom.C;  // a group's first input channel
+    g.b_outer = p.N * p.K; // its filter rows
+    g.o_outer = p.N;       // its first output channel,
+    g.epi_n_outer = p.N;   // which fused per-channel operands see as well
+  }
   g.c_dt = d->y.dtype;
   g.o_dt = d->out.dtype;
   g.tile_rows = p.halo ? p.tile_rows : p.bm;
   g.tiles_m = (int)((p.M + g.tile_rows - 1) / g.tile_rows);
   g.tiles_n = (int)((p.N + p.bn - 1) / p.bn);
   g.o_vec = (p.N * fhip_dtype_size(d->out.dtype)) % 16 == 0 &&
+            (p.channels_out * fhip_dtype_size(d->out.dtype)) % 16 == 0 &&
             ((uintptr_t)out & 15) == 0;
   g.epi = epi;
   g.epi.rank = 3;

@@ -95,7 +95,8 @@ constexpr int kThreads = 256;
 // the GEMM is output pixel (n, p, q) and K-slice kt is filter tap (r, s) with a
 // 128-byte run of channels, gathered from the NHWC input (zero outside it).
 struct ConvGeom {
-  int32_t H, W, C;        // input spatial extents and channels
+  int32_t H, W, C;        // input spatial extents and channels (of one group)
+  int32_t x_pitch;        // bytes between input pixels (all groups' channels)
   int32_t P, Q;           // output spatial extents
   int32_t S;              // filter width (taps per filter row)
   int32_t pad_h, pad_w, str_h, str_w, dil_h, dil_w;
@@ -143,6 +144,9 @@ struct GemmArgs {
   // optional outer batch dim (grid z) with strides of its own; fused operands
   // do not see it
   int64_t a_outer, b_outer, o_outer;
+  // column offset per outer index that fused operands DO see (grouped
+  // convolution: the group's first output channel); 0 otherwise
+  int64_t epi_n_outer;
   int32_t outer; // extent (0 or 1: none)
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
@@ -537,10 +541,10 @@ gemm_kernel(GemmArgs g) {
   int32_t h_row[HALO ? TM : 1];
   uint32_t h_mask[HALO ? TM : 1];
   if constexpr (HALO) {
-    a_base = g.a;
+    a_base = g.a + outer * g.a_outer * ELEM; // a group's first channel
     a_step = 0;
   } else if constexpr (A_MODE == A_CONV) {
-    a_base = g.a;
+    a_base = g.a + outer * g.a_outer * ELEM;
     a_step = 0;
 #pragma unroll
     for (int j = 0; j < GA::kLoads; ++j) {
@@ -614,7 +618,7 @@ gemm_kernel(GemmArgs g) {
       const int32_t fr = conv_div(tap, g.conv.S, g.conv.magic_s);
       const int32_t fs = tap - fr * g.conv.S;
       const int32_t dpix = fr * g.conv.dil_h * g.conv.W + fs * g.conv.dil_w;
-      const int32_t cbytes = g.conv.C * ELEM;
+      const int32_t cbytes = g.conv.x_pitch;
       uint32_t off[GA::kLoads];
 #pragma unroll
       for (int j = A0; j < A1; ++j) {
@@ -641,7 +645,7 @@ gemm_kernel(GemmArgs g) {
     // its end read as zeros, rows of other image lines are masked at use.
     const int32_t pix0 =
         (int32_t)m0 - g.conv.pad_h * g.conv.W - g.conv.pad_w;
-    const int32_t cbytes = g.conv.C * ELEM;
+    const int32_t cbytes = g.conv.x_pitch;
     const int groups = g.conv.halo_rows / 8;
     const uint64_t b64 = (uint64_t)a_base;
     const uint32_t blo = __builtin_amdgcn_readfirstlane((uint32_t)b64);
@@ -957,7 +961,7 @@ gemm_kernel(GemmArgs g) {
           if (o.kind == FHIP_OPERAND_TENSOR) {
             int64_t n = n0 + wn * WN + j * 32 + (l & 31);
             n = n < gN ? n : gN - 1;
-            const int64_t off[1] = {n * o.stride[2]};
+            const int64_t off[1] = {(n + outer * g.epi_n_outer) * o.stride[2]};
             float one[1];
             load_operand_vec<1>(o.ptr, o.operand_dtype, off, one);
             ov = one[0];
@@ -1144,7 +1148,7 @@ gemm_kernel(GemmArgs g) {
               for (int c = 0; c < 8; ++c) {
                 int64_t n = ncol + c;
                 n = n < g.N ? n : g.N - 1; // edge tiles stay in bounds
-                off[c] = base + n * o.stride[2];
+                off[c] = base + (n + outer * g.epi_n_outer) * o.stride[2];
               }
               load_operand_vec<8>(o.ptr, o.operand_dtype, off, other);
             }
@@ -1355,7 +1359,8 @@ int conv_launch_halo(fhip_ctx *ctx, const GemmArgs &g) {
                             160 * 1024));
     configured.mark(ctx->device);
   }
-  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1);
+  const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1,
+                  (unsigned)(g.outer > 1 ? g.outer : 1));
   hipLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, g);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   return 0;

@@ -2,7 +2,7 @@
 
 Shapes here satisfy the tuned kernel's contract (channels-last bf16/f16,
 C a multiple of 8 -- channel counts that are no multiple of 64 run on
-zero-padded copies --, groups = 1); each test asserts that the tuned kernel is
+zero-padded copies --, one group or groups of a multiple of 64 channels); each test asserts that the tuned kernel is
 the one chosen, so a silent fall back to the generic kernel fails.
 """
 import numpy as np
@@ -182,16 +182,58 @@ def test_conv_igemm_bias_relu_residual(ctx):
     assert_close(out.logical(), ref, capi.BFLOAT16)
 
 
+GROUPED_CASES = [
+    # two groups of 64 -> 64 channels, same geometry (halo tiles, 64 wide)
+    dict(x=[2, 128, 9, 11], w=[128, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    # four groups of 64 -> 24 channels (ragged columns), stride 2 (gather)
+    dict(x=[2, 256, 8, 8], w=[96, 64, 3, 3], pad=[1, 1], s=[2, 2], d=[1, 1]),
+    # three groups of 128 -> 136 channels (two column tiles per group), 1x1
+    dict(x=[1, 384, 7, 6], w=[408, 128, 1, 1], pad=[0, 0], s=[1, 1], d=[1, 1]),
+    # 1-D, two groups of 64 -> 16, dilation 2
+    dict(x=[3, 128, 40], w=[32, 64, 5], pad=[4], s=[1], d=[2]),
+    # many groups: 16 groups of 64 -> 8 channels
+    dict(x=[1, 1024, 6, 5], w=[128, 64, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+]
+
+
+@pytest.mark.parametrize("case", GROUPED_CASES)
+@pytest.mark.parametrize("halo", ["auto", "0"])
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_conv_grouped_vs_oracle(ctx, case, halo, dtype, knobs):
+    # Reference: conv with groups = C / filter channels (aten.convolution's
+    # groups operand, reference support/asm_emitter.h:690-701).  One GEMM per
+    # group on the MFMA kernels; the fused bias is indexed by the channel of
+    # the whole output, not of the group.
+    if halo != "auto":
+        knobs(CONV_HALO=halo)
+    x = cl(case["x"], 48, 0, dtype)
+    w = cl(case["w"], 48, 1, dtype, std=0.1)
+    k = case["w"][0]
+    bdims = [1, k] + [1] * len(case["pad"])
+    bias = HT.from_logical(rand(48, 2, bdims), dtype, oracle.channels_last_strides(bdims))
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT)]
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT, out_dtype=dtype,
+              epilogue=epi, epi_tensors=[bias])
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"], case["d"])
+    ref = np.maximum(ref + bias.logical(), 0.0)
+    assert_close(out.logical(), ref, dtype, f"halo={halo} {case}")
+    # no epilogue, f32 out
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"], case["d"])
+    assert_close(out.logical(), ref, capi.FLOAT, f"halo={halo} {case}", rtol=1e-4)
+
+
 def test_conv_igemm_not_chosen_outside_contract(ctx):
-    # C = 44 (not whole 16-byte chunks per pixel) and grouped filters keep the
-    # generic kernel
+    # C = 44 (not whole 16-byte chunks per pixel) and groups of 32 channels
+    # (half a K slice) keep the generic kernel
     x = cl([1, 44, 8, 8], 44, 0, capi.BFLOAT16)
     w = cl([16, 44, 3, 3], 44, 1, capi.BFLOAT16, std=0.1)
     out = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.BFLOAT16, expect_tuned=False)
     ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
     assert_close(out.logical(), ref, capi.BFLOAT16)
     x = cl([1, 128, 8, 8], 44, 2, capi.BFLOAT16)
-    w = cl([16, 64, 3, 3], 44, 3, capi.BFLOAT16, std=0.1)
+    w = cl([16, 32, 3, 3], 44, 3, capi.BFLOAT16, std=0.1)
     out = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.BFLOAT16, expect_tuned=False)
     ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
     assert_close(out.logical(), ref, capi.BFLOAT16)
