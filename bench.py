@@ -509,6 +509,35 @@ def bench_conv_grouped(ctx, steps, warmup):
             "call_us": round(ev_ms * 1e3, 2), "work": flop, "kernels_per_call": 1}
 
 
+def bench_conv_depthwise(ctx, steps, warmup):
+    """Depthwise 3x3 convolution (groups = channels), N32 C128 56x56, padding 1,
+    bf16 channels-last: the channels-last small-group kernel; bound by HBM
+    (X read once, OUT written once)."""
+    n, c, h, w, r = 32, 128, 56, 56, 3
+    cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
+    xd, wd, yd = [n, c, h, w], [c, 1, r, r], [n, c, h, w]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.FLOAT)
+    d.out = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_conv_fprop_supported(d) == 2, "small-group kernel not chosen"
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 7, n * c * h * w)))
+    wt = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 8, c * r * r, 0.0, 0.3)))
+    out = ctx.alloc(n * c * h * w * 2)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.conv_fprop(d, x, wt, out),
+                                steps, warmup)
+    nbytes = 2 * n * c * h * w * 2 + c * r * r * 2
+    return {"value": round(nbytes / ev_ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "call_us": round(ev_ms * 1e3, 2), "bytes": nbytes, "kernels_per_call": 1}
+
+
 def calibrate_copy(ctx, steps):
     """Plain copy of known size (pointwise IDENTITY over 64 Mi int32 = 256 MiB
     read + 256 MiB written, on the strided kernel: one ordinary 4-byte load
@@ -730,6 +759,8 @@ def main():
              lambda: bench_layernorm_long(ctx, max(20, args.steps // 4), kwarm)),
             ("conv_fprop_bf16_n32c256h56w56_k256r3s3_groups4",
              lambda: bench_conv_grouped(ctx, max(20, args.steps // 10), kwarm)),
+            ("conv_fprop_bf16_n32c128h56w56_depthwise_r3s3",
+             lambda: bench_conv_depthwise(ctx, max(20, args.steps // 10), kwarm)),
             ("conv_fprop_f16_n16c48h48w32_k48r3s3_padded_channels",
              lambda: bench_conv_padded(ctx, max(20, args.steps // 4), kwarm)),
         ]

@@ -142,6 +142,216 @@ __global__ __launch_bounds__(256) void direct_conv_fprop_kernel(
   }
 }
 
+// ---- channels-last groups of 1, 2, 4 or 8 channels (depthwise, ResNeXt) ------
+// 16-bit channels-last X, W and OUT (f32 OUT too) with as many output as input
+// channels per group.  A thread owns one output pixel and 8 consecutive
+// channels -- whole groups -- so that every tap is ONE 16-byte load of X (the
+// lanes of a pixel are consecutive chunks: coalesced) feeding 8 x CG
+// multiply-adds, and the 8 results leave as one 16-byte store.  A workgroup is
+// 16 pixels x 16 channel blocks; it keeps the f32 filter of its 128 channels in
+// LDS as [block][tap][8][CG] (blocks 4 words past a multiple of 64 apart: the
+// 16 blocks of a wavefront read different banks, its 4 pixels the same words)
+// and walks `iters` groups of 16 pixels.
+struct DcClArgs {
+  int32_t N, H, W, C, K, P, Q, R, S;
+  int32_t pad_h, pad_w, str_h, str_w, dil_h, dil_w;
+  int32_t cbs;     // 8-channel blocks of a pixel
+  int32_t stride;  // LDS words between the blocks' filters
+  int32_t iters;
+  int32_t y_dt, o_dt, sp;
+  uint32_t pixels;
+  DevEpilogue epi;
+};
+
+template <bool BF16, int CG>
+__global__ __launch_bounds__(256) void direct_conv_fprop_cl_kernel(
+    DcClArgs g, const void *x, const void *w, void *out) {
+  extern __shared__ __attribute__((aligned(16))) float wcl[];
+  const int tid = threadIdx.x;
+  const int cbl = tid & 15, pl = tid >> 4;
+  const int cb0 = blockIdx.y * 16;
+  const int fvol = g.R * g.S;
+  const int per_block = fvol * 8 * CG;
+  auto to_f32 = [](uint32_t h) __attribute__((always_inline)) {
+    if constexpr (BF16)
+      return __builtin_bit_cast(float, h << 16);
+    else
+      return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+  };
+  for (int e = tid; e < 16 * per_block; e += 256) {
+    const int b = e / per_block, rest = e - b * per_block; // rest = (tap * 8 + k) * CG + j
+    const int j = rest % CG, tk = rest / CG;
+    const int k = tk & 7, tap = tk >> 3;
+    const int kg = (cb0 + b) * 8 + k;
+    float v = 0.f;
+    if (kg < g.K)
+      v = to_f32(((const uint16_t *)w)[((int64_t)kg * fvol + tap) * CG + j]);
+    wcl[b * g.stride + rest] = v;
+  }
+  __syncthreads();
+  const int cb = cb0 + cbl;
+  if (cb >= g.cbs)
+    return;
+  const float *wl = wcl + cbl * g.stride;
+  const uint32_t first = blockIdx.x * (uint32_t)(16 * g.iters) + (uint32_t)pl;
+  for (int it = 0; it < g.iters; ++it) {
+    const uint32_t pix = first + (uint32_t)it * 16u;
+    if (pix >= g.pixels)
+      break;
+    const int q = pix % (uint32_t)g.Q;
+    const uint32_t t = pix / (uint32_t)g.Q;
+    const int p = t % (uint32_t)g.P, n = t / (uint32_t)g.P;
+    const int ih0 = p * g.str_h - g.pad_h, iw0 = q * g.str_w - g.pad_w;
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      acc[k] = 0.f;
+    for (int r = 0; r < g.R; ++r) {
+      const int ih = ih0 + r * g.dil_h;
+      if ((unsigned)ih >= (unsigned)g.H)
+        continue;
+      const int64_t row = ((int64_t)n * g.H + ih) * g.W;
+      for (int s = 0; s < g.S; ++s) {
+        const int iw = iw0 + s * g.dil_w;
+        if ((unsigned)iw >= (unsigned)g.W)
+          continue;
+        const uint4 xv = *(const uint4 *)((const uint16_t *)x + (row + iw) * g.C + cb * 8);
+        const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+        float xf[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          xf[2 * i] = to_f32(xw[i] & 0xffffu);
+          xf[2 * i + 1] = to_f32(xw[i] >> 16);
+        }
+        // (16-byte aligned: the blocks' distance and a tap's 8 * CG words are
+        // multiples of 4 words)
+        const float4 *wt4 = (const float4 *)(wl + (r * g.S + s) * 8 * CG);
+        float wt[8 * CG];
+#pragma unroll
+        for (int i = 0; i < 2 * CG; ++i) {
+          const float4 v = wt4[i];
+          wt[4 * i] = v.x, wt[4 * i + 1] = v.y, wt[4 * i + 2] = v.z, wt[4 * i + 3] = v.w;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+#pragma unroll
+          for (int j = 0; j < CG; ++j)
+            acc[k] = __builtin_fmaf(xf[k / CG * CG + j], wt[k * CG + j], acc[k]);
+      }
+    }
+    int64_t coord[FHIP_MAX_RANK];
+    coord[0] = n;
+    if (g.sp == 2) {
+      coord[2] = p;
+      coord[3] = q;
+    } else {
+      coord[2] = q;
+    }
+    float y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      coord[1] = cb * 8 + k;
+      y[k] = fhip_apply_epilogue<float>(g.epi, fhip_round_through<float>(g.y_dt, acc[k]), coord);
+    }
+    const int64_t ob = (int64_t)pix * g.K + cb * 8;
+    if (g.o_dt == FHIP_FLOAT) {
+      float4 *o = (float4 *)((float *)out + ob);
+      o[0] = make_float4(y[0], y[1], y[2], y[3]);
+      o[1] = make_float4(y[4], y[5], y[6], y[7]);
+    } else {
+      uint32_t ow[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t lo, hi;
+        if (g.o_dt == FHIP_BFLOAT16) {
+          lo = __builtin_bit_cast(uint16_t, (__bf16)y[2 * i]);
+          hi = __builtin_bit_cast(uint16_t, (__bf16)y[2 * i + 1]);
+        } else {
+          lo = __builtin_bit_cast(uint16_t, (_Float16)y[2 * i]);
+          hi = __builtin_bit_cast(uint16_t, (_Float16)y[2 * i + 1]);
+        }
+        ow[i] = lo | (hi << 16);
+      }
+      *(uint4 *)((uint16_t *)out + ob) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+  }
+}
+
+// dense channels-last strides of dims [d0, C, spatial...] (unit dims are free)
+bool dc_channels_last(const fhip_tensor_desc &t) {
+  int64_t expect = t.dim[1];
+  if (t.dim[1] != 1 && t.stride[1] != 1)
+    return false;
+  for (int i = t.rank - 1; i >= 2; --i) {
+    if (t.dim[i] != 1 && t.stride[i] != expect)
+      return false;
+    expect *= t.dim[i];
+  }
+  return t.dim[0] == 1 || t.stride[0] == expect;
+}
+
+constexpr int kDcClLds = 64 * 1024;
+
+bool make_cl_args(const fhip_conv_desc *d, DcClArgs &g) {
+  const int sp = d->spatial_rank;
+  if ((sp != 1 && sp != 2) || d->x.rank != 2 + sp)
+    return false;
+  if (d->x.dtype != d->w.dtype ||
+      (d->x.dtype != FHIP_BFLOAT16 && d->x.dtype != FHIP_HALF))
+    return false;
+  if (d->out.dtype != FHIP_BFLOAT16 && d->out.dtype != FHIP_HALF &&
+      d->out.dtype != FHIP_FLOAT)
+    return false;
+  const int64_t C = d->x.dim[1], K = d->w.dim[0], CG = d->w.dim[1];
+  if (C != K || C % 8 != 0 || (CG != 1 && CG != 2 && CG != 4 && CG != 8))
+    return false;
+  if (!dc_channels_last(d->x) || !dc_channels_last(d->w) || !dc_channels_last(d->out) ||
+      d->out.rank != d->y.rank)
+    return false;
+  const int64_t lim = 1ll << 30;
+  const int64_t pixels = fhip_desc_volume(d->y) / (K > 0 ? K : 1);
+  if (fhip_desc_volume(d->x) >= lim || fhip_desc_volume(d->y) >= lim * 2 || pixels < 1)
+    return false;
+  g.N = (int32_t)d->x.dim[0];
+  g.C = (int32_t)C;
+  g.K = (int32_t)K;
+  g.H = sp == 2 ? (int32_t)d->x.dim[2] : 1;
+  g.W = (int32_t)d->x.dim[1 + sp];
+  g.P = sp == 2 ? (int32_t)d->y.dim[2] : 1;
+  g.Q = (int32_t)d->y.dim[1 + sp];
+  g.R = sp == 2 ? (int32_t)d->w.dim[2] : 1;
+  g.S = (int32_t)d->w.dim[1 + sp];
+  g.pad_h = sp == 2 ? (int32_t)d->padding[0] : 0;
+  g.str_h = sp == 2 ? (int32_t)d->stride[0] : 1;
+  g.dil_h = sp == 2 ? (int32_t)d->dilation[0] : 1;
+  g.pad_w = (int32_t)d->padding[sp - 1];
+  g.str_w = (int32_t)d->stride[sp - 1];
+  g.dil_w = (int32_t)d->dilation[sp - 1];
+  if (d->padding[sp - 1] >= lim || d->stride[sp - 1] >= lim || d->dilation[sp - 1] >= lim ||
+      (sp == 2 && (d->padding[0] >= lim || d->stride[0] >= lim || d->dilation[0] >= lim)))
+    return false;
+  const int64_t per_block = (int64_t)g.R * g.S * 8 * CG;
+  // blocks 4 words past a multiple of 64 apart
+  const int64_t stride = (per_block + 59) / 64 * 64 + 4;
+  if (16 * stride * 4 > kDcClLds)
+    return false;
+  g.stride = (int32_t)stride;
+  g.cbs = (int32_t)(C / 8);
+  if ((g.cbs + 15) / 16 > 65535)
+    return false;
+  g.pixels = (uint32_t)pixels;
+  g.y_dt = d->y.dtype;
+  g.o_dt = d->out.dtype;
+  g.sp = sp;
+  // about eight workgroups per compute unit, at most 16 pixel groups each
+  const int64_t ygrid = (g.cbs + 15) / 16;
+  int64_t iters = pixels * ygrid / (16 * 2048);
+  g.iters = (int32_t)(iters < 1 ? 1 : iters > 16 ? 16 : iters);
+  g.epi.count = 0;
+  g.epi.rank = 0;
+  return true;
+}
+
 // DX[n, c, i..] = sum over the k of c's group and the taps f with
 // i + pad - f * dil = o * stride:  DY[n, k, o..] * W[k, c % fC, f..]
 template <int DT>
@@ -473,9 +683,50 @@ bool fhip_direct_conv_applicable(const fhip_conv_desc *d) {
          (g.fC * fvol + kWgJ - 1) / kWgJ <= 65535;
 }
 
+bool fhip_direct_conv_cl_applicable(const fhip_conv_desc *d) {
+  DcClArgs g{};
+  // (tensors that are not 16-byte aligned run on the general kernel)
+  return make_cl_args(d, g) && fhip_direct_conv_applicable(d);
+}
+
 int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
                            const void *x, const void *w, const DevEpilogue &epi,
                            void *out) {
+  {
+    DcClArgs c{};
+    if (make_cl_args(d, c) && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0) {
+      c.epi = epi;
+      const dim3 grid((unsigned)((c.pixels + 16u * c.iters - 1) / (16u * c.iters)),
+                      (unsigned)((c.cbs + 15) / 16));
+      const size_t lds = (size_t)16 * c.stride * 4;
+      const bool bf16 = d->x.dtype == FHIP_BFLOAT16;
+      auto go = [&](auto cg) {
+        constexpr int CG = decltype(cg)::value;
+        if (bf16)
+          hipLaunchKernelGGL((direct_conv_fprop_cl_kernel<true, CG>), grid, dim3(256), lds,
+                             ctx->stream, c, x, w, out);
+        else
+          hipLaunchKernelGGL((direct_conv_fprop_cl_kernel<false, CG>), grid, dim3(256), lds,
+                             ctx->stream, c, x, w, out);
+      };
+      switch ((int)d->w.dim[1]) {
+      case 1:
+        go(std::integral_constant<int, 1>{});
+        break;
+      case 2:
+        go(std::integral_constant<int, 2>{});
+        break;
+      case 4:
+        go(std::integral_constant<int, 4>{});
+        break;
+      default:
+        go(std::integral_constant<int, 8>{});
+        break;
+      }
+      FHIP_HIP_CHECK(ctx, hipGetLastError());
+      return 0;
+    }
+  }
   DcArgs g{};
   FHIP_REQUIRE(ctx, make_args(d, g),
                "conv: descriptor not supported by the direct kernel");

@@ -74,6 +74,8 @@ int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
 // kernels do not take.  The weight gradient keeps its partial sums in the
 // context's scratch buffer.
 bool fhip_direct_conv_applicable(const fhip_conv_desc *d);
+// forward: the channels-last kernel for groups of 1, 2, 4 or 8 channels
+bool fhip_direct_conv_cl_applicable(const fhip_conv_desc *d);
 int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
                            const void *x, const void *w, const DevEpilogue &epi,
                            void *out);

@@ -1189,7 +1189,7 @@ int fhip_conv_fprop_workspace_size(const fhip_conv_desc *d, size_t *bytes) {
 int fhip_conv_fprop_supported(const fhip_conv_desc *d) {
   if (!d || conv_validate(nullptr, d) != 0)
     return 0;
-  return fhip_fast_conv_applicable(d) ? 2 : 1;
+  return fhip_fast_conv_applicable(d) || fhip_direct_conv_cl_applicable(d) ? 2 : 1;
 }
 
 int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,

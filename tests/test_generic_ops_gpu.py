@@ -352,6 +352,55 @@ def test_conv_direct_kernels_vs_oracle(ctx, case, dtype, nhwc):
                  dtype, f"wgrad {case}")
 
 
+SMALL_GROUP_CASES = [
+    # depthwise 3x3 (ConvNeXt / MobileNet style), ragged pixel count
+    dict(x=[2, 40, 9, 7], w=[40, 1, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    # depthwise 7x7, more than one workgroup of channel blocks (136 channels)
+    dict(x=[1, 136, 12, 10], w=[136, 1, 7, 7], pad=[3, 3], s=[1, 1], d=[1, 1]),
+    # ResNeXt: 32 groups of 4 -> 4 channels; stride 2
+    dict(x=[2, 128, 10, 11], w=[128, 4, 3, 3], pad=[1, 1], s=[2, 2], d=[1, 1]),
+    # groups of 8 and of 2, dilation, asymmetric padding
+    dict(x=[1, 64, 8, 9], w=[64, 8, 3, 2], pad=[2, 0], s=[1, 1], d=[2, 1]),
+    dict(x=[3, 16, 6, 5], w=[16, 2, 1, 3], pad=[0, 1], s=[1, 2], d=[1, 1]),
+    # 1-D depthwise
+    dict(x=[2, 24, 50], w=[24, 1, 5], pad=[2], s=[1], d=[1]),
+]
+
+
+@pytest.mark.parametrize("case", SMALL_GROUP_CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("out_dtype", ["same", "f32"])
+def test_conv_small_groups_channels_last_vs_oracle(ctx, case, dtype, out_dtype):
+    # Channels-last 16-bit convolutions whose groups have 1, 2, 4 or 8 input
+    # and as many output channels: the kernel that owns whole groups per
+    # thread (one 16-byte load per tap), with a per-channel bias and ReLU.
+    lay = oracle.channels_last_strides
+    x = HT.from_logical(rand(35, 0, case["x"]), dtype, lay(case["x"]))
+    w = HT.from_logical(rand(35, 1, case["w"], std=0.3), dtype, lay(case["w"]))
+    k = case["w"][0]
+    bdims = [1, k] + [1] * len(case["pad"])
+    bias = HT.from_logical(rand(35, 3, bdims), dtype)
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT)]
+    od = dtype if out_dtype == "same" else capi.FLOAT
+    ydims = oracle.conv_output_dims(case["x"], case["w"], case["pad"], case["s"], case["d"])
+    d = capi.ConvDesc()
+    d.x, d.w = x.desc(), w.desc()
+    d.y = capi.TensorDesc.make(ydims, lay(ydims), capi.FLOAT)
+    d.out = capi.TensorDesc.make(ydims, lay(ydims), od)
+    d.out_dtype = od
+    d.spatial_rank = len(case["pad"])
+    for i in range(len(case["pad"])):
+        d.padding[i], d.stride[i], d.dilation[i] = case["pad"][i], case["s"][i], case["d"][i]
+    d.epilogue = capi.make_epilogue(epi)
+    assert ctx.lib.fhip_conv_fprop_supported(d) == 2
+    y = run_conv(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT, out_dtype=od,
+                 epilogue=epi, epi_tensors=[bias], channels_last_out=True)
+    ref = np.maximum(oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"],
+                                       case["d"]) + bias.logical(), 0.0)
+    assert_close(y.logical(), ref, od, f"{case}")
+
+
 def test_conv_direct_kernels_mixed_dtypes(ctx):
     # bf16 X against an f32 filter, f32 result: the run-time dtype path
     xd, wd = [2, 5, 8, 9], [7, 5, 3, 3]
