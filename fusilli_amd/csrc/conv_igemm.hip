@@ -484,8 +484,12 @@ DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
   const int sp = d->spatial_rank;
   if (sp != 1 && sp != 2)
     return p;
-  if (d->w.dim[1] != d->x.dim[1]) // groups
+  // groups: the forward problem is grouped the same way (a group's K / groups
+  // gradient channels in, its C / groups channels out)
+  const int64_t Cg = d->w.dim[1];
+  if (Cg < 1 || d->x.dim[1] % Cg != 0 || d->w.dim[0] % (d->x.dim[1] / Cg) != 0)
     return p;
+  const int64_t groups = d->x.dim[1] / Cg;
   if (d->y.dtype != d->w.dtype)
     return p;
   fhip_conv_desc &f = p.fwd;
@@ -522,11 +526,11 @@ DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
   f.y = d->x; // DX plays the output
   f.out = d->x;
   f.out_dtype = d->x.dtype;
-  // W' [C, K, F...], dense channels-last
+  // W' [C, K / groups, F...], dense channels-last
   f.w.rank = d->w.rank;
   f.w.dtype = d->w.dtype;
-  f.w.dim[0] = d->w.dim[1];
-  f.w.dim[1] = d->w.dim[0];
+  f.w.dim[0] = d->x.dim[1];
+  f.w.dim[1] = d->w.dim[0] / groups;
   int64_t st = f.w.dim[1];
   f.w.stride[1] = 1;
   for (int i = sp - 1; i >= 0; --i) {
@@ -569,11 +573,12 @@ __global__ void conv_spread_kernel(SpreadArgs a, const uint4 *src, uint4 *dst) {
 }
 
 struct FlipArgs {
-  int64_t K, C, R, S;         // R = 1 for one spatial dim
-  int64_t sk, sc, sr, ss;     // element strides of W [K, C, R, S]
+  int64_t K, C, R, S;         // of one group; R = 1 for one spatial dim
+  int64_t sk, sc, sr, ss;     // element strides of W [groups * K, C, R, S]
 };
 
-// dst[c][r'][s'][k] = src[k][c][R - 1 - r'][S - 1 - s'], 16-bit elements
+// dst[g * C + c][r'][s'][k] = src[g * K + k][c][R - 1 - r'][S - 1 - s'], 16-bit
+// elements
 __global__ void conv_flip_filter_kernel(FlipArgs a, const uint16_t *src,
                                         uint16_t *dst, int64_t total) {
   const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -584,8 +589,9 @@ __global__ void conv_flip_filter_kernel(FlipArgs a, const uint16_t *src,
   const int64_t s2 = rem % a.S;
   rem /= a.S;
   const int64_t r2 = rem % a.R;
-  const int64_t c = rem / a.R;
-  dst[lin] = src[k * a.sk + c * a.sc + (a.R - 1 - r2) * a.sr +
+  const int64_t gc = rem / a.R;
+  const int64_t grp = gc / a.C, c = gc - grp * a.C;
+  dst[lin] = src[(grp * a.K + k) * a.sk + c * a.sc + (a.R - 1 - r2) * a.sr +
                  (a.S - 1 - s2) * a.ss];
 }
 
@@ -638,7 +644,8 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                "conv dgrad: workspace must be 16-byte aligned");
   const int sp = d->spatial_rank;
   FlipArgs a;
-  a.K = d->w.dim[0];
+  const int64_t groups = d->x.dim[1] / d->w.dim[1];
+  a.K = d->w.dim[0] / groups;
   a.C = d->w.dim[1];
   a.R = sp == 2 ? d->w.dim[2] : 1;
   a.S = d->w.dim[1 + sp];
@@ -646,7 +653,7 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   a.sc = d->w.dim[1] == 1 ? 0 : d->w.stride[1];
   a.sr = sp == 2 ? d->w.stride[2] : 0;
   a.ss = d->w.stride[1 + sp];
-  const int64_t total = a.K * a.C * a.R * a.S;
+  const int64_t total = groups * a.K * a.C * a.R * a.S;
   hipLaunchKernelGGL(conv_flip_filter_kernel,
                      dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                      ctx->stream, a, (const uint16_t *)w, (uint16_t *)workspace,

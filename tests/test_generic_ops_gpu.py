@@ -430,12 +430,17 @@ def test_conv_direct_kernels_mixed_dtypes(ctx):
     dict(x=[3, 24, 23, 31], w=[64, 24, 4, 3], pad=[2, 1], d=[2, 1], s=[3, 2]),
     dict(x=[2, 128, 16, 16], w=[256, 128, 1, 1], pad=[0, 0], d=[1, 1], s=[2, 2]),
     dict(x=[2, 16, 101], w=[64, 16, 5], pad=[2], d=[1], s=[4]),
+    # groups whose K / groups is a multiple of 64: 2 groups of 24 <- 64
+    # channels, 3 groups of 8 <- 128 with a stride, 1-D
+    dict(x=[2, 48, 13, 12], w=[128, 24, 3, 3], pad=[1, 1], d=[1, 1]),
+    dict(x=[1, 24, 15, 14], w=[384, 8, 3, 3], pad=[1, 1], d=[1, 1], s=[2, 2]),
+    dict(x=[3, 32, 60], w=[128, 16, 5], pad=[2], d=[1]),
 ])
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
 @pytest.mark.parametrize("w_nhwc", [True, False])
 def test_conv_dgrad_mfma_vs_oracle(ctx, case, dtype, w_nhwc):
-    # unit strides, one group, 16-bit channels-last gradients: the forward
-    # MFMA kernel on the mirrored filter (any filter layout)
+    # 16-bit channels-last gradients: the forward MFMA kernel on the mirrored
+    # filter (any filter layout), grouped when the convolution is
     sp = len(case["pad"])
     ones = case.get("s", [1] * sp)
     yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], ones, case["d"])
