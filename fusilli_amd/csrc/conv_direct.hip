@@ -151,15 +151,17 @@ __global__ __launch_bounds__(256) void direct_conv_fprop_kernel(
 // 16 pixels x 16 channel blocks; it keeps the f32 filter of its 128 channels in
 // LDS as [block][tap][8][CG] (blocks 4 words past a multiple of 64 apart: the
 // 16 blocks of a wavefront read different banks, its 4 pixels the same words)
-// and walks `iters` groups of 16 pixels.
+// and four groups of 16 pixels (a thread's four pixels go tap by tap together).
+constexpr int kDcClPix = 4; // pixels per thread
+
 struct DcClArgs {
   int32_t N, H, W, C, K, P, Q, R, S;
   int32_t pad_h, pad_w, str_h, str_w, dil_h, dil_w;
   int32_t cbs;     // 8-channel blocks of a pixel
   int32_t stride;  // LDS words between the blocks' filters
-  int32_t iters;
   int32_t y_dt, o_dt, sp;
   uint32_t pixels;
+  uint32_t x_bytes;
   DevEpilogue epi;
 };
 
@@ -193,67 +195,108 @@ __global__ __launch_bounds__(256) void direct_conv_fprop_cl_kernel(
   if (cb >= g.cbs)
     return;
   const float *wl = wcl + cbl * g.stride;
-  const uint32_t first = blockIdx.x * (uint32_t)(16 * g.iters) + (uint32_t)pl;
-  for (int it = 0; it < g.iters; ++it) {
-    const uint32_t pix = first + (uint32_t)it * 16u;
-    if (pix >= g.pixels)
-      break;
-    const int q = pix % (uint32_t)g.Q;
-    const uint32_t t = pix / (uint32_t)g.Q;
-    const int p = t % (uint32_t)g.P, n = t / (uint32_t)g.P;
+  // kDcClPix pixels per thread, 16 apart, tap by tap together: their loads are
+  // in flight at the same time and a tap's filter is read from LDS once for
+  // all of them.
+  const uint32_t first = blockIdx.x * (uint32_t)(16 * kDcClPix) + (uint32_t)pl;
+  // Per pixel: the byte offset of tap (0, 0) and one bit per filter row and
+  // column that lies inside the image; a tap's own offset is the same for
+  // every lane.  X is read through a buffer descriptor, so a tap outside the
+  // image (offset 2^31) reads zeros.
+  uint32_t base[kDcClPix], rmask[kDcClPix], cmask[kDcClPix];
+  float acc[kDcClPix][8];
+  const uint32_t chan = (uint32_t)cb * 8u;
+#pragma unroll
+  for (int u = 0; u < kDcClPix; ++u) {
+    const uint32_t pix = first + (uint32_t)u * 16u;
+    const bool live = pix < g.pixels;
+    const uint32_t px = live ? pix : 0u;
+    const int q = px % (uint32_t)g.Q;
+    const uint32_t t = px / (uint32_t)g.Q;
+    const int p = t % (uint32_t)g.P;
+    const int n = (int)(t / (uint32_t)g.P);
     const int ih0 = p * g.str_h - g.pad_h, iw0 = q * g.str_w - g.pad_w;
-    float acc[8];
+    // (modulo 2^32: taps above or left of the image are masked)
+    base[u] = ((uint32_t)((n * g.H + ih0) * g.W + iw0) * (uint32_t)g.C + chan) * 2u;
+    uint32_t rm = 0, cm = 0;
+    for (int r = 0; r < g.R; ++r)
+      rm |= (uint32_t)(live && (unsigned)(ih0 + r * g.dil_h) < (unsigned)g.H) << r;
+    for (int s2 = 0; s2 < g.S; ++s2)
+      cm |= (uint32_t)((unsigned)(iw0 + s2 * g.dil_w) < (unsigned)g.W) << s2;
+    rmask[u] = rm;
+    cmask[u] = cm;
 #pragma unroll
     for (int k = 0; k < 8; ++k)
-      acc[k] = 0.f;
-    for (int r = 0; r < g.R; ++r) {
-      const int ih = ih0 + r * g.dil_h;
-      if ((unsigned)ih >= (unsigned)g.H)
-        continue;
-      const int64_t row = ((int64_t)n * g.H + ih) * g.W;
-      for (int s = 0; s < g.S; ++s) {
-        const int iw = iw0 + s * g.dil_w;
-        if ((unsigned)iw >= (unsigned)g.W)
-          continue;
-        const uint4 xv = *(const uint4 *)((const uint16_t *)x + (row + iw) * g.C + cb * 8);
-        const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+      acc[u][k] = 0.f;
+  }
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void *>(x), 0, (int)g.x_bytes, 0x00020000);
+  for (int r = 0; r < g.R; ++r)
+    for (int s = 0; s < g.S; ++s) {
+      const int toff = ((r * g.dil_h * g.W + s * g.dil_w) * g.C) * 2;
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      u32x4 xv[kDcClPix];
+#pragma unroll
+      for (int u = 0; u < kDcClPix; ++u) {
+        const bool in = (rmask[u] >> r) & (cmask[u] >> s) & 1u;
+        // (the sum, not a scalar offset: the range check sees only the lane's
+        // offset, and base alone may lie before the tensor)
+        xv[u] = __builtin_amdgcn_raw_buffer_load_b128(
+            rx, in ? (int)(base[u] + (uint32_t)toff) : (int)0x80000000, 0, 0);
+      }
+      // (16-byte aligned: the blocks' distance and a tap's 8 * CG words are
+      // multiples of 4 words)
+      const float4 *wt4 = (const float4 *)(wl + (r * g.S + s) * 8 * CG);
+      float wt[8 * CG];
+#pragma unroll
+      for (int i = 0; i < 2 * CG; ++i) {
+        const float4 v = wt4[i];
+        wt[4 * i] = v.x, wt[4 * i + 1] = v.y, wt[4 * i + 2] = v.z, wt[4 * i + 3] = v.w;
+      }
+#pragma unroll
+      for (int u = 0; u < kDcClPix; ++u) {
+        const uint32_t xw[4] = {xv[u].x, xv[u].y, xv[u].z, xv[u].w};
         float xf[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           xf[2 * i] = to_f32(xw[i] & 0xffffu);
           xf[2 * i + 1] = to_f32(xw[i] >> 16);
         }
-        // (16-byte aligned: the blocks' distance and a tap's 8 * CG words are
-        // multiples of 4 words)
-        const float4 *wt4 = (const float4 *)(wl + (r * g.S + s) * 8 * CG);
-        float wt[8 * CG];
-#pragma unroll
-        for (int i = 0; i < 2 * CG; ++i) {
-          const float4 v = wt4[i];
-          wt[4 * i] = v.x, wt[4 * i + 1] = v.y, wt[4 * i + 2] = v.z, wt[4 * i + 3] = v.w;
-        }
 #pragma unroll
         for (int k = 0; k < 8; ++k)
 #pragma unroll
           for (int j = 0; j < CG; ++j)
-            acc[k] = __builtin_fmaf(xf[k / CG * CG + j], wt[k * CG + j], acc[k]);
+            acc[u][k] = __builtin_fmaf(xf[k / CG * CG + j], wt[k * CG + j], acc[u][k]);
       }
     }
-    int64_t coord[FHIP_MAX_RANK];
-    coord[0] = n;
-    if (g.sp == 2) {
-      coord[2] = p;
-      coord[3] = q;
-    } else {
-      coord[2] = q;
-    }
+#pragma unroll
+  for (int u = 0; u < kDcClPix; ++u) {
+    const uint32_t pix = first + (uint32_t)u * 16u;
+    if (pix >= g.pixels)
+      break;
     float y[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      coord[1] = cb * 8 + k;
-      y[k] = fhip_apply_epilogue<float>(g.epi, fhip_round_through<float>(g.y_dt, acc[k]), coord);
+    for (int k = 0; k < 8; ++k)
+      y[k] = g.y_dt == FHIP_FLOAT ? acc[u][k] : fhip_round_through<float>(g.y_dt, acc[u][k]);
+    if (g.epi.count > 0) {
+      const int q = pix % (uint32_t)g.Q;
+      const uint32_t t = pix / (uint32_t)g.Q;
+      int64_t coord[FHIP_MAX_RANK];
+      coord[0] = t / (uint32_t)g.P;
+      if (g.sp == 2) {
+        coord[2] = t % (uint32_t)g.P;
+        coord[3] = q;
+      } else {
+        coord[2] = q;
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        coord[1] = cb * 8 + k;
+        y[k] = fhip_apply_epilogue<float>(g.epi, y[k], coord);
+      }
     }
-    const int64_t ob = (int64_t)pix * g.K + cb * 8;
+    // (OUT has fewer than 2^31 elements)
+    const uint32_t ob = pix * (uint32_t)g.K + chan;
     if (g.o_dt == FHIP_FLOAT) {
       float4 *o = (float4 *)((float *)out + ob);
       o[0] = make_float4(y[0], y[1], y[2], y[3]);
@@ -340,13 +383,12 @@ bool make_cl_args(const fhip_conv_desc *d, DcClArgs &g) {
   if ((g.cbs + 15) / 16 > 65535)
     return false;
   g.pixels = (uint32_t)pixels;
+  g.x_bytes = (uint32_t)(fhip_desc_volume(d->x) * 2);
+  if (g.R > 32 || g.S > 32) // one validity bit per filter row and column
+    return false;
   g.y_dt = d->y.dtype;
   g.o_dt = d->out.dtype;
   g.sp = sp;
-  // about eight workgroups per compute unit, at most 16 pixel groups each
-  const int64_t ygrid = (g.cbs + 15) / 16;
-  int64_t iters = pixels * ygrid / (16 * 2048);
-  g.iters = (int32_t)(iters < 1 ? 1 : iters > 16 ? 16 : iters);
   g.epi.count = 0;
   g.epi.rank = 0;
   return true;
@@ -696,7 +738,7 @@ int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
     DcClArgs c{};
     if (make_cl_args(d, c) && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0) {
       c.epi = epi;
-      const dim3 grid((unsigned)((c.pixels + 16u * c.iters - 1) / (16u * c.iters)),
+      const dim3 grid((unsigned)((c.pixels + 16u * kDcClPix - 1) / (16u * kDcClPix)),
                       (unsigned)((c.cbs + 15) / 16));
       const size_t lds = (size_t)16 * c.stride * 4;
       const bool bf16 = d->x.dtype == FHIP_BFLOAT16;
