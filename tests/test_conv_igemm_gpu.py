@@ -272,6 +272,32 @@ def test_conv_igemm_headline_shape(ctx):
         assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"image {img}")
 
 
+@pytest.mark.parametrize("shape", ["groups4", "depthwise"])
+def test_conv_grouped_benchmark_shapes(ctx, shape):
+    """The two grouped lines of the benchmark at full size (N32 56x56, 3x3,
+    padding 1, bf16): 4 groups of 64 -> 64 channels on the MFMA kernel and a
+    depthwise convolution over 128 channels on the small-group kernel.
+    All-ones tensors have closed-form answers (channels of a group times the
+    taps inside the image) on every pixel; random data is checked against the
+    oracle on the first and last image."""
+    c, cg = (256, 64) if shape == "groups4" else (128, 1)
+    xd, wd = [32, c, 56, 56], [c, cg, 3, 3]
+    pad, st, dil = [1, 1], [1, 1], [1, 1]
+    ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
+    ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
+    lg = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+    taps = np.full(56, 3.0); taps[[0, -1]] = 2.0
+    expect = float(cg) * taps[:, None] * taps[None, :]
+    assert np.array_equal(lg, np.broadcast_to(expect, lg.shape))
+    x = cl(xd, 49, 0, capi.BFLOAT16)
+    w = cl(wd, 49, 1, capi.BFLOAT16, std=0.1)
+    lg = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+    xl = x.logical()
+    for img in (0, 31):
+        ref = oracle.conv_fprop(xl[img:img + 1], w.logical(), pad, st, dil)
+        assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"{shape} image {img}")
+
+
 # ---- register-filter kernel (3 x 3 x 64 filters, unit stride, K % 128 == 0) -----
 RF_CASES = [
     # rows per tile forced (CONV_ROWS): image geometry, channels
