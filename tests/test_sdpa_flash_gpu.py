@@ -216,6 +216,37 @@ def test_flash_headline_shape(ctx):
     assert_close(out[2, 7], ref, capi.BFLOAT16, "uniform head")
 
 
+def test_flash_benchmark_lines_mask_and_head_dim_64(ctx):
+    """The two SDPA lines beside the headline at full size (B4 H32 S2048 bf16):
+    head dim 64 under the causal flag, and head dim 128 under an additive bf16
+    mask [B, 1, S, S] shared by the heads.  The oracle runs on three (batch,
+    head) slices each; q = 0 in one head of the masked call gives the
+    closed form softmax(mask row) . V."""
+    B, H, S = 4, 32, 2048
+    for D, masked in ((64, False), (128, True)):
+        qv = rand(58, 0, [B, H, S, D])
+        if masked:
+            qv[1, 5] = 0.0
+        q = HT.from_logical(qv, capi.BFLOAT16)
+        k = HT.from_logical(rand(58, 1, [B, H, S, D]), capi.BFLOAT16)
+        v = HT.from_logical(rand(58, 2, [B, H, S, D]), capi.BFLOAT16)
+        mask = HT.from_logical(rand(58, 3, [B, 1, S, S]), capi.BFLOAT16) if masked else None
+        out = run(ctx, q, k, v, causal=not masked, mask=mask).logical()
+        assert np.all(np.isfinite(out))
+        ql, kl, vl = q.logical(), k.logical(), v.logical()
+        ml = mask.logical() if masked else None
+        for b, h in [(0, 0), (2, 17), (3, 31)]:
+            ref = oracle.sdpa(ql[b:b + 1, h:h + 1], kl[b:b + 1, h:h + 1], vl[b:b + 1, h:h + 1],
+                              mask=ml[b:b + 1] if masked else None, is_causal=not masked)
+            assert_close(out[b:b + 1, h:h + 1], ref, capi.BFLOAT16, f"D{D} b{b} h{h}")
+        if masked:
+            m = ml[1, 0].astype(np.float64)
+            p = np.exp(m - m.max(axis=1, keepdims=True))
+            p /= p.sum(axis=1, keepdims=True)
+            assert_close(out[1, 5], p @ vl[1, 5].astype(np.float64), capi.BFLOAT16,
+                         "uniform scores under the mask")
+
+
 def test_flash_head_dim_64_many_tiles(ctx):
     """Head dim 64, causal, eight query tiles per head: every key-tile count
     from 1 to 32 occurs, and the paired query tiles (long + short) share one
