@@ -70,6 +70,8 @@ RESHAPED_CASES = [
     # or 1), a wider one with a ragged channel tail, 1-D
     dict(x=[3, 48, 20, 16], w=[48, 48, 3, 3], pad=[2, 2], s=[1, 1], d=[2, 2]),
     dict(x=[2, 48, 20, 16], w=[48, 48, 3, 3], pad=[2, 2], s=[1, 1], d=[1, 1]),
+    # (that shape at full size, as the benchmark line runs it)
+    dict(x=[16, 48, 48, 32], w=[48, 48, 3, 3], pad=[2, 2], s=[1, 1], d=[1, 1]),
     dict(x=[2, 200, 9, 7], w=[72, 200, 2, 3], pad=[1, 0], s=[2, 1], d=[1, 1]),
     dict(x=[2, 24, 70], w=[40, 24, 5], pad=[2], s=[1], d=[1]),
     # 3-D convolutions with a 1 x 1 filter in H and W fold into 2-D ones: the
