@@ -85,3 +85,12 @@ def test_runner_contract_on_reference_test_commands(tmp_path):
     for r in rows:
         assert r["iter"] == "2" and r["dispatch_count"] == "1"
         assert 0 < float(r["min (us)"]) <= float(r["mean (us)"]) <= float(r["max (us)"])
+
+
+def test_bench_refuses_more_than_one_gpu():
+    # bench.py measures one GPU; a multi-GPU request ends before anything is
+    # loaded, with a message that says so
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
