@@ -259,9 +259,9 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
     else if (want > 0)
       bm = fits128 ? 128 : 0;
     else // a slab past 80 KB (one workgroup per compute unit) still beats
-         // the gather on large outputs: 55.6 vs 74 us for C = K = 128, 56 x 56
-      bm = small256 && big ? 256
-                           : (small128 || (fits128 && big) ? 128 : 0);
+         // the gather: 55.6 vs 74 us for C = K = 128, 56 x 56; 24 vs 32 us for
+         // C = K = 256, 14 x 14 at N = 32 and 46 vs 52 us at N = 128
+      bm = small256 && big ? 256 : (fits128 ? 128 : 0);
     if (bm) {
       p.halo = true;
       p.bm = bm;
