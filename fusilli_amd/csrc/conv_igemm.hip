@@ -31,6 +31,10 @@ struct ConvPlan {
   // N and K are a group's
   int groups = 1;
   int64_t channels_out = 0; // of all groups
+  // gather mode, one group, few tiles: the reduction is cut into ksplit parts
+  // on workgroups of their own, whose f32 results a second kernel adds (and
+  // applies the epilogue to); needs the context's scratch
+  int ksplit = 1;
 };
 
 // strides equal the dense channels-last strides of dims (unit dims are free)
@@ -119,7 +123,8 @@ bool fold_3d(const fhip_conv_desc *d, fhip_conv_desc *f) {
 
 // `d` is the geometry that runs (possibly folded and channel-padded); the
 // fused operands are described over `orig`'s output dims.
-ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr) {
+ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr,
+                   bool allow_scratch = true) {
   ConvPlan p;
   if (!orig)
     orig = d;
@@ -281,6 +286,21 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
       }
     }
   }
+  if (!p.halo && p.groups == 1 && allow_scratch && p.N % 4 == 0) {
+    // (C512 7 x 7 -> K512 at N32: 52 tiles of 72 K slices 73 us; 4 x 52
+    // workgroups of 18 slices and the sum 27 us)
+    const int64_t tiles = ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn);
+    const int64_t slices = p.K * elem / kTileKBytes;
+    if (tiles < 128 && slices >= 16) {
+      int64_t want = 256 / tiles;
+      want = want > 8 ? 8 : want;
+      for (int64_t sk = want; sk >= 2; --sk)
+        if (slices % sk == 0 && slices / sk >= 6) {
+          p.ksplit = (int)sk;
+          break;
+        }
+    }
+  }
   p.ok = true;
   return p;
 }
@@ -296,13 +316,13 @@ struct ConvResolved {
   size_t x_bytes = 0, w_bytes = 0;
 };
 
-ConvResolved resolve(const fhip_conv_desc *d) {
+ConvResolved resolve(const fhip_conv_desc *d, bool allow_scratch = true) {
   ConvResolved r;
   fhip_conv_desc folded;
   const fhip_conv_desc *g = fold_3d(d, &folded) ? &folded : d;
   r.run = *g;
-  r.plan = make_plan(g, d);
-  if (r.plan.ok)
+  r.plan = make_plan(g, d, allow_scratch);
+  if (r.plan.ok || !allow_scratch)
     return r;
   // channel padding: 16-bit channels-last tensors, whole 16-byte chunks
   const int64_t C = g->x.dim[1];
@@ -354,6 +374,49 @@ __global__ void conv_pad_channels_kernel(const uint4 *src, uint4 *dst, int64_t p
   dst[lin] = chunk < c8 ? src[pixel * c8 + chunk] : make_uint4(0, 0, 0, 0);
 }
 
+struct SplitSumArgs {
+  const float *part; // [parts][M][N]
+  void *out;         // [M][N], dense
+  int64_t mn4;       // M * N / 4
+  int64_t mn;        // M * N
+  int32_t N, parts, P, Q, sp;
+  int32_t y_dt, o_dt;
+  DevEpilogue epi;   // strides over the convolution's Y dims
+};
+
+// OUT[m][n] = epilogue(round(sum over the parts)), four columns per thread
+__global__ void conv_splitk_sum_kernel(SplitSumArgs a) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= a.mn4)
+    return;
+  float4 acc = ((const float4 *)a.part)[lin];
+  for (int z = 1; z < a.parts; ++z) {
+    const float4 v = ((const float4 *)(a.part + (int64_t)z * a.mn))[lin];
+    acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+  }
+  const int64_t e = lin * 4;
+  const int64_t m = e / a.N;
+  const int n0 = (int)(e - m * a.N);
+  int64_t coord[FHIP_MAX_RANK];
+  const int64_t q = m % a.Q, t = m / a.Q;
+  if (a.sp == 2) {
+    coord[0] = t / a.P;
+    coord[2] = t % a.P;
+    coord[3] = q;
+  } else {
+    coord[0] = t;
+    coord[2] = q;
+  }
+  const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    coord[1] = n0 + i;
+    float y = fhip_round_through<float>(a.y_dt, v[i]);
+    y = fhip_apply_epilogue<float>(a.epi, y, coord);
+    fhip_store<float>(a.out, a.o_dt, e + i, y);
+  }
+}
+
 } // namespace
 
 int conv_launch_bf16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
@@ -371,13 +434,13 @@ int conv_launch_f16(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
   return conv_launch_kind<GK_F16>(ctx, bm, bn, g);
 }
 
-bool fhip_fast_conv_applicable(const fhip_conv_desc *d) {
-  return fhip_fast_conv_rf_applicable(d) || resolve(d).plan.ok;
+bool fhip_fast_conv_applicable(const fhip_conv_desc *d, bool allow_scratch) {
+  return fhip_fast_conv_rf_applicable(d) || resolve(d, allow_scratch).plan.ok;
 }
 
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                    const void *w, const DevEpilogue &epi, void *out,
-                   bool *handled) {
+                   bool *handled, bool allow_scratch) {
   if (handled)
     *handled = true;
   bool taken = false;
@@ -385,7 +448,7 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     return 1;
   if (taken)
     return 0;
-  const ConvResolved res = resolve(d);
+  const ConvResolved res = resolve(d, allow_scratch);
   const ConvPlan &p = res.plan;
   if (handled) {
     *handled = p.ok;
@@ -395,12 +458,21 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   FHIP_REQUIRE(ctx, p.ok, "conv: descriptor not supported by the MFMA kernel");
   FHIP_REQUIRE(ctx, ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0,
                "conv: X and W must be 16-byte aligned");
+  // the context's scratch: zero-padded copies of X and W, then the parts of a
+  // split reduction
+  const size_t pad_bytes = res.padded ? res.x_bytes + res.w_bytes : 0;
+  const size_t part_bytes =
+      p.ksplit > 1 ? (size_t)p.ksplit * (size_t)(p.M * p.N) * sizeof(float) : 0;
+  char *scratch = nullptr;
+  if (pad_bytes + part_bytes > 0) {
+    void *sp = nullptr;
+    if (fhip_ctx_scratch(ctx, pad_bytes + part_bytes, &sp) != 0)
+      return 1;
+    scratch = (char *)sp;
+  }
   if (res.padded) {
     // channel counts that are no multiple of 64: zero-padded copies of X and W
-    void *scratch = nullptr;
-    if (fhip_ctx_scratch(ctx, res.x_bytes + res.w_bytes, &scratch) != 0)
-      return 1;
-    char *xp = (char *)scratch, *wp = xp + res.x_bytes;
+    char *xp = scratch, *wp = xp + res.x_bytes;
     const int32_t c8 = (int32_t)(res.C / 8), cp8 = (int32_t)(res.Cp / 8);
     const int64_t xt = res.x_pixels * cp8, wt = res.w_pixels * cp8;
     hipLaunchKernelGGL(conv_pad_channels_kernel, dim3((unsigned)((xt + 255) / 256)),
@@ -457,6 +529,42 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     o.stride[1] = sm;          // per-pixel step (0 for channel vectors)
     o.stride[2] = s.stride[1]; // per-channel step
   }
+  if (p.ksplit > 1) {
+    // every part writes plain f32 sums; rounding and the fused operations
+    // follow in the kernel that adds them
+    float *part = (float *)(scratch + pad_bytes);
+    g.out = (char *)part;
+    g.c_dt = g.o_dt = FHIP_FLOAT;
+    g.o_sm = p.N;
+    g.o_vec = 1;
+    g.epi = DevEpilogue{};
+    g.epi.rank = 3;
+    g.outer = p.ksplit;
+    g.o_outer = p.M * p.N;
+    g.kt_split = (int32_t)(p.K * 2 / kTileKBytes / p.ksplit);
+    gemm_fill_linear(fhip_epilogue{}, g);
+    const int rc = p.kind == GK_BF16 ? conv_launch_bf16(ctx, p.bm, p.bn, g)
+                                     : conv_launch_f16(ctx, p.bm, p.bn, g);
+    if (rc != 0)
+      return rc;
+    SplitSumArgs a{};
+    a.part = part;
+    a.out = out;
+    a.mn = p.M * p.N;
+    a.mn4 = a.mn / 4;
+    a.N = (int32_t)p.N;
+    a.parts = p.ksplit;
+    a.P = p.geom.P;
+    a.Q = p.geom.Q;
+    a.sp = sp;
+    a.y_dt = d->y.dtype;
+    a.o_dt = d->out.dtype;
+    a.epi = epi;
+    hipLaunchKernelGGL(conv_splitk_sum_kernel, dim3((unsigned)((a.mn4 + 255) / 256)),
+                       dim3(256), 0, ctx->stream, a);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    return 0;
+  }
   gemm_fill_linear(d->epilogue, g);
   if (p.halo)
     return p.kind == GK_BF16 ? conv_launch_halo_bm<GK_BF16>(ctx, p.bm, p.bn, g)
@@ -492,7 +600,7 @@ struct DgradPlan {
   size_t spread_bytes = 0;
 };
 
-DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
+DgradPlan make_dgrad_plan(const fhip_conv_desc *d, bool allow_scratch = true) {
   DgradPlan p;
   const int sp = d->spatial_rank;
   if (sp != 1 && sp != 2)
@@ -552,7 +660,7 @@ DgradPlan make_dgrad_plan(const fhip_conv_desc *d) {
     st *= f.w.dim[2 + i];
   }
   f.w.stride[0] = st;
-  if (!fhip_fast_conv_applicable(&f))
+  if (!fhip_fast_conv_applicable(&f, allow_scratch))
     return p;
   p.filter_bytes =
       ((size_t)(st * f.w.dim[0]) * fhip_dtype_size(f.w.dtype) + 255) / 256 * 256;
@@ -638,16 +746,16 @@ int fhip_conv_dgrad_static_setup(fhip_ctx *ctx) {
 }
 
 bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
-                                     size_t *workspace_bytes) {
-  const DgradPlan p = make_dgrad_plan(d);
+                                     size_t *workspace_bytes, bool allow_scratch) {
+  const DgradPlan p = make_dgrad_plan(d, allow_scratch);
   if (workspace_bytes)
     *workspace_bytes = p.ok ? p.filter_bytes + p.spread_bytes : 0;
   return p.ok;
 }
 
 int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
-                         const void *w, void *dx, void *workspace) {
-  const DgradPlan p = make_dgrad_plan(d);
+                         const void *w, void *dx, void *workspace, bool allow_scratch) {
+  const DgradPlan p = make_dgrad_plan(d, allow_scratch);
   FHIP_REQUIRE(ctx, p.ok, "conv dgrad: descriptor not supported by the MFMA kernel");
   // the register-filter kernel needs neither the mirrored filter nor workspace
   if (fhip_fast_conv_dgrad_rf_applicable(d) &&
@@ -689,7 +797,7 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                        dim3((unsigned)((sa.total + 255) / 256)), dim3(256), 0,
                        ctx->stream, sa, (const uint4 *)dy, (uint4 *)grid);
     FHIP_HIP_CHECK(ctx, hipGetLastError());
-    return fhip_fast_conv(ctx, &p.fwd, grid, workspace, epi, dx);
+    return fhip_fast_conv(ctx, &p.fwd, grid, workspace, epi, dx, nullptr, allow_scratch);
   }
-  return fhip_fast_conv(ctx, &p.fwd, dy, workspace, epi, dx);
+  return fhip_fast_conv(ctx, &p.fwd, dy, workspace, epi, dx, nullptr, allow_scratch);
 }

@@ -17,12 +17,15 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
                            void *out, int outer, int64_t a_outer,
                            int64_t b_outer, int64_t o_outer);
 
-bool fhip_fast_conv_applicable(const fhip_conv_desc *d);
+// `allow_scratch` false: only plans that leave the context's scratch alone
+// (no zero-padded channel copies, no split reduction) -- for the entry point
+// that must not allocate.
+bool fhip_fast_conv_applicable(const fhip_conv_desc *d, bool allow_scratch = true);
 // With `handled` the call plans once and reports whether a tuned kernel was
 // launched; a descriptor that none takes is then no error.
 int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
                    const void *w, const DevEpilogue &epi, void *out,
-                   bool *handled = nullptr);
+                   bool *handled = nullptr, bool allow_scratch = true);
 
 // The same problem on the register-filter kernel (unit stride and dilation,
 // 3 x 3 x 64 filters, K a multiple of 128, 16-bit output, linear epilogue that
@@ -37,9 +40,11 @@ int fhip_fast_conv_rf(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
 // Data gradient through the forward kernel (unit strides, one group); needs
 // `*workspace_bytes` of 16-byte aligned workspace for the mirrored filter.
 bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
-                                     size_t *workspace_bytes);
+                                     size_t *workspace_bytes,
+                                     bool allow_scratch = true);
 int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
-                         const void *w, void *dx, void *workspace);
+                         const void *w, void *dx, void *workspace,
+                         bool allow_scratch = true);
 
 // Data gradient of 3 x 3 convolutions over 128 output channels with the filter
 // in registers (conv_rf_dgrad.hip): one kernel, W read as it lies, no

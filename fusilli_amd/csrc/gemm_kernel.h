@@ -148,6 +148,10 @@ struct GemmArgs {
   // convolution: the group's first output channel); 0 otherwise
   int64_t epi_n_outer;
   int32_t outer; // extent (0 or 1: none)
+  // implicit-GEMM convolution with the reduction cut into `outer` parts of
+  // kt_split K slices each (0: not cut): part z accumulates slices z * kt_split
+  // .. and writes its own f32 result, which the caller adds up
+  int32_t kt_split;
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
   // rows of an M tile that are computed and stored (0: all BM); a smaller
@@ -520,7 +524,10 @@ gemm_kernel(GemmArgs g) {
   // first row past this tile's share of the output
   const int64_t m_end = m0 + tile_rows < g.M ? m0 + tile_rows : g.M;
   const int64_t a_ldb = g.a_ld * ELEM, b_ldb = g.b_ld * ELEM;
-  const int kt_count = (int)(g.K * ELEM / kTileKBytes);
+  const int kt_count = A_MODE == A_CONV && g.kt_split > 0
+                           ? g.kt_split
+                           : (int)(g.K * ELEM / kTileKBytes);
+  const int kt_base = A_MODE == A_CONV && g.kt_split > 0 ? (int)outer * g.kt_split : 0;
 
   const int wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -584,7 +591,8 @@ gemm_kernel(GemmArgs g) {
   const char *b_base;
   int64_t b_step;
   if constexpr (B_KC) {
-    b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * b_ldb;
+    b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * b_ldb +
+             (int64_t)kt_base * kTileKBytes;
     b_step = kTileKBytes;
   } else {
     b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * ELEM;
@@ -612,9 +620,10 @@ gemm_kernel(GemmArgs g) {
     if constexpr (HALO) {
       // only the filter streams
     } else if constexpr (A_MODE == A_CONV) {
-      const int32_t tap = conv_div(kt, g.conv.slices_per_tap, g.conv.magic_spt);
+      const int32_t ktg = kt + kt_base;
+      const int32_t tap = conv_div(ktg, g.conv.slices_per_tap, g.conv.magic_spt);
       const int32_t cb =
-          (kt - tap * g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
+          (ktg - tap * g.conv.slices_per_tap) * kTileKBytes + cv_chunk;
       const int32_t fr = conv_div(tap, g.conv.S, g.conv.magic_s);
       const int32_t fs = tap - fr * g.conv.S;
       const int32_t dpix = fr * g.conv.dil_h * g.conv.W + fs * g.conv.dil_w;

@@ -1357,7 +1357,8 @@ int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
   FHIP_REQUIRE(ctx, dy && w && dx, "fhip_conv_dgrad_static: null tensor pointer");
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
   size_t need = 0;
-  if (fhip_fast_conv_dgrad_applicable(d, &need)) {
+  // (only plans that leave the context's growable scratch alone)
+  if (fhip_fast_conv_dgrad_applicable(d, &need, false)) {
     FHIP_REQUIRE(ctx, need <= (size_t)FHIP_CONV_DGRAD_STATIC_MAX_BYTES,
                  "fhip_conv_dgrad_static: this descriptor needs %zu bytes of "
                  "scratch, the static array holds %zu; use fhip_conv_dgrad "
@@ -1365,7 +1366,7 @@ int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
                  need, (size_t)FHIP_CONV_DGRAD_STATIC_MAX_BYTES);
     FHIP_REQUIRE(ctx, ctx->dgrad_static_scratch != nullptr,
                  "fhip_conv_dgrad_static: scratch address not resolved");
-    return fhip_fast_conv_dgrad(ctx, d, dy, w, dx, ctx->dgrad_static_scratch);
+    return fhip_fast_conv_dgrad(ctx, d, dy, w, dx, ctx->dgrad_static_scratch, false);
   }
   // the direct and the strided kernel use no scratch at all
   if (fhip_direct_conv_applicable(d))

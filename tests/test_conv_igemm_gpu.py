@@ -226,6 +226,35 @@ def test_conv_grouped_vs_oracle(ctx, case, halo, dtype, knobs):
     assert_close(out.logical(), ref, capi.FLOAT, f"halo={halo} {case}", rtol=1e-4)
 
 
+SPLIT_CASES = [
+    # few output pixels and a long reduction: the K slices are cut into parts
+    # on workgroups of their own and a second kernel adds them
+    dict(x=[2, 512, 7, 7], w=[512, 512, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),    # 8 parts
+    dict(x=[2, 1024, 5, 5], w=[64, 1024, 1, 1], pad=[0, 0], s=[1, 1], d=[1, 1]),   # 2 parts
+    dict(x=[3, 192, 9, 9], w=[40, 192, 3, 3], pad=[0, 0], s=[2, 2], d=[1, 1]),     # ragged tile, stride
+    dict(x=[1, 256, 40], w=[72, 256, 5], pad=[2], s=[1], d=[1]),                   # 1-D
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_conv_split_reduction_vs_oracle(ctx, case, dtype, knobs):
+    knobs(CONV_HALO="0")  # the gather kernel (the halo kernel does not split)
+    x = cl(case["x"], 50, 0, dtype)
+    w = cl(case["w"], 50, 1, dtype, std=0.05)
+    k = case["w"][0]
+    bdims = [1, k] + [1] * len(case["pad"])
+    bias = HT.from_logical(rand(50, 2, bdims), dtype, oracle.channels_last_strides(bdims))
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT)]
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT, out_dtype=dtype,
+              epilogue=epi, epi_tensors=[bias])
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"], case["d"])
+    assert_close(out.logical(), np.maximum(ref + bias.logical(), 0.0), dtype, f"{case}")
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT)
+    assert_close(out.logical(), ref, capi.FLOAT, f"{case}", rtol=1e-4)
+
+
 def test_conv_igemm_not_chosen_outside_contract(ctx):
     # C = 44 (not whole 16-byte chunks per pixel) and groups of 32 channels
     # (half a K slice) keep the generic kernel
