@@ -148,9 +148,9 @@ struct GemmArgs {
   // convolution: the group's first output channel); 0 otherwise
   int64_t epi_n_outer;
   int32_t outer; // extent (0 or 1: none)
-  // implicit-GEMM convolution with the reduction cut into `outer` parts of
-  // kt_split K slices each (0: not cut): part z accumulates slices z * kt_split
-  // .. and writes its own f32 result, which the caller adds up
+  // The reduction cut into `outer` parts of kt_split K slices each (0: not
+  // cut; not in halo mode): part z accumulates slices z * kt_split .. and
+  // writes its own f32 result, which the caller adds up
   int32_t kt_split;
   int32_t c_dt, o_dt;
   int32_t tiles_m, tiles_n;
@@ -524,10 +524,9 @@ gemm_kernel(GemmArgs g) {
   // first row past this tile's share of the output
   const int64_t m_end = m0 + tile_rows < g.M ? m0 + tile_rows : g.M;
   const int64_t a_ldb = g.a_ld * ELEM, b_ldb = g.b_ld * ELEM;
-  const int kt_count = A_MODE == A_CONV && g.kt_split > 0
-                           ? g.kt_split
-                           : (int)(g.K * ELEM / kTileKBytes);
-  const int kt_base = A_MODE == A_CONV && g.kt_split > 0 ? (int)outer * g.kt_split : 0;
+  const int kt_count =
+      !HALO && g.kt_split > 0 ? g.kt_split : (int)(g.K * ELEM / kTileKBytes);
+  const int kt_base = !HALO && g.kt_split > 0 ? (int)outer * g.kt_split : 0;
 
   const int wave = threadIdx.x >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -580,12 +579,14 @@ gemm_kernel(GemmArgs g) {
       cv_chunk = ((l & 7) ^ kc_swz(row)) * 16; // same for every j
     }
   } else if constexpr (A_KC) {
-    a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * a_ldb;
     a_step = kTileKBytes;
+    a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * a_ldb +
+             kt_base * a_step;
     dma_setup<BM, ELEM, true, NW>(a_ldb, m0, m_end, off_a);
   } else {
-    a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * ELEM;
     a_step = (int64_t)GA::kKRows * a_ldb;
+    a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * ELEM +
+             kt_base * a_step;
     dma_setup<BM, ELEM, false, NW>(a_ldb, m0, m_end, off_a);
   }
   const char *b_base;
@@ -595,8 +596,9 @@ gemm_kernel(GemmArgs g) {
              (int64_t)kt_base * kTileKBytes;
     b_step = kTileKBytes;
   } else {
-    b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * ELEM;
     b_step = (int64_t)GB::kKRows * b_ldb;
+    b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * ELEM +
+             kt_base * b_step;
   }
   dma_setup<BN, ELEM, B_KC, NW>(b_ldb, n0, g.N, off_b);
 
@@ -1277,6 +1279,9 @@ struct GemmPlan {
   int64_t a_ld = 0, b_ld = 0, a_batch = 0, b_batch = 0;
   int64_t o_sm = 0, o_sn = 0, o_batch = 0;
   int bm = 256, bn = 256;
+  // parts the reduction is cut into (f32 partial results in the context's
+  // scratch, added by a second kernel); 1: none
+  int ksplit = 1;
 };
 
 // Stage count per tile: as many as fit the 160 KB LDS, at most 4.

@@ -50,7 +50,7 @@ bool kind_for(int a_dt, int b_dt, int *kind) {
   }
 }
 
-GemmPlan make_plan(const fhip_matmul_desc *d) {
+GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
   GemmPlan p;
   const int r = d->a.rank;
   if (r != 2 && r != 3)
@@ -137,6 +137,7 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
   // tile shape: biggest tile that still gives every CU work
   p.bm = p.M >= 256 ? 256 : 128;
   p.bn = p.N >= 256 && p.bm == 256 ? 256 : 128;
+  const int bm0 = p.bm, bn0 = p.bn; // the largest tile the shape allows
   const int64_t big_tiles =
       ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn) * p.batch;
   if (big_tiles < 200) {
@@ -147,6 +148,37 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
     if (t2 < 200 && p.bm == 256)
       p.bm = 128;
   }
+  // Few tiles and a long reduction: K is cut into parts on workgroups of their
+  // own, on the large tile, when a rough model says that the parts' f32 round
+  // trip through memory costs less than the idle compute units do.
+  // (1024 x 1024 x 8192 bf16: 64 tiles of 128 x 128 135 us; 16 tiles x 8 parts
+  // 44 us.  512 x 512 x 16384: 269 -> 27 us.)
+  if (p.batch == 1 && p.kind != GK_I8 && p.N % 4 == 0 && p.o_sn == 1 && allow_split) {
+    const double peak = (p.kind == GK_BF16 || p.kind == GK_F16) ? 2.5e15 : 5.0e15;
+    const double flop = 2.0 * (double)p.M * (double)p.N * (double)p.K;
+    auto tiles = [&](int bm, int bn) {
+      return (double)(((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn));
+    };
+    auto busy = [](double t) { return t < 256.0 ? t / 256.0 : 1.0; };
+    auto eff = [](int bm, int bn) {
+      return bm == 256 && bn == 256 ? 0.45 : (bm == 256 ? 0.3 : 0.2);
+    };
+    const double t0 = flop / (eff(p.bm, p.bn) * peak * busy(tiles(p.bm, p.bn)));
+    const int64_t slices = p.K * elem / kTileKBytes;
+    double best = 0.8 * t0;
+    for (int sk = 2; sk <= 32; ++sk) {
+      if (slices % sk != 0 || slices / sk < 8)
+        continue;
+      const double t = flop / (eff(bm0, bn0) * peak * busy(tiles(bm0, bn0) * sk)) +
+                       2.0 * sk * (double)p.M * (double)p.N * 4.0 / 3.0e12;
+      if (t < best) {
+        best = t;
+        p.ksplit = sk;
+      }
+    }
+    if (p.ksplit > 1)
+      p.bm = bm0, p.bn = bn0;
+  }
   if (fhip_knobs().gemm_tile_bm) {
     const int bm = fhip_knobs().gemm_tile_bm, bn = fhip_knobs().gemm_tile_bn;
     if ((bm == 128 || bm == 256) &&
@@ -155,6 +187,41 @@ GemmPlan make_plan(const fhip_matmul_desc *d) {
   }
   p.ok = true;
   return p;
+}
+
+struct GemmSumArgs {
+  const float *part; // [parts][M][N]
+  void *out;
+  int64_t mn, mn4, o_sm;
+  int32_t N, parts, rank;
+  int32_t c_dt, o_dt;
+  DevEpilogue epi; // strides over the matmul's result dims
+};
+
+// OUT[m][n] = epilogue(round(sum over the parts)), four columns per thread
+__global__ void gemm_splitk_sum_kernel(GemmSumArgs a) {
+  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (lin >= a.mn4)
+    return;
+  float4 acc = ((const float4 *)a.part)[lin];
+  for (int z = 1; z < a.parts; ++z) {
+    const float4 v = ((const float4 *)(a.part + (int64_t)z * a.mn))[lin];
+    acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+  }
+  const int64_t e = lin * 4;
+  const int64_t m = e / a.N;
+  const int64_t n0 = e - m * a.N;
+  int64_t coord[FHIP_MAX_RANK];
+  coord[0] = 0;
+  coord[a.rank - 2] = m;
+  const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    coord[a.rank - 1] = n0 + i;
+    float y = fhip_round_through<float>(a.c_dt, v[i]);
+    y = fhip_apply_epilogue<float>(a.epi, y, coord);
+    fhip_store<float>(a.out, a.o_dt, m * a.o_sm + n0 + i, y);
+  }
 }
 
 } // namespace
@@ -172,7 +239,7 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
                            const void *a, const void *b, const DevEpilogue &epi,
                            void *out, int outer, int64_t a_outer,
                            int64_t b_outer, int64_t o_outer) {
-  const GemmPlan p = make_plan(d);
+  const GemmPlan p = make_plan(d, outer == 1);
   FHIP_REQUIRE(ctx, outer >= 1 && outer <= 65535 && (outer == 1 || epi.count == 0),
                "gemm: outer batch extent %d (no fused operands with it)", outer);
   FHIP_REQUIRE(ctx, p.ok, "gemm: descriptor not supported by the MFMA kernel");
@@ -216,6 +283,57 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     o.stride[0] = r == 3 ? s.stride[0] : 0;
     o.stride[1] = s.stride[r - 2];
     o.stride[2] = s.stride[r - 1];
+  }
+  auto launch = [&]() {
+    switch (p.kind) {
+    case GK_BF16:
+      return gemm_launch_bf16(ctx, p, g);
+    case GK_F16:
+      return gemm_launch_f16(ctx, p, g);
+    case GK_I8:
+      return gemm_launch_i8(ctx, p, g);
+    case GK_FP8E4M3:
+      return gemm_launch_fp8e4m3(ctx, p, g);
+    default:
+      return gemm_launch_fp8e5m2(ctx, p, g);
+    }
+  };
+  if (p.ksplit > 1) {
+    // every part writes plain f32 sums; rounding and the fused operations
+    // follow in the kernel that adds them
+    void *sp = nullptr;
+    if (fhip_ctx_scratch(ctx, (size_t)p.ksplit * (size_t)(p.M * p.N) * sizeof(float), &sp) != 0)
+      return 1;
+    g.out = (char *)sp;
+    g.c_dt = g.o_dt = FHIP_FLOAT;
+    g.o_sm = p.N;
+    g.o_sn = 1;
+    g.o_vec = 1;
+    g.epi = DevEpilogue{};
+    g.epi.rank = 3;
+    g.outer = p.ksplit;
+    g.o_outer = p.M * p.N;
+    g.kt_split = (int32_t)(p.K * fhip_dtype_size(d->a.dtype) / kTileKBytes / p.ksplit);
+    gemm_fill_linear(fhip_epilogue{}, g);
+    const int rc = launch();
+    if (rc != 0)
+      return rc;
+    GemmSumArgs sa{};
+    sa.part = (const float *)sp;
+    sa.out = out;
+    sa.mn = p.M * p.N;
+    sa.mn4 = sa.mn / 4;
+    sa.o_sm = p.o_sm;
+    sa.N = (int32_t)p.N;
+    sa.parts = p.ksplit;
+    sa.rank = r;
+    sa.c_dt = d->c.dtype;
+    sa.o_dt = d->out.dtype;
+    sa.epi = epi;
+    hipLaunchKernelGGL(gemm_splitk_sum_kernel, dim3((unsigned)((sa.mn4 + 255) / 256)),
+                       dim3(256), 0, ctx->stream, sa);
+    FHIP_HIP_CHECK(ctx, hipGetLastError());
+    return 0;
   }
   gemm_fill_linear(d->epilogue, g);
   switch (p.kind) {

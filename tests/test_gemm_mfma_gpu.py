@@ -102,6 +102,28 @@ def test_gemm_bf16_bias_activation_epilogue(ctx, act):
     assert_close(out.logical(), ref, capi.BFLOAT16)
 
 
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF, capi.FP8E4M3])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 8192), (300, 512, 4096), (512, 260, 16384)])
+def test_gemm_split_reduction(ctx, dtype, ta, tb, m, n, k):
+    # Few output tiles and a long K: the reduction is cut into parts on
+    # workgroups of their own and a second kernel adds them, rounds to the C
+    # type and applies the fused bias + GELU.
+    a = make_operand(73, 0, m, k, dtype, ta)
+    b = make_operand(73, 1, k, n, dtype, tb)
+    bias = HT.from_logical(rand(73, 2, [1, n]), capi.BFLOAT16)
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["GELU_FWD"], capi.FLOAT)]
+    elem = capi.DTYPE_SIZE[dtype]
+    fast = (not ta or (m * elem) % 16 == 0) and (tb or (n * elem) % 16 == 0)
+    out = run(ctx, a, b, capi.FLOAT, out_dtype=capi.BFLOAT16, epilogue=epi,
+              epi_tensors=[bias], expect_fast=fast)
+    ref = oracle.pointwise(capi.PW["GELU_FWD"], [ref_matmul(a, b) + bias.logical()])
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+    out = run(ctx, a, b, capi.FLOAT, expect_fast=fast)
+    assert_close(out.logical(), ref_matmul(a, b), capi.FLOAT, rtol=1e-4)
+
+
 def test_gemm_fp8_per_tensor_scales_bf16_out(ctx):
     # benchmark config 5b at reduced size: x ~ U[-1,1], per-tensor scale
     # s = max|x| / 448, saturating RNE cast, C = (A8 B8) * (sa * sb) -> bf16.
