@@ -509,6 +509,46 @@ def bench_conv_grouped(ctx, steps, warmup):
             "call_us": round(ev_ms * 1e3, 2), "work": flop, "kernels_per_call": 1}
 
 
+def bench_conv_deep_layer(ctx, steps, warmup):
+    """A late ResNet layer: N32 C512 7x7 -> K512, 3x3, padding 1, bf16
+    channels-last.  1568 output pixels make 52 tiles, so the planner cuts the
+    reduction into four parts on workgroups of their own and a second kernel
+    adds them (two kernels per call)."""
+    n, c, h, w, k, r = 32, 512, 7, 7, 512, 3
+    cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
+    xd, wd, yd = [n, c, h, w], [k, c, r, r], [n, k, h, w]
+    d = capi.ConvDesc()
+    d.x = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
+    d.w = capi.TensorDesc.make(wd, cl(wd), capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(yd, cl(yd), capi.FLOAT)
+    d.out = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
+    d.out_dtype = capi.BFLOAT16
+    d.spatial_rank = 2
+    for i in range(2):
+        d.padding[i], d.stride[i], d.dilation[i] = 1, 1, 1
+    d.epilogue = capi.make_epilogue([])
+    assert ctx.lib.fhip_conv_fprop_supported(d) == 2, "MFMA conv not chosen"
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 9, n * c * h * w)))
+    wt = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(8, 10, k * c * r * r, 0.0, 0.02)))
+    out = ctx.alloc(n * k * h * w * 2)
+    wall_ms, ev_ms = timed_loop(ctx, lambda i: ctx.conv_fprop(d, x, wt, out),
+                                steps, warmup)
+    flop = 2.0 * n * h * w * k * c * r * r
+    return {"value": round(flop / ev_ms / 1e9, 1), "unit": "TFLOP/s",
+            "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / PEAK_TFLOPS["bf16"], 4),
+            "call_us": round(ev_ms * 1e3, 2), "work": flop, "kernels_per_call": 2}
+
+
+def bench_matmul_split(ctx, steps, warmup):
+    """bf16 1024 x 1024 x 8192: 16 tiles of 256 x 256, so the planner cuts K
+    into parts on workgroups of their own (f32 partial sums in the context's
+    scratch) and a second kernel adds them: two kernels per call."""
+    r = bench_matmul(ctx, steps, warmup, "bf16", 1024, 1024, 8192)
+    r["call_us"] = r.pop("kernel_us")
+    r["kernels_per_call"] = 2
+    return r
+
+
 def bench_conv_depthwise(ctx, steps, warmup):
     """Depthwise 3x3 convolution (groups = channels), N32 C128 56x56, padding 1,
     bf16 channels-last: the channels-last small-group kernel; bound by HBM
@@ -759,6 +799,10 @@ def main():
              lambda: bench_layernorm_long(ctx, max(20, args.steps // 4), kwarm)),
             ("conv_fprop_bf16_n32c256h56w56_k256r3s3_groups4",
              lambda: bench_conv_grouped(ctx, max(20, args.steps // 10), kwarm)),
+            ("conv_fprop_bf16_n32c512h7w7_k512r3s3_split_reduction",
+             lambda: bench_conv_deep_layer(ctx, max(20, args.steps // 10), kwarm)),
+            ("matmul_bf16_1024x1024x8192_split_reduction",
+             lambda: bench_matmul_split(ctx, max(20, args.steps // 10), kwarm)),
             ("conv_fprop_bf16_n32c128h56w56_depthwise_r3s3",
              lambda: bench_conv_depthwise(ctx, max(20, args.steps // 10), kwarm)),
             ("conv_fprop_f16_n16c48h48w32_k48r3s3_padded_channels",

@@ -255,6 +255,25 @@ def test_conv_split_reduction_vs_oracle(ctx, case, dtype, knobs):
     assert_close(out.logical(), ref, capi.FLOAT, f"{case}", rtol=1e-4)
 
 
+def test_conv_split_reduction_benchmark_shape(ctx):
+    """N32 C512 7x7 -> K512, 3x3, padding 1, bf16 at full size (the
+    benchmark's late-layer line): closed form on all-ones tensors for every
+    pixel, the oracle on the first and last image for random ones."""
+    xd, wd = [32, 512, 7, 7], [512, 512, 3, 3]
+    pad, st, dil = [1, 1], [1, 1], [1, 1]
+    ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
+    ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
+    lg = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+    taps = np.full(7, 3.0); taps[[0, -1]] = 2.0
+    assert np.array_equal(lg, np.broadcast_to(512.0 * taps[:, None] * taps[None, :], lg.shape))
+    x = cl(xd, 51, 0, capi.BFLOAT16)
+    w = cl(wd, 51, 1, capi.BFLOAT16, std=0.02)
+    lg = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+    for img in (0, 31):
+        ref = oracle.conv_fprop(x.logical()[img:img + 1], w.logical(), pad, st, dil)
+        assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"image {img}")
+
+
 def test_conv_igemm_not_chosen_outside_contract(ctx):
     # C = 44 (not whole 16-byte chunks per pixel) and groups of 32 channels
     # (half a K slice) keep the generic kernel

@@ -124,6 +124,14 @@ def test_gemm_split_reduction(ctx, dtype, ta, tb, m, n, k):
     assert_close(out.logical(), ref_matmul(a, b), capi.FLOAT, rtol=1e-4)
 
 
+def test_gemm_split_reduction_benchmark_shape(ctx):
+    # bf16 1024 x 1024 x 8192 -> bf16, as the benchmark line runs it
+    a = make_operand(74, 0, 1024, 8192, capi.BFLOAT16, False)
+    b = make_operand(74, 1, 8192, 1024, capi.BFLOAT16, False)
+    out = run(ctx, a, b, capi.FLOAT, out_dtype=capi.BFLOAT16)
+    assert_close(out.logical(), ref_matmul(a, b), capi.BFLOAT16)
+
+
 def test_gemm_fp8_per_tensor_scales_bf16_out(ctx):
     # benchmark config 5b at reduced size: x ~ U[-1,1], per-tensor scale
     # s = max|x| / 448, saturating RNE cast, C = (A8 B8) * (sa * sb) -> bf16.
