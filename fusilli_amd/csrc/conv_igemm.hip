@@ -219,7 +219,10 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
     };
     if (tiles(256, 256) < 192)
       p.bn = 128;
-    if (p.bn == 128 && tiles(256, 128) < 192)
+    // (256 x 128 runs on eight wavefronts in two phases at about twice the
+    // rate of the four in-order wavefronts of a 128 x 128 tile)
+    const int64_t small = tiles(128, 128) < 256 ? tiles(128, 128) : 256;
+    if (p.bn == 128 && tiles(256, 128) < 192 && 2 * tiles(256, 128) < small)
       p.bm = 128;
   }
   const FhipKnobs &knobs = fhip_knobs();

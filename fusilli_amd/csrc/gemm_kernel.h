@@ -442,11 +442,12 @@ __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
 // LDS bytes of the kernel: NSTAGE stages of (A slice + B slice); the epilogue
 // reuses it for four 32-row accumulator bands (one per wavefront).
 // Wavefront grid of a tile.  8 wavefronts (two per SIMD, scheduled in
-// alternating memory / MFMA phases) where each still owns 128 x 64 outputs:
-// 256 x 256 as 2 x 4 and 512 x 128 as 4 x 2; otherwise 2 x 2.
-template <int BM, int BN> struct GemmLayout {
+// alternating memory / MFMA phases): 256 x 256 as 2 x 4 and 512 x 128 as 4 x 2,
+// each wavefront owning 128 x 64 outputs, and 256 x 128 as 4 x 2 of 64 x 64;
+// 4 wavefronts as 2 x 2.
+template <int BM, int BN, int NW = 0> struct GemmLayout {
   static constexpr bool kWide = BM == 256 && BN == 256;
-  static constexpr bool kTall = BM == 512 && BN == 128;
+  static constexpr bool kTall = (BM == 512 || (BM == 256 && NW == 8)) && BN == 128;
   static constexpr int kWavesM = kTall ? 4 : 2;
   static constexpr int kWavesN = kWide ? 4 : 2;
   static constexpr int kWaves = kWavesM * kWavesN;
@@ -454,10 +455,10 @@ template <int BM, int BN> struct GemmLayout {
 
 template <int BM, int BN, int NSTAGE, int NW, bool HALO = false> struct GemmLds {
   static constexpr int kStage = (BM + BN) * kTileKBytes;
-  static constexpr int kWN = BN / GemmLayout<BM, BN>::kWavesN; // wave columns
+  static constexpr int kWN = BN / GemmLayout<BM, BN, NW>::kWavesN; // wave columns
   static constexpr int kEpiPitch = kWN * 4 + 32;
   static constexpr int kBand = 32 * kEpiPitch; // one wavefront, one tile row
-  static constexpr int kTM = BM / GemmLayout<BM, BN>::kWavesM / 32;
+  static constexpr int kTM = BM / GemmLayout<BM, BN, NW>::kWavesM / 32;
   // tile rows that leave together: as many as fit 160 KB, or 80 KB where the
   // stages leave room for two workgroups per compute unit
   static constexpr int kCap =
@@ -484,8 +485,8 @@ gemm_kernel(GemmArgs g) {
   using GA = SliceGeom<BM, ELEM, A_KC, NW>;
   using GB = SliceGeom<BN, ELEM, B_KC, NW>;
   using L = GemmLds<BM, BN, NSTAGE, NW, A_MODE == A_HALO>;
-  constexpr int WAVES_M = GemmLayout<BM, BN>::kWavesM;
-  constexpr int WAVES_N = GemmLayout<BM, BN>::kWavesN;
+  constexpr int WAVES_M = GemmLayout<BM, BN, NW>::kWavesM;
+  constexpr int WAVES_N = GemmLayout<BM, BN, NW>::kWavesN;
   static_assert(WAVES_M * WAVES_N == NW, "wavefront grid");
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N; // wavefront tile
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -1290,8 +1291,12 @@ template <int BM, int BN> struct GemmStages {
   static constexpr int value = 160 * 1024 / kStage >= 4 ? 4 : 160 * 1024 / kStage;
 };
 
+template <> struct GemmStages<256, 128> {
+  static constexpr int value = 2; // the ping-pong loop alternates two stages
+};
+
 template <int BM, int BN> struct GemmWaves {
-  static constexpr int value = GemmLayout<BM, BN>::kWaves;
+  static constexpr int value = BM == 256 && BN == 128 ? 8 : GemmLayout<BM, BN>::kWaves;
 };
 
 template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int STAGES = 0>

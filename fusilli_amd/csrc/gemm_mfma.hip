@@ -134,20 +134,26 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
         return p;
     }
   }
-  // tile shape: biggest tile that still gives every CU work
-  p.bm = p.M >= 256 ? 256 : 128;
-  p.bn = p.N >= 256 && p.bm == 256 ? 256 : 128;
-  const int bm0 = p.bm, bn0 = p.bn; // the largest tile the shape allows
-  const int64_t big_tiles =
-      ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn) * p.batch;
-  if (big_tiles < 200) {
-    if (p.bm == 256 && p.bn == 256)
-      p.bn = 128;
-    const int64_t t2 =
-        ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn) * p.batch;
-    if (t2 < 200 && p.bm == 256)
-      p.bm = 128;
-  }
+  // Tile shape: the one with the shortest estimated run -- the MFMA work at
+  // the tile's usual share of the peak (256 x 256 and 256 x 128 on eight
+  // wavefronts in two phases: a half and four tenths; 128 x 128 on four in
+  // order: a fifth) over the share of the 256 compute units that have a tile.
+  auto tiles = [&](int bm, int bn) {
+    return (double)(((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch);
+  };
+  auto busy = [](double t) { return t < 256.0 ? t / 256.0 : 1.0; };
+  auto eff = [](int bm, int bn) {
+    return bm == 256 && bn == 256 ? 0.5 : (bm == 256 ? 0.4 : 0.2);
+  };
+  p.bm = p.bn = 128;
+  // (ties go to the larger tile: compute units run faster when others idle)
+  if (p.M >= 256 && eff(256, 128) * busy(tiles(256, 128)) >= eff(p.bm, p.bn) * busy(tiles(p.bm, p.bn)))
+    p.bm = 256, p.bn = 128;
+  if (p.M >= 256 && p.N >= 256 &&
+      eff(256, 256) * busy(tiles(256, 256)) >= eff(p.bm, p.bn) * busy(tiles(p.bm, p.bn)))
+    p.bm = 256, p.bn = 256;
+  // the largest tile the shape allows (for the cut below)
+  const int bm0 = p.M >= 256 ? 256 : 128, bn0 = p.N >= 256 && bm0 == 256 ? 256 : 128;
   // Few tiles and a long reduction: K is cut into parts on workgroups of their
   // own, on the large tile, when a rough model says that the parts' f32 round
   // trip through memory costs less than the idle compute units do.
@@ -156,13 +162,6 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
   if (p.batch == 1 && p.kind != GK_I8 && p.N % 4 == 0 && p.o_sn == 1 && allow_split) {
     const double peak = (p.kind == GK_BF16 || p.kind == GK_F16) ? 2.5e15 : 5.0e15;
     const double flop = 2.0 * (double)p.M * (double)p.N * (double)p.K;
-    auto tiles = [&](int bm, int bn) {
-      return (double)(((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn));
-    };
-    auto busy = [](double t) { return t < 256.0 ? t / 256.0 : 1.0; };
-    auto eff = [](int bm, int bn) {
-      return bm == 256 && bn == 256 ? 0.45 : (bm == 256 ? 0.3 : 0.2);
-    };
     const double t0 = flop / (eff(p.bm, p.bn) * peak * busy(tiles(p.bm, p.bn)));
     const int64_t slices = p.K * elem / kTileKBytes;
     double best = 0.8 * t0;
