@@ -104,7 +104,8 @@ def test_gemm_bf16_bias_activation_epilogue(ctx, act):
 
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF, capi.FP8E4M3])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
-@pytest.mark.parametrize("m,n,k", [(256, 256, 8192), (300, 512, 4096), (512, 260, 16384)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 8192), (300, 512, 4096), (512, 260, 16384),
+                                   (128, 520, 8192)])
 def test_gemm_split_reduction(ctx, dtype, ta, tb, m, n, k):
     # Few output tiles and a long K: the reduction is cut into parts on
     # workgroups of their own and a second kernel adds them, rounds to the C
