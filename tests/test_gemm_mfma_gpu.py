@@ -133,6 +133,23 @@ def test_gemm_split_reduction_benchmark_shape(ctx):
     assert_close(out.logical(), ref_matmul(a, b), capi.BFLOAT16)
 
 
+def test_gemm_tile_shapes_agree_bit_for_bit(ctx, knobs):
+    # 1024 x 2048 x 4096 bf16 takes 256 x 128 tiles (eight wavefronts, 64 x 64
+    # outputs each).  Every output element accumulates its K slices in the same
+    # order on every tile shape, so repeated runs and the other tile shapes
+    # must give the same bits; a wavefront reading a stage that another is
+    # still filling would not.
+    a = make_operand(75, 0, 1024, 4096, capi.BFLOAT16, False)
+    b = make_operand(75, 1, 4096, 2048, capi.BFLOAT16, True)
+    first = run(ctx, a, b, capi.FLOAT).logical()
+    assert_close(first, ref_matmul(a, b), capi.FLOAT, rtol=1e-4)
+    for _ in range(8):
+        assert np.array_equal(run(ctx, a, b, capi.FLOAT).logical(), first)
+    for tile in ("256,256", "256,128", "128,128"):
+        knobs(GEMM_TILE=tile)
+        assert np.array_equal(run(ctx, a, b, capi.FLOAT).logical(), first), tile
+
+
 def test_gemm_fp8_per_tensor_scales_bf16_out(ctx):
     # benchmark config 5b at reduced size: x ~ U[-1,1], per-tensor scale
     # s = max|x| / 448, saturating RNE cast, C = (A8 B8) * (sa * sb) -> bf16.
