@@ -165,7 +165,7 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
     const double t0 = flop / (eff(p.bm, p.bn) * peak * busy(tiles(p.bm, p.bn)));
     const int64_t slices = p.K * elem / kTileKBytes;
     double best = 0.8 * t0;
-    for (int sk = 2; sk <= 32; ++sk) {
+    for (int sk = 2; sk <= 128; ++sk) {
       if (slices % sk != 0 || slices / sk < 8)
         continue;
       const double t = flop / (eff(bm0, bn0) * peak * busy(tiles(bm0, bn0) * sk)) +

@@ -1401,9 +1401,59 @@ static bool conv_wgrad_grid(const fhip_conv_desc *d, dim3 *grid) {
   return true;
 }
 
+// The weight gradient of a 1 x 1 convolution (unit stride, no padding, one
+// group, dense channels-last 16-bit X and DY) is the matrix product DY^T X
+// over the pixels: M = K, N = C, both operands with the reduction dim as the
+// slow one.  The MFMA GEMM takes it as it lies and cuts the long reduction
+// into parts (needs no caller workspace).
+static bool conv_wgrad_as_matmul(const fhip_conv_desc *d, fhip_matmul_desc *m) {
+  const int sp = d->spatial_rank;
+  if (d->w.dim[1] != d->x.dim[1] || d->x.dtype != d->y.dtype ||
+      (d->x.dtype != FHIP_BFLOAT16 && d->x.dtype != FHIP_HALF))
+    return false;
+  int64_t pixels = d->x.dim[0];
+  for (int i = 0; i < sp; ++i) {
+    if (d->w.dim[2 + i] != 1 || d->stride[i] != 1 || d->padding[i] != 0)
+      return false;
+    pixels *= d->x.dim[2 + i];
+  }
+  const int64_t C = d->x.dim[1], K = d->w.dim[0];
+  auto dense_cl = [&](const fhip_tensor_desc &t, int64_t ch) {
+    // [N, ch, spatial...] with the channel as the fastest dim and pixels dense
+    if (ch != 1 && t.stride[1] != 1)
+      return false;
+    int64_t expect = ch;
+    for (int i = t.rank - 1; i >= 2; --i) {
+      if (t.dim[i] != 1 && t.stride[i] != expect)
+        return false;
+      expect *= t.dim[i];
+    }
+    return t.dim[0] == 1 || t.stride[0] == expect;
+  };
+  if (!dense_cl(d->x, C) || !dense_cl(d->y, K))
+    return false;
+  // DW [K, C, 1...]: rows of C contiguous elements
+  if ((C != 1 && d->w.stride[1] != 1) || (K != 1 && d->w.stride[0] != C))
+    return false;
+  std::memset(m, 0, sizeof(*m));
+  m->a.rank = m->b.rank = m->c.rank = m->out.rank = 2;
+  m->a.dtype = m->b.dtype = d->x.dtype;
+  m->a.dim[0] = K, m->a.dim[1] = pixels, m->a.stride[0] = 1, m->a.stride[1] = K;
+  m->b.dim[0] = pixels, m->b.dim[1] = C, m->b.stride[0] = C, m->b.stride[1] = 1;
+  m->c.dim[0] = K, m->c.dim[1] = C, m->c.stride[0] = C, m->c.stride[1] = 1;
+  m->c.dtype = FHIP_FLOAT;
+  m->out = m->c;
+  m->out.dtype = d->w.dtype;
+  m->out_dtype = d->w.dtype;
+  return fhip_fast_matmul_applicable(m);
+}
+
 int fhip_conv_wgrad_supported(const fhip_conv_desc *d) {
   if (!d || conv_bwd_validate(nullptr, d, "fhip_conv_wgrad") != 0)
     return 0;
+  fhip_matmul_desc md;
+  if (conv_wgrad_as_matmul(d, &md))
+    return 2;
   if (fhip_fast_conv_wgrad_applicable(d, nullptr))
     return 2;
   dim3 grid;
@@ -1417,6 +1467,14 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   if (conv_bwd_validate(ctx, d, "fhip_conv_wgrad") != 0)
     return 1;
   FHIP_REQUIRE(ctx, dy && x && dw, "fhip_conv_wgrad: null tensor pointer");
+  {
+    fhip_matmul_desc md;
+    if (conv_wgrad_as_matmul(d, &md) &&
+        (((uintptr_t)dy | (uintptr_t)x | (uintptr_t)dw) & 15) == 0) {
+      FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+      return fhip_fast_matmul(ctx, &md, dy, x, DevEpilogue{}, dw);
+    }
+  }
   size_t need = 0;
   if (fhip_fast_conv_wgrad_applicable(d, &need)) {
     FHIP_REQUIRE(ctx, workspace && workspace_bytes >= need,
