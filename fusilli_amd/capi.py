@@ -176,6 +176,7 @@ SYMBOLS = {
     "fhip_ctx_create": (c_int, [c_int, _P, POINTER(_P)]),
     "fhip_ctx_destroy": (c_int, [_P]),
     "fhip_last_error": (c_char_p, [_P]),
+    "fhip_last_kernel": (c_char_p, [_P]),
     "fhip_ctx_stream": (_P, [_P]),
     "fhip_ctx_device": (c_int, [_P]),
     "fhip_malloc": (c_int, [_P, c_size_t, POINTER(_P)]),
@@ -348,6 +349,10 @@ class Context:
     def _check(self, rc: int):
         if rc != 0:
             raise FusilliHipError(self.lib.fhip_last_error(self.handle).decode())
+
+    def last_kernel(self) -> str:
+        """Kernel variant the last operator call on this context launched."""
+        return self.lib.fhip_last_kernel(self.handle).decode()
 
     def arch(self) -> str:
         buf = ctypes.create_string_buffer(256)

@@ -267,6 +267,8 @@ const char *fhip_last_error(fhip_ctx *ctx) {
 void *fhip_ctx_stream(fhip_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 int fhip_ctx_device(fhip_ctx *ctx) { return ctx ? ctx->device : -1; }
 
+const char *fhip_last_kernel(fhip_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+
 int fhip_malloc(fhip_ctx *ctx, size_t bytes, void **out) {
   FHIP_REQUIRE(ctx, ctx && out, "fhip_malloc: null argument");
   *out = nullptr;

@@ -29,7 +29,20 @@ struct fhip_ctx {
   void *scratch = nullptr;
   size_t scratch_bytes = 0;
   std::string err;
+  // name and shape parameters of the kernel variant that the last operator
+  // call on this context chose (fhip_last_kernel)
+  char last_kernel[96] = {0};
 };
+// Records the variant the running call has chosen; a call that launches
+// helpers around one main kernel names the main kernel.
+inline void fhip_note_kernel(fhip_ctx *ctx, const char *fmt, ...) {
+  if (!ctx)
+    return;
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(ctx->last_kernel, sizeof(ctx->last_kernel), fmt, ap);
+  va_end(ap);
+}
 // At least `bytes` of 256-byte aligned scratch in *out.  Growing it allocates
 // (after the stream has drained): not for callers under graph capture.
 int fhip_ctx_scratch(fhip_ctx *ctx, size_t bytes, void **out);

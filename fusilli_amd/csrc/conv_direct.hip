@@ -766,9 +766,11 @@ int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
         break;
       }
       FHIP_HIP_CHECK(ctx, hipGetLastError());
+      fhip_note_kernel(ctx, "conv_direct channels_last group_width=%d", (int)d->w.dim[1]);
       return 0;
     }
   }
+  fhip_note_kernel(ctx, "conv_direct");
   DcArgs g{};
   FHIP_REQUIRE(ctx, make_args(d, g),
                "conv: descriptor not supported by the direct kernel");
@@ -788,6 +790,7 @@ int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
 
 int fhip_direct_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d,
                            const void *dy, const void *w, void *dx) {
+  fhip_note_kernel(ctx, "conv_direct_dgrad");
   DcArgs g{};
   FHIP_REQUIRE(ctx, make_args(d, g),
                "conv: descriptor not supported by the direct kernel");
@@ -807,6 +810,7 @@ int fhip_direct_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d,
 
 int fhip_direct_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d,
                            const void *dy, const void *x, void *dw) {
+  fhip_note_kernel(ctx, "conv_direct_wgrad");
   DcArgs g{};
   FHIP_REQUIRE(ctx, make_args(d, g),
                "conv: descriptor not supported by the direct kernel");

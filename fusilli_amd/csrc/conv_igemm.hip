@@ -382,9 +382,9 @@ struct SplitSumArgs {
   void *out;         // [M][N], dense
   int64_t mn4;       // M * N / 4
   int64_t mn;        // M * N
-  int32_t N, parts, P, Q, sp;
+  int32_t N, parts;
   int32_t y_dt, o_dt;
-  DevEpilogue epi;   // strides over the convolution's Y dims
+  DevEpilogue epi;   // rank 3: strides {0, per pixel, per channel} over (0, m, n)
 };
 
 // OUT[m][n] = epilogue(round(sum over the parts)), four columns per thread
@@ -400,20 +400,14 @@ __global__ void conv_splitk_sum_kernel(SplitSumArgs a) {
   const int64_t e = lin * 4;
   const int64_t m = e / a.N;
   const int n0 = (int)(e - m * a.N);
-  int64_t coord[FHIP_MAX_RANK];
-  const int64_t q = m % a.Q, t = m / a.Q;
-  if (a.sp == 2) {
-    coord[0] = t / a.P;
-    coord[2] = t % a.P;
-    coord[3] = q;
-  } else {
-    coord[0] = t;
-    coord[2] = q;
-  }
+  // fused operands are addressed as base + m * pixel step + n * channel step,
+  // whatever the rank of the convolution (a folded 3-D problem included)
+  int64_t coord[FHIP_MAX_RANK] = {};
+  coord[1] = m;
   const float v[4] = {acc.x, acc.y, acc.z, acc.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    coord[1] = n0 + i;
+    coord[2] = n0 + i;
     float y = fhip_round_through<float>(a.y_dt, v[i]);
     y = fhip_apply_epilogue<float>(a.epi, y, coord);
     fhip_store<float>(a.out, a.o_dt, e + i, y);
@@ -535,6 +529,7 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   if (p.ksplit > 1) {
     // every part writes plain f32 sums; rounding and the fused operations
     // follow in the kernel that adds them
+    const DevEpilogue by_pixel = g.epi; // the remapped (0, pixel, channel) strides
     float *part = (float *)(scratch + pad_bytes);
     g.out = (char *)part;
     g.c_dt = g.o_dt = FHIP_FLOAT;
@@ -557,18 +552,19 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     a.mn4 = a.mn / 4;
     a.N = (int32_t)p.N;
     a.parts = p.ksplit;
-    a.P = p.geom.P;
-    a.Q = p.geom.Q;
-    a.sp = sp;
     a.y_dt = d->y.dtype;
     a.o_dt = d->out.dtype;
-    a.epi = epi;
+    a.epi = by_pixel;
     hipLaunchKernelGGL(conv_splitk_sum_kernel, dim3((unsigned)((a.mn4 + 255) / 256)),
                        dim3(256), 0, ctx->stream, a);
     FHIP_HIP_CHECK(ctx, hipGetLastError());
+    fhip_note_kernel(ctx, "conv_igemm gather %dx%d split=%d padded=%d groups=%d", p.bm, p.bn,
+                     p.ksplit, (int)res.padded, (int)p.groups);
     return 0;
   }
   gemm_fill_linear(d->epilogue, g);
+  fhip_note_kernel(ctx, "conv_igemm %s %dx%d split=1 padded=%d groups=%d",
+                   p.halo ? "halo" : "gather", p.bm, p.bn, (int)res.padded, (int)p.groups);
   if (p.halo)
     return p.kind == GK_BF16 ? conv_launch_halo_bm<GK_BF16>(ctx, p.bm, p.bn, g)
                              : conv_launch_halo_bm<GK_F16>(ctx, p.bm, p.bn, g);
@@ -748,6 +744,13 @@ int fhip_conv_dgrad_static_setup(fhip_ctx *ctx) {
   return 0;
 }
 
+// the forward kernel's name, marked as the data gradient's
+static void dgrad_note(fhip_ctx *ctx, const char *prefix) {
+  char inner[sizeof(ctx->last_kernel)];
+  std::snprintf(inner, sizeof(inner), "%s", ctx->last_kernel);
+  fhip_note_kernel(ctx, "%s%s", prefix, inner);
+}
+
 bool fhip_fast_conv_dgrad_applicable(const fhip_conv_desc *d,
                                      size_t *workspace_bytes, bool allow_scratch) {
   const DgradPlan p = make_dgrad_plan(d, allow_scratch);
@@ -800,7 +803,11 @@ int fhip_fast_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
                        dim3((unsigned)((sa.total + 255) / 256)), dim3(256), 0,
                        ctx->stream, sa, (const uint4 *)dy, (uint4 *)grid);
     FHIP_HIP_CHECK(ctx, hipGetLastError());
-    return fhip_fast_conv(ctx, &p.fwd, grid, workspace, epi, dx, nullptr, allow_scratch);
+    const int rc = fhip_fast_conv(ctx, &p.fwd, grid, workspace, epi, dx, nullptr, allow_scratch);
+    dgrad_note(ctx, "dgrad spread + ");
+    return rc;
   }
-  return fhip_fast_conv(ctx, &p.fwd, dy, workspace, epi, dx, nullptr, allow_scratch);
+  const int rc = fhip_fast_conv(ctx, &p.fwd, dy, workspace, epi, dx, nullptr, allow_scratch);
+  dgrad_note(ctx, "dgrad ");
+  return rc;
 }

@@ -649,6 +649,8 @@ int rf_launch(fhip_ctx *ctx, const RfPlan &p) {
   hipLaunchKernelGGL(kernel, dim3((unsigned)p.grid), dim3(kRfThreads), p.lds,
                      ctx->stream, p.a);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
+  fhip_note_kernel(ctx, "conv_rf c=%d r=%d s=%d rows=%d relu=%d unit=%d", C, R, S, p.a.TR,
+                   (int)RELU, (int)UNIT);
   return 0;
 }
 

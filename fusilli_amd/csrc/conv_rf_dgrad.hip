@@ -600,6 +600,7 @@ template <int KIND> int rd_launch(fhip_ctx *ctx, const RdPlan &p) {
   hipLaunchKernelGGL(kernel, dim3((unsigned)p.grid), dim3(kRdThreads), p.lds,
                      ctx->stream, p.a);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
+  fhip_note_kernel(ctx, "conv_rf_dgrad rows=%d cols=%d", p.a.TR, p.a.TQ);
   return 0;
 }
 

@@ -243,5 +243,6 @@ int fhip_fast_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   hipLaunchKernelGGL(conv_wgrad_sum_kernel, dim3((unsigned)((total + 255) / 256)),
                      dim3(256), 0, ctx->stream, as, part, dw, total);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
+  fhip_note_kernel(ctx, "conv_wgrad batched gemm");
   return 0;
 }

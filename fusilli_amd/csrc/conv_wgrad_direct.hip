@@ -585,5 +585,6 @@ int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
   hipLaunchKernelGGL(conv_wgrad_direct_sum_kernel, dim3((unsigned)(total / 64)),
                      dim3(256), 0, ctx->stream, s, (const float *)p.a.part, dw);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
+  fhip_note_kernel(ctx, "conv_wgrad_direct");
   return 0;
 }

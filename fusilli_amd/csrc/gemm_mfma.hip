@@ -283,6 +283,9 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     o.stride[1] = s.stride[r - 2];
     o.stride[2] = s.stride[r - 1];
   }
+  static const char *const kKindName[] = {"bf16", "f16", "i8", "fp8e4m3", "fp8e5m2"};
+  fhip_note_kernel(ctx, "gemm_mfma %s %dx%d waves=%d split=%d", kKindName[p.kind], p.bm, p.bn,
+                   p.bm == 128 ? 4 : 8, p.ksplit);
   auto launch = [&]() {
     switch (p.kind) {
     case GK_BF16:

@@ -102,6 +102,22 @@ __global__ void generic_matmul_kernel(MatmulArgs g, const void *a,
 // global loads are in flight while the current one is multiplied.
 constexpr int kF32Tile = 64, kF32K = 16, kF32Pitch = kF32Tile + 4;
 
+// Operand element as f32.  DT is the element type fixed at compile time (both
+// operands f32, bf16 or f16: a plain load and at most one conversion); -1
+// takes the type from the descriptor per element (mixed operand types).
+template <int DT>
+__device__ __forceinline__ float matmul_operand(const void *p, int dt, int64_t idx) {
+  if constexpr (DT == FHIP_FLOAT)
+    return ((const float *)p)[idx];
+  else if constexpr (DT == FHIP_BFLOAT16)
+    return (float)((const __bf16 *)p)[idx];
+  else if constexpr (DT == FHIP_HALF)
+    return (float)((const _Float16 *)p)[idx];
+  else
+    return fhip_load<float>(p, dt, idx);
+}
+
+template <int DT>
 __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
     MatmulArgs g, const void *a, const void *b, void *out, int tiles_n) {
   typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -145,10 +161,10 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
       const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
       const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
       ra[i] = m < M && ka < g.K
-                  ? fhip_load<float>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
+                  ? matmul_operand<DT>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
                   : 0.f;
       rb[i] = n < N && kb < g.K
-                  ? fhip_load<float>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
+                  ? matmul_operand<DT>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
                   : 0.f;
     }
   };
@@ -197,6 +213,7 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
 // A / B sub-tiles in a private LDS region (no workgroup barriers in the loop);
 // the partial sums meet in LDS and every wavefront finishes a quarter of the
 // accumulator registers.
+template <int DT>
 __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
     MatmulArgs g, const void *a, const void *b, void *out, int tiles_n) {
   typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -239,10 +256,10 @@ __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
       const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
       const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
       ra[i] = m < M && ka < g.K
-                  ? fhip_load<float>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
+                  ? matmul_operand<DT>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
                   : 0.f;
       rb[i] = n < N && kb < g.K
-                  ? fhip_load<float>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
+                  ? matmul_operand<DT>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
                   : 0.f;
     }
   };
@@ -1080,6 +1097,7 @@ int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
     return 1;
   if (fhip_fast_matmul_applicable(d))
     return fhip_fast_matmul(ctx, d, a, b, epi, out);
+  fhip_note_kernel(ctx, "matmul_generic");
 
   MatmulArgs g{};
   g.out = make_dims(d->c);
@@ -1107,19 +1125,42 @@ int fhip_matmul(fhip_ctx *ctx, const fhip_matmul_desc *d, const void *a,
     const int64_t tm = (M + kF32Tile - 1) / kF32Tile, tn = (N + kF32Tile - 1) / kF32Tile;
     const int64_t batch = total / (M * N);
     const int64_t sm = (M + 31) / 32, sn = (N + 31) / 32;
+    // the operands' common element type, compiled into the kernel (-1: mixed)
+    const int same_dt = d->a.dtype == d->b.dtype ? (int)d->a.dtype : -1;
     if (tm * tn * batch < 128 && g.K >= 8 * kF32K && batch <= 65535 &&
         sm * sn < (1ll << 31)) {
       // few tiles: 32 x 32 tiles with K split over the wavefronts
-      hipLaunchKernelGGL(splitk_matmul_f32_kernel,
-                         dim3((unsigned)(sm * sn), (unsigned)batch), dim3(256),
-                         0, ctx->stream, g, a, b, out, (int)sn);
+      const dim3 grid((unsigned)(sm * sn), (unsigned)batch);
+      auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, ctx->stream, g, a, b, out, (int)sn);
+      };
+      if (same_dt == FHIP_FLOAT)
+        go(splitk_matmul_f32_kernel<FHIP_FLOAT>);
+      else if (same_dt == FHIP_BFLOAT16)
+        go(splitk_matmul_f32_kernel<FHIP_BFLOAT16>);
+      else if (same_dt == FHIP_HALF)
+        go(splitk_matmul_f32_kernel<FHIP_HALF>);
+      else
+        go(splitk_matmul_f32_kernel<-1>);
       FHIP_HIP_CHECK(ctx, hipGetLastError());
+      fhip_note_kernel(ctx, "matmul_f32_splitk");
       return 0;
     }
     if (tm * tn < (1ll << 31) && batch <= 65535 && tn < (1ll << 31)) {
-      hipLaunchKernelGGL(tiled_matmul_f32_kernel, dim3((unsigned)(tm * tn), (unsigned)batch),
-                         dim3(256), 0, ctx->stream, g, a, b, out, (int)tn);
+      const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
+      auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, ctx->stream, g, a, b, out, (int)tn);
+      };
+      if (same_dt == FHIP_FLOAT)
+        go(tiled_matmul_f32_kernel<FHIP_FLOAT>);
+      else if (same_dt == FHIP_BFLOAT16)
+        go(tiled_matmul_f32_kernel<FHIP_BFLOAT16>);
+      else if (same_dt == FHIP_HALF)
+        go(tiled_matmul_f32_kernel<FHIP_HALF>);
+      else
+        go(tiled_matmul_f32_kernel<-1>);
       FHIP_HIP_CHECK(ctx, hipGetLastError());
+      fhip_note_kernel(ctx, "matmul_f32_tiled");
       return 0;
     }
   }
@@ -1213,6 +1254,7 @@ int fhip_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     return 0;
   if (fhip_direct_conv_applicable(d))
     return fhip_direct_conv_fprop(ctx, d, x, w, epi, out);
+  fhip_note_kernel(ctx, "conv_generic");
 
   ConvArgs g{};
   g.y = make_dims(d->y);
@@ -1341,6 +1383,7 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   }
   if (fhip_direct_conv_applicable(d))
     return fhip_direct_conv_dgrad(ctx, d, dy, w, dx);
+  fhip_note_kernel(ctx, "conv_dgrad_generic");
   const ConvBwdArgs g = conv_bwd_args(d, true);
   const int64_t total = fhip_desc_volume(d->x);
   hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),
@@ -1371,6 +1414,7 @@ int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
   // the direct and the strided kernel use no scratch at all
   if (fhip_direct_conv_applicable(d))
     return fhip_direct_conv_dgrad(ctx, d, dy, w, dx);
+  fhip_note_kernel(ctx, "conv_dgrad_generic");
   const ConvBwdArgs g = conv_bwd_args(d, true);
   const int64_t total = fhip_desc_volume(d->x);
   hipLaunchKernelGGL(generic_conv_dgrad_kernel, dim3(grid_for(total, 256)),
@@ -1472,7 +1516,11 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
     if (conv_wgrad_as_matmul(d, &md) &&
         (((uintptr_t)dy | (uintptr_t)x | (uintptr_t)dw) & 15) == 0) {
       FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
-      return fhip_fast_matmul(ctx, &md, dy, x, DevEpilogue{}, dw);
+      const int rc = fhip_fast_matmul(ctx, &md, dy, x, DevEpilogue{}, dw);
+      char inner[sizeof(ctx->last_kernel)];
+      std::snprintf(inner, sizeof(inner), "%s", ctx->last_kernel);
+      fhip_note_kernel(ctx, "wgrad 1x1 as %s", inner);
+      return rc;
     }
   }
   size_t need = 0;
@@ -1492,6 +1540,7 @@ int fhip_conv_wgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
   if (fhip_direct_conv_applicable(d))
     return fhip_direct_conv_wgrad(ctx, d, dy, x, dw);
+  fhip_note_kernel(ctx, "conv_wgrad_generic");
   const ConvBwdArgs g = conv_bwd_args(d, false);
   if (fhip_desc_volume(d->w) == 0)
     return 0;
@@ -1608,6 +1657,7 @@ int fhip_sdpa_fwd(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
   if (fhip_fast_sdpa_applicable(d))
     return fhip_fast_sdpa(ctx, d, q, k, v, mask, o);
+  fhip_note_kernel(ctx, "sdpa_generic");
 
   SdpaArgs g{};
   g.B = d->q.dim[0];
@@ -1714,6 +1764,7 @@ int fhip_norm_fwd(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
     return 1;
   if (fhip_fast_norm_applicable(d))
     return fhip_fast_norm(ctx, d, x, scale, bias, epi, out, mean, inv_variance);
+  fhip_note_kernel(ctx, "norm_generic");
 
   NormArgs g{};
   g.x = make_dims(d->x);
@@ -1810,6 +1861,7 @@ int fhip_batchnorm_fwd(fhip_ctx *ctx, const fhip_batchnorm_desc *d,
   (void)workspace;
   (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  fhip_note_kernel(ctx, "batchnorm_generic training=%d", (int)d->training);
   BatchNormArgs g{};
   g.x = make_dims(d->x);
   g.xs = make_strides(d->x);
@@ -1878,6 +1930,7 @@ int fhip_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
   // the row kernel moves 16-byte chunks: an unaligned base takes the generic one
   if (fhip_fast_reduce_applicable(d) && ((uintptr_t)x & 15) == 0)
     return fhip_fast_reduce(ctx, d, x, y);
+  fhip_note_kernel(ctx, "reduce_generic");
   ReduceArgs g{};
   g.y = make_dims(d->y);
   g.red.rank = d->x.rank;
@@ -2020,6 +2073,7 @@ int fhip_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d, const void *in0,
     if (aligned && fhip_fast_pointwise_applicable(d))
       return fhip_fast_pointwise(ctx, d, in0, in1, in2, out);
   }
+  fhip_note_kernel(ctx, "pointwise_generic");
   PointwiseArgs g{};
   g.out = make_dims(d->out);
   g.os = make_strides(d->out);

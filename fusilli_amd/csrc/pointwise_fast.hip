@@ -445,6 +445,7 @@ int fhip_fast_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d,
   PwFastArgs &g = p.g;
   g.in[0] = in0, g.in[1] = in1, g.in[2] = in2;
   g.out = out;
+  fhip_note_kernel(ctx, "pointwise_fast inputs=%d mode=%d", (int)d->num_inputs, (int)d->mode);
   // the common modes get kernels of their own
 #define PW_CASE(NIN, MODE)                                                     \
   case MODE:                                                                   \

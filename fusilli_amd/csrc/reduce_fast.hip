@@ -375,6 +375,7 @@ int fhip_fast_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
   g.y_dt = d->y.dtype;
   g.post = p.post;
   g.inv_count = 1.0f / (float)p.cols;
+  fhip_note_kernel(ctx, "reduce_rows");
   switch (d->x.dtype) {
   case FHIP_FLOAT:
     return launch_mode<float>(ctx, p, g);

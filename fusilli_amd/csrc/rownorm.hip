@@ -232,5 +232,6 @@ int fhip_fast_norm(fhip_ctx *ctx, const fhip_norm_desc *d, const void *x,
   FHIP_REQUIRE(ctx, launched, "rownorm: no kernel for shape (%d, %d)", wpr,
                chunks);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
+  fhip_note_kernel(ctx, "rownorm chunks=%d waves_per_row=%d variant=%d", chunks, wpr, variant);
   return 0;
 }

@@ -120,6 +120,10 @@ __global__ __launch_bounds__(kRlThreads) void rownorm_long_stats_kernel(RowNormL
     float *p = g.partial + (row * g.splits + s) * 2;
     p[0] = s1;
     p[1] = s2;
+    // the pivot travels with the sums: when OUT is X, the second kernel's
+    // workgroups must not re-read it from a row that one of them is rewriting
+    if (s == 0)
+      g.partial[g.rows * g.splits * 2 + row] = pivot;
   }
 }
 
@@ -129,7 +133,7 @@ __global__ __launch_bounds__(kRlThreads) void rownorm_long_apply_kernel(RowNormL
   __shared__ float lds[kRlThreads / 64][2];
   const int64_t row = blockIdx.y, s = blockIdx.x;
   const T *xr = (const T *)g.x + row * g.x_row_stride;
-  const float pivot = g.is_layernorm ? (float)xr[0] : 0.f;
+  const float pivot = g.partial[g.rows * g.splits * 2 + row];
   // the row's statistics from its segments' sums (at most one per thread)
   float s1 = 0.f, s2 = 0.f;
   if ((int)threadIdx.x < g.splits) {
@@ -221,7 +225,8 @@ int fhip_norm_long(fhip_ctx *ctx, const fhip_norm_desc *d, int64_t inner,
   g.seg = seg;
   g.splits = (int32_t)splits;
   void *scratch = nullptr;
-  if (fhip_ctx_scratch(ctx, (size_t)(g.rows * splits * 2) * sizeof(float), &scratch) != 0)
+  // per row: a pair of sums per segment, and behind all pairs the rows' pivots
+  if (fhip_ctx_scratch(ctx, (size_t)(g.rows * splits * 2 + g.rows) * sizeof(float), &scratch) != 0)
     return 1;
   g.partial = (float *)scratch;
   auto aligned = [](const void *p) { return ((uintptr_t)p & 15u) == 0; };
@@ -239,5 +244,6 @@ int fhip_norm_long(fhip_ctx *ctx, const fhip_norm_desc *d, int64_t inner,
     break;
   }
   FHIP_HIP_CHECK(ctx, hipGetLastError());
+  fhip_note_kernel(ctx, "rownorm_long segments=%d", g.splits);
   return 0;
 }

@@ -58,6 +58,7 @@ constexpr int kWaves = 8;
 constexpr int kStages = 3;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kMaxSlack = 8.0f; // see the softmax phase
+constexpr float kRedoSum = 8192.0f; // 32 probabilities of 2^kMaxSlack
 
 // Sizes that follow from the head dimension HD (Q/K and V), 64 or 128.
 template <int HD> struct SdShape {
@@ -85,6 +86,9 @@ struct SdpaArgs {
   int64_t o_sb, o_sh, o_ss;
   int32_t Sq, Skv, group; // group = Hq / Hkv
   int32_t causal;
+  // XCD-aware order of a one-dimensional grid (0: the grid is heads x batch x
+  // query-tile groups): heads and query-tile groups per head
+  int32_t xcd_heads, xcd_groups;
   float scale_log2e; // softmax scale * log2(e)
   float scale;       // softmax scale
   // mask tensor (kernels with MASK): strides in elements, 0 where broadcast;
@@ -254,9 +258,19 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   // Causal masks: a workgroup runs query tile (last - z) and then tile z, a
   // long and a short one, so all workgroups do the same work (tiles of one
   // head need 1 .. n key-tile rows).  Otherwise one tile per workgroup.
-  const int h = blockIdx.x, b = blockIdx.y;
+  // Hardware deals consecutive workgroup ids to the 8 XCDs in turn.  All query
+  // tiles of a (batch, head) read the same K and V: the remapped order runs
+  // them side by side on one XCD, so that its L2 fetches every K / V tile once
+  // for all of them.
+  int h = blockIdx.x, b = blockIdx.y, z = blockIdx.z;
+  if (g.xcd_heads) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    z = slot % g.xcd_groups;
+    const int head = (slot / g.xcd_groups) * 8 + xcd;
+    h = head % g.xcd_heads;
+    b = head / g.xcd_heads;
+  }
   const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
-  const int z = blockIdx.z;
   const int passes = CAUSAL && n_qtiles - 1 - z != z ? 2 : 1;
   for (int pass = 0; pass < passes; ++pass) {
   const int qtile = CAUSAL && pass == 0 ? n_qtiles - 1 - z : z;
@@ -425,23 +439,21 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
 
   // ---- fragment addressing ----------------------------------------------------
   // K (A operand of S^T): row lq of a 32-key block, 16-byte chunk 2*ds + half
-  uint32_t kaddr[kD / 16];
-#pragma unroll
-  for (int ds = 0; ds < kD / 16; ++ds)
-    kaddr[ds] =
-        (uint32_t)(lq * kRowB + (((ds * 2 + half) ^ sd_kswz<HD>(lq)) << 4));
+  // (the chunk index is ds * 2 + half XOR a value below 16: K-step ds moves
+  // the address by XOR with ds << 5, which costs one instruction per read and
+  // saves a register per K-step; the stages start on multiples of 16 KB)
+  const uint32_t kaddr0 = (uint32_t)(lq * kRowB + ((half ^ sd_kswz<HD>(lq)) << 4));
   // V^T (A operand of O^T += V^T P^T): the keys a lane needs are those whose
   // probabilities it holds: key = 32*kb + 8*(i/4) + 4*half + i%4 for score
   // register i; one transposing read returns 4 consecutive keys of one column
-  uint32_t vaddr[kD / 32];
+  // (chunk dt * 4 + x with x < 4: both permutations leave the dt bits alone,
+  // so feature block dt moves the address by XOR with dt << 6)
+  uint32_t vaddr0;
   {
     const int L = l & 15, h16 = (l >> 4) & 1;
     const int row = half * 4 + (L >> 2);
-#pragma unroll
-    for (int dt = 0; dt < kD / 32; ++dt) {
-      const int c = dt * 4 + h16 * 2 + ((L & 3) >> 1);
-      vaddr[dt] = (uint32_t)(row * kRowB + (sd_vpos<HD>(row, c) << 4) + (L & 1) * 8);
-    }
+    const int c = h16 * 2 + ((L & 3) >> 1);
+    vaddr0 = (uint32_t)(row * kRowB + (sd_vpos<HD>(row, c) << 4) + (L & 1) * 8);
   }
 
   f32x16 o[kD / 32];
@@ -466,6 +478,11 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   // the top of round t (K tile t + 2, V tile t + 1) reuse the stages of K tile
   // t - 1 and V tile t - 2 and have to land by barrier t + 1.
   const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
+  constexpr bool kLoadsInValuPhase = MASK == 0 && HD == 128;
+#ifndef SD_FUSE_PLAIN
+#define SD_FUSE_PLAIN 0
+#endif
+  constexpr bool kFusedPipeline = MASK != 0 || SD_FUSE_PLAIN;
   if constexpr (MASK == 2)
     issue_mask(0); // older than every K / V load: landed by the first wait
   issue_k(0, 0);
@@ -477,106 +494,145 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
-  f32x16 s[2];
   uint32_t pf[4][4]; // probabilities as B-operand fragments, 16 keys each
   // a wavefront whose rows all lie above a tile has nothing to add
   auto active = [&](int t) { return !(CAUSAL && t * kBKV > qw0 + 31); };
   // ring slots of tile t - 1, t, t + 1, t + 2 (slot of t + 2 == slot of t - 1)
   int sl_prev = kStages - 1, sl_cur = 0, sl_next = 1;
-#pragma clang loop unroll(disable)
-  for (int t = 0; t <= tiles; ++t) {
+  // One round.  The first (tile 0: no O^T update, and the softmax always takes
+  // its full route) and the last (t == tiles: only the O^T update of the last
+  // tile) are peeled off the loop as straight-line code, so that the loop holds
+  // a single variant of the MFMA pipeline.
+  auto round = [&](const int t, auto which_c) __attribute__((always_inline)) {
+    constexpr bool FIRST = decltype(which_c)::value == 0;
+    constexpr bool LAST = decltype(which_c)::value == 2;
+    f32x16 s[2]; // scores of tile t: written by the MFMA phase, read by the softmax
     // (the mask first: the waits below count the K / V loads issued after it)
     if constexpr (MASK == 1)
       if (t < tiles)
         load_mask(t);
-    issue_k(t + 2, sl_prev);
-    issue_v(t + 1, sl_next);
+    // This round's loads, K tile t + 2 and V tile t + 1.  Under memory
+    // back-pressure every LDS-DMA instruction holds its wavefront at issue for
+    // tens of clocks.  They go in front of the shorter of a round's two phases:
+    // the MFMA phase with a mask tensor or head dim 64, the vector-ALU phase
+    // otherwise (the SIMD's other wavefront feeds the matrix pipe meanwhile).
+    if constexpr (!kLoadsInValuPhase) {
+      issue_k(t + 2, sl_prev);
+      issue_v(t + 1, sl_next);
+    }
     // ---- MFMA phase -----------------------------------------------------------
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_setprio(2);
-    // Fragment reads of both blocks are written as asm: the compiler neither
+    // The phase is one software pipeline over up to 32 MFMAs: NS for S^T of
+    // tile t (ds-major, kb-minor: K fragment m, Q fragment m / 2), then NP for
+    // O^T += V^T P^T of tile t - 1 (j-major, dt-minor).  Every MFMA takes a
+    // fresh A fragment from LDS (one 16-byte read of K, or two transposing
+    // 8-byte reads of V).  The reads are written as asm: the compiler neither
     // sees them as LDS accesses (it would make the transposing reads wait for
     // every outstanding global -> LDS load, the tiles fetched ahead included)
-    // nor waits for them; reads run kAhead MFMAs ahead, and one sd_wait_pin
-    // per kGroup MFMAs waits for that group's fragments.
+    // nor waits for them; they run kAhead MFMAs ahead, straight across the
+    // boundary between the two products, and one sd_wait_pin per kGroup MFMAs
+    // waits for that group's fragments.
     constexpr int kAhead = 8, kGroup = 4;
-    if (t < tiles && active(t)) {
-      const uint32_t sk = k_stage(sl_cur);
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          s[kb][r] = 0.f;
-      constexpr int kMfmas = 2 * (kD / 16); // ds-major, kb-minor
-      u32x4 kr[kMfmas];
-      auto read = [&](auto mc) {
+    constexpr int NS = 2 * (kD / 16), NP = 4 * (kD / 32);
+    static_assert(NS % kGroup == 0 && NP % kGroup == 0 && NS >= kAhead && NP >= kAhead,
+                  "groups do not straddle the two products");
+    auto mfma_range = [&](auto first_c, auto last_c) __attribute__((always_inline)) {
+      constexpr int M0 = decltype(first_c)::value, M1 = decltype(last_c)::value;
+      const uint32_t sk = k_stage(sl_cur) + kaddr0, sv = v_stage(sl_prev) + vaddr0;
+      u32x4 kr[NS];
+      u32x2 vr[NP][2];
+      auto read = [&](auto mc) __attribute__((always_inline)) {
         constexpr int m = decltype(mc)::value;
-        sd_read_b128<(m % 2) * 32 * kRowB>(kr[m], sk + kaddr[m / 2]);
+        if constexpr (m < NS) {
+          sd_read_b128<(m % 2) * 32 * kRowB>(kr[m], sk ^ (uint32_t)((m / 2) << 5));
+        } else {
+          constexpr int j = (m - NS) / (kD / 32), dt = (m - NS) % (kD / 32);
+          const uint32_t ad = sv ^ (uint32_t)(dt << 6);
+          sd_read_tr16<(j * 16 + 0) * kRowB>(vr[m - NS][0], ad);
+          sd_read_tr16<(j * 16 + 8) * kRowB>(vr[m - NS][1], ad);
+        }
       };
-      sd_static_for<kAhead>(read);
-      sd_static_for<kMfmas / kGroup>([&](auto gc) {
-        constexpr int m0 = decltype(gc)::value * kGroup;
-        constexpr int rest = kMfmas - (m0 + kGroup);
-        constexpr int left = rest < kAhead - kGroup ? rest : kAhead - kGroup;
-        sd_wait_pin<left>(kr[m0], kr[m0 + 1], kr[m0 + 2], kr[m0 + 3]);
+      sd_static_for<kAhead>([&](auto ic) {
+        read(std::integral_constant<int, M0 + decltype(ic)::value>{});
+      });
+      sd_static_for<(M1 - M0) / kGroup>([&](auto gc) {
+        constexpr int m0 = M0 + decltype(gc)::value * kGroup;
+        // LDS operations younger than this group's: the next group's reads
+        constexpr int n1 = m0 + 2 * kGroup < M1 ? m0 + 2 * kGroup : M1;
+        constexpr int young_k = n1 < NS ? n1 - (m0 + kGroup) : (m0 + kGroup < NS ? NS - (m0 + kGroup) : 0);
+        constexpr int young = n1 <= m0 + kGroup ? 0 : young_k + 2 * ((n1 - (m0 + kGroup)) - young_k);
+        if constexpr (m0 < NS) {
+          sd_wait_pin<young>(kr[m0], kr[m0 + 1], kr[m0 + 2], kr[m0 + 3]);
 #pragma unroll
-        for (int i = 0; i < kGroup; ++i) {
-          const int m = m0 + i;
-          const uint32_t kf[4] = {kr[m].x, kr[m].y, kr[m].z, kr[m].w};
-          s[m % 2] = sd_mfma<BF16>(kf, qf[m / 2], s[m % 2]);
+          for (int i = 0; i < kGroup; ++i) {
+            const int m = m0 + i;
+            const uint32_t kf[4] = {kr[m].x, kr[m].y, kr[m].z, kr[m].w};
+            f32x16 zero;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              zero[r] = 0.f;
+            s[m % 2] = sd_mfma<BF16>(kf, qf[m / 2], m < 2 ? zero : s[m % 2]);
+          }
+        } else {
+          constexpr int v0 = m0 - NS;
+          sd_wait_pin<young>(vr[v0][0], vr[v0][1], vr[v0 + 1][0], vr[v0 + 1][1],
+                             vr[v0 + 2][0], vr[v0 + 2][1], vr[v0 + 3][0], vr[v0 + 3][1]);
+#pragma unroll
+          for (int i = 0; i < kGroup; ++i) {
+            const int m = v0 + i;
+            const int j = m / (kD / 32), dt = m % (kD / 32);
+            const uint32_t vf[4] = {vr[m][0].x, vr[m][0].y, vr[m][1].x, vr[m][1].y};
+            o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
+          }
         }
         __builtin_amdgcn_sched_barrier(0); // keep the MFMAs at their wait
         sd_static_for<kGroup>([&](auto ic) {
           constexpr int m = m0 + kAhead + decltype(ic)::value;
-          if constexpr (m < kMfmas)
+          if constexpr (m < M1)
             read(std::integral_constant<int, m>{});
         });
       });
-    }
-    if (t > 0 && active(t - 1)) {
-      const uint32_t sv = v_stage(sl_prev);
-      constexpr int kMfmas = 4 * (kD / 32); // j-major, dt-minor
-      u32x2 vr[kMfmas][2];
-      auto read = [&](auto mc) {
-        constexpr int m = decltype(mc)::value;
-        constexpr int j = m / (kD / 32), dt = m % (kD / 32);
-        const uint32_t ad = sv + vaddr[dt];
-        sd_read_tr16<(j * 16 + 0) * kRowB>(vr[m][0], ad);
-        sd_read_tr16<(j * 16 + 8) * kRowB>(vr[m][1], ad);
-      };
-      sd_static_for<kAhead>(read);
-      sd_static_for<kMfmas / kGroup>([&](auto gc) {
-        constexpr int m0 = decltype(gc)::value * kGroup;
-        constexpr int rest = kMfmas - (m0 + kGroup);
-        constexpr int left = rest < kAhead - kGroup ? rest : kAhead - kGroup;
-        sd_wait_pin<2 * left>(vr[m0][0], vr[m0][1], vr[m0 + 1][0], vr[m0 + 1][1],
-                              vr[m0 + 2][0], vr[m0 + 2][1], vr[m0 + 3][0],
-                              vr[m0 + 3][1]);
-#pragma unroll
-        for (int i = 0; i < kGroup; ++i) {
-          const int m = m0 + i;
-          const int j = m / (kD / 32), dt = m % (kD / 32);
-          const uint32_t vf[4] = {vr[m][0].x, vr[m][0].y, vr[m][1].x, vr[m][1].y};
-          o[dt] = sd_mfma<BF16>(vf, pf[j], o[dt]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        sd_static_for<kGroup>([&](auto ic) {
-          constexpr int m = m0 + kAhead + decltype(ic)::value;
-          if constexpr (m < kMfmas)
-            read(std::integral_constant<int, m>{});
-        });
-      });
+    };
+    {
+      using I0 = std::integral_constant<int, 0>;
+      using IS = std::integral_constant<int, NS>;
+      using IE = std::integral_constant<int, NS + NP>;
+      // A tile that is live for a wavefront has a live predecessor.  In the
+      // round after a wavefront's last live tile S^T of a dead tile is computed
+      // along with the O^T update and never looked at: a second variant of the
+      // pipeline inside the loop costs registers the kernel does not have.
+      if constexpr (FIRST) {
+        mfma_range(I0{}, IS{});
+      } else if constexpr (LAST) {
+        if (active(t - 1))
+          mfma_range(IS{}, IE{});
+      } else if constexpr (kFusedPipeline) {
+        if (active(t - 1))
+          mfma_range(I0{}, IE{});
+      } else {
+        if (active(t))
+          mfma_range(I0{}, IS{});
+        if (active(t - 1))
+          mfma_range(IS{}, IE{});
+      }
     }
     __builtin_amdgcn_s_setprio(0);
     __builtin_amdgcn_sched_barrier(0);
     // wavefronts 4..7 end their round here: everything but the loads of this
-    // round has landed
+    // round has landed (which, in the vector-ALU phase, have not been issued
+    // yet)
     if (team) {
-      __builtin_amdgcn_s_waitcnt(sd_wait_imm(2 * kLoadsPerTile));
+      __builtin_amdgcn_s_waitcnt(sd_wait_imm(kLoadsInValuPhase ? 0 : 2 * kLoadsPerTile));
       sd_barrier();
     }
-    if (t == tiles)
-      break;
+    if constexpr (LAST)
+      return;
+    if constexpr (kLoadsInValuPhase) {
+      issue_k(t + 2, sl_prev);
+      issue_v(t + 1, sl_next);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 
     // ---- vector-ALU phase -------------------------------------------------------
     if (active(t)) {
@@ -671,42 +727,111 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
             s[kb][r] = dead ? gone : s[kb][r];
           }
       }
-      float mx = s[0][0];
+      // Exponentials of the tile's scores against reference point `ref` (raw
+      // score units): the probabilities, rounded to the input type, go into
+      // the fragments of the next MFMA phase; returns this lane's sum.  (Summing
+      // the rounded pairs with v_dot2c_f32_bf16 measured slower than two adds.)
+      auto exps = [&](float ref) __attribute__((always_inline)) {
+        const float mc = ref * sl2;
+        float psum = 0.f;
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          mx = fmaxf(mx, s[kb][r]);
-      mx = sd_half_max(mx);
+          for (int r = 0; r < 16; r += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * sl2 - mc);
+            const float p1 = __builtin_amdgcn_exp2f(s[kb][r + 1] * sl2 - mc);
+            const uint32_t pk = sd_pack<BF16>(p0, p1);
+            pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = pk;
+            psum += p0 + p1;
+          }
+        return psum;
+      };
       // The reference point of the exponentials follows the row maximum
-      // lazily: it moves only when the maximum has risen by more than
-      // kMaxSlack (in log2 units of the scaled scores).  Probabilities are
-      // then at most 2^kMaxSlack, sums and outputs stay far inside float
-      // range, and O = sum(p v) / sum(p) does not depend on the reference
-      // point; the rescaling of O^T becomes rare.
-      const bool moved = (mx - m_run) * sl2 > kMaxSlack;
-      const float m_new = moved ? mx : m_run;
-      const float mc = m_new * sl2;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
-      m_run = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * sl2 - mc);
-          const float p1 = __builtin_amdgcn_exp2f(s[kb][r + 1] * sl2 - mc);
-          psum += p0 + p1;
-          pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = sd_pack<BF16>(p0, p1);
+      // lazily.  Without a mask tensor a tile first runs against the reference
+      // point it inherits, with no maximum taken at all: as long as no lane's
+      // sum exceeds kRedoSum every probability is at most that, sums and
+      // outputs stay far inside float range, and O = sum(p v) / sum(p) does not
+      // depend on the reference point.  Only the first tile, and a tile in which
+      // some row's scores rose that far above the reference, take the full
+      // route: row maximum, a reference point that moves when the maximum has
+      // risen by more than kMaxSlack (log2 units of the scaled scores), O^T
+      // rescaled, the exponentials (again).  One copy of the code serves both:
+      // the second trip of the loop is the full route.
+      if constexpr (HD == 128) {
+        bool full = FIRST || MASK != 0;
+        float psum;
+  #pragma clang loop unroll(disable)
+        for (;;) {
+          if (full) {
+            float mx = s[0][0];
+  #pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+  #pragma unroll
+              for (int r = 0; r < 16; ++r)
+                mx = fmaxf(mx, s[kb][r]);
+            mx = sd_half_max(mx);
+            const bool moved = (mx - m_run) * sl2 > kMaxSlack;
+            const float m_new = moved ? mx : m_run;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
+            m_run = m_new;
+            l_run *= alpha;
+            // O^T holds tiles 0 .. t - 1 here (their MFMA phases are over).  In
+            // place, as asm with tied operands: written as o *= alpha the
+            // compiler gives the rescaled O^T registers of its own and copies
+            // all 64 accumulators on the common route.  (The MFMAs that wrote
+            // O^T lie a whole row maximum behind: no hazard.)
+            if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+  #pragma unroll
+              for (int dt = 0; dt < kD / 32; ++dt)
+  #pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                  float x = o[dt][r];
+                  asm volatile("v_mul_f32 %0, %1, %0" : "+v"(x) : "v"(alpha));
+                  o[dt][r] = x;
+                }
+            }
+          }
+          psum = exps(m_run);
+          if (full || __builtin_amdgcn_ballot_w64(!(psum <= kRedoSum)) == 0)
+            break;
+          full = true;
         }
-      l_run = l_run * alpha + psum;
-      // O^T holds tiles 0 .. t - 1 here (their MFMA phases are over)
-      if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+        l_run += psum;
+      } else {
+        // Head dim 64, where this phase is the longer one: the same steps as
+        // two straight-line copies (fast route, then the full one if needed).
+        // The compiler copies registers around whichever form it likes less:
+        // all of O^T on the fast route of this form at head dim 128, the
+        // scores in the loop form at head dim 64.
+        bool full = true;
+        if constexpr (MASK == 0 && !FIRST) {
+          const float psum = exps(m_run);
+          full = __builtin_amdgcn_ballot_w64(!(psum <= kRedoSum)) != 0;
+          if (!full)
+            l_run += psum;
+        }
+        if (full) {
+          float mx = s[0][0];
 #pragma unroll
-        for (int dt = 0; dt < kD / 32; ++dt)
+          for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            o[dt][r] *= alpha;
+            for (int r = 0; r < 16; ++r)
+              mx = fmaxf(mx, s[kb][r]);
+          mx = sd_half_max(mx);
+          const bool moved = (mx - m_run) * sl2 > kMaxSlack;
+          const float m_new = moved ? mx : m_run;
+          const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
+          m_run = m_new;
+          const float psum = exps(m_new);
+          l_run = l_run * alpha + psum;
+          if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+              for (int r = 0; r < 16; ++r)
+                o[dt][r] *= alpha;
+          }
+        }
       }
     }
     // wavefronts 0..3 end their round here
@@ -717,7 +842,12 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
     sl_prev = sl_cur;
     sl_cur = sl_next;
     sl_next = next_slot(sl_next);
-  }
+  };
+  round(0, std::integral_constant<int, 0>{});
+#pragma clang loop unroll(disable)
+  for (int t = 1; t < tiles; ++t)
+    round(t, std::integral_constant<int, 1>{});
+  round(tiles, std::integral_constant<int, 2>{});
   if (!team) // pairs with the last barrier of wavefronts 4..7
     __builtin_amdgcn_s_barrier();
 
@@ -882,8 +1012,15 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   g.scale_log2e = scale * 1.4426950408889634f;
   g.scale = scale;
   const int n_qtiles = (g.Sq + kBQ - 1) / kBQ;
-  const dim3 grid((unsigned)d->q.dim[1], (unsigned)d->q.dim[0],
-                  (unsigned)(d->is_causal ? (n_qtiles + 1) / 2 : n_qtiles));
+  const int64_t groups = d->is_causal ? (n_qtiles + 1) / 2 : n_qtiles;
+  const int64_t heads = d->q.dim[1] * d->q.dim[0];
+  dim3 grid((unsigned)d->q.dim[1], (unsigned)d->q.dim[0], (unsigned)groups);
+  if (heads % 8 == 0 && groups > 1 && heads * groups < (1ll << 31) &&
+      std::getenv("FUSILLI_HIP_SDPA_GRID") == nullptr) {
+    g.xcd_heads = (int32_t)d->q.dim[1];
+    g.xcd_groups = (int32_t)groups;
+    grid = dim3((unsigned)(heads * groups));
+  }
   auto launch = [&](auto kernel, int lds_bytes, FhipOncePerDevice &configured) {
     if (!configured.done(ctx->device)) {
       if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -900,6 +1037,8 @@ int fhip_fast_sdpa(fhip_ctx *ctx, const fhip_sdpa_desc *d, const void *q,
   // one flag per kernel instance: [head dim][type][plain / causal / mask in
   // registers / mask staged in LDS]
   static FhipOncePerDevice configured[2][2][4];
+  fhip_note_kernel(ctx, "sdpa_fwd d=%d causal=%d mask=%d", p.hd, (int)(d->is_causal != 0),
+                   p.mask ? (staged_mask ? 2 : 1) : 0);
   auto pick = [&](auto hd) {
     constexpr int HD = decltype(hd)::value;
     FhipOncePerDevice(&cfg)[2][4] = configured[HD == 128];

@@ -193,6 +193,14 @@ int fhip_tuning_reload(void);
 int fhip_ctx_create(int device_id, void *external_stream, fhip_ctx **out);
 int fhip_ctx_destroy(fhip_ctx *ctx);
 const char *fhip_last_error(fhip_ctx *ctx);
+/* Name of the kernel variant that the last operator call on this context
+ * launched, with its shape parameters (e.g. "conv_rf rows=7",
+ * "gemm_mfma 256x256 w8", "sdpa_fwd d=128 causal=1 mask=0"); "" before the
+ * first call.  The string lives in the context and is overwritten by the next
+ * call.  It has no counterpart in the reference, where one IREE dispatch list
+ * serves every shape: here several tuned kernels stand behind one operator,
+ * and tests and benchmarks assert that the one they mean to cover has run. */
+const char *fhip_last_kernel(fhip_ctx *ctx);
 void *fhip_ctx_stream(fhip_ctx *ctx);
 int fhip_ctx_device(fhip_ctx *ctx);
 

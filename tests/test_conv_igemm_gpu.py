@@ -255,6 +255,48 @@ def test_conv_split_reduction_vs_oracle(ctx, case, dtype, knobs):
     assert_close(out.logical(), ref, capi.FLOAT, f"{case}", rtol=1e-4)
 
 
+SPLIT_OPERAND_CASES = [
+    # 2-D, split reduction
+    dict(x=[2, 512, 7, 7], w=[128, 512, 3, 3], pad=[1, 1], s=[1, 1], d=[1, 1]),
+    # 3-D with a 1 x 1 filter in H and W (folded into 2-D) and a split reduction
+    dict(x=[2, 512, 4, 7, 7], w=[128, 512, 3, 1, 1], pad=[1, 0, 0], s=[1, 1, 1], d=[1, 1, 1]),
+    dict(x=[8, 512, 4, 7, 7], w=[512, 512, 3, 1, 1], pad=[1, 0, 0], s=[1, 1, 1], d=[1, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_OPERAND_CASES)
+@pytest.mark.parametrize("operand", ["bias", "residual", "bias_relu_residual"])
+def test_conv_split_reduction_fused_operands(ctx, case, operand, knobs):
+    """Fused operands on the split-reduction path, whose second kernel applies
+    them: a per-channel vector, a tensor of the output's shape (residual add,
+    addressed by pixel), and both around a ReLU; 2-D and folded 3-D problems.
+    Reference: pointwise nodes consuming the convolution's output
+    (reference samples/convolution/conv_fprop_with_relu_and_bias.cpp)."""
+    knobs(CONV_HALO="0")
+    dt = capi.BFLOAT16
+    x = cl(case["x"], 61, 0, dt)
+    w = cl(case["w"], 61, 1, dt, std=0.05)
+    yd = oracle.conv_output_dims(case["x"], case["w"], case["pad"], case["s"], case["d"])
+    bd = [1, case["w"][0]] + [1] * len(case["pad"])
+    bias = HT.from_logical(rand(61, 2, bd), dt, oracle.channels_last_strides(bd))
+    res = cl(yd, 61, 3, dt)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"], case["d"])
+    add = lambda t, i, rd=capi.FLOAT: capi.epilogue_op(capi.PW["ADD"], rd, operand_index=i,
+                                                       operand=t.desc())
+    if operand == "bias":
+        epi, tensors, ref = [add(bias, 0)], [bias], ref + bias.logical()
+    elif operand == "residual":
+        epi, tensors, ref = [add(res, 0)], [res], ref + res.logical()
+    else:
+        epi = [add(bias, 0), capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT), add(res, 1)]
+        tensors = [bias, res]
+        ref = np.maximum(ref + bias.logical(), 0.0) + res.logical()
+    out = run(ctx, x, w, case["pad"], case["s"], case["d"], capi.FLOAT, out_dtype=dt,
+              epilogue=epi, epi_tensors=tensors)
+    assert "split=" in ctx.last_kernel() and "split=1" not in ctx.last_kernel(), ctx.last_kernel()
+    assert_close(out.logical(), ref, dt, f"{operand} {case}")
+
+
 def test_conv_split_reduction_benchmark_shape(ctx):
     """N32 C512 7x7 -> K512, 3x3, padding 1, bf16 at full size (the
     benchmark's late-layer line): closed form on all-ones tensors for every
@@ -264,6 +306,8 @@ def test_conv_split_reduction_benchmark_shape(ctx):
     ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
     ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
     lg = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+    assert ctx.last_kernel().startswith("conv_igemm gather") and "split=8" in ctx.last_kernel(), \
+        ctx.last_kernel()
     taps = np.full(7, 3.0); taps[[0, -1]] = 2.0
     assert np.array_equal(lg, np.broadcast_to(512.0 * taps[:, None] * taps[None, :], lg.shape))
     x = cl(xd, 51, 0, capi.BFLOAT16)
@@ -314,12 +358,27 @@ def test_conv_igemm_headline_shape(ctx):
     w = cl(wd, 45, 1, capi.BFLOAT16, std=0.05)
     out = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16,
               epilogue=epi, epi_tensors=[bias])
+    # the kernel that the benchmark's headline convolution line times
+    assert ctx.last_kernel().startswith("conv_rf c=64 r=3 s=3"), ctx.last_kernel()
     lg = out.logical()
     xl = x.logical()
     for img in (0, 31):
         ref = oracle.conv_fprop(xl[img:img + 1], w.logical(), pad, st, dil)
         ref = np.maximum(ref + bias.logical(), 0.0)
         assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"image {img}")
+
+    # Every workgroup slot: the same random image in all 32 batch entries must
+    # give 32 bit-identical outputs, and image 0's has just been compared with
+    # the oracle's arithmetic on the same kernel.
+    xs = np.broadcast_to(rand(45, 3, [1] + xd[1:]), xd)
+    x = HT.from_logical(xs, capi.BFLOAT16, oracle.channels_last_strides(xd))
+    out = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16,
+              epilogue=epi, epi_tensors=[bias])
+    lg = out.logical()
+    ref = oracle.conv_fprop(x.logical()[:1], w.logical(), pad, st, dil)
+    assert_close(lg[:1], np.maximum(ref + bias.logical(), 0.0), capi.BFLOAT16, "shared image")
+    for img in range(1, 32):
+        assert np.array_equal(lg[img], lg[0]), f"image {img} differs from image 0"
 
 
 @pytest.mark.parametrize("shape", ["groups4", "depthwise"])

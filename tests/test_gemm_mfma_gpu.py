@@ -190,6 +190,9 @@ def _full_size_rows_check(ctx, dtype):
     b = make_operand(5 if dtype == capi.INT8 else 6, 1, k, n, dtype, False)
     cdt = capi.INT32 if dtype == capi.INT8 else capi.FLOAT
     out = run(ctx, a, b, cdt).logical()
+    # one 256 x 256 tile per compute unit on eight wavefronts
+    kind = "i8" if dtype == capi.INT8 else "fp8e4m3"
+    assert ctx.last_kernel() == f"gemm_mfma {kind} 256x256 waves=8 split=1", ctx.last_kernel()
     rows = np.array([0, 1, 31, 32, 255, 256, 1023, 2048, 2049, 3071, 4064, 4095])
     al, bl = a.logical(), b.logical()
     if dtype == capi.INT8:

@@ -36,6 +36,9 @@ def test_matmul_config1_f32(ctx):
     b = HT.from_logical(rand(1, 1, [1, 512, 256], "uniform"), capi.FLOAT)
     out = run_matmul(ctx, a, b, capi.FLOAT)
     assert_close(out.logical(), oracle.matmul(a.logical(), b.logical()), capi.FLOAT)
+    # 16 tiles of 64 x 64: the f32 matrix-instruction kernel that splits K
+    # over the wavefronts of a 32 x 32 tile
+    assert ctx.last_kernel() == "matmul_f32_splitk", ctx.last_kernel()
 
 
 @pytest.mark.parametrize("transpose_b", [False, True])

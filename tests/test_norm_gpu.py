@@ -266,6 +266,9 @@ def test_rmsnorm_config2_full_size_all_rows(ctx):
                    expect_path=2)
     ref = oracle.rmsnorm(x.logical(), s.logical(), 1e-6) * 0.5
     assert_close(out.logical(), ref, capi.BFLOAT16, "config 2 full size")
+    # rows held in registers, the variant with the scalar multiply compiled in
+    assert ctx.last_kernel().startswith("rownorm chunks="), ctx.last_kernel()
+    assert ctx.last_kernel().endswith("variant=2"), ctx.last_kernel()
 
 
 def test_rmsnorm_config2_full_size_full_operand_mul(ctx):

@@ -214,6 +214,20 @@ def test_flash_headline_shape(ctx):
         assert_close(out[b:b + 1, h:h + 1], ref, capi.BFLOAT16, f"b{b} h{h}")
     ref = np.cumsum(vl[2, 7], axis=0) / np.arange(1, S + 1)[:, None]
     assert_close(out[2, 7], ref, capi.BFLOAT16, "uniform head")
+    assert ctx.last_kernel() == "sdpa_fwd d=128 causal=1 mask=0", ctx.last_kernel()
+
+    # Every workgroup slot: the same random head in all 128 (batch, head)
+    # entries must give 128 bit-identical outputs; entry (0, 0) is compared
+    # with the oracle.
+    one = lambda tid: np.broadcast_to(rand(57, tid, [1, 1, S, D]), [B, H, S, D])
+    q, k, v = (HT.from_logical(one(i), capi.BFLOAT16) for i in range(3))
+    out = run(ctx, q, k, v, causal=True).logical()
+    ref = oracle.sdpa(q.logical()[:1, :1], k.logical()[:1, :1], v.logical()[:1, :1],
+                      is_causal=True)
+    assert_close(out[:1, :1], ref, capi.BFLOAT16, "shared head")
+    for b in range(B):
+        for h in range(H):
+            assert np.array_equal(out[b, h], out[0, 0]), f"b{b} h{h} differs from b0 h0"
 
 
 def test_flash_benchmark_lines_mask_and_head_dim_64(ctx):
