@@ -612,7 +612,10 @@ bool fhip_fast_conv_dgrad_rf_applicable(const fhip_conv_desc *d) {
 
 int fhip_fast_conv_dgrad_rf(fhip_ctx *ctx, const fhip_conv_desc *d,
                             const void *dy, const void *w, void *dx) {
-  RdPlan p = make_rd_plan(d, ctx->num_cus);
+  // planned for 256 compute units, like the applicability query that the
+  // caller went by: on a device or partition of another size the tile choice
+  // must not flip between the two (the grid runs anywhere)
+  RdPlan p = make_rd_plan(d, 256);
   FHIP_REQUIRE(ctx, p.ok,
                "conv: descriptor not supported by the register-filter data gradient");
   FHIP_REQUIRE(ctx, ((uintptr_t)dy & 15) == 0 && ((uintptr_t)w & 15) == 0 &&

@@ -153,18 +153,22 @@ private:
   bool remove_ = false;
 };
 
-// The files of one compiled graph (reference support/cache.h:272-300).
+// The files of one compiled graph (reference support/cache.h:303-335).
 struct CachedAssets {
-  CacheFile input;   // description of the planned graph
-  CacheFile output;  // the artifact
-  CacheFile command; // planner key (backend, plan format)
+  CacheFile input;      // description of the planned graph
+  CacheFile output;     // the artifact
+  CacheFile command;    // planner key (backend, plan format)
+  CacheFile statistics; // JSON: dispatch count and workspace bytes of the plan
+                        // (the reference keeps iree-compile's statistics here)
 };
 
-enum class CachedAssetsType { Input, Output, Command };
+// (reference support/cache.h:306-312)
+enum class CachedAssetsType { Input, Output, Command, Statistics };
 
 inline constexpr const char *kCacheInputFileName = "fusilli_plan_input.txt";
 inline constexpr const char *kCacheOutputFileName = "fusilli_plan_output.bin";
 inline constexpr const char *kCacheCommandFileName = "fusilli_plan_command.txt";
+inline constexpr const char *kCacheStatisticsFileName = "fusilli_plan_statistics.json";
 
 } // namespace fusilli
 

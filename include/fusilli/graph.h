@@ -163,11 +163,15 @@ public:
     FUSILLI_ASSIGN_OR_RETURN(
         CacheFile command,
         CacheFile::create(getName(), kCacheCommandFileName, remove));
+    FUSILLI_ASSIGN_OR_RETURN(
+        CacheFile statistics,
+        CacheFile::create(getName(), kCacheStatisticsFileName, remove));
     FUSILLI_CHECK_ERROR(input.write(generatedAsm));
     FUSILLI_CHECK_ERROR(output.write(bytes));
     FUSILLI_CHECK_ERROR(command.write(plannerKey(backend)));
+    FUSILLI_CHECK_ERROR(statistics.write(planStatistics(p)));
     cache_.emplace(CachedAssets{std::move(input), std::move(output),
-                                std::move(command)});
+                                std::move(command), std::move(statistics)});
     if (reCompiled)
       *reCompiled = true;
     return ok(cache_->output.path);
@@ -182,9 +186,24 @@ public:
       return cache_->input.read();
     case CachedAssetsType::Output:
       return cache_->output.read();
-    default:
+    case CachedAssetsType::Command:
       return cache_->command.read();
+    case CachedAssetsType::Statistics:
+      return cache_->statistics.read();
     }
+    return error(ErrorCode::InvalidAttribute, "Unknown CachedAssetsType");
+  }
+
+  // What the statistics file holds: the plan's dispatch count (one per fused
+  // step; the figure the reference reads out of iree-compile's statistics
+  // JSON, graph/graph.h:449-468 and benchmarks/driver.cpp) and its workspace.
+  static std::string planStatistics(const plan::Plan &p) {
+    std::ostringstream os;
+    os << "{\n  \"dispatch-count\": " << p.steps.size()
+       << ",\n  \"workspace-bytes\": " << p.workspaceBytes
+       << ",\n  \"plan-signature\": \"0x" << std::hex << p.signature << std::dec
+       << "\"\n}\n";
+    return os.str();
   }
 
   // Loads a plan produced by this or an identically built graph.  Replaces
@@ -245,7 +264,9 @@ public:
       return ok(false);
     if (cache_->input.path != CacheFile::getPath(getName(), kCacheInputFileName) ||
         cache_->output.path != CacheFile::getPath(getName(), kCacheOutputFileName) ||
-        cache_->command.path != CacheFile::getPath(getName(), kCacheCommandFileName))
+        cache_->command.path != CacheFile::getPath(getName(), kCacheCommandFileName) ||
+        cache_->statistics.path !=
+            CacheFile::getPath(getName(), kCacheStatisticsFileName))
       return ok(false);
     FUSILLI_ASSIGN_OR_RETURN(CacheFile input,
                              CacheFile::open(getName(), kCacheInputFileName));
@@ -253,7 +274,10 @@ public:
                              CacheFile::open(getName(), kCacheOutputFileName));
     FUSILLI_ASSIGN_OR_RETURN(CacheFile command,
                              CacheFile::open(getName(), kCacheCommandFileName));
+    FUSILLI_ASSIGN_OR_RETURN(CacheFile statistics,
+                             CacheFile::open(getName(), kCacheStatisticsFileName));
     (void)output;
+    (void)statistics;
     FUSILLI_ASSIGN_OR_RETURN(std::string inputContents, input.read());
     if (inputContents != generatedAsm)
       return ok(false);

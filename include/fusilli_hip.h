@@ -289,9 +289,14 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
  * loops, harnesses that forbid hipMalloc).  The mirrored filter (and DY's zero
  * grid for strides above one) live in a per-device static array of
  * FHIP_CONV_DGRAD_STATIC_MAX_BYTES inside the library; descriptors whose
- * fhip_conv_dgrad_workspace_size exceeds that fail with a message.  Same
- * kernels and results as fhip_conv_dgrad.  All calls on one GPU share the
- * array: calls that overlap on one GPU (two streams, two contexts) race. */
+ * fhip_conv_dgrad_workspace_size exceeds that fail with a message.  It plans
+ * without the context's growable scratch: descriptors that fhip_conv_dgrad
+ * runs on zero-padded channel copies or with a split reduction take the
+ * direct (slower) kernels here, and their results may differ from
+ * fhip_conv_dgrad's in the last bit (another summation order); every other
+ * descriptor runs the same kernel with bit-identical results.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams, two
+ * contexts) race. */
 #define FHIP_CONV_DGRAD_STATIC_MAX_BYTES (8u << 20)
 int fhip_conv_dgrad_static(fhip_ctx *ctx, const fhip_conv_desc *d,
                            const void *dy, const void *w, void *dx);

@@ -1081,6 +1081,13 @@ TEST("cache: files, RAII removal, hit and miss") {
   CHECK(cmd.find("--backend=CPU") != std::string::npos);
   REQUIRE_ASSIGN(std::string in, g.readCompilationCacheFile(CachedAssetsType::Input));
   CHECK(in == text + " ");
+  // the statistics asset (reference graph/graph.h:449-468): one dispatch for
+  // conv + bias + relu, as Graph::getKernelCount reports after compile()
+  REQUIRE_ASSIGN(std::string stats, g.readCompilationCacheFile(CachedAssetsType::Statistics));
+  CHECK(stats.find("\"dispatch-count\": 1") != std::string::npos);
+  CHECK(stats.find("\"workspace-bytes\": 0") != std::string::npos);
+  CHECK_ERROR(g.readCompilationCacheFile(static_cast<CachedAssetsType>(99)),
+              ErrorCode::InvalidAttribute, "Unknown CachedAssetsType");
   // a deleted file is a miss, not an error of the second kind
   fs::remove(artifact);
   CHECK(isError(g.getCompiledArtifact(Backend::CPU, text + " ", true, &re)));
@@ -1103,6 +1110,7 @@ TEST("cache: files, RAII removal, hit and miss") {
     CHECK(fs::exists(compiled_dir / kCacheOutputFileName));
     CHECK(fs::exists(compiled_dir / kCacheInputFileName));
     CHECK(fs::exists(compiled_dir / kCacheCommandFileName));
+    CHECK(fs::exists(compiled_dir / kCacheStatisticsFileName));
     // the artifact in the cache is what compileToArtifact returns
     REQUIRE_ASSIGN(auto bytes, tmp.graph->compileToArtifact(Backend::CPU, true));
     REQUIRE_ASSIGN(CacheFile f, CacheFile::open("cache_compile", kCacheOutputFileName));

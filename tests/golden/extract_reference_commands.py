@@ -1,11 +1,11 @@
-"""Writes reference_commands.txt: the argument lists of every
+"""Writes fusilli_amd/bench/reference_commands.txt: the argument lists of every
 add_fusilli_benchmark(...) entry of the reference's benchmarks/CMakeLists.txt
 (:49-392), one command per line in the format of test_commands.txt.  Entries
 the reference has commented out (it disables them for a compiler issue of its
 own backend) are kept and marked in their comment line.  Run once in the
 container that holds the reference; the output is committed data.
 
-    python fusilli_amd/bench/extract_reference_commands.py [/root/reference]
+    python tests/golden/extract_reference_commands.py [/root/reference]
 """
 import os
 import re
@@ -31,8 +31,8 @@ def main():
         out.append("")
         out.append(f"# {name}" + ("  (disabled in the reference)" if m.group("c") else ""))
         out.append(args)
-    here = os.path.dirname(os.path.abspath(__file__))
-    with open(os.path.join(here, "reference_commands.txt"), "w") as f:
+    root = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    with open(os.path.join(root, "fusilli_amd", "bench", "reference_commands.txt"), "w") as f:
         f.write("\n".join(out) + "\n")
     print(f"{(len(out) - 1) // 3} commands")
 

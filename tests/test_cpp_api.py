@@ -34,6 +34,13 @@ def test_cpp_host_api():
     assert "19 cases" in out or "cases, 0 failed" in out
 
 
+def test_cpp_node_validation():
+    """The reference's node / attribute validation expectations (codes, exact
+    messages, order of checks): tests/cpp/test_node_validation.cpp."""
+    out = _run("test_node_validation", 120)
+    assert "cases, 0 failed" in out
+
+
 @pytest.mark.gpu
 def test_cpp_device_api():
     _run("test_device_api", 300)
