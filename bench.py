@@ -37,6 +37,71 @@ HBM_PEAK_GBS = 8000.0
 RMSNORM_TRAFFIC_BYTES = (65608 + 65536) * 1024
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}
 
+# HBM bytes per launch of the dominant kernel of a line (FETCH_SIZE + WRITE_SIZE
+# of rocprofv3 --pmc runs of this script, each scaled by what the same counter
+# reads for `--calibrate-copy`), with the summary under profiles/ that records
+# the run.  Counters cannot be read from inside this process: these are the
+# figures of the recorded runs, not of this one.
+TRAFFIC = {
+    "conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu":
+        (int((8486.5 * 1.9985 + 25088) * 1024),
+         "profiles/conv_rf_dgrad_wgrad_direct_bf16_n32c64h56w56_k128r3s3.md"),
+    "sdpa_fwd_bf16_causal_b4h32s2048d128":
+        (436_000_000 + 64 * 1024 * 1024, "profiles/sdpa_fwd_bf16_causal_b4h32s2048d128.md"),
+    "matmul_int8_4096x8192x4096_i32":
+        (201_000_000 + 64 * 1024 * 1024, "profiles/gemm_mfma_4096x8192x4096_int8_fp8_bf16.md"),
+    "matmul_fp8e4m3_4096x8192x4096_scaled_bf16_out":
+        (201_000_000 + 32 * 1024 * 1024, "profiles/gemm_mfma_4096x8192x4096_int8_fp8_bf16.md"),
+}
+
+# The benchmark's configurations: line of `others` (None: the headline), the
+# north-star target for its roofline fraction (None: plumbing case without a
+# target), the kernel variant that must have run (prefix of fhip_last_kernel),
+# and the driver command that times the same problem through Graph::execute.
+CONFIGS = {
+    "C1": ("matmul_f32_1x256x512x256", None, "matmul_f32_splitk",
+           "matmul -M 256 -N 256 -K 512 --a_type f32 --b_type f32 --out_type f32"),
+    "C2": (None, 0.70, "rownorm chunks=",
+           "rmsnorm -X 8192x4096 -t bf16 -e 1e-6 --mul 0.5"),
+    "C3": ("conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu", 0.60, "conv_rf c=64 r=3 s=3",
+           "conv -F 1 -n 32 -c 64 -H 56 -W 56 -k 128 -y 3 -x 3 -p 1 -q 1 -u 1 -v 1 -l 1 -j 1 "
+           "--in_layout NHWC --out_layout NHWC --fil_layout NHWC --spatial_dim 2 --bf16 --bias --relu"),
+    "C4": ("sdpa_fwd_bf16_causal_b4h32s2048d128", 0.60, "sdpa_fwd d=128 causal=1 mask=0",
+           "sdpa -B 4 --heads_q 32 --heads_kv 32 --seq_q 2048 --seq_kv 2048 -d 128 -t bf16 --causal"),
+    "C5a": ("matmul_int8_4096x8192x4096_i32", 0.60, "gemm_mfma i8 256x256 waves=8 split=1",
+            "matmul -M 4096 -N 4096 -K 8192 --a_type i8 --b_type i8 --out_type i32"),
+    "C5b": ("matmul_fp8e4m3_4096x8192x4096_scaled_bf16_out", 0.60,
+            "gemm_mfma fp8e4m3 256x256 waves=8 split=1",
+            "matmul -M 4096 -N 4096 -K 8192 --a_type fp8 --b_type fp8 --out_type bf16 "
+            "--out_scale 0.0000049824617"),
+}
+FLOOR_FILE = os.path.join(ROOT, "bench_floor.json")
+DRIVER = os.path.join(ROOT, "fusilli_amd", "bench", "bin", "driver")
+
+
+def graph_api_us(command, iters=200):
+    """Average time of one Graph::execute of `command`'s graph (HIP events
+    around --iter back-to-back executes inside the benchmark driver, a child
+    process: variant-pack lookup, plan and argument set-up included), or None
+    when the driver binary is not built."""
+    import shlex
+    import subprocess
+    if not os.path.exists(DRIVER):
+        return None
+    try:
+        # (--fill random: constant operands toggle fewer bits and let the MFMA
+        # kernels clock higher than real data does)
+        proc = subprocess.run([DRIVER, "--iter", str(iters), "--warmup", "50", "--fill", "random"]
+                              + shlex.split(command),
+                              capture_output=True, text=True, timeout=120)
+        if proc.returncode != 0:
+            return None
+        lines = proc.stdout.strip().splitlines()
+        rec = dict(zip(lines[-2].split(","), lines[-1].split(",")))
+        return round(float(rec["avg_us"]), 2)
+    except Exception:  # a missing figure, not a failed benchmark
+        return None
+
 
 # The secondary workloads warm up for at least this long (the GPU's clocks take
 # tens of milliseconds of load to settle: a short MFMA kernel timed right after
@@ -198,8 +263,8 @@ def bench_matmul_f32_c1(ctx, steps, warmup):
     return {"value": round(flop / ev_ms / 1e9, 3), "unit": "TFLOP/s",
             "frac_of_mfma_peak": round(flop / ev_ms / 1e9 / 157.3, 5),
             "kernel_us": round(ev_ms * 1e3, 2), "work": flop,
-            "kernel": "stride-generic f32 MFMA tiles (fhip_matmul_supported == %d)"
-                      % ctx.lib.fhip_matmul_supported(d)}
+            "kernel_note": "stride-generic f32 MFMA tiles (fhip_matmul_supported == %d)"
+                           % ctx.lib.fhip_matmul_supported(d)}
 
 
 def bench_conv(ctx, steps, warmup):
@@ -702,6 +767,10 @@ def main():
     ap.add_argument("--only", default="",
                     help="comma-separated substrings: run only the matching "
                          "lines of `others` (tuning runs; skips the CPU baseline)")
+    ap.add_argument("--write-floors", type=float, default=0.0, metavar="FRACTION",
+                    help="after the run, write bench_floor.json: FRACTION x this "
+                         "run's roofline fraction per line (later runs list the "
+                         "lines that fall below their floor under `regressions`)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain copy kernel of known size (counter "
                          "calibration) and print its figures")
@@ -718,6 +787,7 @@ def main():
         ctx.close()
         return
     r = bench_rmsnorm(ctx, args.steps, args.warmup, "scalar")
+    headline_kernel = ctx.last_kernel()
     line = {
         "metric": "GB/s (norms) on 1 MI355X, % roofline",
         "value": round(r["gbs_wall"], 1),
@@ -754,6 +824,11 @@ def main():
         def other(name, result):
             result["warmup_launches"] = LAST_WARMUP
             result["roofline"] = roofline_of(result)
+            # (the variant of the line's last call: a line of two kernels names
+            # the second)
+            result.setdefault("kernel", ctx.last_kernel())
+            if name in TRAFFIC:
+                result["roofline"]["traffic"], result["roofline"]["traffic_source"] = TRAFFIC[name]
             others[name] = result
 
         def rms_full():
@@ -814,6 +889,44 @@ def main():
                 continue
             other(name, fn())
         line["others"] = others
+        # ---- the configurations side by side, and the floors --------------------
+        if not wanted:
+            configs = {}
+            for cfg, (name, target, variant, command) in CONFIGS.items():
+                if name is None:
+                    frac, us, kernel = line["roofline"]["frac"], line["roofline"]["kernel_us"], headline_kernel
+                else:
+                    res = others[name]
+                    frac, us, kernel = res["roofline"]["frac"], res["roofline"]["kernel_us"], res["kernel"]
+                configs[cfg] = {"line": name or "headline", "frac": frac, "target": target,
+                                "met": None if target is None else bool(frac >= target),
+                                "kernel_us": us, "kernel": kernel,
+                                "expected_kernel": bool(kernel.startswith(variant)),
+                                "graph_api_us": graph_api_us(command)}
+            line["configs"] = configs
+            floors = json.load(open(FLOOR_FILE)) if os.path.exists(FLOOR_FILE) else {}
+            regressions = []
+            for name, floor in floors.items():
+                if name == "headline":
+                    frac = line["roofline"]["frac"]
+                elif name in others:
+                    frac = others[name]["roofline"]["frac"]
+                else:
+                    continue
+                if frac < floor:
+                    regressions.append({"line": name, "frac": frac, "floor": floor})
+            for cfg, c in configs.items():
+                if not c["expected_kernel"]:
+                    regressions.append({"line": cfg, "kernel": c["kernel"],
+                                        "expected": CONFIGS[cfg][2]})
+            line["regressions"] = regressions
+            if args.write_floors > 0:
+                new = {"headline": round(line["roofline"]["frac"] * args.write_floors, 4)}
+                for name, res in others.items():
+                    new[name] = round(res["roofline"]["frac"] * args.write_floors, 4)
+                with open(FLOOR_FILE, "w") as f:
+                    json.dump(new, f, indent=1, sort_keys=True)
+                    f.write("\n")
     if not args.no_cpu_baseline and not args.only:
         line["cpu_baseline"] = cpu_baseline_rmsnorm()
         if not args.no_others:

@@ -11,9 +11,11 @@
 // for conv, int8 / fp8 matmul types, `--out_scale s` (matmul output x scalar).
 #include <fusilli.h>
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <map>
 #include <optional>
 #include <set>
@@ -136,13 +138,64 @@ TensorAttr mk(const std::string &name, const Dims &dim, const Dims &stride,
   return TensorAttr().setName(name).setDim(dim).setStride(stride).setDataType(dt);
 }
 
-// constant-filled device buffer shaped like the tensor's physical dims
+bool g_random = false; // --fill random: pseudo-random inputs instead of constants
+
+// Values of a random fill: a 64-bit mix of the element index (splitmix64),
+// uniform in [-1, 1) (integers: -127 .. 127).
+struct RandomFill {
+  uint64_t seed;
+  double operator()(size_t i) const {
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (uint64_t)(i + 1);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (double)(z >> 11) * (1.0 / 9007199254740992.0) * 2.0 - 1.0;
+  }
+};
+
+// device buffer shaped like the tensor's physical dims, filled with the
+// constant `v` (the reference driver's fills), or with pseudo-random values
+// under --fill random (outputs, v == 0, stay zero)
 std::shared_ptr<Buffer> constant(const Handle &h, const TensorPtr &t, float v) {
   std::vector<size_t> shape;
   size_t n = 1;
   for (int64_t d : t->getPhysicalDim()) {
     shape.push_back((size_t)d);
     n *= (size_t)d;
+  }
+  if (g_random && v != 0.f) {
+    static uint64_t tensors = 0;
+    const RandomFill rnd{0x5eed0000ull + 977 * ++tensors};
+    auto wrapr = [&](auto e) {
+      if (isError(e))
+        die("allocate " + t->getName() + ": " + ErrorObject(e).getMessage());
+      return std::make_shared<Buffer>(std::move(*e));
+    };
+    auto fill = [&](auto tag, double scale) {
+      using T = decltype(tag);
+      std::vector<T> data(n);
+      for (size_t i = 0; i < n; ++i)
+        data[i] = (T)(float)(rnd(i) * scale);
+      return wrapr(Buffer::allocate(h, shape, data));
+    };
+    switch (t->getDataType()) {
+    case DataType::Float:
+      return fill(float{}, 1.0);
+    case DataType::Half:
+      return fill(half{}, 1.0);
+    case DataType::BFloat16:
+      return fill(bf16{}, 1.0);
+    case DataType::Int8:
+      return fill(int8_t{}, 127.0);
+    case DataType::FP8E4M3: {
+      std::vector<fp8e4m3> data(n);
+      for (size_t i = 0; i < n; ++i) // any finite bit pattern: sign, exponent < 15, mantissa
+        data[i] = fp8e4m3{(uint8_t)((uint64_t)((rnd(i) + 1.0) * 63.0) | (rnd(i + n) < 0 ? 0x80 : 0))};
+      return wrapr(Buffer::allocate(h, shape, data));
+    }
+    default:
+      break; // other types keep their constant
+    }
   }
   auto wrap = [&](auto e) {
     if (isError(e))
@@ -183,13 +236,110 @@ struct LazyHandle {
   }
 };
 
+// One output to check after the timed loop (--verify): the tensor, and the
+// value every element must have as a function of its logical coordinates.
+// With the constant fills of the inputs every answer here is a closed form
+// (the reference's samples check the same ones: convolution = taps inside the
+// image x channels of a group, matmul = K, attention over constant tensors = V,
+// samples/sdpa_utils.cpp:49-102, tests/test_graph.cpp:198-223).
+struct Expect {
+  TensorPtr tensor;
+  std::function<double(const Dims &)> value;
+  double rtol = 0; // 0: by the tensor's type (1e-4 f32, 2e-2 16-bit / fp8, 0 integers)
+  double atol = 0;
+};
+
 struct Run {
   std::string name;
   double work = 0; // FLOP or bytes
   const char *unit = "TFLOP/s";
+  std::vector<Expect> expect;
 };
 
 int g_warmup = 3; // untimed executes before the --iter loop (--warmup)
+bool g_verify = false; // --verify: compare the outputs with their closed forms
+
+// The buffer's elements as doubles, in storage order.
+std::vector<double> readAsDouble(const Handle &h, Buffer &b, DataType dt) {
+  std::vector<double> out;
+  auto pull = [&](auto tag) {
+    using T = decltype(tag);
+    std::vector<T> v;
+    OK(b.read(h, v));
+    out.reserve(v.size());
+    for (const T &x : v)
+      out.push_back((double)(float)x);
+  };
+  switch (dt) {
+  case DataType::Float:
+    pull(float{});
+    break;
+  case DataType::Half:
+    pull(half{});
+    break;
+  case DataType::BFloat16:
+    pull(bf16{});
+    break;
+  case DataType::Int32:
+    pull(int32_t{});
+    break;
+  case DataType::Int8:
+    pull(int8_t{});
+    break;
+  default:
+    die("--verify: no reader for this output type");
+  }
+  return out;
+}
+
+// Compares every element of the expectation's tensor; prints the verdict line
+// `verify,<tensor>,<elements>,<mismatches>,<max abs error>` and fails the run
+// on a mismatch.
+void verifyOutputs(const Handle &h, Pack &pack, const Run &r) {
+  for (const Expect &e : r.expect) {
+    const TensorPtr &t = e.tensor;
+    const DataType dt = t->getDataType();
+    const std::vector<double> got = readAsDouble(h, *pack.at(t), dt);
+    const Dims &dim = t->getDim(), &st = t->getStride();
+    double rtol = e.rtol;
+    if (rtol == 0)
+      rtol = dt == DataType::Float ? 1e-4 : (dt == DataType::Int32 || dt == DataType::Int8) ? 0 : 2e-2;
+    Dims c(dim.size(), 0);
+    size_t bad = 0, n = 0;
+    double worst = 0;
+    for (;;) {
+      int64_t off = 0;
+      for (size_t i = 0; i < dim.size(); ++i)
+        off += c[i] * st[i];
+      const double want = e.value(c), have = got.at((size_t)off);
+      const double err = std::fabs(have - want);
+      if (!(err <= rtol * std::fabs(want) + e.atol)) {
+        if (bad < 5) {
+          std::string at;
+          for (int64_t x : c)
+            at += (at.empty() ? "" : ",") + std::to_string(x);
+          std::fprintf(stderr, "verify: %s[%s] = %.6g, expected %.6g\n", t->getName().c_str(),
+                       at.c_str(), have, want);
+        }
+        ++bad;
+      }
+      worst = err > worst ? err : worst;
+      ++n;
+      int i = (int)dim.size() - 1;
+      for (; i >= 0; --i) {
+        if (++c[i] < dim[i])
+          break;
+        c[i] = 0;
+      }
+      if (i < 0)
+        break;
+    }
+    std::printf("verify,%s,%zu,%zu,%.6g\n", t->getName().c_str(), n, bad, worst);
+    if (bad)
+      die("--verify: " + std::to_string(bad) + " of " + std::to_string(n) + " elements of " +
+          t->getName() + " differ from the closed form");
+  }
+}
 
 void timeGraph(const Handle &h, Graph &g, Pack &pack, const Run &r, int iter) {
   OK(g.validate());
@@ -222,6 +372,8 @@ void timeGraph(const Handle &h, Graph &g, Pack &pack, const Run &r, int iter) {
   std::printf("name,iter,dispatch_count,avg_us,work,%s\n", r.unit);
   std::printf("%s,%d,%zu,%.3f,%.0f,%.3f\n", r.name.c_str(), iter, kernels, us,
               r.work, r.work / us / 1e6);
+  if (g_verify)
+    verifyOutputs(h, pack, r);
 }
 
 // Strides of `dims` under a layout name of the reference's list
@@ -339,6 +491,42 @@ void runConv(LazyHandle &lh, const Args &a, int iter) {
     if (DB)
       pack[DB] = constant(h, DB, 0.f);
     Run r{mode == 2 ? "conv_dgrad" : "conv_wgrad", flop};
+    // all-ones DY and W / X: every gradient element counts the (tap, output)
+    // pairs that touch it, per spatial dim, times the channels summed over
+    const size_t sp = (size_t)sdim;
+    if (mode == 2) {
+      // DX[n, c, i..] = (K / groups) x prod_dims #{(f, o): i + pad - f dil = o stride, 0 <= o < P}
+      r.expect.push_back({OUT, [=](const Dims &at) {
+        double v = (double)(k / gcount);
+        for (size_t d = 0; d < sp; ++d) {
+          int cnt = 0;
+          for (int64_t f = 0; f < wd[2 + d]; ++f) {
+            const int64_t num = at[2 + d] + cp[d] - f * cd[d];
+            if (num >= 0 && num % cs[d] == 0 && num / cs[d] < yd[2 + d])
+              ++cnt;
+          }
+          v *= cnt;
+        }
+        return v;
+      }});
+    } else {
+      // DW[k, c, f..] = N x prod_dims #{o: 0 <= o stride - pad + f dil < H}
+      r.expect.push_back({OUT, [=](const Dims &at) {
+        double v = (double)n;
+        for (size_t d = 0; d < sp; ++d) {
+          int cnt = 0;
+          for (int64_t o2 = 0; o2 < yd[2 + d]; ++o2) {
+            const int64_t in = o2 * cs[d] - cp[d] + at[2 + d] * cd[d];
+            if (in >= 0 && in < xd[2 + d])
+              ++cnt;
+          }
+          v *= cnt;
+        }
+        return v;
+      }});
+    }
+    if (DB) // the bias gradient sums DY over batch and space
+      r.expect.push_back({DB, [=](const Dims &) { return (double)n * opix; }});
     timeGraph(h, g, pack, r, iter);
     return;
   }
@@ -380,6 +568,25 @@ void runConv(LazyHandle &lh, const Args &a, int iter) {
     pack[B] = constant(h, B, 1.f);
   pack[Y] = constant(h, Y, 0.f);
   Run r{"conv_fprop", flop};
+  {
+    // all-ones X, W and bias: Y = (filter taps inside the image) x (channels of
+    // a group) (+ 1) (x the scalar); ReLU leaves the positive values alone
+    const size_t sp = (size_t)sdim;
+    const double add = bias ? 1.0 : 0.0, scale = mul ? (double)mulBy : 1.0;
+    r.expect.push_back({Y, [=](const Dims &at) {
+      double v = (double)fc;
+      for (size_t d = 0; d < sp; ++d) {
+        int cnt = 0;
+        for (int64_t f = 0; f < wd[2 + d]; ++f) {
+          const int64_t in = at[2 + d] * cs[d] - cp[d] + f * cd[d];
+          if (in >= 0 && in < xd[2 + d])
+            ++cnt;
+        }
+        v *= cnt;
+      }
+      return (v + add) * scale;
+    }});
+  }
   timeGraph(h, g, pack, r, iter);
 }
 
@@ -431,6 +638,11 @@ void runMatmul(LazyHandle &lh, const Args &a, int iter) {
   if (bias)
     pack[bias] = constant(h, bias, 1.f);
   Run r{"matmul", 2.0 * Bt * M * N * K};
+  {
+    // all-ones operands (and bias): C = K (+ 1) (x the scalar)
+    const double want = ((double)K + (withBias ? 1.0 : 0.0)) * (outScale ? (double)outScaleBy : 1.0);
+    r.expect.push_back({C, [=](const Dims &) { return want; }});
+  }
   timeGraph(h, g, pack, r, iter);
 }
 
@@ -481,6 +693,10 @@ void runSdpa(LazyHandle &lh, const Args &a, int iter) {
   if (Mk)
     pack[Mk] = constant(h, Mk, -1.f);
   Run r{"sdpa", 4.0 * B * Hq * Sq * Skv * D * (causal ? 0.5 : 1.0)};
+  // constant Q, K, V (and mask): every softmax is uniform over its live keys
+  // and the output equals V's constant (reference samples/sdpa_utils.cpp:49-102,
+  // tolerance 1e-2 there); dropout is not applied by the inference graph
+  r.expect.push_back({O, [](const Dims &) { return 0.01; }, 1e-2, 1e-4});
   timeGraph(h, g, pack, r, iter);
 }
 
@@ -587,6 +803,22 @@ void runNorm(LazyHandle &lh, const Args &a, int iter, bool layer) {
     n *= (double)d;
   const double es = dt == DataType::Float ? 4 : 2;
   Run r{layer ? "layernorm" : "rmsnorm", 2.0 * n * es, "TB/s"};
+  {
+    // constant X = 1, scale = 2, bias = 0.5.  LayerNorm: x - mean = 0, so Y is
+    // the bias (0 without the affine pair), mean = 1 and 1/sqrt(0 + eps);
+    // RMSNorm: Y = scale / sqrt(1 + eps) (x the scalar)
+    const double scale = fuseMul ? (double)mulBy : 1.0;
+    if (layer) {
+      const double yv = (affine ? 0.5 : 0.0) * scale;
+      r.expect.push_back({Y, [=](const Dims &) { return yv; }, 0, 1e-3});
+      r.expect.push_back({Mean, [](const Dims &) { return 1.0; }});
+      const double rs = 1.0 / std::sqrt((double)epsv);
+      r.expect.push_back({Rstd, [=](const Dims &) { return rs; }});
+    } else {
+      const double yv = (affine ? 2.0 : 1.0) / std::sqrt(1.0 + (double)epsv) * scale;
+      r.expect.push_back({Y, [=](const Dims &) { return yv; }});
+    }
+  }
   timeGraph(h, g, pack, r, iter);
 }
 
@@ -602,13 +834,23 @@ int main(int argc, char **argv) {
       device = std::atoi(argv[++i]);
     else if (k == "--warmup" && i + 1 < argc)
       g_warmup = std::atoi(argv[++i]);
+    else if (k == "--verify")
+      g_verify = true;
+    else if (k == "--fill" && i + 1 < argc) {
+      const std::string f = argv[++i];
+      if (f != "random" && f != "constant")
+        die("--fill takes `constant` (the default) or `random`");
+      g_random = f == "random";
+    }
     else if (k == "--dump" || k == "-d")
       ; // nothing to dump: there is no intermediate IR
     else
       break;
   }
   if (i >= argc)
-    die("usage: driver [--device N] [--iter N] [--warmup N] <conv|matmul|sdpa|layernorm|rmsnorm> flags...");
+    die("usage: driver [--device N] [--iter N] [--warmup N] [--verify] [--fill constant|random] <conv|matmul|sdpa|layernorm|rmsnorm> flags...");
+  if (g_verify && g_random)
+    die("--verify checks the closed forms of the constant fills: it excludes --fill random");
   const std::string cmd = argv[i];
   const Args a = parse(argc, argv, i + 1);
   LazyHandle h;

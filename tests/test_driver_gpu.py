@@ -27,18 +27,32 @@ def commands(path=COMMANDS):
     return out
 
 
+def run_verified(cmd):
+    """Runs one driver command with --verify: besides timing, the driver then
+    compares every element of every output with the closed form its constant
+    fills imply (convolution: taps inside the image x channels of a group;
+    matmul: K; attention over constant tensors: V; the norms' constant-row
+    answers) and fails on a mismatch.  Returns the CSV row as a dict."""
+    proc = subprocess.run([DRIVER, "--verify"] + shlex.split(cmd), capture_output=True,
+                          text=True, timeout=180)
+    assert proc.returncode == 0, (proc.stdout[-1500:] + proc.stderr[-2000:])
+    lines = proc.stdout.strip().splitlines()
+    checks = [ln.split(",") for ln in lines if ln.startswith("verify,")]
+    assert checks, "no output was verified"
+    for _, name, elements, mismatches, _worst in checks:
+        assert int(elements) > 0 and int(mismatches) == 0, (name, mismatches)
+    timing = [ln for ln in lines if not ln.startswith("verify,")]
+    header, row = timing[-2].split(","), timing[-1].split(",")
+    assert header[:4] == ["name", "iter", "dispatch_count", "avg_us"]
+    return dict(zip(header, row))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("cmd", commands())
 def test_driver_command(cmd):
     assert os.path.exists(DRIVER), \
         f"{DRIVER} missing: run `python -c 'import __graft_entry__ as g; g.build()'`"
-    proc = subprocess.run([DRIVER] + shlex.split(cmd), capture_output=True,
-                          text=True, timeout=120)
-    assert proc.returncode == 0, proc.stderr[-2000:]
-    lines = proc.stdout.strip().splitlines()
-    header, row = lines[-2].split(","), lines[-1].split(",")
-    assert header[:4] == ["name", "iter", "dispatch_count", "avg_us"]
-    rec = dict(zip(header, row))
+    rec = run_verified(cmd)
     want_iter = shlex.split(cmd)[shlex.split(cmd).index("--iter") + 1]
     assert rec["iter"] == want_iter
     assert rec["dispatch_count"] == "1"  # producer + pointwise chain fused
@@ -51,11 +65,7 @@ def test_driver_runs_the_reference_benchmark_commands(cmd):
     # 2-D and 3-D convolutions in every direction and layout, layer norms of
     # rank 2 to 4, (batched, transposed, mixed-type) matmuls, attention with
     # mask / GQA / explicit scale: each must run unchanged and print its row.
-    proc = subprocess.run([DRIVER] + shlex.split(cmd), capture_output=True,
-                          text=True, timeout=120)
-    assert proc.returncode == 0, proc.stderr[-2000:]
-    lines = proc.stdout.strip().splitlines()
-    rec = dict(zip(lines[-2].split(","), lines[-1].split(",")))
+    rec = run_verified(cmd)
     assert rec["iter"] == "10"
     # gradients with --bias add the bias-gradient reduction as a second step
     steps = 2 if ("--bias" in cmd and (" -F 2 " in cmd or " -F 4 " in cmd)) else 1
