@@ -8,8 +8,10 @@
 //     image and 128 output channels; the wavefronts w and w + 4 share 32 of
 //     those channels, both keep that 32 x (R*S*C) filter slice in registers as
 //     ready-made MFMA A operands for the kernel's whole life (staged once
-//     through LDS, so that the global reads are whole 64-byte runs of a filter
-//     row), and they take alternate blocks of 16 pixels;
+//     through LDS, all of it at once -- one part in a stage of its own, the
+//     other where the slab will be -- by LDS-DMA instructions that each cover
+//     eight whole 128-byte lines of filter rows), and they draw blocks of 16
+//     pixels from a counter they share;
 //   * the tile's input rows plus halo go into LDS once, by LDS-DMA, into a
 //     zero-padded image (W + S - 1 pixels per row, rows above / below the image
 //     as zeros) with a pixel pitch of C * 2 + 16 bytes: every filter tap is then
@@ -33,20 +35,20 @@
 #include "fast_paths.h"
 #include "gemm_kernel.h"
 
-#ifdef RF_PROFILE // experiment builds: cycle stamps of workgroup 0
-__device__ uint64_t rf_prof[64];
+#ifdef RF_PROFILE // experiment builds (-DRF_PROFILE=<workgroup>): cycle stamps per wavefront
+__device__ uint64_t rf_prof[128];
 #define RF_STAMP(i)                                                            \
   do {                                                                         \
-    if (blockIdx.x == 0 && threadIdx.x == 0)                                   \
-      rf_prof[i] = __builtin_amdgcn_s_memtime();                               \
+    if (blockIdx.x == RF_PROFILE && (threadIdx.x & 63) == 0)                   \
+      rf_prof[(threadIdx.x >> 6) * 16 + (i)] = __builtin_amdgcn_s_memtime();   \
   } while (0)
+extern "C" int fhip_debug_rf_prof(unsigned long long *out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rf_prof), sizeof(rf_prof));
+}
 #else
 #define RF_STAMP(i)                                                            \
   do {                                                                         \
   } while (0)
-#endif
-#ifndef RF_VARIANT_NAME
-#define RF_VARIANT_NAME "default"
 #endif
 
 namespace {
@@ -58,13 +60,17 @@ constexpr int kRfThreads = kRfWaves * 64;
 constexpr int kRfChannels = 128; // output channels per workgroup
 constexpr int kRfMaxNI = 16;     // KB of LDS per slab row, at most
 
+// s_waitcnt immediate: lgkmcnt <= n, the other counters untouched
+constexpr int rf_wait_lgkm_imm(int n) { return 0xF | (0x7 << 4) | (n << 8) | (0x3 << 14); }
+
 // Compile-time geometry shared by the kernel and the host's LDS budget.
 template <int C, int R, int S> struct RfGeom {
   static constexpr int kCPP = C * 2 / 16 + 1;   // chunks per slab pixel (one is padding)
   static constexpr int kNK = R * S * (C / 32);  // K-steps of 32 channels
-  static constexpr int kNKA = (kNK + 1) / 2;    // K-steps staged first
-  // filter stage: per wavefront one KB per (K-step, tile) of the larger part
+  static constexpr int kNKA = kNK / 4 * 2;      // K-steps staged in front of the slab
+  // filter stages: per channel slice two KB per K-step (one per 16-channel tile)
   static constexpr int kStageBytes = 4 * kNKA * 2 * 1024;
+  static constexpr int kStage2Bytes = 4 * (kNK - kNKA) * 2 * 1024; // in the slab's place
 };
 
 struct ConvRfArgs {
@@ -81,7 +87,6 @@ struct ConvRfArgs {
   uint32_t magic_q, magic_ni;
   uint32_t x_bytes, w_bytes;
   int32_t o_dt;
-  int32_t lds_spare;  // byte offset of a spare KB behind the slab
   int32_t unit_scale; // every op of the chain is additive with factor 1
   // linear epilogue before the optional ReLU: per op y = mul ? y * o : a * y + b * o
   int32_t nops;
@@ -130,7 +135,6 @@ conv_rf_kernel(ConvRfArgs g) {
   const int a_pad_w = g.pad_w;
   const int a_pad_h = g.pad_h;
   const uint32_t a_magic_q = g.magic_q;
-  const uint32_t a_magic_ni = g.magic_ni;
   const uint32_t a_x_bytes = g.x_bytes;
   const uint32_t a_w_bytes = g.w_bytes;
   const int a_nops = g.nops;
@@ -143,7 +147,7 @@ conv_rf_kernel(ConvRfArgs g) {
   // K-step j always sits in buffer j % RING
   constexpr int RING = NK % 6 == 0 ? 6 : (NK % 4 == 0 ? 4 : 3);
   constexpr int FROW = R * S * C * 2;        // bytes of a filter row
-  static_assert(C % 32 == 0 && NK % RING == 0 && NKA >= RING, "filter too small for this kernel");
+  static_assert(C % 64 == 0 && NK % RING == 0 && NKA % 2 == 0, "filter shape outside this kernel");
   static_assert((S - 1) * PITCH + (KPT - 1) * 64 + 48 < 65536, "ds offset range");
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -154,9 +158,9 @@ conv_rf_kernel(ConvRfArgs g) {
   const int l = threadIdx.x & 63;
   const int px = l & 15, q = l >> 4;
   const uint32_t rowpitch = (uint32_t)a_NI * 1024u;
-  // LDS: [filter stage, one part per channel slice | slab]
-  const uint32_t lds_f = lds0 + (uint32_t)slice * (NKA * 2 * 1024);
-  const uint32_t lds_s = lds0 + RfGeom<C, R, S>::kStageBytes;
+  // LDS: [block counters, 1 KB | filter stage | slab (first: rest of the filter)]
+  const uint32_t lds_f = lds0 + 1024u + (uint32_t)slice * (NKA * 2 * 1024);
+  const uint32_t lds_s = lds0 + 1024u + RfGeom<C, R, S>::kStageBytes;
 
   // this workgroup's channel group stays fixed; tiles are strided over
   const int kg = (int)(blockIdx.x % (unsigned)a_kgroups);
@@ -172,49 +176,68 @@ conv_rf_kernel(ConvRfArgs g) {
   // channel's R * S * C run; MFMA lane (rho, kq) takes the 16 bytes of K
   // quarter kq.  Loading those straight into registers would touch four cache
   // lines per lane quad (adjacent lanes are adjacent rho: rows FROW bytes
-  // apart), so each (K-step, tile) fragment is first written to one KB of LDS
-  // by one LDS-DMA instruction whose lane quads each fetch the 64 contiguous
-  // bytes of one row: DMA lane d carries row d / 4, quarter (d % 4) ^ (row / 4
-  // % 4) -- the XOR spreads the 16 rows that a fragment read of one quarter
-  // touches over all banks -- and the MFMA lane reads its 16 bytes back from
-  // position rho * 4 + (kq ^ (rho / 4 % 4)).  The two wavefronts of a slice
-  // stage one tile each and both read all fragments.  The K-step is the
-  // instructions' scalar offset (the immediate offset would also move the LDS
-  // destination), so there is no address arithmetic per instruction.
+  // apart), so the fragments go through LDS: per (pair of K-steps, tile) two
+  // LDS-DMA instructions, one per eight MFMA rows, each fetching the 128
+  // contiguous bytes that the pair covers of its eight filter rows.  The two
+  // wavefronts of a slice stage one tile each and both read all fragments.
+  // The pair is the instructions' scalar offset (the immediate offset would
+  // also move the LDS destination), so there is no address arithmetic per
+  // instruction.
   u32x4 filt[NK][2];
   const __amdgpu_buffer_rsrc_t rw = rf_rsrc(g.w, a_w_bytes);
-  uint32_t fvoff;
-  {
-    const int rho = l >> 2, kq = (l & 3) ^ ((rho >> 2) & 3);
+  // DMA lane d of the instruction for (K-step pair jp, row half h) carries
+  // MFMA row 8 h + d / 8 and the 16-byte chunk (d % 8) ^ (d / 16 | 4 h) of the
+  // 128 bytes at jp * 128 of that row: eight whole lines per instruction.  The
+  // MFMA lane (rho, kq) of K-step 2 jp + jo finds its chunk jo * 4 + kq at
+  // position ((jo ^ h) * 4 + (kq ^ (rho % 8 / 2))) of its row's eight: the 16
+  // lanes of a quarter wavefront then read 16 different bank groups.
+  uint32_t fvoff[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r8 = l >> 3, cpos = l & 7;
+    const int rho = 8 * h + r8;
+    const int chunk = cpos ^ ((r8 >> 1) | (h << 2));
     const int ch = ch_wave + 8 * (rho >> 2) + 4 * half + (rho & 3);
-    fvoff = (uint32_t)ch * (uint32_t)FROW + (uint32_t)kq * 16u;
+    fvoff[h] = (uint32_t)ch * (uint32_t)FROW + (uint32_t)chunk * 16u;
   }
-  const uint32_t fread = lds_f + (uint32_t)(px * 4 + (q ^ ((px >> 2) & 3))) * 16u;
-  auto filter_dma = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
+  const uint32_t lds_f2 = lds_s + (uint32_t)slice * ((NK - NKA) * 2 * 1024);
+  uint32_t fread[2]; // per K-step parity, relative to the stage of the slice
+#pragma unroll
+  for (int jo = 0; jo < 2; ++jo) {
+    const int h = px >> 3, r8 = px & 7;
+    fread[jo] = (uint32_t)(h * 1024 + (r8 * 8 + ((jo ^ h) * 4 + (q ^ (r8 >> 1)))) * 16);
+  }
+  auto filter_dma = [&](auto j0c, auto j1c, uint32_t stage) __attribute__((always_inline)) {
     constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
-    gemm_static_for<J1 - J0>([&](auto dc) {
-      constexpr int j = J0 + decltype(dc)::value;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rw,
-          (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(
-              lds_f + (uint32_t)(((j - J0) * 2 + half) * 1024)),
-          16, (int)fvoff, j * 64, 0, 0);
+    gemm_static_for<(J1 - J0) / 2>([&](auto dc) {
+      constexpr int jp = decltype(dc)::value;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rw,
+            (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(
+                stage + (uint32_t)((jp * 2 + half) * 2048 + h * 1024)),
+            16, (int)fvoff[h], (J0 / 2 + jp) * 128, 0, 0);
     });
   };
-  auto filter_read = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
+  auto filter_read = [&](auto j0c, auto j1c, uint32_t from) __attribute__((always_inline)) {
     constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
     gemm_static_for<J1 - J0>([&](auto dc) {
       constexpr int j = J0 + decltype(dc)::value;
+      constexpr int jp = (j - J0) / 2, jo = j % 2;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
         filt[j][t] = *(const GEMM_AS3 u32x4 *)(uintptr_t)(
-            fread + (uint32_t)(((j - J0) * 2 + t) * 1024));
+            from + fread[jo] + (uint32_t)((jp * 2 + t) * 2048));
     });
   };
   using JA0 = std::integral_constant<int, 0>;
   using JA1 = std::integral_constant<int, NKA>;
   using JB1 = std::integral_constant<int, NK>;
-  filter_dma(JA0{}, JA1{});
+  // Both parts are requested at once: the first into the stage, the second
+  // into the slab's place (the slab is loaded after the filter has left LDS).
+  filter_dma(JA0{}, JA1{}, lds_f);
+  filter_dma(JA1{}, JB1{}, lds_f2);
   RF_STAMP(14);
 
   const __amdgpu_buffer_rsrc_t rx = rf_rsrc(g.x, a_x_bytes);
@@ -222,7 +245,57 @@ conv_rf_kernel(ConvRfArgs g) {
   float sc[8], sh[8];
   f32x4 acc0[2];
 
-  bool first = true; // the filter's second part is still on its way
+  // ---- slab: rows of NI KB by LDS-DMA; wavefront w carries the KBs w and w + 8
+  // of every row.  LDS chunk x = i * 64 + lane of a slab row is chunk x % CPP of
+  // slab pixel x / CPP, i.e. input column x / CPP - pad_w; the padding chunk,
+  // columns outside the image and the tail of the row's last KB read as
+  // zeros.  The lane offsets are the same for every row, the row is the
+  // instructions' scalar offset.
+  uint32_t rel[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int xk = (wave + 8 * i) * 64 + l;
+    const int sp = (xk * (65536 / CPP + 1)) >> 16; // xk / CPP for xk < 2^12
+    const int c = xk - sp * CPP;
+    const int iw = sp - a_pad_w;
+    const bool ok = c < CPP - 1 && (unsigned)iw < (unsigned)a_W;
+    rel[i] = ok ? (uint32_t)(iw * (C * 2) + c * 16) : 0x80000000u;
+  }
+  const int npr = wave + 8 < a_NI ? 2 : (wave < a_NI ? 1 : 0); // instructions per row
+  auto slab_rows = [&](int rows_in, int n, int ih0) __attribute__((always_inline)) {
+    for (int sr = 0; sr < rows_in; ++sr) {
+      const int ih = ih0 + sr;
+      const bool row_ok = (unsigned)ih < (unsigned)a_H;
+      const __amdgpu_buffer_rsrc_t rs = row_ok ? rx : rnone;
+      const int soff = row_ok ? ((n * a_H + ih) * a_W) * (C * 2) : 0;
+      const uint32_t dst = lds_s + (uint32_t)sr * rowpitch + (uint32_t)wave * 1024u;
+      if (npr > 0)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16, (int)rel[0], soff, 0, 0);
+      if (npr > 1)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst + 8192u), 16, (int)rel[1],
+            soff, 0, 0);
+    }
+  };
+
+  // block counter of the slice, in the KB at the bottom of LDS
+  const uint32_t draw = lds0 + (uint32_t)slice * 4u;
+  auto draw_block = [&]() __attribute__((always_inline)) {
+    // one LDS atomic of lane 0; the result is in flight when this returns (the
+    // compiler does not know: the reader waits by count, LDS answers in order)
+    uint32_t v;
+    uint64_t saved;
+    asm volatile("s_mov_b64 %1, exec\n\t"
+                 "s_mov_b64 exec, 1\n\t"
+                 "ds_add_rtn_u32 %0, %2, %3\n\t"
+                 "s_mov_b64 exec, %1"
+                 : "=&v"(v), "=&s"(saved)
+                 : "v"(draw), "v"(1u)
+                 : "memory");
+    return v;
+  };
+  bool first = true; // the filter is still on its way
   for (int tile = tile0; tile < a_ntiles; tile += tile_step) {
     const int n = tile / a_tiles_per_image;
     const int p0 = (tile - n * a_tiles_per_image) * a_TR;
@@ -231,39 +304,8 @@ conv_rf_kernel(ConvRfArgs g) {
     const int rows_in = tr + R - 1;
     const int ih0 = p0 - a_pad_h;
 
-    // ---- slab: rows_in rows of NI KB by LDS-DMA; wavefront w loads rows w, w + 8, ...
-    // LDS chunk x = i * 64 + lane of a slab row is chunk x % CPP of slab pixel
-    // x / CPP, i.e. input column x / CPP - pad_w; the padding chunk, columns
-    // outside the image and the tail of the row's last KB read as zeros.  The
-    // lane offsets are the same for every row, the row is the instructions'
-    // scalar offset: nothing but the LDS address changes between instructions.
-    {
-      uint32_t rel[kRfMaxNI];
-#pragma unroll
-      for (int i = 0; i < kRfMaxNI; ++i) {
-        const int xk = i * 64 + l;
-        const int sp = (xk * (65536 / CPP + 1)) >> 16; // xk / CPP for xk < 2^12
-        const int c = xk - sp * CPP;
-        const int iw = sp - a_pad_w;
-        const bool ok = c < CPP - 1 && (unsigned)iw < (unsigned)a_W;
-        rel[i] = ok ? (uint32_t)(iw * (C * 2) + c * 16) : 0x80000000u;
-      }
-      for (int sr = wave; sr < rows_in; sr += kRfWaves) {
-        const int ih = ih0 + sr;
-        const bool row_ok = (unsigned)ih < (unsigned)a_H;
-        const __amdgpu_buffer_rsrc_t rs = row_ok ? rx : rnone;
-        const int soff = row_ok ? ((n * a_H + ih) * a_W) * (C * 2) : 0;
-        const uint32_t dst = lds_s + (uint32_t)sr * rowpitch;
-#pragma unroll
-        for (int i = 0; i < kRfMaxNI; ++i)
-          if (i < a_NI)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                rs, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst + i * 1024u),
-                16, (int)rel[i], soff, 0, 0);
-      }
-    }
-    RF_STAMP(15);
     if (first) {
+      RF_STAMP(15);
       // ---- epilogue constants: y = acc * sc[c] + sh[c] for the lane's 8 channels
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
@@ -304,21 +346,34 @@ conv_rf_kernel(ConvRfArgs g) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           acc0[t][i] = UNIT ? sh[4 * t + i] : 0.f;
-    }
-    RF_STAMP(1);
-    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
-    RF_STAMP(2);
-    gemm_barrier();
-    RF_STAMP(3);
-    if (first) {
-      // first part of the filter into registers; the stage is refilled with
-      // the second part once every wavefront has read the first
-      filter_read(JA0{}, JA1{});
+      RF_STAMP(1);
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+      RF_STAMP(2);
+      gemm_barrier();
+      RF_STAMP(3);
+      // the second part leaves the slab's place first; the first part is read
+      // while the slab's loads are in flight
+      filter_read(JA1{}, JB1{}, lds_f2);
       asm volatile("" ::: "memory");
       __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
+      RF_STAMP(6);
       gemm_barrier();
-      filter_dma(JA1{}, JB1{});
     }
+    slab_rows(rows_in, n, ih0);
+    RF_STAMP(7);
+    if (first) {
+      filter_read(JA0{}, JA1{}, lds_f);
+      first = false;
+    }
+    // the two wavefronts of a slice draw their blocks from a counter (the
+    // first two are dealt out): the SIMD serves its older wavefront first, so
+    // equal shares would leave the younger one to finish alone
+    if (half == 0 && l == 0)
+      *(GEMM_AS3 uint32_t *)(uintptr_t)draw = 2u;
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+    RF_STAMP(9);
+    gemm_barrier();
+    RF_STAMP(10);
 
     // outputs of this tile: dense rows of K channels, pixel index tile-relative
     const __amdgpu_buffer_rsrc_t ro =
@@ -347,22 +402,35 @@ conv_rf_kernel(ConvRfArgs g) {
     };
     f32x4 acc[2];
     uint32_t base, ooff, nbase, nooff;
-    // K-steps [J0, J1) of the block at `base`; the first fragments of the next
+    uint32_t drawn;
+    int nb;
+    // The K-steps of the block at `base`; the first fragments of the next
     // block (at `nbase`) are fetched during the last steps.
-    auto ksteps = [&](auto j0c, auto j1c) __attribute__((always_inline)) {
-      constexpr int J0 = decltype(j0c)::value, J1 = decltype(j1c)::value;
-      gemm_static_for<J1 - J0>([&](auto dc) {
-        constexpr int j = J0 + decltype(dc)::value;
+    auto ksteps = [&]() __attribute__((always_inline)) {
+      gemm_static_for<NK>([&](auto dc) {
+        constexpr int j = decltype(dc)::value;
         constexpr int ahead = j + RING - 1;
-#ifndef RF_EXP_NOFETCH
+        if constexpr (ahead == NK) {
+          // the block drawn at the top of this one: j fragment reads have been
+          // issued since, so "at most j outstanding" says the draw is back
+          // (one statement: nothing may move between the wait and the read)
+          asm volatile("s_waitcnt lgkmcnt(%2)\n\t"
+                       "v_readfirstlane_b32 %0, %1\n\t"
+                       "s_nop 4"
+                       : "=s"(nb)
+                       : "v"(drawn), "n"(j < 15 ? j : 15));
+          block_setup(nb, nbase, nooff);
+        }
         if constexpr (ahead < NK)
           fetch(std::integral_constant<int, ahead>{}, base);
         else
           fetch(std::integral_constant<int, ahead - NK>{}, nbase);
-#endif
 #pragma unroll
         for (int t = 0; t < 2; ++t)
           acc[t] = rf_mfma<KIND>(filt[j][t], frag[j % RING], j == 0 ? acc0[t] : acc[t]);
+        // (keeps the fragment reads where they are written: RING - 1 K-steps
+        // ahead of their MFMAs)
+        __builtin_amdgcn_sched_barrier(0);
       });
     };
     // scale / ReLU, rounding and the 16-byte store of a finished block
@@ -400,46 +468,23 @@ conv_rf_kernel(ConvRfArgs g) {
         }
       }
       const u32x4 pk = {w[0], w[1], w[2], w[3]};
-#ifdef RF_EXP_NOSTORE
-      if (pk[0] == 0x12345678u) // (experiment: keeps the epilogue alive, stores nothing)
-#endif
       // (sc0 sc1 nt: the output is written once and not read back here;
       // measured 8 % faster end to end than the default write-back policy)
       __builtin_amdgcn_raw_buffer_store_b128(pk, ro, (int)off, 0, 19);
     };
 
-    // This wavefront's blocks: half, half + 2, ...  (block indices past the
-    // last one address the last pixel and store nothing).
+    // This wavefront's blocks: `half`, then whatever it draws (block indices
+    // past the last one address the last pixel and store nothing).
     int b = half;
     block_setup(b, base, ooff);
-    gemm_static_for<RING - 1>([&](auto jc) { fetch(jc, base); });
+    gemm_static_for<RING - 1>([&](auto jc) {
+      fetch(jc, base);
+      __builtin_amdgcn_sched_barrier(0); // (in this order: the loop waits for the oldest)
+    });
     RF_STAMP(4);
-    if (first) {
-      // The first block (of every wavefront: the barrier in its middle is the
-      // workgroup's) runs its first K-steps on the first part of the filter.
-      block_setup(b + 2, nbase, nooff);
-      ksteps(JA0{}, JA1{});
-      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
-      gemm_barrier();
-      filter_read(JA1{}, JB1{});
-      ksteps(JA1{}, JB1{});
-      float y[8];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          y[4 * t + i] = acc[t][i];
-      const uint32_t done_off = ooff;
-      b += 2;
-      base = nbase;
-      ooff = nooff;
-      first = false;
-      finish(y, done_off);
-    }
-    RF_STAMP(5);
-    for (; b < nblocks; b += 2) {
-      block_setup(b + 2, nbase, nooff);
-      ksteps(JA0{}, JB1{});
+    while (b < nblocks) {
+      drawn = draw_block();
+      ksteps();
       float y[8];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -450,6 +495,9 @@ conv_rf_kernel(ConvRfArgs g) {
       base = nbase;
       ooff = nooff;
       finish(y, done_off);
+      if (b == half)
+        RF_STAMP(5);
+      b = nb;
     }
     RF_STAMP(12);
     // every wavefront is done with the slab before the next tile overwrites it
@@ -586,9 +634,11 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   (void)wp;
   if (a.NI > kRfMaxNI)
     return p;
-  // LDS: the filter stage (one KB per K-step and tile of the larger filter
-  // part, per wavefront) in front of the slab
-  const int stage = 4 * (int)((R * S * (C / 32) + 1) / 2) * 2 * 1024;
+  // LDS: a KB of block counters, the stage of the filter's first part, and
+  // the slab, whose place first stages the filter's second part
+  const int nk = (int)(R * S * (C / 32));
+  const int stage = 4 * (nk / 4 * 2) * 2 * 1024;
+  const int stage2 = 4 * (nk - nk / 4 * 2) * 2 * 1024;
   const int64_t lds_cap = 160 * 1024 - stage - 1024;
   // rows per tile: the choice that fills whole rounds of the machine best
   const int cus = num_cus > 0 ? num_cus : 256;
@@ -626,8 +676,9 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   a.magic_q = conv_magic(a.Q);
   a.magic_ni = conv_magic(a.NI);
   p.C = (int)C, p.R = (int)R, p.S = (int)S;
-  a.lds_spare = stage + (a.TR + (int)R - 1) * a.NI * 1024;
-  p.lds = a.lds_spare + 1024;
+  // (the slab's place also stages the second part of the filter)
+  const int slab_bytes = (a.TR + (int)R - 1) * a.NI * 1024;
+  p.lds = 1024 + stage + (slab_bytes > stage2 ? slab_bytes : stage2);
   const int64_t items = (int64_t)a.ntiles * kgroups;
   const int64_t slots = (int64_t)cus / kgroups * kgroups > 0 ? (int64_t)cus / kgroups * kgroups : kgroups;
   p.grid = (int)(items < slots ? items : slots);
