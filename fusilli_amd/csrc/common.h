@@ -52,6 +52,7 @@ int fhip_ctx_scratch(fhip_ctx *ctx, size_t bytes, void **out);
 struct FhipKnobs {
   bool has_rownorm_wgs = false;
   int rownorm_wgs_per_cu = 0;       // FUSILLI_HIP_ROWNORM_WGS_PER_CU
+  int pointwise_wgs_per_cu = 0;     // FUSILLI_HIP_POINTWISE_WGS_PER_CU (0: built-in)
   int rownorm_shape_w = 0, rownorm_shape_c = 0; // FUSILLI_HIP_ROWNORM_SHAPE "w,c"
   bool rownorm_general = false;     // FUSILLI_HIP_ROWNORM_GENERAL
   int conv_tile_bm = 0, conv_tile_bn = 0; // FUSILLI_HIP_CONV_TILE "bm,bn"

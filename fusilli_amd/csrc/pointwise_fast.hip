@@ -73,9 +73,18 @@ __device__ __forceinline__ void fetch_raw(const PwFastArgs &g, int i,
     if (kind == IN_ROW)
       rv = vec - div_magic(vec, g.span[i], g.magic[i]) * g.span[i];
     const char *p = base + (int64_t)rv * (8 * ES);
-    raw.lo = *(const u32x4 *)p;
-    if constexpr (ES == 4)
-      raw.hi = *(const u32x4 *)(p + 16);
+#ifdef PW_NT_LOADS
+    if (kind == IN_FULL) {
+      raw.lo = __builtin_nontemporal_load((const u32x4 *)p);
+      if constexpr (ES == 4)
+        raw.hi = __builtin_nontemporal_load((const u32x4 *)(p + 16));
+    } else
+#endif
+    {
+      raw.lo = *(const u32x4 *)p;
+      if constexpr (ES == 4)
+        raw.hi = *(const u32x4 *)(p + 16);
+    }
   } else if (kind == IN_COL) {
     const char *p =
         base + (int64_t)div_magic(vec, g.span[i], g.magic[i]) * ES;
@@ -165,18 +174,24 @@ __device__ __forceinline__ void store8(void *out, int32_t vec,
 
 // erf-based GELU for 16-bit outputs: erf by Abramowitz & Stegun 7.1.26
 // (|error| <= 1.5e-7, far below bf16 / f16 resolution) on the hardware's
-// exp2 and reciprocal -- a third of the instructions of the library erff.
+// exp2 and reciprocal.  With w = (1 - erf(|x| / sqrt 2)) / 2 = p(t) t e / 2 the
+// result is x (1 - w) for x >= 0 and x w below, i.e. max(x, 0) - |x| w: eleven
+// multiply-adds and the two transcendentals per element, no cancellation on
+// the negative side.
 __device__ __forceinline__ float gelu_erf_16bit(float x) {
-  const float z = x * 0.70710678118654752440f, az = __builtin_fabsf(z);
-  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, az, 1.f));
-  float p = __builtin_fmaf(1.061405429f, t, -1.453152027f);
-  p = __builtin_fmaf(p, t, 1.421413741f);
-  p = __builtin_fmaf(p, t, -0.284496736f);
-  p = __builtin_fmaf(p, t, 0.254829592f);
-  const float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * az * az);
-  const float erf_abs = __builtin_fmaf(-p * t, e, 1.f);
-  const float erf = z < 0.f ? -erf_abs : erf_abs;
-  return 0.5f * x * (1.f + erf);
+  const float ax = __builtin_fabsf(x);
+  // t = 1 / (1 + 0.3275911 |x| / sqrt 2)
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.23164189f, ax, 1.f));
+  // half of the polynomial's coefficients
+  float p = __builtin_fmaf(0.5307027145f, t, -0.7265760135f);
+  p = __builtin_fmaf(p, t, 0.7107068705f);
+  p = __builtin_fmaf(p, t, -0.142248368f);
+  p = __builtin_fmaf(p, t, 0.127414796f);
+  // e = exp(-x^2 / 2) = exp2(-(|x| sqrt(log2(e) / 2))^2)
+  const float u = ax * 0.84932180028801904272f;
+  const float e = __builtin_amdgcn_exp2f(-u * u);
+  const float w = p * t * e;
+  return __builtin_fmaf(-ax, w, __builtin_fmaxf(x, 0.f));
 }
 
 // One lane evaluates 8 elements.  MODE >= 0 fixes the mode at compile time;
@@ -302,7 +317,8 @@ void launch_dt(fhip_ctx *ctx, const PwFastArgs &g0) {
   // chunks of a large tensor
   const int64_t chunk = 256 * kUnroll;
   int64_t blocks = (g.nvec + chunk - 1) / chunk;
-  const int64_t cap = 256 * kWgsPerCu;
+  const int knob = fhip_knobs().pointwise_wgs_per_cu;
+  const int64_t cap = 256 * (knob > 0 ? knob : kWgsPerCu);
   if (blocks > cap)
     blocks = cap;
   // broadcast rows: a grid that is a multiple of `need` workgroups puts every
