@@ -73,18 +73,10 @@ __device__ __forceinline__ void fetch_raw(const PwFastArgs &g, int i,
     if (kind == IN_ROW)
       rv = vec - div_magic(vec, g.span[i], g.magic[i]) * g.span[i];
     const char *p = base + (int64_t)rv * (8 * ES);
-#ifdef PW_NT_LOADS
-    if (kind == IN_FULL) {
-      raw.lo = __builtin_nontemporal_load((const u32x4 *)p);
-      if constexpr (ES == 4)
-        raw.hi = __builtin_nontemporal_load((const u32x4 *)(p + 16));
-    } else
-#endif
-    {
-      raw.lo = *(const u32x4 *)p;
-      if constexpr (ES == 4)
-        raw.hi = *(const u32x4 *)(p + 16);
-    }
+    // (plain loads: nontemporal ones measured the same)
+    raw.lo = *(const u32x4 *)p;
+    if constexpr (ES == 4)
+      raw.hi = *(const u32x4 *)(p + 16);
   } else if (kind == IN_COL) {
     const char *p =
         base + (int64_t)div_magic(vec, g.span[i], g.magic[i]) * ES;
