@@ -44,10 +44,11 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}
 # figures of the recorded runs, not of this one.
 TRAFFIC = {
     "conv_fprop_bf16_n32c64h56w56_k128r3s3_bias_relu":
-        (int((8486.5 * 1.9985 + 25088) * 1024),
+        (int((8467.5 * 1.9985 + 25088) * 1024),
          "profiles/conv_rf_dgrad_wgrad_direct_bf16_n32c64h56w56_k128r3s3.md"),
     "sdpa_fwd_bf16_causal_b4h32s2048d128":
-        (436_000_000 + 64 * 1024 * 1024, "profiles/sdpa_fwd_bf16_causal_b4h32s2048d128.md"),
+        (int(149207.4 * 1.9985 * 1024) + 64 * 1024 * 1024,
+         "profiles/sdpa_fwd_bf16_causal_b4h32s2048d128.md"),
     "matmul_int8_4096x8192x4096_i32":
         (201_000_000 + 64 * 1024 * 1024, "profiles/gemm_mfma_4096x8192x4096_int8_fp8_bf16.md"),
     "matmul_fp8e4m3_4096x8192x4096_scaled_bf16_out":
