@@ -413,28 +413,36 @@ struct WgDirectSumArgs {
 // A partial block is [entry e = 4 * tap + i / 4][lane][i % 4].
 __global__ __launch_bounds__(256) void
 conv_wgrad_direct_sum_kernel(WgDirectSumArgs a, const float *part, void *dw) {
-  __shared__ float red[4][64];
+  // A workgroup adds 256 results: thread (o, j) the parts j, j + 4, ... of
+  // four consecutive ones (16-byte loads; a wavefront reads 1 KB runs), then
+  // the four j of a group meet in LDS, always in the same order.
+  __shared__ f32x4 red[4][64];
   const int o = threadIdx.x & 63, j = threadIdx.x >> 6;
-  const int64_t lin = (int64_t)blockIdx.x * 64 + o;
+  const int64_t lin = ((int64_t)blockIdx.x * 64 + o) * 4;
   const int type = (int)(lin / kWdBlock);
   const int within = (int)(lin - (int64_t)type * kWdBlock);
   const float *src = part + (int64_t)type * a.nparts * kWdBlock + within;
-  float acc = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
   for (int p = j; p < a.nparts; p += 4)
-    acc += src[(int64_t)p * kWdBlock];
+    acc += *(const f32x4 *)(src + (int64_t)p * kWdBlock);
   red[j][o] = acc;
   __syncthreads();
   if (j != 0)
     return;
   acc = ((red[0][o] + red[1][o]) + red[2][o]) + red[3][o];
-  const int comp = within & 3, lane = (within >> 2) & 63, e = within >> 8;
-  const int tap = e >> 2, i = 4 * (e & 3) + comp;
+  // within = [entry e = 4 * tap + i / 4][lane][i % 4]: the four values are i % 4 = 0 .. 3
+  const int lane = (within >> 2) & 63, e = within >> 8;
+  const int tap = e >> 2;
   const int kb = type / a.ctypes, cb = type - kb * a.ctypes;
-  const int64_t k = kb * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
   const int64_t c = cb * 32 + (lane & 31);
   const int r = tap / 3, sx = tap - r * 3;
-  fhip_store<float>(dw, a.dt, k * a.sk + c * a.sc + r * a.sr + sx * a.ss, acc);
+#pragma unroll
+  for (int comp = 0; comp < 4; ++comp) {
+    const int i = 4 * (e & 3) + comp;
+    const int64_t k = kb * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+    fhip_store<float>(dw, a.dt, k * a.sk + c * a.sc + r * a.sr + sx * a.ss, acc[comp]);
+  }
 }
 
 struct WgDirectPlan {
@@ -582,7 +590,7 @@ int fhip_fast_conv_wgrad_direct(fhip_ctx *ctx, const fhip_conv_desc *d,
   s.ss = d->w.dim[3] == 1 ? 0 : d->w.stride[3];
   s.dt = d->w.dtype;
   const int64_t total = (int64_t)(p.a.C / 32) * (p.a.K / 32) * kWdBlock;
-  hipLaunchKernelGGL(conv_wgrad_direct_sum_kernel, dim3((unsigned)(total / 64)),
+  hipLaunchKernelGGL(conv_wgrad_direct_sum_kernel, dim3((unsigned)(total / 256)),
                      dim3(256), 0, ctx->stream, s, (const float *)p.a.part, dw);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
   fhip_note_kernel(ctx, "conv_wgrad_direct");
