@@ -162,16 +162,33 @@ __global__ __launch_bounds__(kRlThreads) void rownorm_long_apply_kernel(RowNormL
   T *orow = (T *)g.out + row * g.out_row_stride;
   const int64_t lo = s * g.seg;
   const int64_t hi = lo + g.seg < g.inner ? lo + g.seg : g.inner;
+  // scale and bias of the row's own type come as whole vectors, like the row
+  const bool scale_vec = g.scale && g.scale_dt == V::kDt;
+  const bool bias_vec = g.bias && g.bias_dt == V::kDt;
   for (int64_t i = lo + (int64_t)threadIdx.x * V::kN; i < hi; i += (int64_t)kRlThreads * V::kN) {
-    float v[V::kN];
+    float v[V::kN], sc[V::kN], bi[V::kN];
     V::load(xr, i, v);
+    if (scale_vec) {
+      V::load(g.scale, i, sc);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V::kN; ++k)
+        sc[k] = g.scale ? fhip_load<float>(g.scale, g.scale_dt, i + k) : 1.f;
+    }
+    if (bias_vec) {
+      V::load(g.bias, i, bi);
+    } else {
+#pragma unroll
+      for (int k = 0; k < V::kN; ++k)
+        bi[k] = g.bias ? fhip_load<float>(g.bias, g.bias_dt, i + k) : 0.f;
+    }
 #pragma unroll
     for (int k = 0; k < V::kN; ++k) {
       float y = (v[k] - mean) * rstd;
       if (g.scale)
-        y *= fhip_load<float>(g.scale, g.scale_dt, i + k);
+        y *= sc[k];
       if (g.bias)
-        y += fhip_load<float>(g.bias, g.bias_dt, i + k);
+        y += bi[k];
       v[k] = fhip_round_through<float>(g.y_dt, y);
     }
     V::store(orow, i, v);
