@@ -895,15 +895,17 @@ def main():
             configs = {}
             for cfg, (name, target, variant, command) in CONFIGS.items():
                 if name is None:
-                    frac, us, kernel = line["roofline"]["frac"], line["roofline"]["kernel_us"], headline_kernel
+                    roof, kernel = line["roofline"], headline_kernel
                 else:
-                    res = others[name]
-                    frac, us, kernel = res["roofline"]["frac"], res["roofline"]["kernel_us"], res["kernel"]
+                    roof, kernel = others[name]["roofline"], others[name]["kernel"]
+                frac, us = roof["frac"], roof["kernel_us"]
                 configs[cfg] = {"line": name or "headline", "frac": frac, "target": target,
                                 "met": None if target is None else bool(frac >= target),
                                 "kernel_us": us, "kernel": kernel,
                                 "expected_kernel": bool(kernel.startswith(variant)),
-                                "graph_api_us": graph_api_us(command)}
+                                "graph_api_us": graph_api_us(command),
+                                "traffic": roof.get("traffic"),
+                                "traffic_source": roof.get("traffic_source")}
             line["configs"] = configs
             floors = json.load(open(FLOOR_FILE)) if os.path.exists(FLOOR_FILE) else {}
             regressions = []
