@@ -250,16 +250,27 @@ __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
     b_kk[i] = b_kfast ? e % kF32K : e / T;
     b_n[i] = b_kfast ? e / kF32K : e % T;
   }
+  // element offsets at K-step 0 (a step adds k0 times the K stride) and the
+  // rows / columns that exist
+  int64_t a_off[8], b_off[8];
+  uint32_t a_live = 0, b_live = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
+    a_off[i] = ab + m * a_sm + a_kk[i] * g.a_k;
+    b_off[i] = bb + n * b_sn + b_kk[i] * g.b_k;
+    a_live |= (uint32_t)(m < M) << i;
+    b_live |= (uint32_t)(n < N) << i;
+  }
   auto fetch = [&](int64_t k0, float (&ra)[8], float (&rb)[8]) {
+    const int64_t ka0 = k0 * g.a_k, kb0 = k0 * g.b_k;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int64_t m = m0 + a_m[i], n = n0 + b_n[i];
-      const int64_t ka = k0 + a_kk[i], kb = k0 + b_kk[i];
-      ra[i] = m < M && ka < g.K
-                  ? matmul_operand<DT>(a, g.a_dt, ab + m * a_sm + ka * g.a_k)
+      ra[i] = ((a_live >> i) & 1) && k0 + a_kk[i] < g.K
+                  ? matmul_operand<DT>(a, g.a_dt, a_off[i] + ka0)
                   : 0.f;
-      rb[i] = n < N && kb < g.K
-                  ? matmul_operand<DT>(b, g.b_dt, bb + n * b_sn + kb * g.b_k)
+      rb[i] = ((b_live >> i) & 1) && k0 + b_kk[i] < g.K
+                  ? matmul_operand<DT>(b, g.b_dt, b_off[i] + kb0)
                   : 0.f;
     }
   };
