@@ -175,6 +175,10 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
         p.ksplit = sk;
       }
     }
+    // (a forced count must still divide the slices into runs of at least 8)
+    const int forced = fhip_knobs().gemm_split;
+    if (forced > 1 && slices % forced == 0 && slices / forced >= 8)
+      p.ksplit = forced;
     if (p.ksplit > 1)
       p.bm = bm0, p.bn = bn0;
   }
