@@ -16,6 +16,8 @@ FhipKnobs parse_knobs() {
     k.has_rownorm_wgs = true;
     k.rownorm_wgs_per_cu = atoi(e);
   }
+  if (const char *e = getenv("FUSILLI_HIP_CONV_DEPTHWISE_STRIPS"))
+    k.conv_depthwise_strips = atoi(e) != 0;
   if (const char *e = getenv("FUSILLI_HIP_GEMM_SPLIT"))
     k.gemm_split = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_POINTWISE_WGS_PER_CU"))

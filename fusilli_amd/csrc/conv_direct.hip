@@ -320,6 +320,146 @@ __global__ __launch_bounds__(256) void direct_conv_fprop_cl_kernel(
   }
 }
 
+// ---- depthwise 3 x 3, unit stride and dilation, channels-last ------------------
+// A thread owns a strip of kDwQ consecutive output pixels of one row and 8
+// consecutive channels.  Its 9 x 8 filter values stay in registers (72 floats,
+// loaded as nine 16-byte vectors: the 8 channels' taps are contiguous in W),
+// and the strip's 3 x (kDwQ + 2) input vectors are loaded once -- each feeds up
+// to three output pixels -- so a pixel costs 4.5 loads instead of 9 and no LDS
+// at all.  Lanes run over the channel blocks first (a pixel's chunks are
+// coalesced), then over the strips.  Taps outside the image read zeros through
+// the buffer descriptor's range check.
+constexpr int kDwQ = 4;
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void depthwise3x3_cl_kernel(DcClArgs g, const void *x,
+                                                              const void *w, void *out,
+                                                              uint32_t strips, uint32_t strips_q) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  auto to_f32 = [](uint32_t h) __attribute__((always_inline)) {
+    if constexpr (BF16)
+      return __builtin_bit_cast(float, h << 16);
+    else
+      return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+  };
+  const int cb = blockIdx.y * 16 + (threadIdx.x & 15);
+  const uint32_t strip = blockIdx.x * 16u + (threadIdx.x >> 4);
+  if (cb >= g.cbs || strip >= strips)
+    return;
+  const uint32_t chan = (uint32_t)cb * 8u;
+  // filter: wt[tap][k] = W[chan + k][tap]
+  float wt[9][8];
+  {
+    const u32x4 *wp = (const u32x4 *)((const uint16_t *)w + (size_t)chan * 9);
+    uint32_t raw[36];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+      const u32x4 v = wp[i];
+      raw[4 * i] = v.x, raw[4 * i + 1] = v.y, raw[4 * i + 2] = v.z, raw[4 * i + 3] = v.w;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+#pragma unroll
+      for (int t = 0; t < 9; ++t) {
+        const int e = k * 9 + t;
+        wt[t][k] = to_f32((e & 1) ? raw[e >> 1] >> 16 : raw[e >> 1] & 0xffffu);
+      }
+  }
+  const uint32_t qs = strip % strips_q;
+  const uint32_t t1 = strip / strips_q;
+  const int p = (int)(t1 % (uint32_t)g.P);
+  const int n = (int)(t1 / (uint32_t)g.P);
+  const int q0 = (int)qs * kDwQ;
+  const int ih0 = p - g.pad_h, iw0 = q0 - g.pad_w;
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<void *>(x), 0, (int)g.x_bytes, 0x00020000);
+  u32x4 xv[3][kDwQ + 2];
+#pragma unroll
+  for (int r = 0; r < 3; ++r) {
+    const int ih = ih0 + r;
+    const bool row_in = (unsigned)ih < (unsigned)g.H;
+#pragma unroll
+    for (int c = 0; c < kDwQ + 2; ++c) {
+      const int iw = iw0 + c;
+      const bool in = row_in && (unsigned)iw < (unsigned)g.W;
+      const uint32_t off = ((uint32_t)((n * g.H + ih) * g.W + iw) * (uint32_t)g.C + chan) * 2u;
+      xv[r][c] = __builtin_amdgcn_raw_buffer_load_b128(rx, in ? (int)off : (int)0x80000000, 0, 0);
+    }
+  }
+  float acc[kDwQ][8];
+#pragma unroll
+  for (int u = 0; u < kDwQ; ++u)
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      acc[u][k] = 0.f;
+#pragma unroll
+  for (int r = 0; r < 3; ++r)
+#pragma unroll
+    for (int c = 0; c < kDwQ + 2; ++c) {
+      const uint32_t xw[4] = {xv[r][c].x, xv[r][c].y, xv[r][c].z, xv[r][c].w};
+      float xf[8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        xf[2 * i] = to_f32(xw[i] & 0xffffu);
+        xf[2 * i + 1] = to_f32(xw[i] >> 16);
+      }
+      // input column c is tap s = c - u of output pixel u (taps in filter order
+      // per pixel: r ascending, then s ascending -- the order of the other kernels)
+#pragma unroll
+      for (int u = 0; u < kDwQ; ++u) {
+        const int sx = c - u;
+        if (sx < 0 || sx > 2)
+          continue;
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          acc[u][k] = __builtin_fmaf(xf[k], wt[r * 3 + sx][k], acc[u][k]);
+      }
+    }
+#pragma unroll
+  for (int u = 0; u < kDwQ; ++u) {
+    const int qq = q0 + u;
+    if (qq >= g.Q)
+      break;
+    float y[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      y[k] = g.y_dt == FHIP_FLOAT ? acc[u][k] : fhip_round_through<float>(g.y_dt, acc[u][k]);
+    if (g.epi.count > 0) {
+      int64_t coord[FHIP_MAX_RANK];
+      coord[0] = n;
+      coord[2] = p;
+      coord[3] = qq;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        coord[1] = cb * 8 + k;
+        y[k] = fhip_apply_epilogue<float>(g.epi, y[k], coord);
+      }
+    }
+    // (OUT has fewer than 2^31 elements)
+    const uint32_t ob = ((uint32_t)((n * g.P + p) * g.Q + qq)) * (uint32_t)g.K + chan;
+    if (g.o_dt == FHIP_FLOAT) {
+      float4 *o = (float4 *)((float *)out + ob);
+      o[0] = make_float4(y[0], y[1], y[2], y[3]);
+      o[1] = make_float4(y[4], y[5], y[6], y[7]);
+    } else {
+      uint32_t ow[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t lo, hi;
+        if (g.o_dt == FHIP_BFLOAT16) {
+          lo = __builtin_bit_cast(uint16_t, (__bf16)y[2 * i]);
+          hi = __builtin_bit_cast(uint16_t, (__bf16)y[2 * i + 1]);
+        } else {
+          lo = __builtin_bit_cast(uint16_t, (_Float16)y[2 * i]);
+          hi = __builtin_bit_cast(uint16_t, (_Float16)y[2 * i + 1]);
+        }
+        ow[i] = lo | (hi << 16);
+      }
+      *(uint4 *)((uint16_t *)out + ob) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
+  }
+}
+
 // dense channels-last strides of dims [d0, C, spatial...] (unit dims are free)
 bool dc_channels_last(const fhip_tensor_desc &t) {
   int64_t expect = t.dim[1];
@@ -738,6 +878,22 @@ int fhip_direct_conv_fprop(fhip_ctx *ctx, const fhip_conv_desc *d,
     DcClArgs c{};
     if (make_cl_args(d, c) && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0) {
       c.epi = epi;
+      // depthwise 3 x 3 at unit stride and dilation: the strip kernel
+      if (d->w.dim[1] == 1 && c.sp == 2 && c.R == 3 && c.S == 3 && c.str_h == 1 && c.str_w == 1 &&
+          c.dil_h == 1 && c.dil_w == 1 && fhip_knobs().conv_depthwise_strips) {
+        const uint32_t strips_q = (uint32_t)((c.Q + kDwQ - 1) / kDwQ);
+        const uint32_t strips = strips_q * (uint32_t)c.P * (uint32_t)c.N;
+        const dim3 sgrid((strips + 15u) / 16u, (unsigned)((c.cbs + 15) / 16));
+        if (d->x.dtype == FHIP_BFLOAT16)
+          hipLaunchKernelGGL((depthwise3x3_cl_kernel<true>), sgrid, dim3(256), 0, ctx->stream, c, x,
+                             w, out, strips, strips_q);
+        else
+          hipLaunchKernelGGL((depthwise3x3_cl_kernel<false>), sgrid, dim3(256), 0, ctx->stream, c,
+                             x, w, out, strips, strips_q);
+        FHIP_HIP_CHECK(ctx, hipGetLastError());
+        fhip_note_kernel(ctx, "conv_depthwise3x3 channels_last strip=%d", kDwQ);
+        return 0;
+      }
       const dim3 grid((unsigned)((c.pixels + 16u * kDcClPix - 1) / (16u * kDcClPix)),
                       (unsigned)((c.cbs + 15) / 16));
       const size_t lds = (size_t)16 * c.stride * 4;

@@ -368,6 +368,11 @@ SMALL_GROUP_CASES = [
     dict(x=[3, 16, 6, 5], w=[16, 2, 1, 3], pad=[0, 1], s=[1, 2], d=[1, 1]),
     # 1-D depthwise
     dict(x=[2, 24, 50], w=[24, 1, 5], pad=[2], s=[1], d=[1]),
+    # depthwise 3x3 strips: no padding (output narrower than a strip's reach),
+    # padding 2 (output wider than the input), width a multiple of the strip
+    dict(x=[1, 16, 6, 12], w=[16, 1, 3, 3], pad=[0, 0], s=[1, 1], d=[1, 1]),
+    dict(x=[2, 24, 5, 9], w=[24, 1, 3, 3], pad=[2, 2], s=[1, 1], d=[1, 1]),
+    dict(x=[3, 264, 4, 8], w=[264, 1, 3, 3], pad=[1, 0], s=[1, 1], d=[1, 1]),
 ]
 
 
@@ -403,6 +408,28 @@ def test_conv_small_groups_channels_last_vs_oracle(ctx, case, dtype, out_dtype):
     ref = np.maximum(oracle.conv_fprop(x.logical(), w.logical(), case["pad"], case["s"],
                                        case["d"]) + bias.logical(), 0.0)
     assert_close(y.logical(), ref, od, f"{case}")
+
+
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+def test_conv_depthwise_strip_kernel_matches_general_kernel(ctx, knobs, dtype):
+    # depthwise 3x3 at unit stride runs on the strip kernel (4 output pixels
+    # and 8 channels per thread, the filter in registers); with the switch off
+    # the same call runs on the general small-group kernel.  Both add a pixel's
+    # taps in filter order, so the results agree bit for bit.
+    lay = oracle.channels_last_strides
+    xd, wd = [2, 72, 11, 13], [72, 1, 3, 3]
+    x = HT.from_logical(rand(36, 0, xd), dtype, lay(xd))
+    w = HT.from_logical(rand(36, 1, wd, std=0.3), dtype, lay(wd))
+    got = {}
+    for strips in (1, 0):
+        knobs(CONV_DEPTHWISE_STRIPS=strips)
+        got[strips] = run_conv(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.FLOAT, out_dtype=dtype,
+                               channels_last_out=True).logical()
+        name = ctx.last_kernel()
+        assert name.startswith("conv_depthwise3x3" if strips else "conv_direct channels_last"), name
+    assert np.array_equal(got[1], got[0])
+    ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
+    assert_close(got[1], ref, dtype, "depthwise strips")
 
 
 def test_conv_direct_kernels_mixed_dtypes(ctx):
