@@ -514,6 +514,35 @@ def bench_layernorm_long(ctx, steps, warmup, rows=16, cols=128 * 64 * 32):
             "note": "8 MB of X: the whole call is a few launch latencies long"}
 
 
+def bench_batchnorm_train(ctx, steps, warmup):
+    """Training batch norm with scale and bias over N32 C128 56x56 bf16,
+    channels-last: column statistics (one read of X), a per-channel finalize,
+    and the apply pass (a second read of X, mostly from the caches, and the
+    write of Y): 3 kernels per call.  Algorithmic bytes: X once + Y once."""
+    n, c, h, w = 32, 128, 56, 56
+    dims = [n, c, h, w]
+    cl = [c * h * w, 1, w * c, c]
+    d = capi.BatchNormDesc()
+    d.x = capi.TensorDesc.make(dims, cl, capi.BFLOAT16)
+    d.y = capi.TensorDesc.make(dims, cl, capi.BFLOAT16)
+    d.training = 1
+    d.has_scale = d.has_bias = 1
+    d.scale_dtype = d.bias_dtype = d.running_dtype = d.stats_dtype = capi.FLOAT
+    d.epsilon = 1e-5
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 2, "channels-last batch norm not chosen"
+    x = ctx.to_device(synth.f32_to_bf16_bits(synth.normal(12, 0, n * c * h * w)))
+    sc = ctx.to_device(synth.normal(12, 1, c, 1.0, 0.2).astype(np.float32))
+    bi = ctx.to_device(synth.normal(12, 2, c).astype(np.float32))
+    y = ctx.alloc(n * c * h * w * 2)
+    sm, sv = ctx.alloc(c * 4), ctx.alloc(c * 4)
+    wall_ms, ev_ms = timed_loop(
+        ctx, lambda i: ctx.batchnorm_fwd(d, x, y, sc, bi, None, None, sm, sv), steps, warmup)
+    nbytes = 2 * n * c * h * w * 2 + 4 * c * 4
+    return {"value": round(nbytes / ev_ms / 1e6, 1), "unit": "GB/s",
+            "frac_of_hbm_peak": round(nbytes / ev_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "call_us": round(ev_ms * 1e3, 2), "bytes": nbytes, "kernels_per_call": 3}
+
+
 def bench_conv_padded(ctx, steps, warmup):
     """The reference benchmark's conv2d_nhwc_fp16 shape: N16 C48 48x32, K48
     3x3, padding 2 -- a channel count that is no multiple of 64, so X and W
@@ -883,6 +912,8 @@ def main():
              lambda: bench_conv_depthwise(ctx, max(20, args.steps // 10), kwarm)),
             ("conv_fprop_f16_n16c48h48w32_k48r3s3_padded_channels",
              lambda: bench_conv_padded(ctx, max(20, args.steps // 4), kwarm)),
+            ("batchnorm_train_bf16_n32c128h56w56_scale_bias",
+             lambda: bench_batchnorm_train(ctx, max(20, args.steps // 10), kwarm)),
         ]
         wanted = [w for w in args.only.split(",") if w]
         for name, fn in lines:

@@ -109,6 +109,14 @@ bool fhip_fast_reduce_applicable(const fhip_reduce_desc *d);
 int fhip_fast_reduce(fhip_ctx *ctx, const fhip_reduce_desc *d, const void *x,
                      void *y);
 
+// Batch normalisation of dense channels-last tensors (column statistics with
+// whole pixel vectors per load); everything else runs on the generic kernels.
+bool fhip_fast_batchnorm_applicable(const fhip_batchnorm_desc *d);
+int fhip_fast_batchnorm(fhip_ctx *ctx, const fhip_batchnorm_desc *d, const void *x,
+                        const void *scale, const void *bias, const void *running_mean,
+                        const void *running_var, void *y, void *saved_mean,
+                        void *saved_inv_variance);
+
 bool fhip_fast_pointwise_applicable(const fhip_pointwise_desc *d);
 int fhip_fast_pointwise(fhip_ctx *ctx, const fhip_pointwise_desc *d,
                         const void *in0, const void *in1, const void *in2,

@@ -1846,7 +1846,9 @@ int fhip_batchnorm_fwd_workspace_size(const fhip_batchnorm_desc *d,
 }
 
 int fhip_batchnorm_fwd_supported(const fhip_batchnorm_desc *d) {
-  return d && batchnorm_validate(nullptr, d) == 0 ? 1 : 0;
+  if (!d || batchnorm_validate(nullptr, d) != 0)
+    return 0;
+  return fhip_fast_batchnorm_applicable(d) ? 2 : 1;
 }
 
 int fhip_batchnorm_fwd(fhip_ctx *ctx, const fhip_batchnorm_desc *d,
@@ -1872,6 +1874,10 @@ int fhip_batchnorm_fwd(fhip_ctx *ctx, const fhip_batchnorm_desc *d,
   (void)workspace;
   (void)workspace_bytes;
   FHIP_HIP_CHECK(ctx, hipSetDevice(ctx->device));
+  if (fhip_desc_volume(d->x) > 0 && fhip_fast_batchnorm_applicable(d) &&
+      (((uintptr_t)x | (uintptr_t)y) & 15) == 0)
+    return fhip_fast_batchnorm(ctx, d, x, scale, bias, running_mean, running_var, y,
+                               saved_mean, saved_inv_variance);
   fhip_note_kernel(ctx, "batchnorm_generic training=%d", (int)d->training);
   BatchNormArgs g{};
   g.x = make_dims(d->x);

@@ -84,6 +84,6 @@ def test_gradient_and_batchnorm_queries_need_no_gpu():
     b.x = b.y = capi.TensorDesc.make(xd, cl(xd), capi.BFLOAT16)
     b.running_dtype = b.stats_dtype = b.scale_dtype = b.bias_dtype = capi.FLOAT
     b.epsilon = 1e-5
-    assert lib.fhip_batchnorm_fwd_supported(b) == 1
+    assert lib.fhip_batchnorm_fwd_supported(b) == 2  # dense channels-last: the column kernels
     b.y = capi.TensorDesc.make(yd, cl(yd), capi.BFLOAT16)
     assert lib.fhip_batchnorm_fwd_supported(b) == 0

@@ -681,7 +681,7 @@ def run_batchnorm(ctx, x, *, training, eps, scale=None, bias=None, mean=None,
     d.running_dtype = mean.dtype if mean is not None else capi.FLOAT
     d.stats_dtype = stats_dtype
     d.epsilon = eps
-    assert ctx.lib.fhip_batchnorm_fwd_supported(d) == 1
+    assert ctx.lib.fhip_batchnorm_fwd_supported(d) >= 1
     up = lambda t: None if t is None else t.upload(ctx)
     sm, sv = HT.empty([c], stats_dtype), HT.empty([c], stats_dtype)
     by, bsm, bsv = y.upload(ctx), sm.upload(ctx), sv.upload(ctx)
@@ -755,6 +755,44 @@ def test_batchnorm_random_vs_oracle(ctx, dims, training, dtype, nhwc):
     if training:
         assert_close(m, rmean, capi.FLOAT, "saved mean")
         assert_close(v, rinv, capi.FLOAT, "saved inv variance")
+
+
+BN_CL_CASES = [
+    # channels-last shapes of the column kernels: one chunk of channels (256 row
+    # lanes), 17 chunks (15 row lanes, idle threads), fewer rows than row lanes,
+    # 1-D and 3-D space, f32 chunks of 4
+    ([64, 8, 5, 7], capi.BFLOAT16), ([3, 136, 9, 11], capi.HALF), ([2, 128, 1, 3], capi.BFLOAT16),
+    ([5, 40, 33], capi.HALF), ([2, 16, 3, 4, 5], capi.BFLOAT16), ([6, 12, 10, 9], capi.FLOAT),
+    ([16, 256, 28, 28], capi.BFLOAT16),
+]
+
+
+@pytest.mark.parametrize("dims,dtype", BN_CL_CASES)
+@pytest.mark.parametrize("training", [False, True])
+@pytest.mark.parametrize("affine", [False, True])
+def test_batchnorm_channels_last_kernels_vs_oracle(ctx, dims, dtype, training, affine):
+    c, eps = dims[1], 1e-3
+    x = HT.from_logical(rand(43, 0, dims, std=1.5, mean=3.0), dtype,
+                        oracle.channels_last_strides(dims))
+    sc = HT.from_logical(rand(43, 1, [c], mean=1.0, std=0.3), capi.FLOAT) if affine else None
+    b = HT.from_logical(rand(43, 2, [c]), dtype) if affine else None
+    rm = HT.from_logical(rand(43, 3, [c], mean=3.0), capi.FLOAT)
+    rv = HT.from_logical(rand(43, 4, [c], "uniform", lo=0.5, hi=3.0), capi.FLOAT)
+    y, m, v = run_batchnorm(ctx, x, training=training, eps=eps, scale=sc, bias=b,
+                            mean=None if training else rm, var=None if training else rv)
+    assert ctx.last_kernel().startswith("batchnorm_channels_last"), ctx.last_kernel()
+    ry, rmean, rinv = oracle.batchnorm(x.logical(), None if sc is None else sc.logical(),
+                                       None if b is None else b.logical(),
+                                       rm.logical(), rv.logical(), eps, training)
+    assert_close(y, ry, dtype, f"batchnorm channels-last {dims}")
+    if training:
+        assert_close(m, rmean, capi.FLOAT, "saved mean")
+        assert_close(v, rinv, capi.FLOAT, "saved inv variance")
+        # moment invariants of the output: mean_c(y) = bias, var_c(y) = scale^2 var / (var + eps)
+        axes = tuple(i for i in range(len(dims)) if i != 1)
+        tol = 2e-2 if dtype != capi.FLOAT else 1e-4
+        want_mean = 0.0 if b is None else b.logical()
+        assert np.max(np.abs(y.mean(axis=axes) - want_mean)) < tol
 
 
 def test_batchnorm_rejects_bad_descriptors(ctx):
