@@ -63,10 +63,26 @@ class HT:
         return self
 
 
+def worst_violations(got, ref, rtol, limit=8):
+    """Index, value and reference of the entries furthest outside the bar
+    |got - ref| <= rtol |ref| + rtol rms(ref) (for the failure message: where
+    a kernel went wrong says more than how far)."""
+    g = np.asarray(got, np.float64)
+    r = np.asarray(ref, np.float64)
+    finite = np.isfinite(r)
+    rms = float(np.sqrt(np.mean(r[finite] ** 2))) if finite.any() else 0.0
+    excess = np.where(finite, np.abs(g - r) - (rtol * np.abs(r) + rtol * rms), 0.0)
+    excess = np.nan_to_num(excess, nan=np.inf)
+    order = np.argsort(excess, axis=None)[::-1][:limit]
+    return [(tuple(int(i) for i in np.unravel_index(o, g.shape)), float(g.flat[o]), float(r.flat[o]))
+            for o in order if excess.flat[o] > 0]
+
+
 def assert_close(got, ref, dtype, what="", rtol=None):
     rtol = RTOL[dtype] if rtol is None else rtol
     ok, rep = oracle.check_close(got, ref, rtol)
-    assert ok, f"{what}: {rep} (rtol {rtol})"
+    assert ok, (f"{what}: {rep} (rtol {rtol}); worst (index, got, ref): "
+                f"{worst_violations(got, ref, rtol)}")
 
 
 def rand(seed, tid, dims, kind="normal", **kw):
