@@ -28,7 +28,11 @@
 //     MFMAs, across block boundaries, and a block's epilogue and store are
 //     issued while the SIMD's other wavefront keeps the matrix pipe busy.
 //
-// Reference semantics: aten.convolution, groups = 1 (reference
+// Grouped convolutions of 64 -> 64 channels per group run on the same kernel
+// with two groups per workgroup: the slab holds both groups' input channels
+// of a pixel and a wavefront reads the half of its channel slice's group.
+//
+// Reference semantics: aten.convolution (reference
 // support/asm_emitter.h:690-701, node/conv_node.h:38-56) followed by the fused
 // pointwise chain (support/asm_emitter.h:1806-2122).
 #include "common.h"
@@ -64,8 +68,12 @@ constexpr int kRfMaxNI = 16;     // KB of LDS per slab row, at most
 constexpr int rf_wait_lgkm_imm(int n) { return 0xF | (0x7 << 4) | (n << 8) | (0x3 << 14); }
 
 // Compile-time geometry shared by the kernel and the host's LDS budget.
-template <int C, int R, int S> struct RfGeom {
-  static constexpr int kCPP = C * 2 / 16 + 1;   // chunks per slab pixel (one is padding)
+// GW: groups of the convolution that a workgroup's 128 output channels span
+// (1, or 2 groups of 64 -> 64 channels: the slab then holds both groups' C
+// input channels of a pixel, and a channel slice reads its group's half).
+template <int C, int R, int S, int GW = 1> struct RfGeom {
+  static constexpr int kCS = C * GW;            // input channels of a slab pixel
+  static constexpr int kCPP = kCS * 2 / 16 + 1; // chunks per slab pixel (one is padding)
   static constexpr int kNK = R * S * (C / 32);  // K-steps of 32 channels
   static constexpr int kNKA = kNK / 4 * 2;      // K-steps staged in front of the slab
   // filter stages: per channel slice two KB per K-step (one per 16-channel tile)
@@ -77,7 +85,8 @@ struct ConvRfArgs {
   const char *x, *w;
   char *out;
   int32_t N, H, W, P, Q;
-  int32_t K;               // output channels, a multiple of 128
+  int32_t K;               // output channels (of all groups), a multiple of 128
+  int32_t x_pitch;         // bytes between pixels of X (all groups' channels)
   int32_t pad_h, pad_w;
   int32_t TR;              // output rows per tile
   int32_t tiles_per_image; // ceil(P / TR)
@@ -116,7 +125,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rf_rsrc(const void *base,
       (int)__builtin_amdgcn_readfirstlane(bytes), 0x00020000);
 }
 
-template <int KIND, int C, int R, int S, bool RELU, bool UNIT>
+template <int KIND, int C, int R, int S, bool RELU, bool UNIT, int GW>
 __global__ __launch_bounds__(kRfThreads)
 __attribute__((amdgpu_waves_per_eu(2, 2))) void
 conv_rf_kernel(ConvRfArgs g) {
@@ -138,17 +147,18 @@ conv_rf_kernel(ConvRfArgs g) {
   const uint32_t a_x_bytes = g.x_bytes;
   const uint32_t a_w_bytes = g.w_bytes;
   const int a_nops = g.nops;
-  constexpr int CPP = RfGeom<C, R, S>::kCPP; // 16-byte chunks per slab pixel
+  constexpr int CPP = RfGeom<C, R, S, GW>::kCPP; // 16-byte chunks per slab pixel
+  constexpr int CS = RfGeom<C, R, S, GW>::kCS;   // input channels of a slab pixel
   constexpr int PITCH = CPP * 16;
   constexpr int KPT = C / 32;                // K-steps per filter tap
-  constexpr int NK = RfGeom<C, R, S>::kNK;   // K-steps
-  constexpr int NKA = RfGeom<C, R, S>::kNKA; // K-steps of the filter's first part
+  constexpr int NK = RfGeom<C, R, S, GW>::kNK;   // K-steps
+  constexpr int NKA = RfGeom<C, R, S, GW>::kNKA; // K-steps of the filter's first part
   // fragment buffers (K-steps in flight); a divisor of NK, so that a block's
   // K-step j always sits in buffer j % RING
   constexpr int RING = NK % 6 == 0 ? 6 : (NK % 4 == 0 ? 4 : 3);
   constexpr int FROW = R * S * C * 2;        // bytes of a filter row
   static_assert(C % 64 == 0 && NK % RING == 0 && NKA % 2 == 0, "filter shape outside this kernel");
-  static_assert((S - 1) * PITCH + (KPT - 1) * 64 + 48 < 65536, "ds offset range");
+  static_assert((S - 1) * PITCH + (GW - 1) * C * 2 + (KPT - 1) * 64 + 48 < 65536, "ds offset range");
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
@@ -160,7 +170,7 @@ conv_rf_kernel(ConvRfArgs g) {
   const uint32_t rowpitch = (uint32_t)a_NI * 1024u;
   // LDS: [block counters, 1 KB | filter stage | slab (first: rest of the filter)]
   const uint32_t lds_f = lds0 + 1024u + (uint32_t)slice * (NKA * 2 * 1024);
-  const uint32_t lds_s = lds0 + 1024u + RfGeom<C, R, S>::kStageBytes;
+  const uint32_t lds_s = lds0 + 1024u + RfGeom<C, R, S, GW>::kStageBytes;
 
   // this workgroup's channel group stays fixed; tiles are strided over
   const int kg = (int)(blockIdx.x % (unsigned)a_kgroups);
@@ -259,7 +269,8 @@ conv_rf_kernel(ConvRfArgs g) {
     const int c = xk - sp * CPP;
     const int iw = sp - a_pad_w;
     const bool ok = c < CPP - 1 && (unsigned)iw < (unsigned)a_W;
-    rel[i] = ok ? (uint32_t)(iw * (C * 2) + c * 16) : 0x80000000u;
+    rel[i] = ok ? (uint32_t)(iw * g.x_pitch + (GW > 1 ? kg * (CS * 2) : 0) + c * 16)
+                : 0x80000000u;
   }
   const int npr = wave + 8 < a_NI ? 2 : (wave < a_NI ? 1 : 0); // instructions per row
   auto slab_rows = [&](int rows_in, int n, int ih0) __attribute__((always_inline)) {
@@ -267,7 +278,7 @@ conv_rf_kernel(ConvRfArgs g) {
       const int ih = ih0 + sr;
       const bool row_ok = (unsigned)ih < (unsigned)a_H;
       const __amdgpu_buffer_rsrc_t rs = row_ok ? rx : rnone;
-      const int soff = row_ok ? ((n * a_H + ih) * a_W) * (C * 2) : 0;
+      const int soff = row_ok ? ((n * a_H + ih) * a_W) * g.x_pitch : 0;
       const uint32_t dst = lds_s + (uint32_t)sr * rowpitch + (uint32_t)wave * 1024u;
       if (npr > 0)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -389,7 +400,8 @@ conv_rf_kernel(ConvRfArgs g) {
       const int plc = pl < npix ? pl : npix - 1;
       const int prow = (int)conv_div(plc, a_Q, a_magic_q);
       const int pcol = plc - prow * a_Q;
-      base = lds_s + (uint32_t)prow * rowpitch + (uint32_t)pcol * PITCH + (uint32_t)q * 16u;
+      base = lds_s + (uint32_t)prow * rowpitch + (uint32_t)pcol * PITCH + (uint32_t)q * 16u +
+             (GW > 1 ? (uint32_t)(slice >> 1) * (C * 2) : 0u);
       ooff = pl < npix ? (uint32_t)pl * (uint32_t)a_K * 2u + lane_out : 0x80000000u;
     };
     u32x4 frag[RING];
@@ -512,7 +524,8 @@ conv_rf_kernel(ConvRfArgs g) {
 struct RfPlan {
   bool ok = false;
   int kind = 0;
-  int C = 0, R = 0, S = 0;
+  int C = 0, R = 0, S = 0; // C: input channels of a group
+  int gw = 1;              // groups per workgroup
   bool relu = false;
   ConvRfArgs a{};
   int lds = 0;
@@ -558,9 +571,15 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
     return p;
   if (d->y.dtype != FHIP_FLOAT && !(d->epilogue.count == 0 && d->y.dtype == d->out.dtype))
     return p;
-  const int64_t C = d->x.dim[1], K = d->w.dim[0];
-  if (d->w.dim[1] != C || K % kRfChannels != 0)
+  // C: input channels of a group.  One group, or an even number of groups of
+  // 64 -> 64 channels (a workgroup's 128 output channels are then two groups)
+  const int64_t Call = d->x.dim[1], C = d->w.dim[1], K = d->w.dim[0];
+  if (C <= 0 || Call % C != 0 || K % kRfChannels != 0)
     return p;
+  const int64_t groups = Call / C;
+  if (groups != 1 && !(groups % 2 == 0 && C == 64 && K == groups * 64))
+    return p;
+  p.gw = groups == 1 ? 1 : 2;
   const int64_t R = d->w.dim[2], S = d->w.dim[3];
   if (!rf_instance((int)C, (int)R, (int)S))
     return p;
@@ -576,7 +595,8 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   a.pad_h = (int32_t)d->padding[0], a.pad_w = (int32_t)d->padding[1];
   if (a.P != a.H + 2 * a.pad_h - (int)R + 1 || a.Q != a.W + 2 * a.pad_w - (int)S + 1)
     return p;
-  const int64_t x_bytes = (int64_t)a.N * a.H * a.W * C * 2;
+  const int64_t x_bytes = (int64_t)a.N * a.H * a.W * Call * 2;
+  a.x_pitch = (int32_t)(Call * 2);
   const int64_t o_tile_max = (int64_t)a.P * a.Q * K * 2;
   if (x_bytes >= (1ll << 31) || o_tile_max >= (1ll << 31) || K * R * S * C * 2 >= (1ll << 31))
     return p;
@@ -626,7 +646,7 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   a.nops = nops;
   a.o_dt = d->out.dtype;
   // slab geometry
-  const int cpp = (int)C * 2 / 16 + 1;
+  const int cpp = (int)C * p.gw * 2 / 16 + 1;
   const int wp = a.W + (int)S - 1 + 0; // = W + 2 * pad_w
   if (a.W + 2 * a.pad_w != a.Q + (int)S - 1)
     return p;
@@ -686,9 +706,9 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   return p;
 }
 
-template <int KIND, int C, int R, int S, bool RELU, bool UNIT>
+template <int KIND, int C, int R, int S, bool RELU, bool UNIT, int GW>
 int rf_launch(fhip_ctx *ctx, const RfPlan &p) {
-  auto kernel = conv_rf_kernel<KIND, C, R, S, RELU, UNIT>;
+  auto kernel = conv_rf_kernel<KIND, C, R, S, RELU, UNIT, GW>;
   static FhipOncePerDevice configured;
   if (!configured.done(ctx->device)) {
     FHIP_HIP_CHECK(ctx, hipFuncSetAttribute(
@@ -700,23 +720,28 @@ int rf_launch(fhip_ctx *ctx, const RfPlan &p) {
   hipLaunchKernelGGL(kernel, dim3((unsigned)p.grid), dim3(kRfThreads), p.lds,
                      ctx->stream, p.a);
   FHIP_HIP_CHECK(ctx, hipGetLastError());
-  fhip_note_kernel(ctx, "conv_rf c=%d r=%d s=%d rows=%d relu=%d unit=%d", C, R, S, p.a.TR,
-                   (int)RELU, (int)UNIT);
+  if (GW > 1)
+    fhip_note_kernel(ctx, "conv_rf c=%d r=%d s=%d rows=%d relu=%d unit=%d groups_per_wg=%d", C, R,
+                     S, p.a.TR, (int)RELU, (int)UNIT, GW);
+  else
+    fhip_note_kernel(ctx, "conv_rf c=%d r=%d s=%d rows=%d relu=%d unit=%d", C, R, S, p.a.TR,
+                     (int)RELU, (int)UNIT);
   return 0;
 }
 
-template <int KIND, int C, int R, int S>
+template <int KIND, int C, int R, int S, int GW>
 int rf_launch_relu(fhip_ctx *ctx, const RfPlan &p) {
   if (p.a.unit_scale)
-    return p.relu ? rf_launch<KIND, C, R, S, true, true>(ctx, p)
-                  : rf_launch<KIND, C, R, S, false, true>(ctx, p);
-  return p.relu ? rf_launch<KIND, C, R, S, true, false>(ctx, p)
-                : rf_launch<KIND, C, R, S, false, false>(ctx, p);
+    return p.relu ? rf_launch<KIND, C, R, S, true, true, GW>(ctx, p)
+                  : rf_launch<KIND, C, R, S, false, true, GW>(ctx, p);
+  return p.relu ? rf_launch<KIND, C, R, S, true, false, GW>(ctx, p)
+                : rf_launch<KIND, C, R, S, false, false, GW>(ctx, p);
 }
 
 template <int KIND> int rf_launch_shape(fhip_ctx *ctx, const RfPlan &p) {
   if (p.C == 64 && p.R == 3 && p.S == 3)
-    return rf_launch_relu<KIND, 64, 3, 3>(ctx, p);
+    return p.gw == 2 ? rf_launch_relu<KIND, 64, 3, 3, 2>(ctx, p)
+                     : rf_launch_relu<KIND, 64, 3, 3, 1>(ctx, p);
   return fhip_fail(ctx, "conv: no register-filter kernel for this filter");
 }
 

@@ -384,7 +384,8 @@ def test_conv_igemm_headline_shape(ctx):
 @pytest.mark.parametrize("shape", ["groups4", "depthwise"])
 def test_conv_grouped_benchmark_shapes(ctx, shape):
     """The two grouped lines of the benchmark at full size (N32 56x56, 3x3,
-    padding 1, bf16): 4 groups of 64 -> 64 channels on the MFMA kernel and a
+    padding 1, bf16): 4 groups of 64 -> 64 channels on the register-filter
+    kernel (two groups per workgroup) and a
     depthwise convolution over 128 channels on the small-group kernel.
     All-ones tensors have closed-form answers (channels of a group times the
     taps inside the image) on every pixel; random data is checked against the
@@ -395,6 +396,9 @@ def test_conv_grouped_benchmark_shapes(ctx, shape):
     ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
     ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
     lg = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+    if shape == "groups4":
+        assert ctx.last_kernel().startswith("conv_rf c=64 r=3 s=3") and \
+            ctx.last_kernel().endswith("groups_per_wg=2"), ctx.last_kernel()
     taps = np.full(56, 3.0); taps[[0, -1]] = 2.0
     expect = float(cg) * taps[:, None] * taps[None, :]
     assert np.array_equal(lg, np.broadcast_to(expect, lg.shape))
@@ -460,6 +464,51 @@ def test_conv_register_filter_kernel_vs_oracle(ctx, knobs, case, dtype, epi_kind
         got[rows] = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=dtype,
                         epilogue=epi, epi_tensors=ops).logical()
         assert_close(got[rows], ref, dtype, f"rows={rows} {case} {epi_kind}")
+
+
+RF_GROUPED_CASES = [
+    # groups of 64 -> 64 channels, two per workgroup; rows per tile forced
+    dict(x=[2, 128, 13, 21], pad=[1, 1], rows=4),   # one pair of groups
+    dict(x=[1, 256, 9, 17], pad=[1, 1], rows=1),    # two pairs, one row per tile
+    dict(x=[3, 384, 12, 19], pad=[0, 0], rows=5),   # three pairs, no padding
+    dict(x=[40, 128, 16, 8], pad=[1, 1], rows=2),   # workgroups walk several tiles
+    dict(x=[2, 256, 6, 50], pad=[1, 2], rows=2),    # wide rows, asymmetric padding
+]
+
+
+@pytest.mark.parametrize("case", RF_GROUPED_CASES)
+@pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
+@pytest.mark.parametrize("epi_kind", ["bias_relu", "none"])
+def test_conv_register_filter_kernel_grouped_vs_oracle(ctx, knobs, case, dtype, epi_kind):
+    # Reference: aten.convolution's groups operand (reference
+    # support/asm_emitter.h:690-701).  The same problem on the register-filter
+    # kernel (two groups per workgroup) and on the tiled kernel (one GEMM per
+    # group), both against the oracle; distinct random data per group, so a
+    # slice reading the other group's half of a slab pixel cannot pass.
+    xd = case["x"]
+    k = xd[1]
+    wd = [k, 64, 3, 3]
+    pad, st, dil = case["pad"], [1, 1], [1, 1]
+    x = cl(xd, 51, 0, dtype)
+    w = cl(wd, 51, 1, dtype, std=0.05)
+    bias = HT.from_logical(rand(51, 2, [1, k, 1, 1]), dtype,
+                           oracle.channels_last_strides([1, k, 1, 1]))
+    ref = oracle.conv_fprop(x.logical(), w.logical(), pad, st, dil)
+    if epi_kind == "bias_relu":
+        epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0,
+                                operand=bias.desc()),
+               capi.epilogue_op(capi.PW["RELU_FWD"], dtype)]
+        ops = [bias]
+        ref = np.maximum(ref + bias.logical(), 0.0)
+    else:
+        epi, ops = [], []
+    for rows in (case["rows"], 0):
+        knobs(CONV_ROWS=rows)
+        got = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=dtype,
+                  epilogue=epi, epi_tensors=ops).logical()
+        name = ctx.last_kernel()
+        assert ("groups_per_wg=2" in name) == (rows != 0), name
+        assert_close(got, ref, dtype, f"rows={rows} {case} {epi_kind}")
 
 
 def test_conv_register_filter_kernel_chosen_rows(ctx, knobs):
