@@ -93,6 +93,9 @@ struct ConvRfArgs {
   int32_t ntiles;          // N * tiles_per_image
   int32_t kgroups;         // K / 128
   int32_t NI;              // 1 KB LDS-DMA instructions per slab row
+  int32_t slab_org;        // LDS byte offset of slab row 0
+  int32_t slab_rows;       // slab rows that fit LDS from there
+  int32_t first_row;       // slab row of a workgroup's first tile (clear of the filter stage)
   uint32_t magic_q, magic_ni;
   uint32_t x_bytes, w_bytes;
   int32_t o_dt;
@@ -168,14 +171,22 @@ conv_rf_kernel(ConvRfArgs g) {
   const int l = threadIdx.x & 63;
   const int px = l & 15, q = l >> 4;
   const uint32_t rowpitch = (uint32_t)a_NI * 1024u;
-  // LDS: [block counters, 1 KB | filter stage | slab (first: rest of the filter)]
+  // LDS: [block counters, 1 KB | filter stage | rest of the filter]; the slab
+  // is a grid of rows over all of it above the counters, a workgroup's first
+  // tile in the rows behind the filter stage (in the place of the filter's
+  // second part, which has left LDS by then)
   const uint32_t lds_f = lds0 + 1024u + (uint32_t)slice * (NKA * 2 * 1024);
-  const uint32_t lds_s = lds0 + 1024u + RfGeom<C, R, S, GW>::kStageBytes;
+  const uint32_t lds_b = lds0 + 1024u + RfGeom<C, R, S, GW>::kStageBytes;
+  const uint32_t slab_org = lds0 + (uint32_t)g.slab_org;
+  const int a_slab_rows = g.slab_rows;
 
-  // this workgroup's channel group stays fixed; tiles are strided over
+  // this workgroup's channel group stays fixed; it takes a run of consecutive
+  // tiles (consecutive row bands of an image share their halo rows in LDS)
   const int kg = (int)(blockIdx.x % (unsigned)a_kgroups);
-  const int tile0 = (int)(blockIdx.x / (unsigned)a_kgroups);
-  const int tile_step = (int)(gridDim.x / (unsigned)a_kgroups);
+  const int wg = (int)(blockIdx.x / (unsigned)a_kgroups);
+  const int nwg = (int)(gridDim.x / (unsigned)a_kgroups);
+  const int tile_end = (int)(((int64_t)(wg + 1) * a_ntiles) / nwg);
+  int tile = (int)(((int64_t)wg * a_ntiles) / nwg);
   const int ch_wave = kg * kRfChannels + slice * 32;
   RF_STAMP(0);
 
@@ -210,7 +221,7 @@ conv_rf_kernel(ConvRfArgs g) {
     const int ch = ch_wave + 8 * (rho >> 2) + 4 * half + (rho & 3);
     fvoff[h] = (uint32_t)ch * (uint32_t)FROW + (uint32_t)chunk * 16u;
   }
-  const uint32_t lds_f2 = lds_s + (uint32_t)slice * ((NK - NKA) * 2 * 1024);
+  const uint32_t lds_f2 = lds_b + (uint32_t)slice * ((NK - NKA) * 2 * 1024);
   uint32_t fread[2]; // per K-step parity, relative to the stage of the slice
 #pragma unroll
   for (int jo = 0; jo < 2; ++jo) {
@@ -273,13 +284,14 @@ conv_rf_kernel(ConvRfArgs g) {
                 : 0x80000000u;
   }
   const int npr = wave + 8 < a_NI ? 2 : (wave < a_NI ? 1 : 0); // instructions per row
-  auto slab_rows = [&](int rows_in, int n, int ih0) __attribute__((always_inline)) {
-    for (int sr = 0; sr < rows_in; ++sr) {
+  // `count` input rows from row ih0 of image n into the slab rows from `row`
+  auto slab_rows = [&](int count, int n, int ih0, int row) __attribute__((always_inline)) {
+    for (int sr = 0; sr < count; ++sr) {
       const int ih = ih0 + sr;
       const bool row_ok = (unsigned)ih < (unsigned)a_H;
       const __amdgpu_buffer_rsrc_t rs = row_ok ? rx : rnone;
       const int soff = row_ok ? ((n * a_H + ih) * a_W) * g.x_pitch : 0;
-      const uint32_t dst = lds_s + (uint32_t)sr * rowpitch + (uint32_t)wave * 1024u;
+      const uint32_t dst = slab_org + (uint32_t)(row + sr) * rowpitch + (uint32_t)wave * 1024u;
       if (npr > 0)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
             rs, (GEMM_AS3 char *)__builtin_amdgcn_readfirstlane(dst), 16, (int)rel[0], soff, 0, 0);
@@ -290,8 +302,9 @@ conv_rf_kernel(ConvRfArgs g) {
     }
   };
 
-  // block counter of the slice, in the KB at the bottom of LDS
-  const uint32_t draw = lds0 + (uint32_t)slice * 4u;
+  // block counters of the slice (one per tile parity), in the KB at the bottom of LDS
+  const uint32_t draw0 = lds0 + (uint32_t)slice * 8u;
+  uint32_t draw = draw0;
   auto draw_block = [&]() __attribute__((always_inline)) {
     // one LDS atomic of lane 0; the result is in flight when this returns (the
     // compiler does not know: the reader waits by count, LDS answers in order)
@@ -306,76 +319,74 @@ conv_rf_kernel(ConvRfArgs g) {
                  : "memory");
     return v;
   };
-  bool first = true; // the filter is still on its way
-  for (int tile = tile0; tile < a_ntiles; tile += tile_step) {
-    const int n = tile / a_tiles_per_image;
-    const int p0 = (tile - n * a_tiles_per_image) * a_TR;
-    const int tr = a_P - p0 < a_TR ? a_P - p0 : a_TR;
-    const int npix = tr * a_Q;
-    const int rows_in = tr + R - 1;
-    const int ih0 = p0 - a_pad_h;
+  // image, first output row, output rows and first input row of a tile
+  auto tile_geom = [&](int t, int &n, int &p0, int &tr, int &ih0) __attribute__((always_inline)) {
+    n = t / a_tiles_per_image;
+    p0 = (t - n * a_tiles_per_image) * a_TR;
+    tr = a_P - p0 < a_TR ? a_P - p0 : a_TR;
+    ih0 = p0 - a_pad_h;
+  };
+  int n, p0, tr, ih0;
+  tile_geom(tile, n, p0, tr, ih0);
+  int srow = g.first_row; // the tile's first slab row
 
-    if (first) {
-      RF_STAMP(15);
-      // ---- epilogue constants: y = acc * sc[c] + sh[c] for the lane's 8 channels
+  {
+    RF_STAMP(15);
+    // ---- epilogue constants: y = acc * sc[c] + sh[c] for the lane's 8 channels
 #pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        sc[c] = 1.f;
-        sh[c] = 0.f;
-      }
-      for (int e = 0; e < a_nops; ++e) {
-        const DevEpiOp &o = g.epi.op[e];
-        // the 8 operand values of an op are fetched by loads issued back to back
-        float ovs[8];
+    for (int c = 0; c < 8; ++c) {
+      sc[c] = 1.f;
+      sh[c] = 0.f;
+    }
+    for (int e = 0; e < a_nops; ++e) {
+      const DevEpiOp &o = g.epi.op[e];
+      // the 8 operand values of an op are fetched by loads issued back to back
+      float ovs[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        ovs[c] = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
+      if (o.kind == FHIP_OPERAND_TENSOR) {
+        int64_t off[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c)
-          ovs[c] = o.kind == FHIP_OPERAND_SCALAR ? o.scalar : 0.f;
-        if (o.kind == FHIP_OPERAND_TENSOR) {
-          int64_t off[8];
+          off[c] = (int64_t)(ch_wave + 8 * q + c) * o.stride[2];
+        load_operand_vec<8>(o.ptr, o.operand_dtype, off, ovs);
+      }
 #pragma unroll
-          for (int c = 0; c < 8; ++c)
-            off[c] = (int64_t)(ch_wave + 8 * q + c) * o.stride[2];
-          load_operand_vec<8>(o.ptr, o.operand_dtype, off, ovs);
-        }
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-          const float ov = ovs[c];
-          if (g.lin_mul[e]) {
-            sc[c] *= ov;
-            sh[c] *= ov;
-          } else {
-            sc[c] *= g.lin_a[e];
-            sh[c] = sh[c] * g.lin_a[e] + g.lin_b[e] * ov;
-          }
+      for (int c = 0; c < 8; ++c) {
+        const float ov = ovs[c];
+        if (g.lin_mul[e]) {
+          sc[c] *= ov;
+          sh[c] *= ov;
+        } else {
+          sc[c] *= g.lin_a[e];
+          sh[c] = sh[c] * g.lin_a[e] + g.lin_b[e] * ov;
         }
       }
-      // with unit scales (UNIT: the host found every op additive with factor
-      // 1) the shift is the accumulators' start value and the multiply-add
-      // drops out of the epilogue
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          acc0[t][i] = UNIT ? sh[4 * t + i] : 0.f;
-      RF_STAMP(1);
-      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
-      RF_STAMP(2);
-      gemm_barrier();
-      RF_STAMP(3);
-      // the second part leaves the slab's place first; the first part is read
-      // while the slab's loads are in flight
-      filter_read(JA1{}, JB1{}, lds_f2);
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
-      RF_STAMP(6);
-      gemm_barrier();
     }
-    slab_rows(rows_in, n, ih0);
+    // with unit scales (UNIT: the host found every op additive with factor
+    // 1) the shift is the accumulators' start value and the multiply-add
+    // drops out of the epilogue
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        acc0[t][i] = UNIT ? sh[4 * t + i] : 0.f;
+    RF_STAMP(1);
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+    RF_STAMP(2);
+    gemm_barrier();
+    RF_STAMP(3);
+    // the second part leaves the slab's place first; the first part is read
+    // while the slab's loads are in flight
+    filter_read(JA1{}, JB1{}, lds_f2);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
+    RF_STAMP(6);
+    gemm_barrier();
+    slab_rows(tr + R - 1, n, ih0, srow);
     RF_STAMP(7);
-    if (first) {
-      filter_read(JA0{}, JA1{}, lds_f);
-      first = false;
-    }
+    filter_read(JA0{}, JA1{}, lds_f);
     // the two wavefronts of a slice draw their blocks from a counter (the
     // first two are dealt out): the SIMD serves its older wavefront first, so
     // equal shares would leave the younger one to finish alone
@@ -385,6 +396,40 @@ conv_rf_kernel(ConvRfArgs g) {
     RF_STAMP(9);
     gemm_barrier();
     RF_STAMP(10);
+  }
+
+  for (;;) {
+    const int npix = tr * a_Q;
+    const uint32_t lds_s = slab_org + (uint32_t)srow * rowpitch;
+
+    // ---- the next tile's rows are requested now and land during this tile's
+    // blocks.  Below this tile in the same image it starts on this tile's last
+    // R - 1 rows and only the new rows are loaded; otherwise it goes to the
+    // slab rows in front of this tile's or behind them, wherever it fits; when
+    // it fits nowhere its rows are loaded once this tile is done.
+    const bool more = tile + 1 < tile_end;
+    int n2 = n, p02 = p0, tr2 = tr, ih02 = ih0, srow2 = 0;
+    bool deferred = false;
+    if (more) {
+      tile_geom(tile + 1, n2, p02, tr2, ih02);
+      const int rows_in = tr + R - 1, rows_in2 = tr2 + R - 1;
+      int skip = 0;
+      if (n2 == n && srow + tr + rows_in2 <= a_slab_rows) {
+        srow2 = srow + tr;
+        skip = R - 1;
+      } else if (srow >= rows_in2) {
+        srow2 = 0;
+      } else if (srow + rows_in + rows_in2 <= a_slab_rows) {
+        srow2 = srow + rows_in;
+      } else {
+        deferred = true;
+      }
+      if (!deferred)
+        slab_rows(rows_in2 - skip, n2, ih02 + skip, srow2 + skip);
+      // the other counter: its last draws were the tile's before this one
+      if (half == 0 && l == 0)
+        *(GEMM_AS3 uint32_t *)(uintptr_t)(draw ^ 4u) = 2u;
+    }
 
     // outputs of this tile: dense rows of K channels, pixel index tile-relative
     const __amdgpu_buffer_rsrc_t ro =
@@ -512,11 +557,20 @@ conv_rf_kernel(ConvRfArgs g) {
       b = nb;
     }
     RF_STAMP(12);
-    // every wavefront is done with the slab before the next tile overwrites it
-    if (tile + tile_step < a_ntiles) {
+    if (!more)
+      break;
+    if (deferred) {
+      // every wavefront is done with the slab before the next tile overwrites it
       __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
       gemm_barrier();
+      slab_rows(tr2 + R - 1, n2, ih02, 0);
     }
+    // the next tile's rows are in LDS, and every wavefront has left this tile
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
+    gemm_barrier();
+    ++tile;
+    n = n2, p0 = p02, tr = tr2, ih0 = ih02, srow = srow2;
+    draw ^= 4u;
   }
   RF_STAMP(13);
 }
@@ -655,26 +709,88 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   if (a.NI > kRfMaxNI)
     return p;
   // LDS: a KB of block counters, the stage of the filter's first part, and
-  // the slab, whose place first stages the filter's second part
+  // the slab, whose place first stages the filter's second part.  The slab's
+  // rows form a grid anchored so that a row starts right behind the stage:
+  // that row takes a workgroup's first tile, the rows in front of it (over the
+  // stage, free once the filter is in registers) serve later tiles.
   const int nk = (int)(R * S * (C / 32));
   const int stage = 4 * (nk / 4 * 2) * 2 * 1024;
   const int stage2 = 4 * (nk - nk / 4 * 2) * 2 * 1024;
-  const int64_t lds_cap = 160 * 1024 - stage - 1024;
-  // rows per tile: the choice that fills whole rounds of the machine best
+  const int lds_max = 160 * 1024;
+  const int rowpitch = a.NI * 1024;
+  const int first_row = stage / rowpitch;
+  const int slab_org = 1024 + stage - first_row * rowpitch;
+  const int rows_max = (lds_max - slab_org) / rowpitch; // slab rows with all of LDS
+  // rows per tile: the choice that keeps the machine busiest
   const int cus = num_cus > 0 ? num_cus : 256;
   const int kgroups = (int)(K / kRfChannels);
+  const int64_t slots = (int64_t)cus / kgroups * kgroups > 0 ? (int64_t)cus / kgroups * kgroups : kgroups;
+  // Cost of a workgroup's run of tiles [t0, t1), in units of 1/16 of a block of
+  // a wavefront: the placement rules of the kernel, a tile's blocks on the
+  // busier wavefront of a pair, and the rows loaded for the next tile, which
+  // hide behind the blocks unless they had to wait for them.
+  auto run_cost = [&](int tr_full, int t0, int t1) {
+    const int tpi = (a.P + tr_full - 1) / tr_full;
+    double cost = 96; // filter, first slab, pipeline fill
+    int srow = first_row;
+    for (int t = t0; t < t1; ++t) {
+      const int n = t / tpi, p0 = (t - n * tpi) * tr_full;
+      const int tr = a.P - p0 < tr_full ? a.P - p0 : tr_full;
+      const int64_t blocks = ((int64_t)tr * a.Q + 15) / 16;
+      const double compute = (double)((blocks + 1) / 2 * 16 + 8);
+      if (t + 1 == t1) {
+        cost += compute;
+        break;
+      }
+      const int n2 = (t + 1) / tpi, p02 = (t + 1 - n2 * tpi) * tr_full;
+      const int tr2 = a.P - p02 < tr_full ? a.P - p02 : tr_full;
+      const int rows_in = tr + (int)R - 1, rows_in2 = tr2 + (int)R - 1;
+      int loaded = rows_in2;
+      bool deferred = false;
+      if (n2 == n && srow + tr + rows_in2 <= rows_max) {
+        srow += tr;
+        loaded = tr2;
+      } else if (srow >= rows_in2) {
+        srow = 0;
+      } else if (srow + rows_in + rows_in2 <= rows_max) {
+        srow += rows_in;
+      } else {
+        srow = 0;
+        deferred = true;
+      }
+      const double load = (double)loaded * a.NI * 2.5;
+      cost += deferred ? compute + load : (compute > load ? compute : load);
+    }
+    return cost;
+  };
   double best = 0;
   int best_tr = 0;
   for (int tr = 1; tr <= a.P; ++tr) {
-    const int64_t lds = (int64_t)(tr + R - 1) * a.NI * 1024;
-    if (lds > lds_cap)
+    if ((tr + (int)R - 1) * rowpitch > lds_max - 1024 - stage)
       break;
-    const int64_t tiles = (int64_t)a.N * ((a.P + tr - 1) / tr) * kgroups;
-    const int64_t rounds = (tiles + cus - 1) / cus;
-    const int64_t blocks = ((int64_t)tr * a.Q + 15) / 16;
-    // time of a round ~ the blocks of the busier wavefront of a pair plus a
-    // fixed set-up share
-    const double cost = (double)rounds * ((blocks + 1) / 2 * 2 * 16 + 96);
+    const int64_t ntiles = (int64_t)a.N * ((a.P + tr - 1) / tr);
+    if (ntiles >= (1 << 24))
+      continue;
+    const int64_t items = ntiles * kgroups;
+    const int64_t nwg = (items < slots ? items : slots) / kgroups;
+    // the longest runs: the first workgroup with a run of the larger size,
+    // from its first tile (the runs differ in where they meet image borders)
+    double cost = 0;
+    const int64_t probes[3] = {0, nwg / 2, nwg - 1};
+    for (int64_t wi : probes) {
+      const double c = run_cost(tr, (int)(wi * ntiles / nwg), (int)((wi + 1) * ntiles / nwg));
+      cost = c > cost ? c : cost;
+    }
+    if (ntiles % nwg != 0) {
+      int64_t wi = 0;
+      const int64_t big = ntiles / nwg + 1;
+      while (wi < nwg && (wi + 1) * ntiles / nwg - wi * ntiles / nwg != big)
+        ++wi;
+      if (wi < nwg) {
+        const double c = run_cost(tr, (int)(wi * ntiles / nwg), (int)((wi + 1) * ntiles / nwg));
+        cost = c > cost ? c : cost;
+      }
+    }
     const double eff = (double)a.N * a.P * a.Q * kgroups / (cost * cus);
     if (eff > best + 1e-9) {
       best = eff;
@@ -682,7 +798,7 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
     }
   }
   if (knobs.conv_rows > 0 && knobs.conv_rows <= a.P &&
-      (int64_t)(knobs.conv_rows + R - 1) * a.NI * 1024 <= lds_cap)
+      (knobs.conv_rows + (int)R - 1) * rowpitch <= lds_max - 1024 - stage)
     best_tr = knobs.conv_rows;
   if (best_tr == 0)
     return p;
@@ -696,12 +812,15 @@ RfPlan make_rf_plan(const fhip_conv_desc *d, int num_cus) {
   a.magic_q = conv_magic(a.Q);
   a.magic_ni = conv_magic(a.NI);
   p.C = (int)C, p.R = (int)R, p.S = (int)S;
-  // (the slab's place also stages the second part of the filter)
-  const int slab_bytes = (a.TR + (int)R - 1) * a.NI * 1024;
-  p.lds = 1024 + stage + (slab_bytes > stage2 ? slab_bytes : stage2);
   const int64_t items = (int64_t)a.ntiles * kgroups;
-  const int64_t slots = (int64_t)cus / kgroups * kgroups > 0 ? (int64_t)cus / kgroups * kgroups : kgroups;
   p.grid = (int)(items < slots ? items : slots);
+  // one tile per workgroup: the first tile's rows behind the stage (or the
+  // second part of the filter, if that is larger); more: all of LDS
+  const int slab_bytes = (a.TR + (int)R - 1) * rowpitch;
+  p.lds = items > p.grid ? lds_max : 1024 + stage + (slab_bytes > stage2 ? slab_bytes : stage2);
+  a.slab_org = slab_org;
+  a.first_row = first_row;
+  a.slab_rows = (p.lds - slab_org) / rowpitch;
   p.ok = true;
   return p;
 }
