@@ -40,11 +40,11 @@
 #include "gemm_kernel.h"
 
 #ifdef RF_PROFILE // experiment builds (-DRF_PROFILE=<workgroup>): cycle stamps per wavefront
-__device__ uint64_t rf_prof[128];
+__device__ uint64_t rf_prof[8 * 48];
 #define RF_STAMP(i)                                                            \
   do {                                                                         \
-    if (blockIdx.x == RF_PROFILE && (threadIdx.x & 63) == 0)                   \
-      rf_prof[(threadIdx.x >> 6) * 16 + (i)] = __builtin_amdgcn_s_memtime();   \
+    if (blockIdx.x == RF_PROFILE && (threadIdx.x & 63) == 0 && (i) < 48)       \
+      rf_prof[(threadIdx.x >> 6) * 48 + (i)] = __builtin_amdgcn_s_memtime();   \
   } while (0)
 extern "C" int fhip_debug_rf_prof(unsigned long long *out) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rf_prof), sizeof(rf_prof));
@@ -401,6 +401,7 @@ conv_rf_kernel(ConvRfArgs g) {
   for (;;) {
     const int npix = tr * a_Q;
     const uint32_t lds_s = slab_org + (uint32_t)srow * rowpitch;
+    RF_STAMP(16 + 4 * (tile - tile_end + 8)); // (profile builds: per tile, the run's last eight)
 
     // ---- the next tile's rows are requested now and land during this tile's
     // blocks.  Below this tile in the same image it starts on this tile's last
@@ -539,6 +540,7 @@ conv_rf_kernel(ConvRfArgs g) {
       __builtin_amdgcn_sched_barrier(0); // (in this order: the loop waits for the oldest)
     });
     RF_STAMP(4);
+    RF_STAMP(17 + 4 * (tile - tile_end + 8));
     while (b < nblocks) {
       drawn = draw_block();
       ksteps();
@@ -557,6 +559,7 @@ conv_rf_kernel(ConvRfArgs g) {
       b = nb;
     }
     RF_STAMP(12);
+    RF_STAMP(18 + 4 * (tile - tile_end + 8));
     if (!more)
       break;
     if (deferred) {
@@ -568,6 +571,7 @@ conv_rf_kernel(ConvRfArgs g) {
     // the next tile's rows are in LDS, and every wavefront has left this tile
     __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
     gemm_barrier();
+    RF_STAMP(19 + 4 * (tile - tile_end + 8));
     ++tile;
     n = n2, p0 = p02, tr = tr2, ih0 = ih02, srow = srow2;
     draw ^= 4u;
