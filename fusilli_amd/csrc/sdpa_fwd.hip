@@ -644,34 +644,44 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
         // s <- s * scale + mask, or -inf where a boolean mask is false (one
         // multiply-add per score; the softmax below then runs in natural-log
         // units, its scale being log2(e))
-        auto fold = [&](const u32x4 (&mraw)[8]) {
+        // (one loop per element kind: the kind is a run-time value, and a
+        // choice per score would cut the loop into 32 scalar branches)
+        auto fold_with = [&](auto value) __attribute__((always_inline)) {
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const u32x4 w = mraw[kb * 4 + (r >> 2)];
-              const int e = r & 3;
-              if (m_esh == 0) {
-                s[kb][r] = ((w.x >> (8 * e)) & 0xffu) != 0 ? s[kb][r] * g.scale
-                                                           : -INFINITY;
-              } else if (m_esh == 1) {
-                const uint32_t word = e < 2 ? w.x : w.y;
-                float mv;
-                if (g.m_dt == FHIP_BFLOAT16)
-                  mv = __builtin_bit_cast(float, (e & 1) ? (word & 0xffff0000u)
-                                                         : (word << 16));
-                else
-                  mv = (float)__builtin_bit_cast(
-                      _Float16, (uint16_t)((e & 1) ? word >> 16 : word));
-                s[kb][r] = __builtin_fmaf(s[kb][r], g.scale, mv);
-              } else {
-                // (through a scalar: bit-casting a vector's element in place
-                // reads element 0)
-                const uint32_t word = e == 0 ? w.x : e == 1 ? w.y : e == 2 ? w.z : w.w;
-                s[kb][r] = __builtin_fmaf(s[kb][r], g.scale,
-                                          __builtin_bit_cast(float, word));
-              }
-            }
+            for (int r = 0; r < 16; ++r)
+              s[kb][r] = value(kb * 4 + (r >> 2), r & 3, s[kb][r]);
+        };
+        auto fold = [&](const u32x4 (&mraw)[8]) __attribute__((always_inline)) {
+          const float scale = g.scale;
+          if (m_esh == 0) {
+            fold_with([&](int i, int e, float sv) {
+              return ((mraw[i].x >> (8 * e)) & 0xffu) != 0 ? sv * scale : -INFINITY;
+            });
+          } else if (m_esh == 2) {
+            // (through a scalar: bit-casting a vector's element in place
+            // reads element 0)
+            fold_with([&](int i, int e, float sv) {
+              const u32x4 w = mraw[i];
+              const uint32_t word = e == 0 ? w.x : e == 1 ? w.y : e == 2 ? w.z : w.w;
+              return __builtin_fmaf(sv, scale, __builtin_bit_cast(float, word));
+            });
+          } else if (g.m_dt == FHIP_BFLOAT16) {
+            fold_with([&](int i, int e, float sv) {
+              const uint32_t word = e < 2 ? mraw[i].x : mraw[i].y;
+              const float mv =
+                  __builtin_bit_cast(float, (e & 1) ? (word & 0xffff0000u) : (word << 16));
+              return __builtin_fmaf(sv, scale, mv);
+            });
+          } else {
+            fold_with([&](int i, int e, float sv) {
+              const uint32_t word = e < 2 ? mraw[i].x : mraw[i].y;
+              const float mv =
+                  (float)__builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? word >> 16 : word));
+              return __builtin_fmaf(sv, scale, mv);
+            });
+          }
         };
         if constexpr (MASK == 1) {
           fold(mreg);
