@@ -378,11 +378,11 @@ __global__ void conv_pad_channels_kernel(const uint4 *src, uint4 *dst, int64_t p
 }
 
 struct SplitSumArgs {
-  const float *part; // [parts][M][N]
+  const float *part; // [parts][M][pitch]: rows padded to whole column tiles
   void *out;         // [M][N], dense
   int64_t mn4;       // M * N / 4
-  int64_t mn;        // M * N
-  int32_t N, parts;
+  int64_t part_stride; // M * pitch
+  int32_t N, pitch, parts;
   int32_t y_dt, o_dt;
   DevEpilogue epi;   // rank 3: strides {0, per pixel, per channel} over (0, m, n)
 };
@@ -392,14 +392,15 @@ __global__ void conv_splitk_sum_kernel(SplitSumArgs a) {
   const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (lin >= a.mn4)
     return;
-  float4 acc = ((const float4 *)a.part)[lin];
-  for (int z = 1; z < a.parts; ++z) {
-    const float4 v = ((const float4 *)(a.part + (int64_t)z * a.mn))[lin];
-    acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
-  }
   const int64_t e = lin * 4;
   const int64_t m = e / a.N;
   const int n0 = (int)(e - m * a.N);
+  const float *src = a.part + m * a.pitch + n0;
+  float4 acc = *(const float4 *)src;
+  for (int z = 1; z < a.parts; ++z) {
+    const float4 v = *(const float4 *)(src + (int64_t)z * a.part_stride);
+    acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+  }
   // fused operands are addressed as base + m * pixel step + n * channel step,
   // whatever the rank of the convolution (a folded 3-D problem included)
   int64_t coord[FHIP_MAX_RANK] = {};
@@ -458,8 +459,11 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
   // the context's scratch: zero-padded copies of X and W, then the parts of a
   // split reduction
   const size_t pad_bytes = res.padded ? res.x_bytes + res.w_bytes : 0;
+  // (rows of the parts are padded to whole column tiles, which are stored
+  // whole: every cache line of the parts is written by one workgroup)
+  const int64_t part_pitch = (p.N + p.bn - 1) / p.bn * p.bn;
   const size_t part_bytes =
-      p.ksplit > 1 ? (size_t)p.ksplit * (size_t)(p.M * p.N) * sizeof(float) : 0;
+      p.ksplit > 1 ? (size_t)p.ksplit * (size_t)(p.M * part_pitch) * sizeof(float) : 0;
   char *scratch = nullptr;
   if (pad_bytes + part_bytes > 0) {
     void *sp = nullptr;
@@ -533,12 +537,13 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     float *part = (float *)(scratch + pad_bytes);
     g.out = (char *)part;
     g.c_dt = g.o_dt = FHIP_FLOAT;
-    g.o_sm = p.N;
+    g.o_sm = part_pitch;
+    g.n_store = part_pitch;
     g.o_vec = 1;
     g.epi = DevEpilogue{};
     g.epi.rank = 3;
     g.outer = p.ksplit;
-    g.o_outer = p.M * p.N;
+    g.o_outer = p.M * part_pitch;
     g.kt_split = (int32_t)(p.K * 2 / kTileKBytes / p.ksplit);
     gemm_fill_linear(fhip_epilogue{}, g);
     const int rc = p.kind == GK_BF16 ? conv_launch_bf16(ctx, p.bm, p.bn, g)
@@ -548,8 +553,9 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     SplitSumArgs a{};
     a.part = part;
     a.out = out;
-    a.mn = p.M * p.N;
-    a.mn4 = a.mn / 4;
+    a.part_stride = p.M * part_pitch;
+    a.pitch = (int32_t)part_pitch;
+    a.mn4 = p.M * p.N / 4;
     a.N = (int32_t)p.N;
     a.parts = p.ksplit;
     a.y_dt = d->y.dtype;

@@ -158,6 +158,10 @@ struct GemmArgs {
   // value lets the host match the tile count to the machine
   int32_t tile_rows;
   int32_t o_vec;              // output rows allow aligned 16-byte stores
+  // columns that are stored (0: N).  The parts of a split reduction store
+  // whole column tiles into rows padded to the tile width, so that no cache
+  // line of the partial sums is written by two workgroups
+  int64_t n_store;
   // Epilogue applied to the accumulators in registers: every op is one of
   // ADD / SUB / MUL / RELU / NEG / IDENTITY with a scalar or per-column
   // operand: v = mul ? v * o : a * v + b * o, then max(v, 0) if relu.
@@ -938,7 +942,8 @@ gemm_kernel(GemmArgs g) {
   // scale, ReLU ...), the output rows allow aligned 16-byte stores and this
   // wavefront has no ragged columns.  A lane's 8 columns are the same in
   // every pass, so each operand is loaded once, before the passes.
-  const bool lane_full = ncol + 8 <= g.N || ncol >= g.N;
+  const int64_t n_store = g.n_store ? g.n_store : g.N;
+  const bool lane_full = ncol + 8 <= n_store || ncol >= n_store;
   const bool lean = g.epi_reg && g.o_vec != 0 &&
                     __builtin_amdgcn_ballot_w64(!lane_full) == 0;
   const int64_t esz = fhip_dtype_size(g.o_dt);
@@ -948,7 +953,7 @@ gemm_kernel(GemmArgs g) {
   const int64_t lean_m = m0 + wm * WM + l / LPR;
   const int64_t row_bytes = g.o_sm * esz;
   const int nops = g.epi.count;
-  const int64_t gM = m_end, gN = g.N;
+  const int64_t gM = m_end, gN = n_store; // rows and columns that are stored
   const int o_dt = g.o_dt;
 
   // Lean path, step 1: the chain runs on the accumulators where they are.  A
@@ -972,7 +977,7 @@ gemm_kernel(GemmArgs g) {
           float ov;
           if (o.kind == FHIP_OPERAND_TENSOR) {
             int64_t n = n0 + wn * WN + j * 32 + (l & 31);
-            n = n < gN ? n : gN - 1;
+            n = n < g.N ? n : g.N - 1;
             const int64_t off[1] = {(n + outer * g.epi_n_outer) * o.stride[2]};
             float one[1];
             load_operand_vec<1>(o.ptr, o.operand_dtype, off, one);
@@ -1118,9 +1123,9 @@ gemm_kernel(GemmArgs g) {
       const uint32_t src = rd + bi * L::kBand + pp * RPP * PITCH;
       const u32x4 v0 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src);
       const u32x4 v1 = *(const GEMM_AS3 u32x4 *)(uintptr_t)(src + 16);
-      if (m >= m_end || ncol >= g.N)
+      if (m >= m_end || ncol >= n_store)
         continue;
-      const bool full = ncol + 8 <= g.N;
+      const bool full = ncol + 8 <= n_store;
       const int64_t o0 = ob + m * g.o_sm + ncol * g.o_sn;
       if constexpr (std::is_same<Acc, int>::value) {
         GEMM_AS1 int32_t *out = (GEMM_AS1 int32_t *)g.out;
@@ -1131,7 +1136,7 @@ gemm_kernel(GemmArgs g) {
           const uint32_t y[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
           for (int e = 0; e < 8; ++e)
-            if (ncol + e < g.N)
+            if (ncol + e < n_store)
               out[o0 + e * g.o_sn] = (int32_t)y[e];
         }
       } else {
@@ -1177,7 +1182,7 @@ gemm_kernel(GemmArgs g) {
           } else {
 #pragma unroll
             for (int c = 0; c < 8; ++c)
-              if (ncol + c < g.N)
+              if (ncol + c < n_store)
                 out[o0 + c * g.o_sn] = y[c];
           }
         } else if (g.o_dt == FHIP_BFLOAT16) {
@@ -1191,7 +1196,7 @@ gemm_kernel(GemmArgs g) {
           } else {
 #pragma unroll
             for (int c = 0; c < 8; ++c)
-              if (ncol + c < g.N)
+              if (ncol + c < n_store)
                 out[o0 + c * g.o_sn] = (__bf16)y[c];
           }
         } else {
@@ -1205,7 +1210,7 @@ gemm_kernel(GemmArgs g) {
           } else {
 #pragma unroll
             for (int c = 0; c < 8; ++c)
-              if (ncol + c < g.N)
+              if (ncol + c < n_store)
                 out[o0 + c * g.o_sn] = (_Float16)y[c];
           }
         }

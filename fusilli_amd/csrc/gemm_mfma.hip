@@ -193,27 +193,30 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
 }
 
 struct GemmSumArgs {
-  const float *part; // [parts][M][N]
+  const float *part; // [parts][M][pitch]: rows padded to whole column tiles
   void *out;
-  int64_t mn, mn4, o_sm;
-  int32_t N, parts, rank;
+  int64_t part_stride; // M * pitch
+  int64_t mn4, o_sm;   // mn4: M * N / 4
+  int32_t N, pitch, parts, rank;
   int32_t c_dt, o_dt;
   DevEpilogue epi; // strides over the matmul's result dims
 };
 
 // OUT[m][n] = epilogue(round(sum over the parts)), four columns per thread
+// (N is a multiple of 4)
 __global__ void gemm_splitk_sum_kernel(GemmSumArgs a) {
   const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (lin >= a.mn4)
     return;
-  float4 acc = ((const float4 *)a.part)[lin];
-  for (int z = 1; z < a.parts; ++z) {
-    const float4 v = ((const float4 *)(a.part + (int64_t)z * a.mn))[lin];
-    acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
-  }
   const int64_t e = lin * 4;
   const int64_t m = e / a.N;
   const int64_t n0 = e - m * a.N;
+  const float *src = a.part + m * a.pitch + n0;
+  float4 acc = *(const float4 *)src;
+  for (int z = 1; z < a.parts; ++z) {
+    const float4 v = *(const float4 *)(src + (int64_t)z * a.part_stride);
+    acc.x += v.x, acc.y += v.y, acc.z += v.z, acc.w += v.w;
+  }
   int64_t coord[FHIP_MAX_RANK];
   coord[0] = 0;
   coord[a.rank - 2] = m;
@@ -307,18 +310,23 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
   if (p.ksplit > 1) {
     // every part writes plain f32 sums; rounding and the fused operations
     // follow in the kernel that adds them
+    // (rows of the parts are padded to whole column tiles and the tiles are
+    // stored whole: every cache line of the parts is written by one workgroup,
+    // with full 16-byte stores)
     void *sp = nullptr;
-    if (fhip_ctx_scratch(ctx, (size_t)p.ksplit * (size_t)(p.M * p.N) * sizeof(float), &sp) != 0)
+    const int64_t pitch = (int64_t)g.tiles_n * p.bn;
+    if (fhip_ctx_scratch(ctx, (size_t)p.ksplit * (size_t)(p.M * pitch) * sizeof(float), &sp) != 0)
       return 1;
     g.out = (char *)sp;
     g.c_dt = g.o_dt = FHIP_FLOAT;
-    g.o_sm = p.N;
+    g.o_sm = pitch;
+    g.n_store = pitch;
     g.o_sn = 1;
     g.o_vec = 1;
     g.epi = DevEpilogue{};
     g.epi.rank = 3;
     g.outer = p.ksplit;
-    g.o_outer = p.M * p.N;
+    g.o_outer = p.M * pitch;
     g.kt_split = (int32_t)(p.K * fhip_dtype_size(d->a.dtype) / kTileKBytes / p.ksplit);
     gemm_fill_linear(fhip_epilogue{}, g);
     const int rc = launch();
@@ -327,8 +335,9 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     GemmSumArgs sa{};
     sa.part = (const float *)sp;
     sa.out = out;
-    sa.mn = p.M * p.N;
-    sa.mn4 = sa.mn / 4;
+    sa.part_stride = p.M * pitch;
+    sa.pitch = (int32_t)pitch;
+    sa.mn4 = p.M * p.N / 4;
     sa.o_sm = p.o_sm;
     sa.N = (int32_t)p.N;
     sa.parts = p.ksplit;
