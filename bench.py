@@ -80,11 +80,14 @@ FLOOR_FILE = os.path.join(ROOT, "bench_floor.json")
 DRIVER = os.path.join(ROOT, "fusilli_amd", "bench", "bin", "driver")
 
 
-def graph_api_us(command, iters=200):
+def graph_api_us(command, kernel_us):
     """Average time of one Graph::execute of `command`'s graph (HIP events
     around --iter back-to-back executes inside the benchmark driver, a child
     process: variant-pack lookup, plan and argument set-up included), or None
-    when the driver binary is not built."""
+    when the driver binary is not built.  As many untimed executes first as
+    60 ms of the kernel's time (`kernel_us` per launch): the GPU's clocks take
+    tens of milliseconds of load to settle, and a short kernel timed before
+    that reads 10-20 % slow."""
     import shlex
     import subprocess
     if not os.path.exists(DRIVER):
@@ -92,7 +95,9 @@ def graph_api_us(command, iters=200):
     try:
         # (--fill random: constant operands toggle fewer bits and let the MFMA
         # kernels clock higher than real data does)
-        proc = subprocess.run([DRIVER, "--iter", str(iters), "--warmup", "50", "--fill", "random"]
+        warm = max(50, int(60e3 / max(kernel_us, 1.0)))
+        iters = max(200, int(20e3 / max(kernel_us, 1.0)))
+        proc = subprocess.run([DRIVER, "--iter", str(iters), "--warmup", str(warm), "--fill", "random"]
                               + shlex.split(command),
                               capture_output=True, text=True, timeout=120)
         if proc.returncode != 0:
@@ -934,7 +939,7 @@ def main():
                                 "met": None if target is None else bool(frac >= target),
                                 "kernel_us": us, "kernel": kernel,
                                 "expected_kernel": bool(kernel.startswith(variant)),
-                                "graph_api_us": graph_api_us(command),
+                                "graph_api_us": graph_api_us(command, us),
                                 "traffic": roof.get("traffic"),
                                 "traffic_source": roof.get("traffic_source")}
             line["configs"] = configs

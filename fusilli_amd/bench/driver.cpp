@@ -12,6 +12,7 @@
 #include <fusilli.h>
 
 #include <cmath>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -257,6 +258,7 @@ struct Run {
 };
 
 int g_warmup = 3; // untimed executes before the --iter loop (--warmup)
+bool g_host_time = false; // --host-time: also print the calling thread's time per execute (stderr)
 bool g_verify = false; // --verify: compare the outputs with their closed forms
 
 // The buffer's elements as doubles, in storage order.
@@ -359,10 +361,16 @@ void timeGraph(const Handle &h, Graph &g, Pack &pack, const Run &r, int iter) {
   if (fhip_event_create(ctx, &e0) || fhip_event_create(ctx, &e1))
     die(fhip_last_error(ctx));
   fhip_event_record(ctx, e0);
+  const auto t0 = std::chrono::steady_clock::now();
   for (int i = 0; i < iter; ++i)
     OK(g.execute(h, pack, wsBuf));
+  const auto t1 = std::chrono::steady_clock::now();
   fhip_event_record(ctx, e1);
   fhip_stream_sync(ctx);
+  if (g_host_time) // (the enqueue loop alone: what one execute costs the calling thread; the
+                   // launch queue takes a few hundred kernels before a launch waits for the GPU)
+    std::fprintf(stderr, "host_us_per_execute,%s,%.3f\n", r.name.c_str(),
+                 std::chrono::duration<double, std::micro>(t1 - t0).count() / iter);
   float ms = 0;
   fhip_event_elapsed_ms(ctx, e0, e1, &ms);
   fhip_event_destroy(ctx, e0);
@@ -836,6 +844,8 @@ int main(int argc, char **argv) {
       g_warmup = std::atoi(argv[++i]);
     else if (k == "--verify")
       g_verify = true;
+    else if (k == "--host-time")
+      g_host_time = true;
     else if (k == "--fill" && i + 1 < argc) {
       const std::string f = argv[++i];
       if (f != "random" && f != "constant")
@@ -848,7 +858,7 @@ int main(int argc, char **argv) {
       break;
   }
   if (i >= argc)
-    die("usage: driver [--device N] [--iter N] [--warmup N] [--verify] [--fill constant|random] <conv|matmul|sdpa|layernorm|rmsnorm> flags...");
+    die("usage: driver [--device N] [--iter N] [--warmup N] [--verify] [--host-time] [--fill constant|random] <conv|matmul|sdpa|layernorm|rmsnorm> flags...");
   if (g_verify && g_random)
     die("--verify checks the closed forms of the constant fills: it excludes --fill random");
   const std::string cmd = argv[i];
