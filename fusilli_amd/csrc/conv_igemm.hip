@@ -367,11 +367,20 @@ ConvResolved resolve(const fhip_conv_desc *d, bool allow_scratch = true) {
 }
 
 // dst[pixel][0 .. Cp) = src[pixel][0 .. C), zeros behind; one 16-byte chunk per thread
-__global__ void conv_pad_channels_kernel(const uint4 *src, uint4 *dst, int64_t pixels,
+// Both operands in one launch: the chunks of X's copy, then those of W's.
+__global__ void conv_pad_channels_kernel(const uint4 *x, uint4 *xp, int64_t x_pixels,
+                                         const uint4 *w, uint4 *wp, int64_t w_pixels,
                                          int32_t c8, int32_t cp8) {
-  const int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (lin >= pixels * cp8)
-    return;
+  int64_t lin = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const uint4 *src = x;
+  uint4 *dst = xp;
+  if (lin >= x_pixels * cp8) {
+    lin -= x_pixels * cp8;
+    if (lin >= w_pixels * cp8)
+      return;
+    src = w;
+    dst = wp;
+  }
   const int64_t pixel = lin / cp8;
   const int32_t chunk = (int32_t)(lin - pixel * cp8);
   dst[lin] = chunk < c8 ? src[pixel * c8 + chunk] : make_uint4(0, 0, 0, 0);
@@ -476,12 +485,9 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     char *xp = scratch, *wp = xp + res.x_bytes;
     const int32_t c8 = (int32_t)(res.C / 8), cp8 = (int32_t)(res.Cp / 8);
     const int64_t xt = res.x_pixels * cp8, wt = res.w_pixels * cp8;
-    hipLaunchKernelGGL(conv_pad_channels_kernel, dim3((unsigned)((xt + 255) / 256)),
-                       dim3(256), 0, ctx->stream, (const uint4 *)x, (uint4 *)xp,
-                       res.x_pixels, c8, cp8);
-    hipLaunchKernelGGL(conv_pad_channels_kernel, dim3((unsigned)((wt + 255) / 256)),
-                       dim3(256), 0, ctx->stream, (const uint4 *)w, (uint4 *)wp,
-                       res.w_pixels, c8, cp8);
+    hipLaunchKernelGGL(conv_pad_channels_kernel, dim3((unsigned)((xt + wt + 255) / 256)),
+                       dim3(256), 0, ctx->stream, (const uint4 *)x, (uint4 *)xp, res.x_pixels,
+                       (const uint4 *)w, (uint4 *)wp, res.w_pixels, c8, cp8);
     FHIP_HIP_CHECK(ctx, hipGetLastError());
     x = xp;
     w = wp;
