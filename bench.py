@@ -579,11 +579,13 @@ def bench_conv_padded(ctx, steps, warmup):
             "note": "1.4 GFLOP: launch-latency bound"}
 
 
-def bench_conv_grouped(ctx, steps, warmup):
-    """Grouped convolution on the MFMA kernels: N32 C256 56x56 -> K256, 3x3,
-    padding 1, 4 groups of 64 -> 64 channels (bf16 channels-last), one launch
-    whose outer grid dimension is the group."""
-    n, c, h, w, k, r, groups = 32, 256, 56, 56, 256, 3, 4
+def bench_conv_grouped(ctx, steps, warmup, n=32, c=256, h=56, w=56, k=256, groups=4):
+    """3 x 3 convolution, padding 1, bf16 channels-last, no fused operations.
+    The default: N32 C256 56x56 -> K256 in 4 groups of 64 -> 64 channels (the
+    register-filter kernel with two groups per workgroup, runs of 2-row tiles).
+    Also used for one-group shapes around C3: K = 64 (64 output channels per
+    workgroup) and N = 64 (two tiles per workgroup)."""
+    r = 3
     cl = lambda dims: [dims[1] * dims[2] * dims[3], 1, dims[3] * dims[1], dims[1]]
     xd, wd, yd = [n, c, h, w], [k, c // groups, r, r], [n, k, h, w]
     d = capi.ConvDesc()
@@ -909,6 +911,10 @@ def main():
              lambda: bench_layernorm_long(ctx, max(20, args.steps // 4), kwarm)),
             ("conv_fprop_bf16_n32c256h56w56_k256r3s3_groups4",
              lambda: bench_conv_grouped(ctx, max(20, args.steps // 10), kwarm)),
+            ("conv_fprop_bf16_n32c64h56w56_k64r3s3",
+             lambda: bench_conv_grouped(ctx, max(20, args.steps // 10), kwarm, 32, 64, 56, 56, 64, 1)),
+            ("conv_fprop_bf16_n64c64h56w56_k128r3s3",
+             lambda: bench_conv_grouped(ctx, max(20, args.steps // 10), kwarm, 64, 64, 56, 56, 128, 1)),
             ("conv_fprop_bf16_n32c512h7w7_k512r3s3_split_reduction",
              lambda: bench_conv_deep_layer(ctx, max(20, args.steps // 10), kwarm)),
             ("matmul_bf16_1024x1024x8192_split_reduction",

@@ -20,6 +20,8 @@ FhipKnobs parse_knobs() {
     k.conv_depthwise_strips = atoi(e) != 0;
   if (const char *e = getenv("FUSILLI_HIP_GEMM_SPLIT"))
     k.gemm_split = atoi(e);
+  if (const char *e = getenv("FUSILLI_HIP_CONV_SLICES"))
+    k.conv_slices = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_POINTWISE_WGS_PER_CU"))
     k.pointwise_wgs_per_cu = atoi(e);
   if (const char *e = getenv("FUSILLI_HIP_ROWNORM_SHAPE"))

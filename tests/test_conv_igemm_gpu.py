@@ -436,7 +436,10 @@ RF_CASES = [
 @pytest.mark.parametrize("case", RF_CASES)
 @pytest.mark.parametrize("dtype", [capi.BFLOAT16, capi.HALF])
 @pytest.mark.parametrize("epi_kind", ["bias_relu", "none", "scale_bias"])
-def test_conv_register_filter_kernel_vs_oracle(ctx, knobs, case, dtype, epi_kind):
+@pytest.mark.parametrize("slices", [4, 2])
+def test_conv_register_filter_kernel_vs_oracle(ctx, knobs, case, dtype, epi_kind, slices):
+    # slices: 128 output channels per workgroup (two wavefronts per 32-channel
+    # slice) or 64 (four per slice, the filter staged in the slab's place)
     xd, wd = case["x"], [case["k"], 64, 3, 3]
     pad, st, dil = case["pad"], [1, 1], [1, 1]
     x = cl(xd, 47, 0, dtype)
@@ -460,10 +463,28 @@ def test_conv_register_filter_kernel_vs_oracle(ctx, knobs, case, dtype, epi_kind
         epi, ops = [], []
     got = {}
     for rows in (case["rows"], 0):  # the register-filter kernel, then the tiled one
-        knobs(CONV_ROWS=rows)
+        knobs(CONV_ROWS=rows, CONV_SLICES=slices)
         got[rows] = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=dtype,
                         epilogue=epi, epi_tensors=ops).logical()
-        assert_close(got[rows], ref, dtype, f"rows={rows} {case} {epi_kind}")
+        if rows:
+            name = ctx.last_kernel()
+            assert name.startswith("conv_rf c=64 r=3 s=3") and \
+                name.endswith("slices=2") == (slices == 2), name
+        assert_close(got[rows], ref, dtype, f"rows={rows} slices={slices} {case} {epi_kind}")
+
+
+def test_conv_register_filter_kernel_64_output_channels(ctx, knobs):
+    # K = 64 (one pair of channel slices): only the two-slice variant applies;
+    # workgroups walk runs of tiles that share halo rows in LDS
+    xd, wd = [8, 64, 30, 24], [64, 64, 3, 3]
+    x = cl(xd, 52, 0, capi.BFLOAT16)
+    w = cl(wd, 52, 1, capi.BFLOAT16, std=0.05)
+    ref = oracle.conv_fprop(x.logical(), w.logical(), [1, 1], [1, 1], [1, 1])
+    for rows in (3, 7):
+        knobs(CONV_ROWS=rows)
+        got = run(ctx, x, w, [1, 1], [1, 1], [1, 1], capi.FLOAT, out_dtype=capi.BFLOAT16).logical()
+        assert ctx.last_kernel().endswith("slices=2"), ctx.last_kernel()
+        assert_close(got, ref, capi.BFLOAT16, f"rows={rows}")
 
 
 RF_GROUPED_CASES = [
