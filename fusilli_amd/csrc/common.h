@@ -712,6 +712,106 @@ __device__ __forceinline__ CT fhip_apply_epilogue(const DevEpilogue &e, CT v,
   return v;
 }
 
+// N elements of a tensor of runtime dtype at once: one switch for all, so the
+// loads are issued back to back (N calls of fhip_load each wait for their
+// value before the next address is even formed).
+template <typename CT, int N>
+__device__ __forceinline__ void fhip_load_many(const void *p, int dt, const int64_t (&idx)[N],
+                                               CT (&out)[N]) {
+  switch (dt) {
+  case FHIP_FLOAT:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      out[n] = (CT)((const float *)p)[idx[n]];
+    break;
+  case FHIP_BFLOAT16:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      out[n] = (CT)(float)((const __bf16 *)p)[idx[n]];
+    break;
+  case FHIP_HALF:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      out[n] = (CT)(float)((const _Float16 *)p)[idx[n]];
+    break;
+  default:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      out[n] = fhip_load<CT>(p, dt, idx[n]);
+  }
+}
+
+// The chain on N values whose coordinates differ in one dim only (`var_dim`,
+// where value n sits at vals[n]; coord[var_dim] is ignored).  Same results as N
+// calls of fhip_apply_epilogue; an operand's N values are fetched together.
+// Callers pass a valid coordinate also for values they will not store.
+template <typename CT, int N>
+__device__ __forceinline__ void fhip_apply_epilogue_many(const DevEpilogue &e, CT (&v)[N],
+                                                         const int64_t *coord, int var_dim,
+                                                         const int64_t (&vals)[N]) {
+  for (int i = 0; i < e.count; ++i) {
+    const DevEpiOp &o = e.op[i];
+    // (f32 chains of the common modes: the mode is chosen once for the N
+    // values, not per value -- a switch over every mode, inlined N times, is
+    // most of such a kernel's code)
+    constexpr bool kF32 = std::is_same<CT, float>::value;
+    const bool fast = kF32 && fhip_pw_is_fast(o.mode);
+    if (o.kind == FHIP_OPERAND_NONE) {
+      if constexpr (kF32) {
+        if (fast) {
+          fhip_pw_fast_unary_vec<true, N>(o.mode, v, o.params.swish_beta);
+        } else {
+#pragma unroll
+          for (int n = 0; n < N; ++n)
+            v[n] = fhip_pw_unary<CT>(o.mode, v[n], o.params);
+        }
+      } else {
+#pragma unroll
+        for (int n = 0; n < N; ++n)
+          v[n] = fhip_pw_unary<CT>(o.mode, v[n], o.params);
+      }
+    } else {
+      CT other[N];
+      if (o.kind == FHIP_OPERAND_SCALAR) {
+#pragma unroll
+        for (int n = 0; n < N; ++n)
+          other[n] = (CT)o.scalar;
+      } else {
+        int64_t base = 0;
+        for (int r = 0; r < e.rank; ++r)
+          base += r == var_dim ? 0 : coord[r] * o.stride[r];
+        int64_t off[N];
+#pragma unroll
+        for (int n = 0; n < N; ++n)
+          off[n] = base + vals[n] * o.stride[var_dim];
+        fhip_load_many<CT, N>(o.ptr, o.operand_dtype, off, other);
+      }
+      bool done = false;
+      if constexpr (kF32) {
+        if (fast) {
+          fhip_pw_fast_binary_vec<N>(o.mode, o.acc_is_in1 != 0, v, other);
+          done = true;
+        }
+      }
+      if (!done) {
+#pragma unroll
+        for (int n = 0; n < N; ++n)
+          v[n] = o.acc_is_in1 ? fhip_pw_binary<CT>(o.mode, other[n], v[n], o.params)
+                              : fhip_pw_binary<CT>(o.mode, v[n], other[n], o.params);
+      }
+    }
+    const int rd = o.result_dtype;
+    if (kF32 && (rd == FHIP_FLOAT || rd == FHIP_BFLOAT16 || rd == FHIP_HALF)) {
+      if constexpr (kF32)
+        fhip_round_fast_vec<N>(rd, v);
+    } else {
+#pragma unroll
+      for (int n = 0; n < N; ++n)
+        v[n] = fhip_round_through<CT>(rd, v[n]);
+    }
+  }
+}
+
 #endif // __HIPCC__
 
 // ---------------------------------------------------------------------------

@@ -131,14 +131,22 @@ __global__ __launch_bounds__(256) void direct_conv_fprop_kernel(
   for (int i = 0; i < g.sp; ++i)
     coord[2 + i] = o[3 - g.sp + i];
   const int64_t ob = n * g.os[0] + o0 * g.os[2] + o1 * g.os[3] + o2 * g.os[4];
+  // (the channels of a thread together: a fused operand's values are fetched
+  // as one batch of loads)
+  float v[kDcT];
+  int64_t chans[kDcT];
+#pragma unroll
+  for (int t = 0; t < kDcT; ++t) {
+    chans[t] = k0 + (t < kvalid ? t : kvalid - 1);
+    v[t] = fhip_round_through<float>(g.y_dt, acc[t]);
+  }
+  if (g.epi.count > 0)
+    fhip_apply_epilogue_many<float, kDcT>(g.epi, v, coord, 1, chans);
 #pragma unroll
   for (int t = 0; t < kDcT; ++t) {
     if (t >= kvalid)
       break;
-    coord[1] = k0 + t;
-    float v = fhip_round_through<float>(g.y_dt, acc[t]);
-    v = fhip_apply_epilogue<float>(g.epi, v, coord);
-    fhip_store<float>(out, g.o_dt, ob + (k0 + t) * g.os[1], v);
+    fhip_store<float>(out, g.o_dt, ob + (k0 + t) * g.os[1], v[t]);
   }
 }
 
@@ -289,11 +297,11 @@ __global__ __launch_bounds__(256) void direct_conv_fprop_cl_kernel(
       } else {
         coord[2] = q;
       }
+      int64_t chans[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        coord[1] = cb * 8 + k;
-        y[k] = fhip_apply_epilogue<float>(g.epi, y[k], coord);
-      }
+      for (int k = 0; k < 8; ++k)
+        chans[k] = cb * 8 + k;
+      fhip_apply_epilogue_many<float, 8>(g.epi, y, coord, 1, chans);
     }
     // (OUT has fewer than 2^31 elements)
     const uint32_t ob = pix * (uint32_t)g.K + chan;
@@ -429,11 +437,11 @@ __global__ __launch_bounds__(256) void depthwise3x3_cl_kernel(DcClArgs g, const 
       coord[0] = n;
       coord[2] = p;
       coord[3] = qq;
+      int64_t chans[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        coord[1] = cb * 8 + k;
-        y[k] = fhip_apply_epilogue<float>(g.epi, y[k], coord);
-      }
+      for (int k = 0; k < 8; ++k)
+        chans[k] = cb * 8 + k;
+      fhip_apply_epilogue_many<float, 8>(g.epi, y, coord, 1, chans);
     }
     // (OUT has fewer than 2^31 elements)
     const uint32_t ob = ((uint32_t)((n * g.P + p) * g.Q + qq)) * (uint32_t)g.K + chan;

@@ -414,14 +414,17 @@ __global__ void conv_splitk_sum_kernel(SplitSumArgs a) {
   // whatever the rank of the convolution (a folded 3-D problem included)
   int64_t coord[FHIP_MAX_RANK] = {};
   coord[1] = m;
-  const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+  float v[4] = {acc.x, acc.y, acc.z, acc.w};
+  int64_t cols[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    coord[2] = n0 + i;
-    float y = fhip_round_through<float>(a.y_dt, v[i]);
-    y = fhip_apply_epilogue<float>(a.epi, y, coord);
-    fhip_store<float>(a.out, a.o_dt, e + i, y);
+    cols[i] = n0 + i;
+    v[i] = fhip_round_through<float>(a.y_dt, v[i]);
   }
+  fhip_apply_epilogue_many<float, 4>(a.epi, v, coord, 2, cols);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    fhip_store<float>(a.out, a.o_dt, e + i, v[i]);
 }
 
 } // namespace

@@ -220,14 +220,17 @@ __global__ void gemm_splitk_sum_kernel(GemmSumArgs a) {
   int64_t coord[FHIP_MAX_RANK];
   coord[0] = 0;
   coord[a.rank - 2] = m;
-  const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+  float v[4] = {acc.x, acc.y, acc.z, acc.w};
+  int64_t cols[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    coord[a.rank - 1] = n0 + i;
-    float y = fhip_round_through<float>(a.c_dt, v[i]);
-    y = fhip_apply_epilogue<float>(a.epi, y, coord);
-    fhip_store<float>(a.out, a.o_dt, m * a.o_sm + n0 + i, y);
+    cols[i] = n0 + i;
+    v[i] = fhip_round_through<float>(a.c_dt, v[i]);
   }
+  fhip_apply_epilogue_many<float, 4>(a.epi, v, coord, a.rank - 1, cols);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    fhip_store<float>(a.out, a.o_dt, m * a.o_sm + n0 + i, v[i]);
 }
 
 } // namespace

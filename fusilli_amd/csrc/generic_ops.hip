@@ -196,15 +196,26 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
   if (n >= N)
     return;
   coord[rank - 1] = n;
+  // (the 16 rows of a lane together: a fused operand's values are fetched as
+  // one batch of loads, not one after the other)
+  // (in f32, like the accumulators and the tuned kernels' fused chains)
+  float v[16];
+  int64_t rows[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int64_t m = m0 + wm * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+    rows[r] = m < M ? m : M - 1;
+    v[r] = fhip_round_through<float>(g.c_dt, acc[r]);
+  }
+  if (g.epi.count > 0)
+    fhip_apply_epilogue_many<float, 16>(g.epi, v, coord, rank - 2, rows);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int64_t m = m0 + wm * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
     if (m >= M)
       continue;
     coord[rank - 2] = m;
-    double v = fhip_round_through<double>(g.c_dt, (double)acc[r]);
-    v = fhip_apply_epilogue<double>(g.epi, v, coord);
-    fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
+    fhip_store<float>(out, g.o_dt, dot(coord, g.o, rank), v[r]);
   }
 }
 
@@ -306,17 +317,26 @@ __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
   if (n >= N)
     return;
   coord[rank - 1] = n;
+  float v[4];
+  int64_t rows[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int r = wave * 4 + q;
+    const int64_t m = m0 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+    const float sum = (part[0][r][l] + part[1][r][l]) + (part[2][r][l] + part[3][r][l]);
+    rows[q] = m < M ? m : M - 1;
+    v[q] = fhip_round_through<float>(g.c_dt, sum);
+  }
+  if (g.epi.count > 0)
+    fhip_apply_epilogue_many<float, 4>(g.epi, v, coord, rank - 2, rows);
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int r = wave * 4 + q;
     const int64_t m = m0 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
     if (m >= M)
       continue;
-    const float sum = (part[0][r][l] + part[1][r][l]) + (part[2][r][l] + part[3][r][l]);
     coord[rank - 2] = m;
-    double v = fhip_round_through<double>(g.c_dt, (double)sum);
-    v = fhip_apply_epilogue<double>(g.epi, v, coord);
-    fhip_store<double>(out, g.o_dt, dot(coord, g.o, rank), v);
+    fhip_store<float>(out, g.o_dt, dot(coord, g.o, rank), v[q]);
   }
 }
 
