@@ -712,6 +712,45 @@ __device__ __forceinline__ CT fhip_apply_epilogue(const DevEpilogue &e, CT v,
   return v;
 }
 
+// The helpers below handle several values of a thread.  Their rare cases (an
+// element type or mode outside the common ones) run the per-value helper --
+// a switch over every type / mode -- in a loop that is NOT unrolled: inlined
+// once per value those switches are most of a kernel's code (the 64 x 64-tile
+// f32 matmul kernel was 267 KB, refetched by every compute unit a small grid
+// lands on), and an out-of-line call would cost every kernel that contains
+// one its register budget.
+// N values to a tensor of runtime dtype (element n at idx[n] when bit n of
+// `live` is set): one switch for all.
+template <typename CT, int N>
+__device__ __forceinline__ void fhip_store_many(void *p, int dt, const int64_t (&idx)[N],
+                                                const CT (&v)[N], uint32_t live) {
+  switch (dt) {
+  case FHIP_FLOAT:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      if ((live >> n) & 1)
+        ((float *)p)[idx[n]] = (float)v[n];
+    break;
+  case FHIP_BFLOAT16:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      if ((live >> n) & 1)
+        ((__bf16 *)p)[idx[n]] = (__bf16)(float)v[n];
+    break;
+  case FHIP_HALF:
+#pragma unroll
+    for (int n = 0; n < N; ++n)
+      if ((live >> n) & 1)
+        ((_Float16 *)p)[idx[n]] = (_Float16)(float)v[n];
+    break;
+  default:
+#pragma clang loop unroll(disable)
+    for (int n = 0; n < N; ++n)
+      if ((live >> n) & 1)
+        fhip_store<CT>(p, dt, idx[n], v[n]);
+  }
+}
+
 // N elements of a tensor of runtime dtype at once: one switch for all, so the
 // loads are issued back to back (N calls of fhip_load each wait for their
 // value before the next address is even formed).
@@ -735,7 +774,7 @@ __device__ __forceinline__ void fhip_load_many(const void *p, int dt, const int6
       out[n] = (CT)(float)((const _Float16 *)p)[idx[n]];
     break;
   default:
-#pragma unroll
+#pragma clang loop unroll(disable)
     for (int n = 0; n < N; ++n)
       out[n] = fhip_load<CT>(p, dt, idx[n]);
   }
@@ -761,12 +800,12 @@ __device__ __forceinline__ void fhip_apply_epilogue_many(const DevEpilogue &e, C
         if (fast) {
           fhip_pw_fast_unary_vec<true, N>(o.mode, v, o.params.swish_beta);
         } else {
-#pragma unroll
+#pragma clang loop unroll(disable)
           for (int n = 0; n < N; ++n)
             v[n] = fhip_pw_unary<CT>(o.mode, v[n], o.params);
         }
       } else {
-#pragma unroll
+#pragma clang loop unroll(disable)
         for (int n = 0; n < N; ++n)
           v[n] = fhip_pw_unary<CT>(o.mode, v[n], o.params);
       }
@@ -794,7 +833,7 @@ __device__ __forceinline__ void fhip_apply_epilogue_many(const DevEpilogue &e, C
         }
       }
       if (!done) {
-#pragma unroll
+#pragma clang loop unroll(disable)
         for (int n = 0; n < N; ++n)
           v[n] = o.acc_is_in1 ? fhip_pw_binary<CT>(o.mode, other[n], v[n], o.params)
                               : fhip_pw_binary<CT>(o.mode, v[n], other[n], o.params);
@@ -805,7 +844,7 @@ __device__ __forceinline__ void fhip_apply_epilogue_many(const DevEpilogue &e, C
       if constexpr (kF32)
         fhip_round_fast_vec<N>(rd, v);
     } else {
-#pragma unroll
+#pragma clang loop unroll(disable)
       for (int n = 0; n < N; ++n)
         v[n] = fhip_round_through<CT>(rd, v[n]);
     }

@@ -205,18 +205,28 @@ __global__ __launch_bounds__(256) void tiled_matmul_f32_kernel(
   for (int r = 0; r < 16; ++r) {
     const int64_t m = m0 + wm * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
     rows[r] = m < M ? m : M - 1;
-    v[r] = fhip_round_through<float>(g.c_dt, acc[r]);
+    v[r] = acc[r];
+  }
+  if (g.c_dt == FHIP_BFLOAT16 || g.c_dt == FHIP_HALF) {
+    fhip_round_fast_vec<16>(g.c_dt, v);
+  } else if (g.c_dt != FHIP_FLOAT) {
+#pragma clang loop unroll(disable)
+    for (int r = 0; r < 16; ++r)
+      v[r] = fhip_round_through<float>(g.c_dt, v[r]);
   }
   if (g.epi.count > 0)
     fhip_apply_epilogue_many<float, 16>(g.epi, v, coord, rank - 2, rows);
+  coord[rank - 2] = 0;
+  const int64_t ob = dot(coord, g.o, rank), o_sm = g.o.s[rank - 2];
+  int64_t idx[16];
+  uint32_t live = 0;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int64_t m = m0 + wm * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
-    if (m >= M)
-      continue;
-    coord[rank - 2] = m;
-    fhip_store<float>(out, g.o_dt, dot(coord, g.o, rank), v[r]);
+    idx[r] = ob + m * o_sm;
+    live |= (uint32_t)(m < M) << r;
   }
+  fhip_store_many<float, 16>(out, g.o_dt, idx, v, live);
 }
 
 // Small outputs (few 64 x 64 tiles): a workgroup owns a 32 x 32 tile and its 4
@@ -325,19 +335,29 @@ __global__ __launch_bounds__(256) void splitk_matmul_f32_kernel(
     const int64_t m = m0 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
     const float sum = (part[0][r][l] + part[1][r][l]) + (part[2][r][l] + part[3][r][l]);
     rows[q] = m < M ? m : M - 1;
-    v[q] = fhip_round_through<float>(g.c_dt, sum);
+    v[q] = sum;
+  }
+  if (g.c_dt == FHIP_BFLOAT16 || g.c_dt == FHIP_HALF) {
+    fhip_round_fast_vec<4>(g.c_dt, v);
+  } else if (g.c_dt != FHIP_FLOAT) {
+#pragma clang loop unroll(disable)
+    for (int q = 0; q < 4; ++q)
+      v[q] = fhip_round_through<float>(g.c_dt, v[q]);
   }
   if (g.epi.count > 0)
     fhip_apply_epilogue_many<float, 4>(g.epi, v, coord, rank - 2, rows);
+  coord[rank - 2] = 0;
+  const int64_t ob = dot(coord, g.o, rank), o_sm = g.o.s[rank - 2];
+  int64_t idx[4];
+  uint32_t live = 0;
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     const int r = wave * 4 + q;
     const int64_t m = m0 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
-    if (m >= M)
-      continue;
-    coord[rank - 2] = m;
-    fhip_store<float>(out, g.o_dt, dot(coord, g.o, rank), v[q]);
+    idx[q] = ob + m * o_sm;
+    live |= (uint32_t)(m < M) << q;
   }
+  fhip_store_many<float, 4>(out, g.o_dt, idx, v, live);
 }
 
 // --------------------------------------------------------------------------
