@@ -615,11 +615,16 @@ gemm_kernel(GemmArgs g) {
     return ring0 + (uint32_t)st * STAGE + (HALO ? 0 : GA::kBytes);
   };
   // Part PART of PARTS of slice kt's loads (A and B split alike).
-  // Slices past the end of K are "loaded" with zero-sized buffers: nothing
-  // is fetched and the zeros land in a stage that is never read, which keeps
-  // every iteration identical (no tail variants, exact load counts).
+  // Slices past the end of K are not loaded at all; the loops' waits by count
+  // become waits for everything where a batch is missing.  (They used to be
+  // "loaded" through zero-sized buffers, which kept every iteration identical;
+  // but such a load counts as complete before its zeros are written to LDS:
+  // on tiles whose real loads return quickly the zeros of the last batch
+  // could land in the epilogue's bands, after the final wait and barrier.)
   auto issue = [&](int kt, int st, auto part_c, auto parts_c) {
-    const uint32_t lim = kt < kt_count ? 0xffffffffu : 0u;
+    if (kt >= kt_count)
+      return;
+    const uint32_t lim = 0xffffffffu;
     constexpr int PART = decltype(part_c)::value;
     constexpr int PARTS = decltype(parts_c)::value;
     constexpr int A0 = PART * GA::kLoads / PARTS, A1 = (PART + 1) * GA::kLoads / PARTS;
@@ -694,7 +699,7 @@ gemm_kernel(GemmArgs g) {
     static_assert(NSTAGE == 2, "ping-pong tiles alternate two stages");
     issue(0, 0, Zero{}, One{});
     if (wave >= 4)
-      issue(1, 1, Zero{}, One{});
+      issue(1, 1, Zero{}, One{}); // (nothing when there is one slice)
   } else {
 #pragma unroll
     for (int p = 0; p < NSTAGE; ++p)
@@ -744,7 +749,7 @@ gemm_kernel(GemmArgs g) {
   }
   if constexpr (PINGPONG) {
     // slice 0 has landed (wavefronts 4..7 keep their share of slice 1 in flight)
-    if (wave >= 4)
+    if (wave >= 4 && kt_count > 1)
       __builtin_amdgcn_s_waitcnt(gemm_wait_imm(LPS));
     else
       __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
@@ -836,7 +841,10 @@ gemm_kernel(GemmArgs g) {
         __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // the reads returned
         issue(kt + 2, cur, Zero{}, One{});
         // its share of slice kt + 1 (one batch older) has landed
-        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(LPS));
+        if (kt + 2 < kt_count)
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm(LPS));
+        else
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
       } else {
         issue(kt + 1, nxt, Zero{}, One{});
         // the reads returned: the other team may overwrite the stage next
@@ -891,7 +899,12 @@ gemm_kernel(GemmArgs g) {
         // Slice kt + 1 must be in LDS (this thread's DMA, then everyone's),
         // and every fragment read of this stage must have returned before
         // it is refilled.
-        __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
+        // (all but the NSTAGE - 2 slices behind it; everything where slices
+        // past the end were not loaded)
+        if (kt + NSTAGE - 1 < kt_count)
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm((NSTAGE - 2) * LPS));
+        else
+          __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -917,7 +930,7 @@ gemm_kernel(GemmArgs g) {
     cur = nxt;
   }
   }
-  // zero-sized loads of the last iterations may still be writing LDS
+  // (nothing is in flight any more; the stages become the epilogue's bands)
   __builtin_amdgcn_s_waitcnt(gemm_wait_imm(0));
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_s_barrier();

@@ -74,8 +74,16 @@ def worst_violations(got, ref, rtol, limit=8):
     excess = np.where(finite, np.abs(g - r) - (rtol * np.abs(r) + rtol * rms), 0.0)
     excess = np.nan_to_num(excess, nan=np.inf)
     order = np.argsort(excess, axis=None)[::-1][:limit]
-    return [(tuple(int(i) for i in np.unravel_index(o, g.shape)), float(g.flat[o]), float(r.flat[o]))
-            for o in order if excess.flat[o] > 0]
+    worst = [(tuple(int(i) for i in np.unravel_index(o, g.shape)), float(g.flat[o]), float(r.flat[o]))
+             for o in order if excess.flat[o] > 0]
+    # the extent of the damage: per dim the range of indices with a violation
+    # and how many distinct ones (a tile, a row of a wavefront, one column ...)
+    bad = np.argwhere(excess > 0)
+    if len(bad):
+        extent = [(int(bad[:, d].min()), int(bad[:, d].max()), int(len(np.unique(bad[:, d]))))
+                  for d in range(bad.shape[1])]
+        worst.append(("extent per dim (min, max, distinct)", extent))
+    return worst
 
 
 def assert_close(got, ref, dtype, what="", rtol=None):
