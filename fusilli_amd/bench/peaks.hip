@@ -108,6 +108,71 @@ __global__ __launch_bounds__(512) void mfma_loop(int iters, int random,
     sink[blockIdx.x * blockDim.x + threadIdx.x] = out;
 }
 
+// The same with the 16 x 16 MFMA shapes (K = 32 / 64 / 128): 16 independent
+// accumulators of four registers per wavefront.
+template <int KIND>
+__global__ __launch_bounds__(512) void mfma16_loop(int iters, int random, float *sink) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef int i32x4v __attribute__((ext_vector_type(4)));
+  uint32_t a[8], b[8];
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t h = mix(threadIdx.x * 16 + i + blockIdx.x * 8192);
+    if (KIND == K_BF16) {
+      a[i] = random ? ((h & 0x807f807fu) | 0x3f003f00u) : 0x3f803f80u;
+      b[i] = random ? ((mix(h) & 0x807f807fu) | 0x3f003f00u) : 0x3f803f80u;
+    } else if (KIND == K_I8) {
+      a[i] = random ? h : 0x01010101u;
+      b[i] = random ? mix(h) : 0x01010101u;
+    } else {
+      a[i] = random ? (h & 0xb7b7b7b7u) : 0x38383838u;
+      b[i] = random ? (mix(h) & 0xb7b7b7b7u) : 0x38383838u;
+    }
+  }
+  float out = 0.f;
+  if constexpr (KIND == K_I8) {
+    i32x4v acc[16];
+    for (int i = 0; i < 16; ++i)
+      for (int r = 0; r < 4; ++r)
+        acc[i][r] = 0;
+    const i32x4 va = {(int)a[0], (int)a[1], (int)a[2], (int)a[3]};
+    const i32x4 vb = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        acc[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(va, vb, acc[i], 0, 0, 0);
+    for (int i = 0; i < 16; ++i)
+      out += (float)acc[i][0];
+  } else {
+    f32x4 acc[16];
+    for (int i = 0; i < 16; ++i)
+      for (int r = 0; r < 4; ++r)
+        acc[i][r] = 0.f;
+    if constexpr (KIND == K_BF16) {
+      const u32x4 ua = {a[0], a[1], a[2], a[3]}, ub = {b[0], b[1], b[2], b[3]};
+      const bf16x8 va = __builtin_bit_cast(bf16x8, ua);
+      const bf16x8 vb = __builtin_bit_cast(bf16x8, ub);
+      for (int it = 0; it < iters; ++it)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, vb, acc[i], 0, 0, 0);
+    } else {
+      const i32x8 va = {(int)a[0], (int)a[1], (int)a[2], (int)a[3],
+                        (int)a[4], (int)a[5], (int)a[6], (int)a[7]};
+      const i32x8 vb = {(int)b[0], (int)b[1], (int)b[2], (int)b[3],
+                        (int)b[4], (int)b[5], (int)b[6], (int)b[7]};
+      for (int it = 0; it < iters; ++it)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+              va, vb, acc[i], 0, 0, 0, 0, 0, 0);
+    }
+    for (int i = 0; i < 16; ++i)
+      out += acc[i][0];
+  }
+  if (out == 12345.678f)
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = out;
+}
+
 // One contiguous chunk of UNROLL x 4 KiB per workgroup: all loads of a lane are
 // issued before its first store.
 template <int UNROLL>
@@ -205,6 +270,18 @@ double mfma_tops(double seconds, int random, int cus, float *sink) {
   return ops / ms / 1e9;
 }
 
+template <int KIND>
+double mfma16_tops(double seconds, int random, int cus, float *sink) {
+  const int iters = 2048;
+  const double ms = time_launches(seconds, [&] {
+    hipLaunchKernelGGL(mfma16_loop<KIND>, dim3(cus), dim3(512), 0, 0, iters, random, sink);
+  });
+  // per MFMA: 16 x 16 x K x 2 operations, K = 32 / 64 / 128
+  const double k = KIND == K_BF16 ? 32 : KIND == K_I8 ? 64 : 128;
+  const double ops = (double)cus * 8 * iters * 16 * 16 * 16 * k * 2;
+  return ops / ms / 1e9;
+}
+
 int main(int argc, char **argv) {
   const double seconds = argc > 1 ? atof(argv[1]) : 0.3;
   hipDeviceProp_t prop;
@@ -222,6 +299,12 @@ int main(int argc, char **argv) {
     for (int i = 0; i < 3; ++i)
       printf(", \"mfma_%s_%s_operands_tops\": %.1f", names[i],
              random ? "random" : "constant", t[i]);
+    const double u[3] = {mfma16_tops<K_BF16>(seconds, random, cus, sink),
+                         mfma16_tops<K_I8>(seconds, random, cus, sink),
+                         mfma16_tops<K_FP8>(seconds, random, cus, sink)};
+    for (int i = 0; i < 3; ++i)
+      printf(", \"mfma16x16_%s_%s_operands_tops\": %.1f", names[i],
+             random ? "random" : "constant", u[i]);
   }
   // 1 GiB source and destination (far beyond the 256 MB Infinity Cache); a
   // launch moves one 64 MiB window (the size of the benchmark's bf16

@@ -38,6 +38,7 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float gemm_f32x4 __attribute__((ext_vector_type(4)));
 
 // Pointer into LDS (address space 3) at a byte offset from a generic pointer
 // that is known to point into shared memory.
@@ -54,30 +55,35 @@ template <> struct KindTraits<GK_BF16> {
   static constexpr int kStepBytes = 32; // K bytes per row per MFMA
   using Acc = float;
   using AccVec = f32x16;
+  using AccVec4 = gemm_f32x4; // accumulators of a 16 x 16 MFMA
 };
 template <> struct KindTraits<GK_F16> {
   static constexpr int kElemBytes = 2;
   static constexpr int kStepBytes = 32;
   using Acc = float;
   using AccVec = f32x16;
+  using AccVec4 = gemm_f32x4;
 };
 template <> struct KindTraits<GK_I8> {
   static constexpr int kElemBytes = 1;
   static constexpr int kStepBytes = 32;
   using Acc = int;
   using AccVec = i32x16;
+  using AccVec4 = i32x4;
 };
 template <> struct KindTraits<GK_FP8E4M3> {
   static constexpr int kElemBytes = 1;
   static constexpr int kStepBytes = 64;
   using Acc = float;
   using AccVec = f32x16;
+  using AccVec4 = gemm_f32x4;
 };
 template <> struct KindTraits<GK_FP8E5M2> {
   static constexpr int kElemBytes = 1;
   static constexpr int kStepBytes = 64;
   using Acc = float;
   using AccVec = f32x16;
+  using AccVec4 = gemm_f32x4;
 };
 
 template <int N, typename F>
@@ -201,7 +207,36 @@ __device__ __forceinline__ void mfma32(typename KindTraits<KIND>::AccVec &c,
   }
 }
 
+// The 16 x 16 shapes with twice the K of the 32 x 32 ones (16x16x32 16-bit,
+// 16x16x64 int8, 16x16x128 fp8): the same operand bytes per lane, a quarter
+// of the accumulator registers per instruction.  Measured on register-resident
+// loops with random operand bits they sustain 13-21 % more than the 32 x 32
+// shapes (bf16 2.34 against 2.03 PFLOP/s, int8 4.33 / 3.58, fp8 4.74 / 4.20):
+// the matrix pipe is power-limited, and these shapes move less accumulator
+// data per operation.  Lane (row or column l % 16, K block l / 16) holds the
+// K block's STEPB / 2 consecutive bytes.
+template <int KIND>
+__device__ __forceinline__ void mfma16(typename KindTraits<KIND>::AccVec4 &c,
+                                       const Frag<KIND> &a, const Frag<KIND> &b) {
+  if constexpr (KIND == GK_BF16) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+        __builtin_bit_cast(bf16x8, a.r), __builtin_bit_cast(bf16x8, b.r), c, 0, 0, 0);
+  } else if constexpr (KIND == GK_F16) {
+    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+        __builtin_bit_cast(f16x8, a.r), __builtin_bit_cast(f16x8, b.r), c, 0, 0, 0);
+  } else if constexpr (KIND == GK_I8) {
+    c = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a.r),
+                                              __builtin_bit_cast(i32x4, b.r), c, 0, 0, 0);
+  } else {
+    constexpr int fmt = KIND == GK_FP8E4M3 ? 0 : 1; // 0 = e4m3, 1 = e5m2
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+        __builtin_bit_cast(i32x8, a.r), __builtin_bit_cast(i32x8, b.r), c, fmt, fmt, 0, 0, 0, 0);
+  }
+}
 
+#ifndef GEMM_M16
+#define GEMM_M16 1
+#endif
 #define GEMM_AS1 __attribute__((address_space(1)))
 #define GEMM_AS3 __attribute__((address_space(3)))
 
@@ -229,26 +264,32 @@ __device__ __forceinline__ int kc_swz(int r) { return (r & 7) ^ ((r >> 3) & 1); 
 // Chunk permutation of the M/N-contiguous layout.  A 32-lane half-wavefront
 // of a transposing read covers 4 K-rows x 64 bytes (16-bit) or 8 K-rows x
 // 32 bytes (8-bit); the permutation spreads those over all 64 banks.
-template <int ELEM, int RB> __device__ __forceinline__ int nkc_pos(int k, int c) {
+// With the 16 x 16 MFMA shapes the two 16-lane groups of a half-wavefront read
+// the same columns of K-rows that differ in bit XB of k (16 for 16-bit
+// elements, 32 for 8-bit ones): that bit sends them to different banks as
+// well.  XB = 0 for the 32 x 32 shapes.  (A bit of k above the lowest three
+// may only enter where it depends on the lane alone: fragment reads reach the
+// K-rows of later reads and K-steps through immediate offsets from one address.)
+template <int ELEM, int RB, int XB> __device__ __forceinline__ int nkc_pos(int k, int c) {
   if constexpr (ELEM == 2)
-    return c ^ ((k & 3) << 1) ^ ((c & 2) << 2);
+    return c ^ ((k & 3) << 1) ^ ((c & 2) << 2) ^ ((k & XB) ? 8 : 0);
   else if constexpr (RB == 256)
-    return c ^ ((k & 7) << 1);
+    return c ^ ((k & 7) << 1) ^ ((k & XB) ? 1 : 0);
   else
-    return c ^ (((k >> 1) & 3) << 1);
+    return c ^ (((k >> 1) & 3) << 1) ^ ((k & XB) ? 1 : 0);
 }
-template <int ELEM, int RB> __device__ __forceinline__ int nkc_chunk(int k, int p) {
+template <int ELEM, int RB, int XB> __device__ __forceinline__ int nkc_chunk(int k, int p) {
   if constexpr (ELEM == 2) {
-    const int t = p ^ ((k & 3) << 1);
+    const int t = p ^ ((k & 3) << 1) ^ ((k & XB) ? 8 : 0);
     return t ^ ((t & 2) << 2);
   } else {
-    return nkc_pos<ELEM, RB>(k, p);
+    return nkc_pos<ELEM, RB, XB>(k, p);
   }
 }
 
 // Per-thread byte offsets (from the tile's first row / column at K = 0) of the
 // chunks this thread's DMA instructions fetch; the same for every K slice.
-template <int ROWS, int ELEM, bool KCONTIG, int NW>
+template <int ROWS, int ELEM, bool KCONTIG, int NW, int XB>
 __device__ __forceinline__ void
 dma_setup(int64_t ld_bytes, int64_t row0, int64_t rows_total,
           uint32_t (&off)[SliceGeom<ROWS, ELEM, KCONTIG, NW>::kLoads]) {
@@ -265,7 +306,7 @@ dma_setup(int64_t ld_bytes, int64_t row0, int64_t rows_total,
       off[j] = (uint32_t)((r - row0) * ld_bytes + c * 16);
     } else {
       const int k = group * G::kRowsPerLoad + l / G::kCPR;
-      const int c = nkc_chunk<ELEM, G::kRowBytes>(k, l % G::kCPR);
+      const int c = nkc_chunk<ELEM, G::kRowBytes, XB>(k, l % G::kCPR);
       int64_t e = row0 + (int64_t)c * (16 / ELEM);
       const int64_t last = rows_total - 16 / ELEM;
       e = e < last ? e : last;
@@ -341,7 +382,7 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr {
           c = rb * 2 + h;
           sub = (L & 1) * 8;
         }
-        a[i] = (uint32_t)(k * RB + nkc_pos<ELEM, RB>(k, c) * 16 + sub);
+        a[i] = (uint32_t)(k * RB + nkc_pos<ELEM, RB, 0>(k, c) * 16 + sub);
       }
     }
   }
@@ -363,6 +404,106 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr {
         }
     } else {
       constexpr int KPL = STEPB / 2 / ELEM;
+      constexpr int RPK = ELEM == 2 ? 4 : 8; // K values per transposing read
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < KPL / RPK; ++r) {
+          const uint32_t ad = st + a[t] + (S * (STEPB / ELEM) + RPK * r) * RB;
+          if constexpr (ELEM == 2) {
+            const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (GEMM_AS3 s16x4 *)(uintptr_t)ad);
+            const u32x2 w = __builtin_bit_cast(u32x2, v);
+            f[t].r[2 * r + 0] = w.x;
+            f[t].r[2 * r + 1] = w.y;
+          } else {
+            const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                (GEMM_AS3 i32x2 *)(uintptr_t)ad);
+            f[t].r[2 * r + 0] = (uint32_t)v.x;
+            f[t].r[2 * r + 1] = (uint32_t)v.y;
+          }
+        }
+    }
+  }
+};
+
+// Fragment addressing for the 16 x 16 MFMA shapes: NT tiles of 16 rows, K-steps
+// of 2 * STEPB bytes.  Same LDS layouts as above (with the bit XB in the
+// M/N-contiguous one).  The 16-lane group g of a wavefront supplies K block
+// kq(g) of a step.  A 16-byte LDS read serves 16 lanes per clock: lanes
+// 32 h + 4 q + (0..3) for the four q in 0..7 of one parity of bit count; where
+// a block is one 16-byte chunk, kq = (0, 2, 1, 3) keeps each such set of rows
+// and chunks on distinct banks under the K-contiguous layout's swizzle.
+template <int KIND> struct Frag16Geom {
+  static constexpr int ELEM = KindTraits<KIND>::kElemBytes;
+  static constexpr int STEPB = 2 * KindTraits<KIND>::kStepBytes;
+  static constexpr int XB = ELEM == 2 ? 16 : 32;
+  __device__ static __forceinline__ int kq(int l) {
+    const int g = l >> 4;
+    return STEPB == 64 ? ((g & 1) << 1) | (g >> 1) : g;
+  }
+};
+template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr16 {
+  static constexpr int XB = Frag16Geom<KIND>::XB;
+  static constexpr int ELEM = KindTraits<KIND>::kElemBytes;
+  static constexpr int STEPB = 2 * KindTraits<KIND>::kStepBytes; // K bytes per row per MFMA
+  static constexpr int KSTEPS = kTileKBytes / STEPB;
+  static constexpr int CH = STEPB / 16;  // chunks per row per K-step
+  static constexpr int CHQ = CH / 4;     // 16-byte reads per fragment
+  static constexpr int RB = ROWS * ELEM; // M/N-contiguous: bytes per K-row
+  static constexpr int KPL = STEPB / 4 / ELEM; // K values per lane per step
+  static constexpr int N = KCONTIG ? KSTEPS * CHQ : NT;
+  uint32_t a[N];
+
+  __device__ __forceinline__ void setup(int tile0) {
+    const int l = threadIdx.x & 63;
+    if constexpr (KCONTIG) {
+      const int r = tile0 * 16 + (l & 15);
+      const int sw = kc_swz(l & 15);
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+        for (int i = 0; i < CHQ; ++i) {
+          const int c = s * CH + Frag16Geom<KIND>::kq(l) * CHQ + i;
+          a[s * CHQ + i] = (uint32_t)(r * kTileKBytes + ((c ^ sw) << 4));
+        }
+    } else {
+      // a 16-lane group reads the K block l / 16: its lanes address 4 (16-bit)
+      // or 8 (8-bit) K-rows x 16 matrix rows and each receives one matrix
+      // row's run of K values
+      const int L = l & 15;
+      const int k = Frag16Geom<KIND>::kq(l) * KPL + (ELEM == 2 ? (L >> 2) : (L >> 1));
+#pragma unroll
+      for (int i = 0; i < NT; ++i) {
+        const int rb = tile0 + i; // 16 matrix rows: 32 bytes (16-bit) or 16 (8-bit)
+        int c, sub;
+        if constexpr (ELEM == 2) {
+          c = rb * 2 + ((L & 3) >> 1);
+          sub = (L & 1) * 8;
+        } else {
+          c = rb;
+          sub = (L & 1) * 8;
+        }
+        a[i] = (uint32_t)(k * RB + nkc_pos<ELEM, RB, XB>(k, c) * 16 + sub);
+      }
+    }
+  }
+
+  template <int S>
+  __device__ __forceinline__ void load(uint32_t st, Frag<KIND> (&f)[NT]) const {
+    if constexpr (KCONTIG) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < CHQ; ++i) {
+          const u32x4 v = *(const GEMM_AS3 u32x4 *)(uintptr_t)(
+              st + a[S * CHQ + i] + t * 16 * kTileKBytes);
+          f[t].r[4 * i + 0] = v.x;
+          f[t].r[4 * i + 1] = v.y;
+          f[t].r[4 * i + 2] = v.z;
+          f[t].r[4 * i + 3] = v.w;
+        }
+    } else {
       constexpr int RPK = ELEM == 2 ? 4 : 8; // K values per transposing read
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -496,6 +637,13 @@ gemm_kernel(GemmArgs g) {
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr bool HALO = A_MODE == A_HALO;
   static_assert(!HALO || (ELEM == 2 && B_KC && NW == 4), "halo mode: 16-bit, 4 waves");
+  // The ping-pong GEMM tiles use the 16 x 16 MFMA shapes (twice the K per
+  // instruction): on operands with random bits the matrix pipe sustains 13 to
+  // 21 % more with them than with the 32 x 32 shapes.
+  constexpr bool M16 = GEMM_M16 && NW == 8 && (A_MODE == A_KCONTIG || A_MODE == A_MCONTIG);
+  constexpr int XB = M16 ? Frag16Geom<KIND>::XB : 0; // (M/N-contiguous LDS layout)
+  constexpr int KSTEPS16 = KSTEPS / 2;
+  constexpr int TM16 = WM / 16, TN16 = WN / 16;
   // DMA instructions per slice
   constexpr int LPS = (HALO ? 0 : GA::kLoads) + GB::kLoads;
 
@@ -587,12 +735,12 @@ gemm_kernel(GemmArgs g) {
     a_step = kTileKBytes;
     a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * a_ldb +
              kt_base * a_step;
-    dma_setup<BM, ELEM, true, NW>(a_ldb, m0, m_end, off_a);
+    dma_setup<BM, ELEM, true, NW, XB>(a_ldb, m0, m_end, off_a);
   } else {
     a_step = (int64_t)GA::kKRows * a_ldb;
     a_base = g.a + (batch * g.a_batch + outer * g.a_outer) * ELEM + m0 * ELEM +
              kt_base * a_step;
-    dma_setup<BM, ELEM, false, NW>(a_ldb, m0, m_end, off_a);
+    dma_setup<BM, ELEM, false, NW, XB>(a_ldb, m0, m_end, off_a);
   }
   const char *b_base;
   int64_t b_step;
@@ -605,7 +753,7 @@ gemm_kernel(GemmArgs g) {
     b_base = g.b + (batch * g.b_batch + outer * g.b_outer) * ELEM + n0 * ELEM +
              kt_base * b_step;
   }
-  dma_setup<BN, ELEM, B_KC, NW>(b_ldb, n0, g.N, off_b);
+  dma_setup<BN, ELEM, B_KC, NW, XB>(b_ldb, n0, g.N, off_b);
 
   // halo mode: [slab | ring of B slices]; otherwise a ring of (A, B) slices
   constexpr uint32_t STAGE = HALO ? GB::kBytes : L::kStage;
@@ -713,14 +861,29 @@ gemm_kernel(GemmArgs g) {
   fb_addr.setup(wn * TN);
   Frag<KIND> fa[2][TM], fb[2][TN];
 
-  typename KindTraits<KIND>::AccVec acc[TM][TN];
+  // Accumulators: value r of 32 x 32 tile (i, j).  With the 16 x 16 shapes
+  // that is value r & 3 of the 16 x 16 tile (2 i + (r >> 3), 2 j + ((r >> 2) & 1)).
+  typename KindTraits<KIND>::AccVec acc[M16 ? 1 : TM][M16 ? 1 : TN];
+  typename KindTraits<KIND>::AccVec4 acc16[M16 ? TM16 : 1][M16 ? TN16 : 1];
+  auto acc_get = [&](int i, int j, int r) __attribute__((always_inline)) -> Acc {
+    if constexpr (M16)
+      return acc16[i * 2 + (r >> 3)][j * 2 + ((r >> 2) & 1)][r & 3];
+    else
+      return acc[i][j][r];
+  };
+  auto acc_set = [&](int i, int j, int r, Acc v) __attribute__((always_inline)) {
+    if constexpr (M16)
+      acc16[i * 2 + (r >> 3)][j * 2 + ((r >> 2) & 1)][r & 3] = v;
+    else
+      acc[i][j][r] = v;
+  };
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r)
-        acc[i][j][r] = 0;
+        acc_set(i, j, r, 0);
   if constexpr (HALO) {
     // (computed while the prologue's loads are in flight)
 #pragma unroll
@@ -826,17 +989,32 @@ gemm_kernel(GemmArgs g) {
     // has two phases to land.
     const int team = __builtin_amdgcn_readfirstlane(wave >> 2);
     Frag<KIND> pa[KSTEPS][TM], pb[KSTEPS][TN];
+    FragAddr16<KIND, BM, A_KC, TM16> fa16;
+    FragAddr16<KIND, BN, B_KC, TN16> fb16;
+    Frag<KIND> qa[M16 ? KSTEPS16 : 1][TM16], qb[M16 ? KSTEPS16 : 1][TN16];
+    if constexpr (M16) {
+      fa16.setup(wm * TM16);
+      fb16.setup(wn * TN16);
+    }
     if (team)
       gemm_barrier();
     for (int kt = 0; kt < kt_count; ++kt) {
       const int nxt = cur ^ 1;
       // ---- memory phase
       const uint32_t sa = stage_a(cur), sb = stage_b(cur);
-      gemm_static_for<KSTEPS>([&](auto uc) {
-        constexpr int u = decltype(uc)::value;
-        fa_addr.template load<u>(sa, pa[u]);
-        fb_addr.template load<u>(sb, pb[u]);
-      });
+      if constexpr (M16) {
+        gemm_static_for<KSTEPS16>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
+          fa16.template load<u>(sa, qa[u]);
+          fb16.template load<u>(sb, qb[u]);
+        });
+      } else {
+        gemm_static_for<KSTEPS>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
+          fa_addr.template load<u>(sa, pa[u]);
+          fb_addr.template load<u>(sb, pb[u]);
+        });
+      }
       if (team) {
         __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // the reads returned
         issue(kt + 2, cur, Zero{}, One{});
@@ -855,14 +1033,25 @@ gemm_kernel(GemmArgs g) {
       __builtin_amdgcn_sched_barrier(0);
       // ---- MFMA phase
       __builtin_amdgcn_s_setprio(1);
-      gemm_static_for<KSTEPS>([&](auto uc) {
-        constexpr int u = decltype(uc)::value;
+      if constexpr (M16) {
+        gemm_static_for<KSTEPS16>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+          for (int i = 0; i < TM16; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            mfma32<KIND>(acc[i][j], pa[u][i], pb[u][j]);
-      });
+            for (int j = 0; j < TN16; ++j)
+              mfma16<KIND>(acc16[i][j], qa[u][i], qb[u][j]);
+        });
+      } else {
+        gemm_static_for<KSTEPS>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              mfma32<KIND>(acc[i][j], pa[u][i], pb[u][j]);
+        });
+      }
       __builtin_amdgcn_s_setprio(0);
       __builtin_amdgcn_sched_barrier(0);
       if (!team)
@@ -946,7 +1135,12 @@ gemm_kernel(GemmArgs g) {
   constexpr int RPP = 64 / LPR; // rows per pass
   constexpr int PPB = 32 / RPP; // passes per band
   const uint32_t band = lds0 + (uint32_t)wave * (BANDS * L::kBand);
-  const uint32_t wr = band + (uint32_t)((l >> 5) * 4 * PITCH + (l & 31) * 4);
+  // a lane's value r of tile (., j) lands at wr + row_of(r) * PITCH + col_of(j, r)
+  const uint32_t wr =
+      band + (uint32_t)(M16 ? (l >> 4) * 4 * PITCH + (l & 15) * 4
+                            : (l >> 5) * 4 * PITCH + (l & 31) * 4);
+  auto row_of = [](int r) { return M16 ? (r >> 3) * 16 + (r & 3) : (r >> 2) * 8 + (r & 3); };
+  auto col_of = [](int j, int r) { return M16 ? j * 128 + ((r >> 2) & 1) * 64 : j * 128; };
   const uint32_t rd = band + (uint32_t)((l / LPR) * PITCH + (l % LPR) * 32);
   const int64_t ob = batch * g.o_batch + outer * g.o_outer;
   const int64_t ncol = n0 + wn * WN + (l % LPR) * 8;
@@ -975,7 +1169,9 @@ gemm_kernel(GemmArgs g) {
   // (operand, -0) for MUL, (a, b * operand) for the additive modes.
   if constexpr (!std::is_same<Acc, int>::value) {
     if (lean && nops > 0) {
-      float S[FHIP_MAX_EPILOGUE][TN], T[FHIP_MAX_EPILOGUE][TN];
+      // (column tiles of 16 with the 16 x 16 shapes)
+      constexpr int CT = M16 ? TN16 : TN, CW = M16 ? 16 : 32;
+      float S[FHIP_MAX_EPILOGUE][CT], T[FHIP_MAX_EPILOGUE][CT];
       int lin_relu[FHIP_MAX_EPILOGUE];
       gemm_static_for<FHIP_MAX_EPILOGUE>([&](auto ec) {
         constexpr int e = decltype(ec)::value;
@@ -986,10 +1182,10 @@ gemm_kernel(GemmArgs g) {
         const bool mul = g.lin_mul[e] != 0;
         const float a = g.lin_a[e], b = g.lin_b[e];
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < CT; ++j) {
           float ov;
           if (o.kind == FHIP_OPERAND_TENSOR) {
-            int64_t n = n0 + wn * WN + j * 32 + (l & 31);
+            int64_t n = n0 + wn * WN + j * CW + (l & (CW - 1));
             n = n < g.N ? n : g.N - 1;
             const int64_t off[1] = {(n + outer * g.epi_n_outer) * o.stride[2]};
             float one[1];
@@ -1011,8 +1207,10 @@ gemm_kernel(GemmArgs g) {
 #pragma unroll
           for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-              acc[i][j][r] = __builtin_fmaf(acc[i][j][r], S[e][j], T[e][j]);
+            for (int r = 0; r < 16; ++r) {
+              const int c = M16 ? j * 2 + ((r >> 2) & 1) : j;
+              acc_set(i, j, r, __builtin_fmaf(acc_get(i, j, r), S[e][c], T[e][c]));
+            }
         if (lin_relu[e]) {
           // one instruction per value (fmaxf would first quiet its input);
           // NaN -> 0 like fmaxf
@@ -1022,9 +1220,9 @@ gemm_kernel(GemmArgs g) {
             for (int j = 0; j < TN; ++j)
 #pragma unroll
               for (int r = 0; r < 16; ++r) {
-                float y = acc[i][j][r];
+                float y = acc_get(i, j, r);
                 asm("v_max_f32 %0, 0, %0" : "+v"(y));
-                acc[i][j][r] = y;
+                acc_set(i, j, r, y);
               }
         }
       });
@@ -1034,7 +1232,12 @@ gemm_kernel(GemmArgs g) {
   // as packed pairs of consecutive rows (half the LDS traffic and passes).
   const bool packed = !std::is_same<Acc, int>::value && lean &&
                       (o_dt == FHIP_BFLOAT16 || o_dt == FHIP_HALF);
-  const uint32_t wr2 = band + (uint32_t)((l >> 5) * 2 * PITCH + (l & 31) * 4);
+  const uint32_t wr2 =
+      band + (uint32_t)(M16 ? (l >> 4) * 2 * PITCH + (l & 15) * 4
+                            : (l >> 5) * 2 * PITCH + (l & 31) * 4);
+  auto pair_row_of = [](int r) {
+    return M16 ? (r >> 3) * 8 + ((r & 3) >> 1) : (r >> 2) * 4 + ((r & 3) >> 1);
+  };
 
   gemm_static_for<TM / BANDS>([&](auto rc) {
     constexpr int round = decltype(rc)::value;
@@ -1049,8 +1252,8 @@ gemm_kernel(GemmArgs g) {
             for (int j = 0; j < TN; ++j)
 #pragma unroll
               for (int r = 0; r < 16; r += 2) {
-                const float lo = acc[round * BANDS + bi][j][r];
-                const float hi = acc[round * BANDS + bi][j][r + 1];
+                const float lo = acc_get(round * BANDS + bi, j, r);
+                const float hi = acc_get(round * BANDS + bi, j, r + 1);
                 uint32_t pk;
                 if constexpr (OT == 1) {
                   typedef __bf16 b2 __attribute__((ext_vector_type(2)));
@@ -1061,8 +1264,7 @@ gemm_kernel(GemmArgs g) {
                                           h2{(_Float16)lo, (_Float16)hi});
                 }
                 *(GEMM_AS3 uint32_t *)(uintptr_t)(
-                    wr2 + bi * L::kBand +
-                    ((r >> 2) * 4 + ((r & 3) >> 1)) * PITCH + j * 128) = pk;
+                    wr2 + bi * L::kBand + pair_row_of(r) * PITCH + col_of(j, r)) = pk;
               }
           // a pass covers RPP pair-rows = 2 * RPP rows
           constexpr int PPB2 = 16 / RPP;
@@ -1108,9 +1310,9 @@ gemm_kernel(GemmArgs g) {
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          *(GEMM_AS3 Acc *)(uintptr_t)(wr + bi * L::kBand +
-                                       ((r >> 2) * 8 + (r & 3)) * PITCH +
-                                       j * 128) = acc[round * BANDS + bi][j][r];
+          *(GEMM_AS3 Acc *)(uintptr_t)(wr + bi * L::kBand + row_of(r) * PITCH +
+                                       col_of(j, r)) =
+              acc_get(round * BANDS + bi, j, r);
     if (lean) {
       // 4-byte outputs (the chain has already run on the accumulators)
 #pragma unroll
