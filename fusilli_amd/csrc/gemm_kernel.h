@@ -640,7 +640,7 @@ gemm_kernel(GemmArgs g) {
   // The ping-pong GEMM tiles use the 16 x 16 MFMA shapes (twice the K per
   // instruction): on operands with random bits the matrix pipe sustains 13 to
   // 21 % more with them than with the 32 x 32 shapes.
-  constexpr bool M16 = GEMM_M16 && NW == 8 && (A_MODE == A_KCONTIG || A_MODE == A_MCONTIG);
+  constexpr bool M16 = GEMM_M16 && NW == 8;
   constexpr int XB = M16 ? Frag16Geom<KIND>::XB : 0; // (M/N-contiguous LDS layout)
   constexpr int KSTEPS16 = KSTEPS / 2;
   constexpr int TM16 = WM / 16, TN16 = WN / 16;
