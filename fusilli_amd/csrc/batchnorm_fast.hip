@@ -78,7 +78,7 @@ template <> struct BnVec<_Float16> : BnVec16<_Float16> {};
 template <typename T>
 __global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(BnFastArgs g) {
   using V = BnVec<T>;
-  extern __shared__ float red[]; // [row_lanes][2][C]
+  extern __shared__ __attribute__((aligned(16))) float red[]; // [row_lanes][2][C]
   const int chunk = threadIdx.x % g.chunks, lane = threadIdx.x / g.chunks;
   const int c0 = chunk * V::kN;
   float s1[V::kN], s2[V::kN];
@@ -90,27 +90,42 @@ __global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(BnFastArgs g) {
     V::load(g.x, c0, pv); // row 0
     const int64_t r0 = (int64_t)blockIdx.x * g.rows_per_wg;
     const int64_t r1 = r0 + g.rows_per_wg < g.rows ? r0 + g.rows_per_wg : g.rows;
-#pragma unroll 4
-    for (int64_t r = r0 + lane; r < r1; r += g.row_lanes) {
-      float v[V::kN];
-      V::load(g.x, r * g.C + c0, v);
+    // eight rows in flight per lane (a workgroup has a dozen or so in all:
+    // the loop is as long as its loads' latency, not its arithmetic); rows
+    // past the end re-read the last one and count as zero
+    constexpr int kFly = 8;
+    for (int64_t r = r0 + lane; r < r1; r += (int64_t)kFly * g.row_lanes) {
+      float v[kFly][V::kN];
 #pragma unroll
-      for (int k = 0; k < V::kN; ++k) {
-        const float d = v[k] - pv[k];
-        s1[k] += d;
-        s2[k] = __builtin_fmaf(d, d, s2[k]);
+      for (int u = 0; u < kFly; ++u) {
+        const int64_t rr = r + (int64_t)u * g.row_lanes;
+        V::load(g.x, (rr < r1 ? rr : r1 - 1) * g.C + c0, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kFly; ++u) {
+        const bool live = r + (int64_t)u * g.row_lanes < r1;
+#pragma unroll
+        for (int k = 0; k < V::kN; ++k) {
+          const float d = live ? v[u][k] - pv[k] : 0.f;
+          s1[k] += d;
+          s2[k] = __builtin_fmaf(d, d, s2[k]);
+        }
       }
     }
+    // (whole 16-byte stores: scalar ones would meet on the banks eight at a time)
 #pragma unroll
-    for (int k = 0; k < V::kN; ++k) {
-      red[(lane * 2 + 0) * g.C + c0 + k] = s1[k];
-      red[(lane * 2 + 1) * g.C + c0 + k] = s2[k];
+    for (int k = 0; k < V::kN; k += 4) {
+      *(float4 *)&red[(lane * 2 + 0) * g.C + c0 + k] =
+          make_float4(s1[k], s1[k + 1], s1[k + 2], s1[k + 3]);
+      *(float4 *)&red[(lane * 2 + 1) * g.C + c0 + k] =
+          make_float4(s2[k], s2[k + 1], s2[k + 2], s2[k + 3]);
     }
   }
   __syncthreads();
   // the row lanes' sums, in lane order, by the first 2 C threads (in turns)
   for (int o = threadIdx.x; o < 2 * g.C; o += kBnThreads) {
     float acc = 0.f;
+#pragma unroll 8
     for (int l = 0; l < g.row_lanes; ++l)
       acc += red[l * 2 * g.C + o];
     g.partial[(int64_t)blockIdx.x * 2 * g.C + o] = acc;
@@ -119,31 +134,43 @@ __global__ __launch_bounds__(kBnThreads) void bn_stats_kernel(BnFastArgs g) {
 
 // pass 2 / 2': per channel the multiplier inv * scale, the mean and the bias.
 // A workgroup serves 4 channels: 64 lanes per channel add the workgroups'
-// sums w, w + 64, ... and meet in LDS, in lane order.
+// sums w, w + 64, ... and meet through a fixed tree (lanes of a wavefront by
+// cross-lane moves, the four wavefronts in LDS), the same for every run.
 constexpr int kBnFinCh = 4;
 template <typename T>
 __global__ __launch_bounds__(kBnThreads) void bn_finalize_kernel(BnFastArgs g) {
-  __shared__ float red[kBnThreads / kBnFinCh][kBnFinCh][2];
+  __shared__ float red[kBnThreads / 64][kBnFinCh][2];
   const int ci = threadIdx.x % kBnFinCh, wl = threadIdx.x / kBnFinCh;
   const int c = blockIdx.x * kBnFinCh + ci;
   const bool live = c < g.C;
   float s1 = 0.f, s2 = 0.f;
-  if (g.training && live) {
-#pragma unroll 4
-    for (int w = wl; w < g.nwg; w += kBnThreads / kBnFinCh) {
-      s1 += g.partial[(int64_t)w * 2 * g.C + c];
-      s2 += g.partial[(int64_t)w * 2 * g.C + g.C + c];
+  if (g.training) {
+    if (live) {
+#pragma unroll 8
+      for (int w = wl; w < g.nwg; w += kBnThreads / kBnFinCh) {
+        s1 += g.partial[(int64_t)w * 2 * g.C + c];
+        s2 += g.partial[(int64_t)w * 2 * g.C + g.C + c];
+      }
+    }
+    // lanes l, l ^ 4, l ^ 8, ... hold the same channel
+#pragma unroll
+    for (int m = kBnFinCh; m < 64; m <<= 1) {
+      s1 += __shfl_xor(s1, m, 64);
+      s2 += __shfl_xor(s2, m, 64);
+    }
+    if ((threadIdx.x & 63) < kBnFinCh) {
+      red[threadIdx.x >> 6][ci][0] = s1;
+      red[threadIdx.x >> 6][ci][1] = s2;
     }
   }
-  red[wl][ci][0] = s1;
-  red[wl][ci][1] = s2;
   __syncthreads();
   if (wl != 0 || !live)
     return;
   float mean, inv;
   if (g.training) {
     s1 = s2 = 0.f;
-    for (int l = 0; l < kBnThreads / kBnFinCh; ++l) {
+#pragma unroll
+    for (int l = 0; l < kBnThreads / 64; ++l) {
       s1 += red[l][ci][0];
       s2 += red[l][ci][1];
     }
