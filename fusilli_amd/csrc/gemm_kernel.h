@@ -430,18 +430,19 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr {
 // Fragment addressing for the 16 x 16 MFMA shapes: NT tiles of 16 rows, K-steps
 // of 2 * STEPB bytes.  Same LDS layouts as above (with the bit XB in the
 // M/N-contiguous one).  The 16-lane group g of a wavefront supplies K block
-// kq(g) of a step.  A 16-byte LDS read serves 16 lanes per clock: lanes
-// 32 h + 4 q + (0..3) for the four q in 0..7 of one parity of bit count; where
-// a block is one 16-byte chunk, kq = (0, 2, 1, 3) keeps each such set of rows
-// and chunks on distinct banks under the K-contiguous layout's swizzle.
+// g of a step.  A 16-byte LDS read serves 16 lanes per clock: lanes
+// 32 h + 4 q + (0..3) for the four q in 0..7 of one parity of bit count, i.e.
+// lanes 0-3 and 12-15 of one group with lanes 4-11 of the next.  Under the
+// K-contiguous layout's swizzle such a set stays on distinct banks when lane i
+// of a group reads tile row row16(i) = i with the blocks 8-11 and 12-15
+// exchanged; the MFMA's output rows (A) or columns (B) are then permuted the
+// same way, which the epilogue's LDS writes undo.  (The K blocks stay in their
+// natural order: every tile shape adds a slice's products in the same order.)
 template <int KIND> struct Frag16Geom {
   static constexpr int ELEM = KindTraits<KIND>::kElemBytes;
   static constexpr int STEPB = 2 * KindTraits<KIND>::kStepBytes;
-  static constexpr int XB = ELEM == 2 ? 16 : 32;
-  __device__ static __forceinline__ int kq(int l) {
-    const int g = l >> 4;
-    return STEPB == 64 ? ((g & 1) << 1) | (g >> 1) : g;
-  }
+  static constexpr int XB = STEPB / 4 / ELEM; // K values per lane: 8, 16 (int8), 32 (fp8)
+  __device__ static __forceinline__ int row16(int i) { return i ^ ((i >> 1) & 4); }
 };
 template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr16 {
   static constexpr int XB = Frag16Geom<KIND>::XB;
@@ -458,13 +459,14 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr16 {
   __device__ __forceinline__ void setup(int tile0) {
     const int l = threadIdx.x & 63;
     if constexpr (KCONTIG) {
-      const int r = tile0 * 16 + (l & 15);
-      const int sw = kc_swz(l & 15);
+      const int r16 = Frag16Geom<KIND>::row16(l & 15);
+      const int r = tile0 * 16 + r16;
+      const int sw = kc_swz(r16);
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s)
 #pragma unroll
         for (int i = 0; i < CHQ; ++i) {
-          const int c = s * CH + Frag16Geom<KIND>::kq(l) * CHQ + i;
+          const int c = s * CH + (l >> 4) * CHQ + i;
           a[s * CHQ + i] = (uint32_t)(r * kTileKBytes + ((c ^ sw) << 4));
         }
     } else {
@@ -472,7 +474,7 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr16 {
       // or 8 (8-bit) K-rows x 16 matrix rows and each receives one matrix
       // row's run of K values
       const int L = l & 15;
-      const int k = Frag16Geom<KIND>::kq(l) * KPL + (ELEM == 2 ? (L >> 2) : (L >> 1));
+      const int k = (l >> 4) * KPL + (ELEM == 2 ? (L >> 2) : (L >> 1));
 #pragma unroll
       for (int i = 0; i < NT; ++i) {
         const int rb = tile0 + i; // 16 matrix rows: 32 bytes (16-bit) or 16 (8-bit)
@@ -1136,8 +1138,13 @@ gemm_kernel(GemmArgs g) {
   constexpr int PPB = 32 / RPP; // passes per band
   const uint32_t band = lds0 + (uint32_t)wave * (BANDS * L::kBand);
   // a lane's value r of tile (., j) lands at wr + row_of(r) * PITCH + col_of(j, r)
+  // (16 x 16 shapes: a K-contiguous operand's fragments hold the tile rows in
+  // the order row16, so the output's row blocks 2 and 3 (A) or its columns (B)
+  // come out exchanged the same way)
+  const int g16 = A_KC ? (l >> 4) ^ (l >> 5) : l >> 4;
+  const int c16 = B_KC ? Frag16Geom<KIND>::row16(l & 15) : l & 15;
   const uint32_t wr =
-      band + (uint32_t)(M16 ? (l >> 4) * 4 * PITCH + (l & 15) * 4
+      band + (uint32_t)(M16 ? g16 * 4 * PITCH + c16 * 4
                             : (l >> 5) * 4 * PITCH + (l & 31) * 4);
   auto row_of = [](int r) { return M16 ? (r >> 3) * 16 + (r & 3) : (r >> 2) * 8 + (r & 3); };
   auto col_of = [](int j, int r) { return M16 ? j * 128 + ((r >> 2) & 1) * 64 : j * 128; };
@@ -1185,7 +1192,7 @@ gemm_kernel(GemmArgs g) {
         for (int j = 0; j < CT; ++j) {
           float ov;
           if (o.kind == FHIP_OPERAND_TENSOR) {
-            int64_t n = n0 + wn * WN + j * CW + (l & (CW - 1));
+            int64_t n = n0 + wn * WN + j * CW + (M16 ? c16 : l & 31);
             n = n < g.N ? n : g.N - 1;
             const int64_t off[1] = {(n + outer * g.epi_n_outer) * o.stride[2]};
             float one[1];
@@ -1233,7 +1240,7 @@ gemm_kernel(GemmArgs g) {
   const bool packed = !std::is_same<Acc, int>::value && lean &&
                       (o_dt == FHIP_BFLOAT16 || o_dt == FHIP_HALF);
   const uint32_t wr2 =
-      band + (uint32_t)(M16 ? (l >> 4) * 2 * PITCH + (l & 15) * 4
+      band + (uint32_t)(M16 ? g16 * 2 * PITCH + c16 * 4
                             : (l >> 5) * 2 * PITCH + (l & 31) * 4);
   auto pair_row_of = [](int r) {
     return M16 ? (r >> 3) * 8 + ((r & 3) >> 1) : (r >> 2) * 4 + ((r & 3) >> 1);
