@@ -61,7 +61,7 @@ struct FhipKnobs {
   int conv_rows = -1;               // FUSILLI_HIP_CONV_ROWS (-1: unset)
   int gemm_tile_bm = 0, gemm_tile_bn = 0; // FUSILLI_HIP_GEMM_TILE "bm,bn"
   bool conv_depthwise_strips = true; // FUSILLI_HIP_CONV_DEPTHWISE_STRIPS=0: the general small-group kernel
-  int gemm_split = 0;               // FUSILLI_HIP_GEMM_SPLIT (parts of a split reduction; 0: planner)
+  int gemm_split = 0;               // FUSILLI_HIP_GEMM_SPLIT (parts of a split reduction; 0: planner, 1: none)
   int conv_slices = 0;              // FUSILLI_HIP_CONV_SLICES (channel slices per workgroup of the register-filter kernel: 2 or 4; 0: planner)
   int wgrad_direct = -1;            // FUSILLI_HIP_WGRAD_DIRECT (-1: unset, 0: off)
   int dgrad_rf = -1;                // FUSILLI_HIP_DGRAD_ROWS (-1: unset, 0: off, n: rows per

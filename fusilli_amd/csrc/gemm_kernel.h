@@ -403,26 +403,28 @@ template <int KIND, int ROWS, bool KCONTIG, int NT> struct FragAddr {
           f[t].r[4 * i + 3] = v.w;
         }
     } else {
+      // Written as asm: the compiler makes the transposing-read builtins wait
+      // for every global -> LDS load in flight (vmcnt(0)), the prefetched
+      // slices included, and spends an address addition on each.  The caller
+      // waits for these reads itself (lgkmcnt) before it uses the fragments.
       constexpr int KPL = STEPB / 2 / ELEM;
       constexpr int RPK = ELEM == 2 ? 4 : 8; // K values per transposing read
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int r = 0; r < KPL / RPK; ++r) {
-          const uint32_t ad = st + a[t] + (S * (STEPB / ELEM) + RPK * r) * RB;
-          if constexpr (ELEM == 2) {
-            const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (GEMM_AS3 s16x4 *)(uintptr_t)ad);
-            const u32x2 w = __builtin_bit_cast(u32x2, v);
-            f[t].r[2 * r + 0] = w.x;
-            f[t].r[2 * r + 1] = w.y;
-          } else {
-            const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-                (GEMM_AS3 i32x2 *)(uintptr_t)ad);
-            f[t].r[2 * r + 0] = (uint32_t)v.x;
-            f[t].r[2 * r + 1] = (uint32_t)v.y;
-          }
-        }
+      for (int t = 0; t < NT; ++t) {
+        const uint32_t ad = st + a[t];
+        gemm_static_for<KPL / RPK>([&](auto rc) {
+          constexpr int r = decltype(rc)::value;
+          constexpr int OFF = (S * (STEPB / ELEM) + RPK * r) * RB;
+          static_assert(OFF >= 0 && OFF < 65536, "16-bit offset field");
+          u32x2 w;
+          if constexpr (ELEM == 2)
+            asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(w) : "v"(ad), "n"(OFF));
+          else
+            asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(w) : "v"(ad), "n"(OFF));
+          f[t].r[2 * r + 0] = w.x;
+          f[t].r[2 * r + 1] = w.y;
+        });
+      }
     }
   }
 };
@@ -963,6 +965,11 @@ gemm_kernel(GemmArgs g) {
     fa_addr.template load<0>(stage_a(0), fa[0]);
   }
   fb_addr.template load<0>(stage_b(0), fb[0]);
+  if constexpr (!PINGPONG && (!A_KC || !B_KC)) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // (transposing reads are asm)
+    __builtin_amdgcn_sched_barrier(0);
+  }
 
   // Reads per fragment set and the loads of a slice spread over the K-steps
   // that precede the barrier.
@@ -1119,6 +1126,12 @@ gemm_kernel(GemmArgs g) {
       constexpr int NV = LAST ? LPS / 2 : (s == 0 ? LPS - LPS / 2 : 0);
       gemm_interleave<TM * TN, NRA + NRB, NV>();
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (!A_KC || !B_KC) {
+        // the next step's transposing reads (asm: the compiler does not wait
+        // for them), issued a K-step of MFMAs ago
+        __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63));
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
     cur = nxt;
   }

@@ -134,59 +134,79 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
         return p;
     }
   }
-  // Tile shape: the one with the shortest estimated run -- the MFMA work at
-  // the tile's usual share of the peak (256 x 256 and 256 x 128 on eight
-  // wavefronts in two phases: a half and four tenths; 128 x 128 on four in
-  // order: a fifth) over the share of the 256 compute units that have a tile.
+  // Tile shape and reduction split: the pair with the shortest estimated run.
+  // A workgroup's time is a fixed part (prologue, epilogue: not overlapped
+  // between the rounds of eight-wavefront tiles, mostly hidden behind the
+  // second resident workgroup of the 128 x 128 tile) plus its K slices at the
+  // tile's measured pace; the tiles run in rounds of 256 (one per compute
+  // unit), and a round that leaves compute units idle runs at a higher clock
+  // (fitted: 0.65 + 0.35 x the busy share).  Microseconds on this chip, from
+  // 2048^3 ... 8192 x 8192 x 1024 problems of each type.
+  const bool k16 = p.kind == GK_BF16 || p.kind == GK_F16;
+  const int64_t slices = p.K * elem / kTileKBytes;
   auto tiles = [&](int bm, int bn) {
     return (double)(((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * p.batch);
   };
-  auto busy = [](double t) { return t < 256.0 ? t / 256.0 : 1.0; };
-  auto eff = [](int bm, int bn) {
-    return bm == 256 && bn == 256 ? 0.5 : (bm == 256 ? 0.4 : 0.2);
+  auto estimate = [&](int bm, int bn, int sk) {
+    const int shape = bm == 256 && bn == 256 ? 0 : (bm == 256 ? 1 : 2);
+    static const double pace16[3] = {1.36, 0.90, 0.64}, pace8f[3] = {1.275, 0.876, 0.88},
+                        pace8i[3] = {1.38, 0.95, 0.70};
+    static const double fixed16[3] = {11.0, 6.7, 7.4}, fixed8f[3] = {11.0, 5.7, 2.0},
+                        fixed8i[3] = {18.0, 9.0, 8.0};
+    const double pace = (k16 ? pace16 : p.kind == GK_I8 ? pace8i : pace8f)[shape];
+    const double fixed = (k16 ? fixed16 : p.kind == GK_I8 ? fixed8i : fixed8f)[shape];
+    const double t = tiles(bm, bn) * sk;
+    const double full = floor(t / 256.0), rest = t - 256.0 * full;
+    const double rounds = full + (rest > 0 ? 1 : 0);
+    const double work = full + (rest > 0 ? 0.65 + 0.35 * rest / 256.0 : 0.0);
+    double us = (double)(slices / sk) * pace * work +
+                (shape == 2 ? fixed + 3.0 * (rounds - 1) : fixed * rounds);
+    if (sk > 1) // the parts' f32 stores and the kernel that adds them (~5 TB/s each way)
+      us += 2.0 * sk * (double)p.M * (double)p.N * 4.0 / 5.0e6 + 2.5;
+    return us;
   };
-  p.bm = p.bn = 128;
-  // (ties go to the larger tile: compute units run faster when others idle)
-  if (p.M >= 256 && eff(256, 128) * busy(tiles(256, 128)) >= eff(p.bm, p.bn) * busy(tiles(p.bm, p.bn)))
-    p.bm = 256, p.bn = 128;
-  if (p.M >= 256 && p.N >= 256 &&
-      eff(256, 256) * busy(tiles(256, 256)) >= eff(p.bm, p.bn) * busy(tiles(p.bm, p.bn)))
-    p.bm = 256, p.bn = 256;
-  // the largest tile the shape allows (for the cut below)
-  const int bm0 = p.M >= 256 ? 256 : 128, bn0 = p.N >= 256 && bm0 == 256 ? 256 : 128;
-  // Few tiles and a long reduction: K is cut into parts on workgroups of their
-  // own, on the large tile, when a rough model says that the parts' f32 round
-  // trip through memory costs less than the idle compute units do.
-  // (1024 x 1024 x 8192 bf16: 64 tiles of 128 x 128 135 us; 16 tiles x 8 parts
-  // 44 us.  512 x 512 x 16384: 269 -> 27 us.)
-  if (p.batch == 1 && p.kind != GK_I8 && p.N % 4 == 0 && p.o_sn == 1 && allow_split) {
-    const double peak = (p.kind == GK_BF16 || p.kind == GK_F16) ? 2.5e15 : 5.0e15;
-    const double flop = 2.0 * (double)p.M * (double)p.N * (double)p.K;
-    const double t0 = flop / (eff(p.bm, p.bn) * peak * busy(tiles(p.bm, p.bn)));
-    const int64_t slices = p.K * elem / kTileKBytes;
-    double best = 0.8 * t0;
-    for (int sk = 2; sk <= 128; ++sk) {
-      if (slices % sk != 0 || slices / sk < 8)
+  const int forced = fhip_knobs().gemm_split; // (1: never split)
+  const bool may_split = p.batch == 1 && p.kind != GK_I8 && p.N % 4 == 0 && p.o_sn == 1 &&
+                         allow_split && forced != 1;
+  double best = 0;
+  p.bm = p.bn = 0;
+  static const int shapes[3][2] = {{128, 128}, {256, 128}, {256, 256}};
+  for (int i = 0; i < 3; ++i) {
+    const int bm = shapes[i][0], bn = shapes[i][1];
+    if (i > 0 && (p.M < bm || p.N < bn))
+      continue;
+    for (int sk = 1; sk <= 128; ++sk) {
+      if (sk > 1 && (!may_split || slices % sk != 0 || slices / sk < 8))
         continue;
-      const double t = flop / (eff(bm0, bn0) * peak * busy(tiles(bm0, bn0) * sk)) +
-                       2.0 * sk * (double)p.M * (double)p.N * 4.0 / 3.0e12;
-      if (t < best) {
-        best = t;
-        p.ksplit = sk;
+      // (a forced count must still divide the slices into runs of at least 8)
+      if (forced > 1 && may_split && slices % forced == 0 && slices / forced >= 8 && sk != forced)
+        continue;
+      // a split must pay clearly; ties go to the larger tile (compute units
+      // run faster while others idle)
+      const double us = estimate(bm, bn, sk) * (sk > 1 ? 1.1 : 1.0);
+      if (p.bm == 0 || us <= best) {
+        best = us;
+        p.bm = bm, p.bn = bn, p.ksplit = sk;
       }
     }
-    // (a forced count must still divide the slices into runs of at least 8)
-    const int forced = fhip_knobs().gemm_split;
-    if (forced > 1 && slices % forced == 0 && slices / forced >= 8)
-      p.ksplit = forced;
-    if (p.ksplit > 1)
-      p.bm = bm0, p.bn = bn0;
   }
   if (fhip_knobs().gemm_tile_bm) {
     const int bm = fhip_knobs().gemm_tile_bm, bn = fhip_knobs().gemm_tile_bn;
     if ((bm == 128 || bm == 256) &&
-        (bn == 128 || bn == 256) && bm >= bn && bm <= p.M && bn <= p.N)
-      p.bm = bm, p.bn = bn;
+        (bn == 128 || bn == 256) && bm >= bn && bm <= p.M && bn <= p.N) {
+      // the best split for the forced shape
+      p.bm = bm, p.bn = bn, p.ksplit = 1;
+      best = estimate(bm, bn, 1);
+      for (int sk = 2; sk <= 128 && may_split; ++sk) {
+        if (slices % sk != 0 || slices / sk < 8)
+          continue;
+        if (forced > 1 && slices % forced == 0 && slices / forced >= 8 && sk != forced)
+          continue;
+        const double us = estimate(bm, bn, sk) * 1.1;
+        if (us < best || sk == forced)
+          best = us, p.ksplit = sk;
+      }
+    }
   }
   p.ok = true;
   return p;

@@ -134,11 +134,12 @@ def test_gemm_split_reduction_benchmark_shape(ctx):
 
 
 def test_gemm_tile_shapes_agree_bit_for_bit(ctx, knobs):
-    # 1024 x 2048 x 4096 bf16 takes 256 x 128 tiles (eight wavefronts, 64 x 64
-    # outputs each).  Every output element accumulates its K slices in the same
-    # order on every tile shape, so repeated runs and the other tile shapes
-    # must give the same bits; a wavefront reading a stage that another is
-    # still filling would not.
+    # 1024 x 2048 x 4096 bf16 with the reduction in one piece (a split adds
+    # its parts in f32, another order).  Every output element accumulates its
+    # K slices in the same order on every tile shape, so repeated runs and the
+    # other tile shapes must give the same bits; a wavefront reading a stage
+    # that another is still filling would not.
+    knobs(GEMM_SPLIT="1")
     a = make_operand(75, 0, 1024, 4096, capi.BFLOAT16, False)
     b = make_operand(75, 1, 4096, 2048, capi.BFLOAT16, True)
     first = run(ctx, a, b, capi.FLOAT).logical()
@@ -146,7 +147,7 @@ def test_gemm_tile_shapes_agree_bit_for_bit(ctx, knobs):
     for _ in range(8):
         assert np.array_equal(run(ctx, a, b, capi.FLOAT).logical(), first)
     for tile in ("256,256", "256,128", "128,128"):
-        knobs(GEMM_TILE=tile)
+        knobs(GEMM_TILE=tile, GEMM_SPLIT="1")
         assert np.array_equal(run(ctx, a, b, capi.FLOAT).logical(), first), tile
 
 
