@@ -742,14 +742,16 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
       // the fragments of the next MFMA phase; returns this lane's sum.  (Summing
       // the rounded pairs with v_dot2c_f32_bf16 measured slower than two adds.)
       auto exps = [&](float ref) __attribute__((always_inline)) {
-        const float mc = ref * sl2;
+        // (one fused multiply-add per score, spelled out: left to itself the
+        // compiler scales every score first and fuses the reference instead)
+        const float mc = -(ref * sl2);
         float psum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
-            const float p0 = __builtin_amdgcn_exp2f(s[kb][r] * sl2 - mc);
-            const float p1 = __builtin_amdgcn_exp2f(s[kb][r + 1] * sl2 - mc);
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][r], sl2, mc));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][r + 1], sl2, mc));
             const uint32_t pk = sd_pack<BF16>(p0, p1);
             pf[kb * 2 + (r >> 3)][(r & 7) >> 1] = pk;
             psum += p0 + p1;
@@ -773,7 +775,10 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
   #pragma clang loop unroll(disable)
         for (;;) {
           if (full) {
+            // (the asm keeps the row maximum inside this branch: the compiler
+            // would compute it on the common route as well)
             float mx = s[0][0];
+            asm volatile("" : "+v"(mx));
   #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
   #pragma unroll
@@ -822,6 +827,7 @@ __global__ __launch_bounds__(kWaves * 64) void sdpa_fwd_kernel(SdpaArgs g) {
         }
         if (full) {
           float mx = s[0][0];
+          asm volatile("" : "+v"(mx)); // (keeps the maximum off the fast route)
 #pragma unroll
           for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
