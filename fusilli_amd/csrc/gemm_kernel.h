@@ -958,17 +958,23 @@ gemm_kernel(GemmArgs g) {
       f[i].r[3] = v.w;
     }
   };
-  if constexpr (HALO) {
-    halo_tap(0);
-    halo_load(Zero{}, fa[0]);
-  } else {
-    fa_addr.template load<0>(stage_a(0), fa[0]);
-  }
-  fb_addr.template load<0>(stage_b(0), fb[0]);
-  if constexpr (!PINGPONG && (!A_KC || !B_KC)) {
-    __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // (transposing reads are asm)
-    __builtin_amdgcn_sched_barrier(0);
+  // The in-order loop starts with K-step 0's fragments in hand.  (Not the
+  // two-phase loop, which reads whole slices itself: a transposing read is asm
+  // whose result nobody would use there, so its registers would be given to
+  // other values at once -- and be overwritten when the read returns.)
+  if constexpr (!PINGPONG) {
+    if constexpr (HALO) {
+      halo_tap(0);
+      halo_load(Zero{}, fa[0]);
+    } else {
+      fa_addr.template load<0>(stage_a(0), fa[0]);
+    }
+    fb_addr.template load<0>(stage_b(0), fb[0]);
+    if constexpr (!A_KC || !B_KC) {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(gemm_wait_imm(63)); // (transposing reads are asm)
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 
   // Reads per fragment set and the loads of a slice spread over the K-steps
