@@ -270,6 +270,13 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
          // the gather: 55.6 vs 74 us for C = K = 128, 56 x 56; 24 vs 32 us for
          // C = K = 256, 14 x 14 at N = 32 and 46 vs 52 us at N = 128
       bm = small256 && big ? 256 : (fits128 ? 128 : 0);
+    // ... unless the gather would run its 128 x 128 tiles (eight wavefronts,
+    // two workgroups per compute unit) over two rounds of the machine or more:
+    // C256 -> K64 1 x 1 at 56 x 56 24.8 -> 18.0 us, C = K = 128 3 x 3 at 56 x 56
+    // and N = 64 98 -> 84 us (C = K = 128 at 28 x 28, 196 tiles: halo 16.2, gather 20.7)
+    if (want < 0 && bm == 128 && p.bm == 128 && p.bn == 128 &&
+        ((p.M + 127) / 128) * ((p.N + 127) / 128) * p.groups >= 512)
+      bm = 0;
     if (bm) {
       p.halo = true;
       p.bm = bm;

@@ -594,13 +594,15 @@ __device__ __forceinline__ void load_operand_vec(const void *p, int dt,
 // reuses it for four 32-row accumulator bands (one per wavefront).
 // Wavefront grid of a tile.  8 wavefronts (two per SIMD, scheduled in
 // alternating memory / MFMA phases): 256 x 256 as 2 x 4 and 512 x 128 as 4 x 2,
-// each wavefront owning 128 x 64 outputs, and 256 x 128 as 4 x 2 of 64 x 64;
-// 4 wavefronts as 2 x 2.
+// each wavefront owning 128 x 64 outputs, 256 x 128 as 4 x 2 of 64 x 64 and
+// 128 x 128 (GEMM, gather convolution) as 2 x 4 of 64 x 32; 4 wavefronts (the
+// halo convolution) as 2 x 2.
 template <int BM, int BN, int NW = 0> struct GemmLayout {
   static constexpr bool kWide = BM == 256 && BN == 256;
   static constexpr bool kTall = (BM == 512 || (BM == 256 && NW == 8)) && BN == 128;
+  static constexpr bool kSmall8 = BM == 128 && BN == 128 && NW == 8; // 64 x 32 per wavefront
   static constexpr int kWavesM = kTall ? 4 : 2;
-  static constexpr int kWavesN = kWide ? 4 : 2;
+  static constexpr int kWavesN = kWide || kSmall8 ? 4 : 2;
   static constexpr int kWaves = kWavesM * kWavesN;
 };
 
@@ -1555,10 +1557,10 @@ template <int BM, int BN> struct GemmWaves {
   static constexpr int value = BM == 256 && BN == 128 ? 8 : GemmLayout<BM, BN>::kWaves;
 };
 
-template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int STAGES = 0>
+template <int KIND, int BM, int BN, int A_MODE, bool B_KC, int STAGES = 0, int WAVES = 0>
 int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
   constexpr int NSTAGE = STAGES ? STAGES : GemmStages<BM, BN>::value;
-  constexpr int NW = GemmWaves<BM, BN>::value;
+  constexpr int NW = WAVES ? WAVES : GemmWaves<BM, BN>::value;
   constexpr int lds = GemmLds<BM, BN, NSTAGE, NW>::kBytes;
   auto kernel = gemm_kernel<KIND, BM, BN, A_MODE, B_KC, NSTAGE, NW>;
   static FhipOncePerDevice configured;
@@ -1575,15 +1577,15 @@ int launch(fhip_ctx *ctx, const GemmArgs &g, int64_t batch) {
   return 0;
 }
 
-template <int KIND, int BM, int BN>
+template <int KIND, int BM, int BN, int STAGES = 0, int WAVES = 0>
 int launch_orient(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g) {
   if (p.a_kc && p.b_kc)
-    return launch<KIND, BM, BN, A_KCONTIG, true>(ctx, g, p.batch);
+    return launch<KIND, BM, BN, A_KCONTIG, true, STAGES, WAVES>(ctx, g, p.batch);
   if (p.a_kc && !p.b_kc)
-    return launch<KIND, BM, BN, A_KCONTIG, false>(ctx, g, p.batch);
+    return launch<KIND, BM, BN, A_KCONTIG, false, STAGES, WAVES>(ctx, g, p.batch);
   if (!p.a_kc && p.b_kc)
-    return launch<KIND, BM, BN, A_MCONTIG, true>(ctx, g, p.batch);
-  return launch<KIND, BM, BN, A_MCONTIG, false>(ctx, g, p.batch);
+    return launch<KIND, BM, BN, A_MCONTIG, true, STAGES, WAVES>(ctx, g, p.batch);
+  return launch<KIND, BM, BN, A_MCONTIG, false, STAGES, WAVES>(ctx, g, p.batch);
 }
 
 template <int KIND>
@@ -1592,7 +1594,9 @@ int gemm_launch_kind(fhip_ctx *ctx, const GemmPlan &p, const GemmArgs &g) {
     return launch_orient<KIND, 256, 256>(ctx, p, g);
   if (p.bm == 256 && p.bn == 128)
     return launch_orient<KIND, 256, 128>(ctx, p, g);
-  return launch_orient<KIND, 128, 128>(ctx, p, g);
+  // (eight wavefronts of 64 x 32 in two phases, two stages: two workgroups per
+  // compute unit at 116-118 registers a lane)
+  return launch_orient<KIND, 128, 128, 2, 8>(ctx, p, g);
 }
 
 // Implicit-GEMM convolution launchers (A gathered, B = filter, K-contiguous).
@@ -1604,9 +1608,10 @@ int conv_launch_kind(fhip_ctx *ctx, int bm, int bn, const GemmArgs &g) {
     return launch<KIND, 256, 256, A_CONV, true>(ctx, g, 1);
   if (bm == 256 && bn == 128)
     return launch<KIND, 256, 128, A_CONV, true>(ctx, g, 1);
-  // two stages: two workgroups share a compute unit, and one's prologue and
-  // epilogue hide behind the other's K loop (convolutions have short K)
-  return launch<KIND, 128, 128, A_CONV, true, 2>(ctx, g, 1);
+  // eight wavefronts in two phases on two stages: two workgroups share a
+  // compute unit, and one's prologue and epilogue hide behind the other's K
+  // loop (convolutions have short K)
+  return launch<KIND, 128, 128, A_CONV, true, 2, 8>(ctx, g, 1);
 }
 
 // Halo mode: 128 x 128 tiles with three filter stages behind the slab, or

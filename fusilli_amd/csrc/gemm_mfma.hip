@@ -136,8 +136,8 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
   }
   // Tile shape and reduction split: the pair with the shortest estimated run.
   // A workgroup's time is a fixed part (prologue, epilogue: not overlapped
-  // between the rounds of eight-wavefront tiles, mostly hidden behind the
-  // second resident workgroup of the 128 x 128 tile) plus its K slices at the
+  // between the rounds of the large tiles, hidden behind the second resident
+  // workgroup of the 128 x 128 tile) plus its K slices at the
   // tile's measured pace; the tiles run in rounds of 256 (one per compute
   // unit), and a round that leaves compute units idle runs at a higher clock
   // (fitted: 0.65 + 0.35 x the busy share).  Microseconds on this chip, from
@@ -149,10 +149,10 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
   };
   auto estimate = [&](int bm, int bn, int sk) {
     const int shape = bm == 256 && bn == 256 ? 0 : (bm == 256 ? 1 : 2);
-    static const double pace16[3] = {1.36, 0.90, 0.64}, pace8f[3] = {1.275, 0.876, 0.88},
-                        pace8i[3] = {1.38, 0.95, 0.70};
-    static const double fixed16[3] = {11.0, 6.7, 7.4}, fixed8f[3] = {11.0, 5.7, 2.0},
-                        fixed8i[3] = {18.0, 9.0, 8.0};
+    static const double pace16[3] = {1.36, 0.90, 0.625}, pace8f[3] = {1.275, 0.876, 0.7125},
+                        pace8i[3] = {1.38, 0.95, 0.66};
+    static const double fixed16[3] = {11.0, 6.7, 6.4}, fixed8f[3] = {11.0, 5.7, 3.3},
+                        fixed8i[3] = {18.0, 9.0, 7.7};
     const double pace = (k16 ? pace16 : p.kind == GK_I8 ? pace8i : pace8f)[shape];
     const double fixed = (k16 ? fixed16 : p.kind == GK_I8 ? fixed8i : fixed8f)[shape];
     const double t = tiles(bm, bn) * sk;
@@ -160,7 +160,9 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
     const double rounds = full + (rest > 0 ? 1 : 0);
     const double work = full + (rest > 0 ? 0.65 + 0.35 * rest / 256.0 : 0.0);
     double us = (double)(slices / sk) * pace * work +
-                (shape == 2 ? fixed + 3.0 * (rounds - 1) : fixed * rounds);
+                (shape != 2 ? fixed * rounds
+                 : p.kind == GK_I8 ? fixed * (1.0 + 0.5 * (rounds - 1)) // (int32 stores)
+                                   : fixed);
     if (sk > 1) // the parts' f32 stores and the kernel that adds them (~5 TB/s each way)
       us += 2.0 * sk * (double)p.M * (double)p.N * 4.0 / 5.0e6 + 2.5;
     return us;
@@ -314,8 +316,8 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     o.stride[2] = s.stride[r - 1];
   }
   static const char *const kKindName[] = {"bf16", "f16", "i8", "fp8e4m3", "fp8e5m2"};
-  fhip_note_kernel(ctx, "gemm_mfma %s %dx%d waves=%d split=%d", kKindName[p.kind], p.bm, p.bn,
-                   p.bm == 128 ? 4 : 8, p.ksplit);
+  fhip_note_kernel(ctx, "gemm_mfma %s %dx%d waves=8 split=%d", kKindName[p.kind], p.bm, p.bn,
+                   p.ksplit);
   auto launch = [&]() {
     switch (p.kind) {
     case GK_BF16:
