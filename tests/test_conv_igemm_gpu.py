@@ -381,6 +381,44 @@ def test_conv_igemm_headline_shape(ctx):
         assert np.array_equal(lg[img], lg[0]), f"image {img} differs from image 0"
 
 
+LARGE_128_CASES = [
+    # 784 tiles of 128 x 128: 3x3 (halo-eligible), 1x1 reduction, 1x1 stride 2
+    dict(x=[32, 128, 56, 56], w=[128, 128, 3, 3], pad=[1, 1], s=[1, 1]),
+    dict(x=[32, 256, 56, 56], w=[64, 256, 1, 1], pad=[0, 0], s=[1, 1]),
+    dict(x=[32, 64, 112, 112], w=[64, 64, 1, 1], pad=[0, 0], s=[2, 2]),
+]
+
+
+@pytest.mark.parametrize("case", LARGE_128_CASES)
+def test_conv_many_128_wide_tiles_take_the_gather_tile(ctx, case):
+    """The 56 x 56 layers with up to 128 output channels: 512 or more tiles of
+    128 x 128 run on the gather kernel's eight-wavefront tile, also where the
+    halo kernel could take them.  All-ones operands have closed-form answers at
+    every output; random data is checked against the oracle on the first and
+    the last image."""
+    xd, wd, pad, st = case["x"], case["w"], case["pad"], case["s"]
+    dil = [1, 1]
+    ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
+    ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
+    out = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16)
+    assert ctx.last_kernel().startswith("conv_igemm gather 128x128 split=1"), ctx.last_kernel()
+    lg = out.logical()
+    if wd[2] == 3:
+        taps = np.full(xd[2], 3.0); taps[[0, -1]] = 2.0
+        expect = wd[1] * taps[:, None] * taps[None, :]
+    else:
+        expect = np.full(lg.shape[2:], float(wd[1]))
+    assert np.array_equal(lg, np.broadcast_to(expect, lg.shape))
+
+    x = cl(xd, 47, 0, capi.BFLOAT16)
+    w = cl(wd, 47, 1, capi.BFLOAT16, std=0.05)
+    out = run(ctx, x, w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16)
+    lg, xl = out.logical(), x.logical()
+    for img in (0, xd[0] - 1):
+        ref = oracle.conv_fprop(xl[img:img + 1], w.logical(), pad, st, dil)
+        assert_close(lg[img:img + 1], ref, capi.BFLOAT16, f"{case} image {img}")
+
+
 @pytest.mark.parametrize("shape", ["groups4", "depthwise"])
 def test_conv_grouped_benchmark_shapes(ctx, shape):
     """The two grouped lines of the benchmark at full size (N32 56x56, 3x3,
