@@ -219,10 +219,9 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
     };
     if (tiles(256, 256) < 192)
       p.bn = 128;
-    // (256 x 128 runs on eight wavefronts in two phases at about twice the
-    // rate of the four in-order wavefronts of a 128 x 128 tile)
-    const int64_t small = tiles(128, 128) < 256 ? tiles(128, 128) : 256;
-    if (p.bn == 128 && tiles(256, 128) < 192 && 2 * tiles(256, 128) < small)
+    // (both run on eight wavefronts in two phases at the same rate per
+    // output; the 128 x 128 tiles share a compute unit in pairs)
+    if (p.bn == 128 && tiles(256, 128) < 192)
       p.bm = 128;
   }
   const FhipKnobs &knobs = fhip_knobs();
@@ -277,6 +276,12 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
     if (want < 0 && bm == 128 && p.bm == 128 && p.bn == 128 &&
         ((p.M + 127) / 128) * ((p.N + 127) / 128) * p.groups >= 512)
       bm = 0;
+    // a single tap has nothing to reuse in the slab (C128 -> K512 at 28 x 28:
+    // halo 19.6, gather 12.9 us; C256 -> K1024 at 14 x 14: 13.9, 11.4 us);
+    // with one K slice in all the halo kernel's shorter set-up still wins
+    // (C64 -> K256 at 56 x 56: 17.7 against 19.3 us)
+    if (want < 0 && reach == 0 && g.slices_per_tap >= 2)
+      bm = 0;
     if (bm) {
       p.halo = true;
       p.bm = bm;
@@ -301,8 +306,10 @@ ConvPlan make_plan(const fhip_conv_desc *d, const fhip_conv_desc *orig = nullptr
     // workgroups of 18 slices and the sum 27 us)
     const int64_t tiles = ((p.M + p.bm - 1) / p.bm) * ((p.N + p.bn - 1) / p.bn);
     const int64_t slices = p.K * elem / kTileKBytes;
-    if (tiles < 128 && slices >= 16) {
-      int64_t want = 256 / tiles;
+    // (128 x 128 tiles: two workgroups per compute unit, 512 slots)
+    const int64_t slots = p.bm == 128 && p.bn == 128 ? 512 : 256;
+    if (tiles < slots / 2 && slices >= 16) {
+      int64_t want = slots / tiles;
       want = want > 8 ? 8 : want;
       for (int64_t sk = want; sk >= 2; --sk)
         if (slices % sk == 0 && slices / sk >= 6) {
