@@ -162,7 +162,9 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
     double us = (double)(slices / sk) * pace * work +
                 (shape != 2 ? fixed * rounds
                  : p.kind == GK_I8 ? fixed * (1.0 + 0.5 * (rounds - 1)) // (int32 stores)
-                                   : fixed);
+                                   // (a partner with under 4.25 us of K slices does not cover it:
+                                   // fp8 4096 x 4096 x 512 18.9 us against 16.1 on 256 x 256)
+                                   : fixed + (rounds - 1) * fmax(0.0, 4.25 - (double)(slices / sk) * pace));
     if (sk > 1) // the parts' f32 stores and the kernel that adds them (~5 TB/s each way)
       us += 2.0 * sk * (double)p.M * (double)p.N * 4.0 / 5.0e6 + 2.5;
     return us;
