@@ -2,7 +2,8 @@
 // kind in gemm_<kind>.hip.
 //
 // Data path of one workgroup (4 wavefronts as 2 x 2, or 8 as 2 x 4 / 4 x 2, each
-// owning a block of 32x32 MFMA tiles):
+// owning a block of 32x32 MFMA tiles; the eight-wavefront kernels compute them
+// as 16x16 MFMA tiles of twice the K):
 //   * 128-byte K slices of A and B go from global memory straight into LDS
 //     with the LDS-DMA form of the buffer load (no staging registers), into a
 //     ring of NSTAGE stages ahead of the MFMAs; the convolution modes gather A
