@@ -170,7 +170,7 @@ GemmPlan make_plan(const fhip_matmul_desc *d, bool allow_split = true) {
     return us;
   };
   const int forced = fhip_knobs().gemm_split; // (1: never split)
-  const bool may_split = p.batch == 1 && p.kind != GK_I8 && p.N % 4 == 0 && p.o_sn == 1 &&
+  const bool may_split = p.batch == 1 && p.N % 4 == 0 && p.o_sn == 1 &&
                          allow_split && forced != 1;
   double best = 0;
   p.bm = p.bn = 0;
@@ -223,6 +223,7 @@ struct GemmSumArgs {
   int64_t mn4, o_sm;   // mn4: M * N / 4
   int32_t N, pitch, parts, rank;
   int32_t c_dt, o_dt;
+  int32_t ints;    // the parts are int32 sums (int8 operands): added exactly, no epilogue
   DevEpilogue epi; // strides over the matmul's result dims
 };
 
@@ -236,6 +237,16 @@ __global__ void gemm_splitk_sum_kernel(GemmSumArgs a) {
   const int64_t m = e / a.N;
   const int64_t n0 = e - m * a.N;
   const float *src = a.part + m * a.pitch + n0;
+  if (a.ints) {
+    uint4 sum = *(const uint4 *)src; // (unsigned: wraps like the kernel's int32 accumulators)
+    for (int z = 1; z < a.parts; ++z) {
+      const uint4 v = *(const uint4 *)(src + (int64_t)z * a.part_stride);
+      sum.x += v.x, sum.y += v.y, sum.z += v.z, sum.w += v.w;
+    }
+    uint32_t *o = (uint32_t *)a.out + m * a.o_sm + n0;
+    o[0] = sum.x, o[1] = sum.y, o[2] = sum.z, o[3] = sum.w;
+    return;
+  }
   float4 acc = *(const float4 *)src;
   for (int z = 1; z < a.parts; ++z) {
     const float4 v = *(const float4 *)(src + (int64_t)z * a.part_stride);
@@ -335,8 +346,8 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     }
   };
   if (p.ksplit > 1) {
-    // every part writes plain f32 sums; rounding and the fused operations
-    // follow in the kernel that adds them
+    // every part writes plain f32 (int8 operands: int32) sums; rounding and
+    // the fused operations follow in the kernel that adds them
     // (rows of the parts are padded to whole column tiles and the tiles are
     // stored whole: every cache line of the parts is written by one workgroup,
     // with full 16-byte stores)
@@ -345,7 +356,7 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     if (fhip_ctx_scratch(ctx, (size_t)p.ksplit * (size_t)(p.M * pitch) * sizeof(float), &sp) != 0)
       return 1;
     g.out = (char *)sp;
-    g.c_dt = g.o_dt = FHIP_FLOAT;
+    g.c_dt = g.o_dt = p.kind == GK_I8 ? FHIP_INT32 : FHIP_FLOAT;
     g.o_sm = pitch;
     g.n_store = pitch;
     g.o_sn = 1;
@@ -371,6 +382,7 @@ int fhip_fast_matmul_outer(fhip_ctx *ctx, const fhip_matmul_desc *d,
     sa.rank = r;
     sa.c_dt = d->c.dtype;
     sa.o_dt = d->out.dtype;
+    sa.ints = p.kind == GK_I8;
     sa.epi = epi;
     hipLaunchKernelGGL(gemm_splitk_sum_kernel, dim3((unsigned)((sa.mn4 + 255) / 256)),
                        dim3(256), 0, ctx->stream, sa);

@@ -125,6 +125,20 @@ def test_gemm_split_reduction(ctx, dtype, ta, tb, m, n, k):
     assert_close(out.logical(), ref_matmul(a, b), capi.FLOAT, rtol=1e-4)
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 8192), (304, 512, 4096), (512, 260, 16384)])
+def test_gemm_int8_split_reduction_bit_exact(ctx, ta, tb, m, n, k):
+    # int8 operands: the parts are int32 sums and their sum is exact
+    a = make_operand(75, 0, m, k, capi.INT8, ta)
+    b = make_operand(75, 1, k, n, capi.INT8, tb)
+    fast = tb or n % 16 == 0
+    out = run(ctx, a, b, capi.INT32, expect_fast=fast)
+    if fast:
+        name = ctx.last_kernel()
+        assert name.startswith("gemm_mfma i8") and "split=" in name and not name.endswith("split=1"), name
+    assert np.array_equal(out.logical(), ref_matmul(a, b))
+
+
 def test_gemm_split_reduction_benchmark_shape(ctx):
     # bf16 1024 x 1024 x 8192 -> bf16, as the benchmark line runs it
     a = make_operand(74, 0, 1024, 8192, capi.BFLOAT16, False)
