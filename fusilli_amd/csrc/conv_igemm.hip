@@ -553,6 +553,43 @@ int fhip_fast_conv(fhip_ctx *ctx, const fhip_conv_desc *d, const void *x,
     o.stride[1] = sm;          // per-pixel step (0 for channel vectors)
     o.stride[2] = s.stride[1]; // per-channel step
   }
+  // A single tap at unit stride without padding is the matrix product
+  // X[pixels][C] . W[K][C]^T of dense operands: the GEMM entry takes them as
+  // they lie (no pixel decode per K slice, its own tile and split choice).
+  // N32: C1024 -> K256 at 14 x 14 20.5 -> 13.4 us, C512 -> K128 at 28 x 28
+  // 12.5 -> 9.8, C256 -> K128 at 56 x 56 20.1 -> 17.9, C64 -> K256 17.6 -> 16.7.
+  {
+    const ConvGeom &cg = p.geom;
+    const FhipKnobs &knobs = fhip_knobs();
+    const int64_t elem = fhip_dtype_size(d->x.dtype);
+    if (allow_scratch && !res.padded && p.groups == 1 && cg.R == 1 && cg.S == 1 &&
+        cg.str_h == 1 && cg.str_w == 1 && cg.pad_h == 0 && cg.pad_w == 0 && cg.P == cg.H &&
+        cg.Q == cg.W && cg.x_pitch == cg.C * elem && p.channels_out == p.N &&
+        knobs.conv_tile_bm == 0 && knobs.conv_halo < 0) {
+      fhip_matmul_desc md{};
+      auto mat = [](fhip_tensor_desc &t, int64_t rows, int64_t cols, int64_t s_row, int64_t s_col,
+                    int dt) {
+        t.rank = 3;
+        t.dim[0] = 1, t.dim[1] = rows, t.dim[2] = cols;
+        t.stride[0] = rows * cols, t.stride[1] = s_row, t.stride[2] = s_col;
+        t.dtype = dt;
+      };
+      mat(md.a, p.M, p.K, p.K, 1, d->x.dtype);
+      mat(md.b, p.K, p.N, 1, p.K, d->w.dtype); // filter rows are B's columns
+      mat(md.c, p.M, p.N, p.N, 1, d->y.dtype);
+      mat(md.out, p.M, p.N, p.N, 1, d->out.dtype);
+      md.out_dtype = d->out.dtype;
+      md.epilogue = d->epilogue;
+      if (fhip_fast_matmul_applicable(&md)) {
+        if (fhip_fast_matmul(ctx, &md, x, w, g.epi, out) != 0)
+          return 1;
+        char inner[sizeof(ctx->last_kernel)];
+        std::snprintf(inner, sizeof(inner), "%s", ctx->last_kernel);
+        fhip_note_kernel(ctx, "conv_igemm as %s", inner);
+        return 0;
+      }
+    }
+  }
   if (p.ksplit > 1) {
     // every part writes plain f32 sums; rounding and the fused operations
     // follow in the kernel that adds them

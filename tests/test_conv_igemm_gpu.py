@@ -163,6 +163,39 @@ def test_conv_same_geometry_halo_and_gather(ctx, case, halo, dtype, knobs):
     assert_close(out.logical(), ref, capi.FLOAT, f"halo={halo} {case}", rtol=1e-4)
 
 
+@pytest.mark.parametrize("xd,wd,split", [
+    ([2, 128, 10, 12], [136, 128, 1, 1], False),   # ragged columns, 240 pixels
+    ([4, 2048, 7, 7], [256, 2048, 1, 1], True),    # long reduction: cut into parts
+    ([3, 192, 60], [128, 192, 1], False),          # 1-D
+])
+def test_conv_single_tap_as_matrix_product_fused_operands(ctx, xd, wd, split):
+    """1 x 1 filters at unit stride are handed to the GEMM entry; the fused
+    per-channel and per-pixel operands keep their conv layouts (bias[K],
+    residual[N, K, ...] channels-last), also through the split reduction."""
+    sp = len(xd) - 2
+    pad, one = [0] * sp, [1] * sp
+    x = cl(xd, 48, 0, capi.BFLOAT16)
+    w = cl(wd, 48, 1, capi.BFLOAT16, std=0.05)
+    yd = oracle.conv_output_dims(xd, wd, pad, one, one)
+    bd = [1, wd[0]] + one
+    bias = HT.from_logical(rand(48, 2, bd), capi.BFLOAT16, oracle.channels_last_strides(bd))
+    res = cl(yd, 48, 3, capi.BFLOAT16)
+    epi = [capi.epilogue_op(capi.PW["ADD"], capi.FLOAT, operand_index=0, operand=bias.desc()),
+           capi.epilogue_op(capi.PW["RELU_FWD"], capi.FLOAT),
+           capi.epilogue_op(capi.PW["ADD"], capi.BFLOAT16, operand_index=1, operand=res.desc())]
+    out = run(ctx, x, w, pad, one, one, capi.FLOAT, out_dtype=capi.BFLOAT16, epilogue=epi,
+              epi_tensors=[bias, res])
+    name = ctx.last_kernel()
+    assert name.startswith("conv_igemm as gemm_mfma bf16"), name
+    assert name.endswith("split=1") != split, name
+    ref = oracle.conv_fprop(x.logical(), w.logical(), pad, one, one)
+    ref = np.maximum(ref + bias.logical(), 0.0) + res.logical()
+    assert_close(out.logical(), ref, capi.BFLOAT16)
+    out = run(ctx, x, w, pad, one, one, capi.FLOAT)
+    assert_close(out.logical(), oracle.conv_fprop(x.logical(), w.logical(), pad, one, one),
+                 capi.FLOAT, rtol=1e-4)
+
+
 def test_conv_igemm_bias_relu_residual(ctx):
     # conv -> +bias[K] -> relu -> +residual[N,K,P,Q] (channels-last) -> bf16
     xd, wd = [2, 64, 10, 12], [96, 64, 3, 3]
@@ -386,6 +419,8 @@ LARGE_128_CASES = [
     dict(x=[32, 128, 56, 56], w=[128, 128, 3, 3], pad=[1, 1], s=[1, 1]),
     dict(x=[32, 256, 56, 56], w=[64, 256, 1, 1], pad=[0, 0], s=[1, 1]),
     dict(x=[32, 64, 112, 112], w=[64, 64, 1, 1], pad=[0, 0], s=[2, 2]),
+    # 1x1 at unit stride with 128 output channels: a plain matrix product
+    dict(x=[32, 256, 56, 56], w=[128, 256, 1, 1], pad=[0, 0], s=[1, 1]),
 ]
 
 
@@ -393,7 +428,7 @@ LARGE_128_CASES = [
 def test_conv_many_128_wide_tiles_take_the_gather_tile(ctx, case):
     """The 56 x 56 layers with up to 128 output channels: 512 or more tiles of
     128 x 128 run on the gather kernel's eight-wavefront tile, also where the
-    halo kernel could take them.  All-ones operands have closed-form answers at
+    halo kernel could take them (1 x 1 filters at unit stride: the GEMM entry).  All-ones operands have closed-form answers at
     every output; random data is checked against the oracle on the first and
     the last image."""
     xd, wd, pad, st = case["x"], case["w"], case["pad"], case["s"]
@@ -401,7 +436,10 @@ def test_conv_many_128_wide_tiles_take_the_gather_tile(ctx, case):
     ones_x = HT.from_logical(np.ones(xd), capi.BFLOAT16, oracle.channels_last_strides(xd))
     ones_w = HT.from_logical(np.ones(wd), capi.BFLOAT16, oracle.channels_last_strides(wd))
     out = run(ctx, ones_x, ones_w, pad, st, dil, capi.FLOAT, out_dtype=capi.BFLOAT16)
-    assert ctx.last_kernel().startswith("conv_igemm gather 128x128 split=1"), ctx.last_kernel()
+    # (a single tap at unit stride is handed to the GEMM entry as it lies)
+    want = "conv_igemm as gemm_mfma bf16" if wd[2] == 1 and st == [1, 1] and wd[0] >= 128 \
+        else "conv_igemm gather 128x128 split=1"
+    assert ctx.last_kernel().startswith(want), ctx.last_kernel()
     lg = out.logical()
     if wd[2] == 3:
         taps = np.full(xd[2], 3.0); taps[[0, -1]] = 2.0
