@@ -292,8 +292,11 @@ int fhip_conv_dgrad(fhip_ctx *ctx, const fhip_conv_desc *d, const void *dy,
  * fhip_conv_dgrad_workspace_size exceeds that fail with a message.  It plans
  * without the context's growable scratch: descriptors that fhip_conv_dgrad
  * runs on zero-padded channel copies or with a split reduction take the
- * direct (slower) kernels here, and their results may differ from
- * fhip_conv_dgrad's in the last bit (another summation order); every other
+ * direct (slower) kernels here, 1 x 1 filters at unit stride (which
+ * fhip_conv_dgrad hands to the matrix-product kernels, whose planner may use
+ * the scratch) stay on the convolution kernel, and the results of both may
+ * differ from fhip_conv_dgrad's in the last bit (another summation order);
+ * every other
  * descriptor runs the same kernel with bit-identical results.  All calls on
  * one GPU share the array: calls that overlap on one GPU (two streams, two
  * contexts) race. */
